@@ -1,0 +1,110 @@
+/* C ABI of libmi355x_qlinear.so — the gfx950 quantized-linear kernels.
+ *
+ * One function per operator of the reference's custom-kernel packages
+ * (vllm/custom-esimd-kernels-vllm = V/, sglang/custom-esimd-kernels = S/).  The
+ * reference binds its kernels to torch.ops with ATen tensors; the functions here
+ * take what those launchers extract from the tensors: raw device pointers,
+ * sizes, and the stream to enqueue on.  Conventions shared by all of them:
+ *
+ *   - every pointer is device memory; outputs are pre-allocated by the caller;
+ *   - the call enqueues on `stream` (a hipStream_t, 0 = the null stream) and
+ *     returns without synchronising; nothing is allocated or freed;
+ *   - tensors are dense row-major;
+ *   - act_dtype: 0 = fp16, 1 = bf16 (inputs and outputs share it);
+ *   - return value: 0 on success, MI_ERR_ARG (-1) for a null pointer or bad
+ *     enum, MI_ERR_SHAPE (-2) for a shape the kernels do not cover,
+ *     MI_ERR_LAUNCH (-3) if the launch itself failed.
+ */
+#ifndef MI355X_QLINEAR_H_
+#define MI355X_QLINEAR_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_DT_F16 0
+#define MI_DT_BF16 1
+
+/* ---- FP8 (E4M3) weight-only, per-output-channel scale ---------------------
+ * out[M,N] = (x[M,K] @ e4m3(w[N,K])^T) * scale[n].   K % 32 == 0.
+ * Replaces esimd_gemv_fp8_pern (V/csrc/xpu/esimd_kernel.sycl:39-48,
+ * V/csrc/xpu/esimd_kernels/fp8_GEMV_v2.h:123-162), extended to any M and to
+ * fp32 scales (scale_is_f16 = 0).  E4M3 decode is exact (no subnormal flush).
+ * The _multi form runs up to 3 weight matrices that share x in one launch and
+ * replaces esimd_gemv_fp8_pern_fused2/3 (V/csrc/xpu/torch_extension.cc:13-25). */
+int mi_gemm_fp8_pern(const void* x, const void* w, const void* scale, void* out, int M, int N, int K,
+                     int act_dtype, int scale_is_f16, void* stream);
+int mi_gemm_fp8_pern_multi(const void* x, int nmat, const void* const* w, const void* const* scale,
+                           void* const* out, const int* N, int M, int K, int act_dtype,
+                           int scale_is_f16, void* stream);
+
+/* ---- FP8 weight-only, per-tensor scale (fp32 scalar read from device memory)
+ * Replaces esimd_gemv_fp8_pert / _bmg / _fused2/3 and esimd_gemm_fp8_pert
+ * (V/csrc/xpu/esimd_kernel.sycl:88-98, :654-670; esimd_kernel_gemm.sycl:32-49). */
+int mi_gemm_fp8_pert(const void* x, const void* w, const float* scale, void* out, int M, int N, int K,
+                     int act_dtype, void* stream);
+int mi_gemm_fp8_pert_multi(const void* x, int nmat, const void* const* w, const float* const* scale,
+                           void* const* out, const int* N, int M, int K, int act_dtype, void* stream);
+
+/* ---- FP8 weight-only, 128x128 block scale (w8a16) --------------------------
+ * out = x @ (e4m3(w) * S[n/128, k/128])^T, S fp32 [ceil(N/128), K/128], K % 128 == 0.
+ * Replaces esimd_gemm_fp8_blockscale and esimd_gemv_fp8_blockscale_fused2
+ * (V/csrc/xpu/esimd_kernel_gemm.sycl:97-139,
+ * V/csrc/xpu/esimd_kernels/fp8_GEMM_blockscale.h:197-223). */
+int mi_gemm_fp8_blockscale(const void* x, const void* w, const float* scale, void* out, int M, int N,
+                           int K, int act_dtype, void* stream);
+int mi_gemm_fp8_blockscale_multi(const void* x, int nmat, const void* const* w,
+                                 const float* const* scale, void* const* out, const int* N, int M,
+                                 int K, int act_dtype, void* stream);
+
+/* ---- INT4, group 128, weight-streaming (decode) ----------------------------
+ * w [N, K/2] uint8 (== [N, K/8] int32), low nibble = even k, stored value =
+ * signed + 8; scale [N, K/128] fp16; zp [N, K/128] uint8 in 0..15 or NULL for
+ * the implicit zero-point 8.  out = x @ ((nib - zp) * scale)^T.  K % 128 == 0.
+ * Replaces esimd_gemv_int4 / esimd_gemv_int4_fused2
+ * (V/csrc/xpu/esimd_kernel.sycl:200-230,
+ * V/csrc/xpu/esimd_kernels/int4_GEMV.h:267-304, :414-462) and, for M <= 64,
+ * esimd_gemm_int4_pgrp (esimd_kernel_gemm.sycl:55-91).  The zero-point operand
+ * has no counterpart in the reference's kernels. */
+int mi_gemv_int4(const void* x, const void* w, const void* scale, const void* zp, void* out, int M,
+                 int N, int K, int act_dtype, void* stream);
+int mi_gemv_int4_multi(const void* x, int nmat, const void* const* w, const void* const* scale,
+                       const void* const* zp, void* const* out, const int* N, int M, int K,
+                       int act_dtype, void* stream);
+
+/* ---- GGUF Q4_K on the repacked representation, fp16 -------------------------
+ * ql [N, K/2] uint8 interleaved nibbles, scale/qmin [N, K/32] fp16;
+ * w = fp16(fp16(nib * scale) - qmin);  out = x @ w^T.  K % 32 == 0.
+ * Replaces esimd_gemv_q4_k (S/csrc/xpu/esimd_kernel.sycl:224-239,
+ * S/csrc/xpu/esimd_kernels/q4_k_GEMV.h:110-132), extended to any M. */
+int mi_gemv_q4k(const void* x, const void* ql, const void* scale, const void* qmin, void* out, int M,
+                int N, int K, void* stream);
+
+/* ---- dequant-only entries (bit-exactness checks, load-time dense copies) ----
+ * They share the in-register dequant routines of the fused kernels.
+ * mi_dequant_int4: out [N,K] fp16/bf16 = rne((nib - zp) * scale), the value
+ *   V/tests/test_gemv_int4.py:172-212 defines (int4_dequantize_ref).
+ * mi_dequant_fp8: out [N,K] fp32 = e4m3(w) * scale; scale_mode 0 = per-channel
+ *   fp32 [N], 1 = per-channel fp16 [N], 2 = per-tensor fp32 [1], 3 = 128x128
+ *   block fp32 (V/tests/test_fp8_blockscale_gemm.py:31-36, dequant_weight).
+ * mi_decode_e4m3: count codes (multiple of 8) -> fp16/bf16, exact for all 254
+ *   finite codes (V/csrc/xpu/esimd_kernels/fp8_GEMM_blockscale.h:40-49).
+ * mi_dequant_q4k: repacked Q4_K -> dense fp16, two fp16 roundings
+ *   (_xpu_dequant_q4_k, sglang/patches/sglang_for_multi_arc.patch:2576-2587).
+ * mi_q4k_repack: raw GGUF block_q4_K rows [N, K/256*144] -> ql [N,K/2] u8,
+ *   scale/qmin [N,K/32] fp16 (_xpu_repack_q4_k, same patch :2527-2573). */
+int mi_dequant_int4(const void* w, const void* scale, const void* zp, void* out, int N, int K,
+                    int out_dtype, void* stream);
+int mi_dequant_fp8(const void* w, const void* scale, int scale_mode, float* out, int N, int K,
+                   void* stream);
+int mi_decode_e4m3(const void* codes, void* out, long long count, int out_dtype, void* stream);
+int mi_dequant_q4k(const void* ql, const void* scale, const void* qmin, void* out, int N, int K,
+                   void* stream);
+int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_QLINEAR_H_ */

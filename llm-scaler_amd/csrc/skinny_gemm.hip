@@ -1,0 +1,324 @@
+// Weight-streaming ("skinny") quantized GEMV / small-M GEMM for gfx950.
+//
+// Regime: M <= 64 rows of activations against an [N, K] quantized weight.  The
+// weight is read exactly once at full HBM rate; everything else (activations,
+// scales) comes out of L2.  One workgroup owns 16 output columns (weight rows)
+// and all of K; its NW wavefronts interleave 128-wide K granules so that the
+// workgroup as a whole walks each weight row front to back, and every lane
+// issues 128-bit loads.  Weights are dequantized in registers to the activation
+// type and fed to v_mfma_f32_16x16x32_{f16,bf16} with the activations as the A
+// operand (M padded to 16 inside the matrix core — free while HBM-bound).  The
+// NW partial accumulators are reduced through LDS.
+//
+// Lane mapping inside one granule (128 k): lane = (j = lane % 16, g = lane / 16)
+// holds the 32 consecutive k  [128 gi + 32 g, +32)  of weight row n0 + j and of
+// activation row j.  MFMA i (0..3) consumes the i-th 8-k slice of both.
+#include "qlinear_common.hpp"
+#include "../../include/mi355x_qlinear.h"
+
+namespace qlin {
+
+constexpr int kMaxMat = 3;
+
+struct SkinnyArgs {
+  const void* x;
+  const void* w[kMaxMat];
+  const void* s[kMaxMat];     // scales (format specific)
+  const void* z[kMaxMat];     // int4: zero-points (may be null); q4k: mins
+  void* out[kMaxMat];
+  int N[kMaxMat];
+  int tiles[kMaxMat];         // 16-row tiles per matrix
+  int nmat;
+  int M, K;
+  int scale_f16;              // fp8 per-channel: scale is fp16 instead of fp32
+};
+
+enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
+
+// ---------------------------------------------------------------- kernel
+template <class Act, int FMT, int SC, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
+  using V8 = typename Act::v8;
+  using Elem = typename Act::elem;
+  constexpr bool kIsFp8 = (FMT == 0);
+  constexpr bool kIsInt4 = (FMT == 1);
+  constexpr bool kIsQ4K = (FMT == 2);
+  constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
+
+  __shared__ f32x4 red[NW - 1][MT][64];
+
+  int tile = blockIdx.x;
+  int mat = 0;
+#pragma unroll
+  for (int i = 0; i + 1 < kMaxMat; ++i) {
+    if (mat == i && i + 1 < a.nmat && tile >= a.tiles[i]) { tile -= a.tiles[i]; mat = i + 1; }
+  }
+  const int N = a.N[mat];
+  const int K = a.K, M = a.M;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int n0 = tile * 16;
+  const int n = n0 + j;
+  const int nc = n < N ? n : N - 1;                  // clamped row for side loads
+  const int G = (K + 127) >> 7;
+
+  const uint32_t wrow = kIsFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+
+  const _Float16* s16 = (const _Float16*)a.s[mat];
+  const float* s32 = (const float*)a.s[mat];
+  const uint8_t* zp = (const uint8_t*)a.z[mat];
+  const _Float16* qmin = (const _Float16*)a.z[mat];
+  const int Kg = K >> 7;                             // int4 groups per row
+  const int Kb32 = K >> 5;                           // q4k sub-blocks per row
+  const int Kb = G;                                  // fp8 block columns
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int UN = MT == 1 ? 4 : (MT == 2 ? 2 : 1);    // granules in flight per wave
+  for (int gbase = wave; gbase < G; gbase += NW * UN) {
+    u32x4 wa[UN], wb[UN];
+    u32x4 xa[UN][MT][4];
+    float sc[UN];                                    // int4 / q4k scale, block scale
+    float zz[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int gi = gbase + u * NW;
+      const int kl = gi * 128 + g * 32;
+      const bool ok = (gi < G) && (kl < K);
+      const uint32_t woff = ok ? (uint32_t)n * wrow + (kIsFp8 ? (uint32_t)kl : ((uint32_t)kl >> 1)) : kOOB;
+      wa[u] = buf_load16(wr, woff);
+      if constexpr (kIsFp8) wb[u] = buf_load16(wr, ok ? woff + 16 : kOOB);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
+      }
+      const int gic = gi < G ? gi : G - 1;
+      if constexpr (kIsInt4) {
+        sc[u] = (float)s16[(size_t)nc * Kg + gic];
+        zz[u] = zp ? (float)zp[(size_t)nc * Kg + gic] : 8.0f;
+      } else if constexpr (kIsQ4K) {
+        const int sb = gic * 4 + g;
+        const int sbc = sb < Kb32 ? sb : Kb32 - 1;
+        sc[u] = (float)s16[(size_t)nc * Kb32 + sbc];
+        zz[u] = (float)qmin[(size_t)nc * Kb32 + sbc];
+      } else if constexpr (kBlock) {
+        sc[u] = s32[(size_t)(n0 >> 7) * Kb + gic];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int gi = gbase + u * NW;
+      if (gi < G) {                                  // wave-uniform
+        V8 b[4];
+        if constexpr (kIsFp8) {
+          b[0] = fp8x8_to_act<Act>(wa[u][0], wa[u][1]);
+          b[1] = fp8x8_to_act<Act>(wa[u][2], wa[u][3]);
+          b[2] = fp8x8_to_act<Act>(wb[u][0], wb[u][1]);
+          b[3] = fp8x8_to_act<Act>(wb[u][2], wb[u][3]);
+        } else if constexpr (kIsInt4) {
+          if constexpr (Act::dt == DT_F16) {
+            const _Float16 s = (_Float16)sc[u];
+            const _Float16 z = (_Float16)(1024.0f + zz[u]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[u][i], s, z);
+          } else {
+            const float s = sc[u];
+            const float nzs = -zz[u] * s;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[u][i], s, nzs);
+          }
+        } else {
+          if constexpr (Act::dt == DT_F16) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = q4kx8_to_f16(wa[u][i], (_Float16)sc[u], (_Float16)zz[u]);
+          }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          if constexpr (kBlock) {
+            f32x4 t = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], t);
+            acc[mt] += t * sc[u];
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[mt] = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], acc[mt]);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- reduce the NW partial tiles through LDS ----
+  if (wave > 0) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[wave - 1][mt][lane] = acc[mt];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 0; w < NW - 1; ++w)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] += red[w][mt][lane];
+
+  // D layout: lane holds output column n0 + j, rows mt*16 + 4 g + v.
+  float os = 1.0f;
+  if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[nc] : s32[nc];
+  if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
+  if (n < N) {
+    Elem* out = (Elem*)a.out[mat];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = mt * 16 + g * 4 + v;
+        if (m < M) out[(size_t)m * N + n] = Act::from_f32(acc[mt][v] * os);
+      }
+  }
+}
+
+template <class Act, int FMT, int SC>
+static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
+  int tiles = 0;
+  for (int i = 0; i < a.nmat; ++i) tiles += a.tiles[i];
+  if (tiles == 0 || a.M == 0) return MI_OK;
+  constexpr int NW = 8;
+  dim3 grid(tiles), block(NW * 64);
+  if (a.M <= 16)
+    hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, 1, NW>), grid, block, 0, st, a);
+  else if (a.M <= 32)
+    hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, 2, NW>), grid, block, 0, st, a);
+  else
+    hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, 4, NW>), grid, block, 0, st, a);
+  return launch_status();
+}
+
+// Runs M in chunks of 64 rows (the skinny kernel's limit); each chunk streams
+// the weight once, so this is meant for decode-sized M.
+template <int FMT, int SC>
+static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (FMT == 2 && act_dtype != DT_F16) return MI_ERR_ARG;
+  if (a.M < 0 || a.K <= 0) return MI_ERR_SHAPE;
+  if (FMT == 0 && (a.K % 32)) return MI_ERR_SHAPE;
+  if (FMT == 1 && (a.K % 128)) return MI_ERR_SHAPE;
+  if (FMT == 2 && (a.K % 32)) return MI_ERR_SHAPE;
+  for (int i = 0; i < a.nmat; ++i) {
+    if (a.N[i] < 0 || !a.w[i] || !a.out[i]) return MI_ERR_ARG;
+    if ((uint64_t)a.N[i] * (uint64_t)a.K >= (1ull << 31)) return MI_ERR_SHAPE;
+    a.tiles[i] = (a.N[i] + 15) / 16;
+  }
+  if (!a.x) return MI_ERR_ARG;
+  const int M = a.M;
+  const size_t esz = 2;
+  for (int m0 = 0; m0 < M; m0 += 64) {
+    SkinnyArgs c = a;
+    c.M = (M - m0) < 64 ? (M - m0) : 64;
+    c.x = (const char*)a.x + (size_t)m0 * a.K * esz;
+    for (int i = 0; i < a.nmat; ++i) c.out[i] = (char*)a.out[i] + (size_t)m0 * a.N[i] * esz;
+    int rc;
+    if (FMT == 2)
+      rc = launch_mt<ActF16, FMT, SC>(c, st);
+    else
+      rc = act_dtype == DT_F16 ? launch_mt<ActF16, FMT, SC>(c, st) : launch_mt<ActBF16, FMT, SC>(c, st);
+    if (rc != MI_OK) return rc;
+  }
+  return MI_OK;
+}
+
+}  // namespace qlin
+
+using namespace qlin;
+
+extern "C" {
+
+int mi_gemm_fp8_pern_multi(const void* x, int nmat, const void* const* w, const void* const* scale,
+                           void* const* out, const int* N, int M, int K, int act_dtype,
+                           int scale_is_f16, void* stream) {
+  if (nmat < 1 || nmat > kMaxMat || !w || !scale || !out || !N) return MI_ERR_ARG;
+  SkinnyArgs a{};
+  a.x = x; a.nmat = nmat; a.M = M; a.K = K; a.scale_f16 = scale_is_f16;
+  for (int i = 0; i < nmat; ++i) {
+    if (!scale[i]) return MI_ERR_ARG;
+    a.w[i] = w[i]; a.s[i] = scale[i]; a.out[i] = out[i]; a.N[i] = N[i];
+  }
+  return run<0, SC_PERN>(a, act_dtype, (hipStream_t)stream);
+}
+
+int mi_gemm_fp8_pern(const void* x, const void* w, const void* scale, void* out, int M, int N, int K,
+                     int act_dtype, int scale_is_f16, void* stream) {
+  return mi_gemm_fp8_pern_multi(x, 1, &w, &scale, &out, &N, M, K, act_dtype, scale_is_f16, stream);
+}
+
+int mi_gemm_fp8_pert_multi(const void* x, int nmat, const void* const* w, const float* const* scale,
+                           void* const* out, const int* N, int M, int K, int act_dtype, void* stream) {
+  if (nmat < 1 || nmat > kMaxMat || !w || !scale || !out || !N) return MI_ERR_ARG;
+  SkinnyArgs a{};
+  a.x = x; a.nmat = nmat; a.M = M; a.K = K;
+  for (int i = 0; i < nmat; ++i) {
+    if (!scale[i]) return MI_ERR_ARG;
+    a.w[i] = w[i]; a.s[i] = scale[i]; a.out[i] = out[i]; a.N[i] = N[i];
+  }
+  return run<0, SC_PERT>(a, act_dtype, (hipStream_t)stream);
+}
+
+int mi_gemm_fp8_pert(const void* x, const void* w, const float* scale, void* out, int M, int N, int K,
+                     int act_dtype, void* stream) {
+  return mi_gemm_fp8_pert_multi(x, 1, &w, &scale, &out, &N, M, K, act_dtype, stream);
+}
+
+int mi_gemm_fp8_blockscale_multi(const void* x, int nmat, const void* const* w,
+                                 const float* const* scale, void* const* out, const int* N, int M,
+                                 int K, int act_dtype, void* stream) {
+  if (nmat < 1 || nmat > kMaxMat || !w || !scale || !out || !N) return MI_ERR_ARG;
+  if (K % 128) return MI_ERR_SHAPE;
+  SkinnyArgs a{};
+  a.x = x; a.nmat = nmat; a.M = M; a.K = K;
+  for (int i = 0; i < nmat; ++i) {
+    if (!scale[i]) return MI_ERR_ARG;
+    a.w[i] = w[i]; a.s[i] = scale[i]; a.out[i] = out[i]; a.N[i] = N[i];
+  }
+  return run<0, SC_BLOCK>(a, act_dtype, (hipStream_t)stream);
+}
+
+int mi_gemm_fp8_blockscale(const void* x, const void* w, const float* scale, void* out, int M, int N,
+                           int K, int act_dtype, void* stream) {
+  return mi_gemm_fp8_blockscale_multi(x, 1, &w, &scale, &out, &N, M, K, act_dtype, stream);
+}
+
+int mi_gemv_int4_multi(const void* x, int nmat, const void* const* w, const void* const* scale,
+                       const void* const* zp, void* const* out, const int* N, int M, int K,
+                       int act_dtype, void* stream) {
+  if (nmat < 1 || nmat > kMaxMat || !w || !scale || !out || !N) return MI_ERR_ARG;
+  SkinnyArgs a{};
+  a.x = x; a.nmat = nmat; a.M = M; a.K = K;
+  for (int i = 0; i < nmat; ++i) {
+    if (!scale[i]) return MI_ERR_ARG;
+    a.w[i] = w[i]; a.s[i] = scale[i]; a.z[i] = zp ? zp[i] : nullptr; a.out[i] = out[i]; a.N[i] = N[i];
+  }
+  return run<1, 0>(a, act_dtype, (hipStream_t)stream);
+}
+
+int mi_gemv_int4(const void* x, const void* w, const void* scale, const void* zp, void* out, int M,
+                 int N, int K, int act_dtype, void* stream) {
+  const void* zps[1] = {zp};
+  return mi_gemv_int4_multi(x, 1, &w, &scale, zp ? zps : nullptr, &out, &N, M, K, act_dtype, stream);
+}
+
+int mi_gemv_q4k(const void* x, const void* ql, const void* scale, const void* qmin, void* out, int M,
+                int N, int K, void* stream) {
+  if (!scale || !qmin) return MI_ERR_ARG;
+  SkinnyArgs a{};
+  a.x = x; a.nmat = 1; a.M = M; a.K = K;
+  a.w[0] = ql; a.s[0] = scale; a.z[0] = qmin; a.out[0] = out; a.N[0] = N;
+  return run<2, 0>(a, DT_F16, (hipStream_t)stream);
+}
+
+}  // extern "C"

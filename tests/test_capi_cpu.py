@@ -1,0 +1,74 @@
+"""CPU-only checks of the boundary: the shared library loads, exports every
+symbol include/mi355x_qlinear.h declares, the torch.ops schemas carry the
+reference's names and argument order, and there is no silent CPU fallback."""
+import ctypes
+import os
+
+import pytest
+import torch
+
+import mi355x_qlinear  # noqa: F401
+from mi355x_qlinear import capi
+
+
+def test_library_exports_every_declared_symbol():
+    protos = capi.parse_header()
+    assert len(protos) >= 14
+    handle = ctypes.CDLL(capi.LIB_PATH)
+    for name in protos:
+        assert hasattr(handle, name), name
+    # and the loader wires argtypes for all of them
+    lib = capi.lib()
+    for name, types in protos.items():
+        assert getattr(lib, name).argtypes == types
+
+
+def test_header_pointer_and_scalar_mapping():
+    p = capi.parse_header()
+    assert p["mi_gemm_fp8_pern"] == [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_void_p]
+    assert p["mi_decode_e4m3"][2] is ctypes.c_longlong
+
+
+REFERENCE_SCHEMAS = {
+    # name: argument names in the reference's registration order
+    "custom_esimd_kernels_vllm::esimd_gemv_fp8_pern": ["input", "weight", "weight_scale", "output", "N", "K"],
+    "custom_esimd_kernels_vllm::esimd_gemv_fp8_pert": ["input", "weight", "weight_scale", "output"],
+    "custom_esimd_kernels_vllm::esimd_gemv_int4": ["input", "weight", "weight_scale", "output"],
+    "custom_esimd_kernels_vllm::esimd_gemv_int4_fused2": ["input", "w0", "s0", "o0", "w1", "s1", "o1"],
+    "custom_esimd_kernels_vllm::esimd_gemm_fp8_pert": ["input", "weight", "weight_scale", "output"],
+    "custom_esimd_kernels_vllm::esimd_gemm_fp8_blockscale": ["input", "weight", "weight_scale", "output", "block_n", "block_k"],
+    "custom_esimd_kernels_sglang::esimd_gemv_q4_k": ["input", "weight", "weight_scale", "weight_min", "output"],
+    "custom_esimd_kernels::esimd_gemm_fp8_pert": ["input", "weight", "weight_scale", "output"],
+}
+
+
+@pytest.mark.parametrize("qual", sorted(REFERENCE_SCHEMAS))
+def test_schema_matches_reference(qual):
+    ns, name = qual.split("::")
+    op = getattr(getattr(torch.ops, ns), name).default
+    assert [a.name for a in op._schema.arguments] == REFERENCE_SCHEMAS[qual]
+
+
+def test_no_cpu_fallback():
+    x = torch.zeros(1, 128, dtype=torch.float16)
+    w = torch.zeros(16, 64, dtype=torch.uint8)
+    s = torch.zeros(16, 1, dtype=torch.float16)
+    out = torch.zeros(1, 16, dtype=torch.float16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        torch.ops.custom_esimd_kernels_vllm.esimd_gemv_int4(x, w, s, out)
+
+
+def test_meta_kernels_trace():
+    x = torch.zeros(1, 128, dtype=torch.float16, device="meta")
+    w = torch.zeros(16, 64, dtype=torch.uint8, device="meta")
+    s = torch.zeros(16, 1, dtype=torch.float16, device="meta")
+    out = torch.zeros(1, 16, dtype=torch.float16, device="meta")
+    r = torch.ops.custom_esimd_kernels_vllm.esimd_gemv_int4(x, w, s, out)
+    assert r.shape == (1, 16)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", os.path.join(os.path.dirname(capi.LIB_PATH), "nope.so"))
+    with pytest.raises(ImportError):
+        capi.lib()

@@ -1,0 +1,311 @@
+"""GPU parity: dense quantized GEMV / small-M GEMM and the dequant kernels,
+called through torch.ops -> ctypes -> the C ABI, checked against the CPU oracle.
+
+Bars: dequantized weights bit-exact; GEMV / GEMM outputs within max relative
+error 1e-2 of the fp32-accumulated reference on the same dequantized weights
+(denominator floored at the tensor's mean magnitude, see oracle.max_rel_err).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qlinear_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops(dev):
+    import custom_esimd_kernels_vllm as v
+    import custom_esimd_kernels_sglang as s
+    return v, s
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16) if t.element_size() == 2 else t.contiguous().view(torch.int32)
+
+
+def _same_bits(a, b):
+    """bit equality, except that any NaN matches any NaN"""
+    a, b = a.cpu(), b.cpu()
+    nan = torch.isnan(a.float()) & torch.isnan(b.float())
+    return bool(((_bits(a) == _bits(b)) | nan).all())
+
+
+# ----------------------------------------------------------------- dequant, bit-exact
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_e4m3_decode_all_codes(ops, dev, dt):
+    v, _ = ops
+    codes = torch.arange(256, dtype=torch.uint8).repeat(4)
+    out = torch.empty(codes.numel(), dtype=dt, device=dev)
+    v.e4m3_decode(codes.to(dev), out)
+    ref = O.e4m3_decode(codes).to(dt)
+    assert _same_bits(out, ref)
+    assert out[0x80].item() == 0.0
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("asym", [False, True])
+def test_int4_dequant_bit_exact(ops, dev, dt, asym):
+    v, _ = ops
+    N, K = 96, 512
+    x, packed, scale, zp = O.make_int4_case(1, K, N, seed=21, asym=asym)
+    # negative, tiny (subnormal products) and large scales as well
+    scale[0, :] = torch.tensor([-0.875, 6.0e-5, 1.0e-7, 123.0], dtype=torch.float16)
+    out = torch.empty(N, K, dtype=dt, device=dev)
+    v.int4_dequant(packed.to(dev), scale.to(dev), None if zp is None else zp.to(dev), out)
+    ref = O.int4_dequant(packed, scale, out_dtype=dt, zp=zp)
+    assert _same_bits(out, ref)
+    # the int32 view of the same bytes is accepted and gives the same result
+    out2 = torch.empty_like(out)
+    v.int4_dequant(packed.view(torch.int32).to(dev), scale.to(dev), None if zp is None else zp.to(dev), out2)
+    assert torch.equal(_bits(out2.cpu()), _bits(out.cpu()))
+
+
+def test_int4_dequant_all_nibbles(ops, dev):
+    v, _ = ops
+    # every nibble value at every position of a dword, both parities
+    N, K = 16, 128
+    u = torch.zeros(N, K, dtype=torch.int32)
+    for n in range(N):
+        u[n] = (torch.arange(K) + n) % 16
+    packed = ((u[:, 0::2] & 0xF) | ((u[:, 1::2] & 0xF) << 4)).to(torch.uint8)
+    scale = torch.linspace(0.005, 0.02, N).to(torch.float16).reshape(N, 1)
+    for dt in (torch.float16, torch.bfloat16):
+        out = torch.empty(N, K, dtype=dt, device=dev)
+        v.int4_dequant(packed.to(dev), scale.to(dev), None, out)
+        assert _same_bits(out, O.int4_dequant(packed, scale, out_dtype=dt))
+
+
+@pytest.mark.parametrize("mode", ["pern", "pern16", "pert", "block"])
+def test_fp8_dequant_bit_exact(ops, dev, mode):
+    v, _ = ops
+    N, K = 256, 384
+    g = torch.Generator().manual_seed(31)
+    w8 = torch.randint(0, 256, (N, K), generator=g, dtype=torch.int32).to(torch.uint8)
+    w8[(w8 & 0x7F) == 0x7F] = 0x3A            # no NaN codes in weights
+    w8[0, :256] = torch.arange(256, dtype=torch.uint8)
+    w8[0, 0x7F] = 0
+    w8[0, 0xFF] = 0
+    out = torch.empty(N, K, dtype=torch.float32, device=dev)
+    if mode in ("pern", "pern16"):
+        s = (torch.rand(N, generator=g) * 1e-3 + 1e-5)
+        if mode == "pern16":
+            s = s.to(torch.float16)
+        v.fp8_dequant(w8.to(dev), s.to(dev), out, "pern")
+        ref = O.fp8_dequant_per_channel(w8, s)
+    elif mode == "pert":
+        s = torch.tensor([3.3e-4])
+        v.fp8_dequant(w8.to(dev), s.to(dev), out, "pert")
+        ref = O.fp8_dequant_per_tensor(w8, s)
+    else:
+        s = torch.rand(2, 3, generator=g) * 1e-3 + 1e-5
+        v.fp8_dequant(w8.view(torch.float8_e4m3fn).to(dev), s.to(dev), out, "block")
+        ref = O.fp8_dequant_block(w8, s)
+    assert _same_bits(out, ref)
+
+
+def test_q4k_repack_and_dequant_bit_exact(ops, dev):
+    _, s = ops
+    N, K = 48, 1024
+    _, raw = O.make_q4k_case(1, K, N, seed=41)
+    rawt = torch.from_numpy(raw).to(dev)
+    ql = torch.empty(N, K // 2, dtype=torch.uint8, device=dev)
+    sc = torch.empty(N, K // 32, dtype=torch.float16, device=dev)
+    mn = torch.empty(N, K // 32, dtype=torch.float16, device=dev)
+    s.q4_k_repack(rawt, ql, sc, mn)
+    rql, rsc, rmn = O.q4k_repack(raw)
+    assert np.array_equal(ql.cpu().numpy(), rql)
+    assert np.array_equal(sc.cpu().numpy().view(np.uint16), rsc.view(np.uint16))
+    assert np.array_equal(mn.cpu().numpy().view(np.uint16), rmn.view(np.uint16))
+    w = torch.empty(N, K, dtype=torch.float16, device=dev)
+    s.q4_k_dequant(ql, sc, mn, w)
+    ref = O.q4k_dequant(rql, rsc, rmn)
+    assert np.array_equal(w.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
+# ----------------------------------------------------------------- GEMV / GEMM, tolerance
+def _run_int4(v, dev, M, K, N, dt, seed=1234):
+    x, packed, scale, _ = O.make_int4_case(M, K, N, seed=seed, act_dtype=dt)
+    out = torch.empty(M, N, dtype=dt, device=dev)
+    r = v.esimd_gemv_int4(x.to(dev), packed.to(dev), scale.to(dev), out)
+    assert r.data_ptr() == out.data_ptr()
+    ref = O.matmul_ref(x, O.int4_dequant(packed, scale, out_dtype=dt))
+    return O.max_rel_err(out.cpu(), ref)
+
+
+def test_cfg0_w4a16_gemv(ops, dev):
+    v, _ = ops
+    assert _run_int4(v, dev, 1, 4096, 4096, torch.float16) < TOL
+
+
+@pytest.mark.parametrize("M,K,N,dt", [
+    (1, 128, 16, torch.float16), (1, 4096, 1000, torch.float16), (1, 1024, 17, torch.bfloat16),
+    (2, 2048, 512, torch.float16), (7, 4096, 96, torch.bfloat16), (16, 1024, 256, torch.float16),
+    (17, 1024, 256, torch.float16), (33, 2048, 128, torch.bfloat16), (64, 1024, 64, torch.float16),
+    (65, 1024, 64, torch.float16), (100, 512, 48, torch.bfloat16)])
+def test_int4_shapes(ops, dev, M, K, N, dt):
+    v, _ = ops
+    assert _run_int4(v, dev, M, K, N, dt, seed=M * 7 + N) < TOL
+
+
+def test_int4_fused2_equals_two_calls(ops, dev):
+    v, _ = ops
+    K = 2048
+    x, p0, s0, _ = O.make_int4_case(1, K, 1536, seed=51)
+    _, p1, s1, _ = O.make_int4_case(1, K, 72, seed=52)
+    xd = x.to(dev)
+    o0 = torch.empty(1, 1536, dtype=torch.float16, device=dev)
+    o1 = torch.empty(1, 72, dtype=torch.float16, device=dev)
+    r = v.esimd_gemv_int4_fused2(xd, p0.to(dev), s0.to(dev), o0, p1.to(dev), s1.to(dev), o1)
+    assert r.data_ptr() == o0.data_ptr()
+    a0 = torch.empty_like(o0)
+    a1 = torch.empty_like(o1)
+    v.esimd_gemv_int4(xd, p0.to(dev), s0.to(dev), a0)
+    v.esimd_gemv_int4(xd, p1.to(dev), s1.to(dev), a1)
+    assert torch.equal(o0, a0) and torch.equal(o1, a1)
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_cfg1_fp8_pern(ops, dev, M):
+    v, _ = ops
+    K, N = 4096, 14336
+    x, w8, s = O.make_fp8_pern_case(M, K, N)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    v.esimd_gemv_fp8_pern(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), s.to(dev), out, N, K)
+    ref = O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
+@pytest.mark.parametrize("M,K,N,dt,s16", [
+    (1, 256, 8, torch.float16, True), (1, 1056, 2816, torch.float16, True),
+    (3, 512, 1000, torch.bfloat16, False), (16, 4096, 40, torch.float16, False),
+    (48, 1024, 333, torch.bfloat16, False), (130, 512, 64, torch.float16, True)])
+def test_fp8_pern_shapes(ops, dev, M, K, N, dt, s16):
+    v, _ = ops
+    x, w8, s = O.make_fp8_pern_case(M, K, N, seed=M + N, act_dtype=dt)
+    if s16:
+        s = s.to(torch.float16)
+    out = torch.empty(M, N, dtype=dt, device=dev)
+    v.esimd_gemv_fp8_pern(x.to(dev), w8.to(dev), s.to(dev), out, N, K)
+    ref = O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
+def test_fp8_pern_fused3_equals_separate(ops, dev):
+    v, _ = ops
+    K = 2048
+    cases = [O.make_fp8_pern_case(1, K, n, seed=60 + i, act_dtype=torch.float16) for i, n in enumerate((512, 40, 1000))]
+    x = cases[0][0].to(dev)
+    ws = [c[1].to(dev) for c in cases]
+    ss = [c[2].to(dev) for c in cases]
+    Ns = [512, 40, 1000]
+    os_ = [torch.empty(1, n, dtype=torch.float16, device=dev) for n in Ns]
+    v.esimd_gemv_fp8_pern_fused3(x, ws[0], ss[0], os_[0], Ns[0], ws[1], ss[1], os_[1], Ns[1],
+                                 ws[2], ss[2], os_[2], Ns[2], K)
+    for w, s, o, n in zip(ws, ss, os_, Ns):
+        a = torch.empty_like(o)
+        v.esimd_gemv_fp8_pern(x, w, s, a, n, K)
+        assert torch.equal(a, o)
+    o2 = [torch.empty_like(o) for o in os_[:2]]
+    v.esimd_gemv_fp8_pern_fused2(x, ws[0], ss[0], o2[0], Ns[0], ws[1], ss[1], o2[1], Ns[1], K)
+    assert torch.equal(o2[0], os_[0]) and torch.equal(o2[1], os_[1])
+
+
+@pytest.mark.parametrize("M", [1, 5, 64])
+def test_fp8_pert(ops, dev, M):
+    v, _ = ops
+    K, N = 2048, 777
+    x, w8, _ = O.make_fp8_pern_case(M, K, N, seed=70 + M, act_dtype=torch.float16)
+    s = torch.tensor([2.5e-4])
+    ref = O.matmul_ref(x, O.fp8_dequant_per_tensor(w8, s))
+    for fn in (v.esimd_gemv_fp8_pert, v.esimd_gemm_fp8_pert, v.esimd_gemv_fp8_pert_bmg):
+        out = torch.empty(M, N, dtype=torch.float16, device=dev)
+        fn(x.to(dev), w8.to(dev), s.to(dev), out)
+        assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 5120, 1024), (1, 6144, 5120), (2, 5120, 5120), (7, 5120, 5120),
+                                   (9, 5120, 5120), (12, 5120, 5120), (33, 5120, 5120), (64, 5120, 5120),
+                                   (1, 5120, 1000), (4, 5120, 1000)])
+def test_fp8_blockscale_reference_shapes(ops, dev, M, K, N):
+    # shapes of V/tests/test_fp8_blockscale_gemm.py:93-101
+    v, _ = ops
+    x, w8, s = O.make_fp8_block_case(M, K, (N + 127) // 128 * 128, seed=M * 131 + N + K, act_dtype=torch.float16, std=0.3)
+    w8, s = w8[:N].contiguous(), s
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    v.esimd_gemm_fp8_blockscale(x.to(dev), w8.to(dev), s.to(dev), out)
+    ref = O.matmul_ref(x, O.fp8_dequant_block(w8, s))
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
+def test_fp8_blockscale_all_codes_exact(ops, dev):
+    # V/tests/test_fp8_blockscale_moe_prefill.py:54-90: row c = code c x 128, x = ones
+    v, _ = ops
+    raw = torch.arange(256, dtype=torch.uint8).view(256, 1).expand(256, 128).contiguous()
+    scale = torch.ones(2, 1)
+    x = torch.ones(1, 128, dtype=torch.float16)
+    out = torch.empty(1, 256, dtype=torch.float16, device=dev)
+    v.esimd_gemm_fp8_blockscale(x.to(dev), raw.to(dev), scale.to(dev), out)
+    reference = raw[:, 0].view(torch.float8_e4m3fn).float() * 128
+    finite = torch.isfinite(reference)
+    actual = out[0].cpu().float()
+    assert torch.equal(actual[finite], reference[finite])
+    assert actual[0x80].item() == 0.0
+
+
+def test_fp8_blockscale_fused2(ops, dev):
+    v, _ = ops
+    K = 1024
+    x, w0, s0 = O.make_fp8_block_case(1, K, 512, seed=80, act_dtype=torch.bfloat16)
+    _, w1, s1 = O.make_fp8_block_case(1, K, 256, seed=81, act_dtype=torch.bfloat16)
+    o0 = torch.empty(1, 512, dtype=torch.bfloat16, device=dev)
+    o1 = torch.empty(1, 256, dtype=torch.bfloat16, device=dev)
+    v.esimd_gemv_fp8_blockscale_fused2(x.to(dev), w0.to(dev), s0.to(dev), o0, w1.to(dev), s1.to(dev), o1)
+    for w8, s, o in ((w0, s0, o0), (w1, s1, o1)):
+        assert O.max_rel_err(o.cpu(), O.matmul_ref(x, O.fp8_dequant_block(w8, s))) < TOL
+
+
+@pytest.mark.parametrize("M", [1, 64])
+def test_cfg4_q4k(ops, dev, M):
+    _, s = ops
+    K = N = 5120
+    x, raw = O.make_q4k_case(M, K, N)
+    ql, sc, mn = O.q4k_repack(raw)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    s.esimd_gemv_q4_k(x.to(dev), torch.from_numpy(ql).to(dev), torch.from_numpy(sc).to(dev),
+                      torch.from_numpy(mn).to(dev), out)
+    w = torch.from_numpy(O.q4k_dequant(ql, sc, mn))
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, w)) < TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 256, 3), (5, 768, 100), (40, 512, 33)])
+def test_q4k_shapes(ops, dev, M, K, N):
+    _, s = ops
+    x, raw = O.make_q4k_case(M, K, N, seed=M + N)
+    ql, sc, mn = O.q4k_repack(raw)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    s.esimd_gemv_q4_k(x.to(dev), torch.from_numpy(ql).to(dev), torch.from_numpy(sc).to(dev),
+                      torch.from_numpy(mn).to(dev), out)
+    w = torch.from_numpy(O.q4k_dequant(ql, sc, mn))
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, w)) < TOL
+
+
+# ----------------------------------------------------------------- error behaviour
+def test_argument_errors_raise(ops, dev):
+    v, _ = ops
+    x = torch.zeros(1, 256, dtype=torch.float16, device=dev)
+    w = torch.zeros(16, 128, dtype=torch.uint8, device=dev)
+    s = torch.zeros(16, 2, dtype=torch.float16, device=dev)
+    out = torch.zeros(1, 16, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError):
+        v.esimd_gemv_int4(x.float(), w, s, out)                      # fp32 activations
+    with pytest.raises(RuntimeError):
+        v.esimd_gemv_int4(x, w, s, out.to(torch.bfloat16))           # dtype mismatch
+    with pytest.raises(RuntimeError):
+        v.esimd_gemv_int4(x, w[:, :100].contiguous(), s, out)        # K not a multiple of 128
+    with pytest.raises(RuntimeError):
+        v.esimd_gemm_fp8_blockscale(x, torch.zeros(16, 256, dtype=torch.uint8, device=dev),
+                                    torch.zeros(1, 2, device=dev), out, 64, 128)   # block size
