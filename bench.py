@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one launch of the hot-path op on one batch of seeded synthetic input.
+The headline workload (default) is BASELINE.json configs[1]: FP8 per-channel
+weight-only GEMV, M=1, K=4096, N=14336, bf16 activations.  Each step uses the
+next of R distinct weight copies (R x weight bytes >> the 256 MB Infinity Cache)
+so the figure is HBM bandwidth, not cache bandwidth.  The K timed steps are
+issued back to back on one stream as replays of a HIP graph holding R launches,
+bracketed by a device synchronise on both sides; HIP events recorded on that same
+stream give the average per-launch duration used for the roofline fraction.
+
+Prints ONE JSON line.  `value` is the algorithmic bytes moved per second with
+inputs resident in HBM.  `cpu_baseline` times the reference's CPU path (torch
+dequant + fp32 matmul, restated in oracle/) on this host's cores on a bounded
+sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "llm-scaler_amd"))
+
+import torch  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "fp8": 5000.0}
+CACHE_BUST_BYTES = 1 << 30       # rotate over >= 1 GiB of distinct weights (4 x Infinity Cache)
+
+
+# ----------------------------------------------------------------------------
+# workloads: each returns (launch(i), alg_bytes, alg_flops, bound, dtype, descr, cpu_fn)
+# ----------------------------------------------------------------------------
+def _copies(nbytes: int) -> int:
+    return max(2, -(-CACHE_BUST_BYTES // nbytes))
+
+
+def wl_fp8_pern(M: int, dev):
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    K, N = 4096, 14336
+    x, w8, s = O.make_fp8_pern_case(M, K, N)
+    R = _copies(N * K)
+    g = torch.Generator().manual_seed(99)
+    ws = [w8.to(dev)]
+    for _ in range(R - 1):          # distinct contents per copy, same distribution (row permutation)
+        ws.append(w8[torch.randperm(N, generator=g)].to(dev))
+    ws = [w.view(torch.float8_e4m3fn) for w in ws]
+    xd, sd = x.to(dev), s.to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+    def launch(i):
+        v.esimd_gemv_fp8_pern(xd, ws[i % R], sd, out, N, K)
+
+    def cpu():
+        return O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s)).to(torch.bfloat16)
+
+    alg_bytes = N * K + 4 * N + 2 * M * K + 2 * M * N
+    return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="bf16",
+                name=f"cfg1 FP8 e4m3 per-channel weight-only GEMV M={M} K={K} N={N} bf16",
+                kernel="skinny_kernel", cpu=cpu)
+
+
+def wl_int4_gemv(dev):
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    M, K, N = 1, 4096, 4096
+    x, packed, scale, _ = O.make_int4_case(M, K, N)
+    R = _copies(N * K // 2)
+    g = torch.Generator().manual_seed(98)
+    ws, ss = [packed.to(dev)], [scale.to(dev)]
+    for _ in range(R - 1):
+        p = torch.randperm(N, generator=g)
+        ws.append(packed[p].to(dev))
+        ss.append(scale[p].to(dev))
+    xd = x.to(dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        v.esimd_gemv_int4(xd, ws[i % R], ss[i % R], out)
+
+    def cpu():
+        return O.matmul_ref(x, O.int4_dequant(packed, scale)).to(torch.float16)
+
+    alg_bytes = N * K // 2 + N * (K // 128) * 2 + K * 2 + N * 2
+    return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="f16",
+                name=f"cfg0 W4A16 group-128 GEMV M={M} K={K} N={N} fp16", kernel="skinny_kernel", cpu=cpu)
+
+
+def wl_q4k(M: int, dev):
+    import custom_esimd_kernels_sglang as s
+    from oracle import qlinear_oracle as O
+    K = N = 5120
+    x, raw = O.make_q4k_case(M, K, N)
+    ql, sc, mn = O.q4k_repack(raw)
+    qlt, sct, mnt = torch.from_numpy(ql), torch.from_numpy(sc), torch.from_numpy(mn)
+    per = N * K // 2 + 2 * N * (K // 32) * 2
+    R = _copies(per)
+    g = torch.Generator().manual_seed(97)
+    W = [(qlt.to(dev), sct.to(dev), mnt.to(dev))]
+    for _ in range(R - 1):
+        p = torch.randperm(N, generator=g)
+        W.append((qlt[p].to(dev), sct[p].to(dev), mnt[p].to(dev)))
+    xd = x.to(dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        a, b, c = W[i % R]
+        s.esimd_gemv_q4_k(xd, a, b, c, out)
+
+    def cpu():
+        return O.matmul_ref(x, torch.from_numpy(O.q4k_dequant(ql, sc, mn))).to(torch.float16)
+
+    alg_bytes = per + 2 * M * K + 2 * M * N
+    return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="f16",
+                name=f"cfg4 GGUF Q4_K (repacked) dequant-matmul M={M} K={K} N={N} fp16",
+                kernel="skinny_kernel", cpu=cpu)
+
+
+WORKLOADS = {
+    "cfg1_m1": lambda dev: wl_fp8_pern(1, dev),
+    "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
+    "cfg1_m32": lambda dev: wl_fp8_pern(32, dev),
+    "cfg0": wl_int4_gemv,
+    "cfg4_m1": lambda dev: wl_q4k(1, dev),
+    "cfg4_m64": lambda dev: wl_q4k(64, dev),
+}
+HEADLINE = "cfg1_m1"
+
+
+# ----------------------------------------------------------------------------
+def run_gpu(wl, steps: int, warmup: int):
+    """-> (wall seconds for `steps` launches, event ms for the same region)"""
+    R = wl["R"]
+    launch = wl["launch"]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(max(warmup, 1)):
+            launch(i)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(R):
+                launch(i)
+        reps, rem = divmod(steps, R)
+        graph.replay()                      # one untimed replay: graph upload
+        stream.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(reps):
+            graph.replay()
+        for i in range(rem):
+            launch(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    return t1 - t0, e0.elapsed_time(e1)
+
+
+def summarize(wl, steps, wall_s, ev_ms):
+    per_launch_s = ev_ms * 1e-3 / steps
+    if wl["bound"] == "hbm":
+        achieved = wl["bytes"] / per_launch_s / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = wl["flops"] / per_launch_s / 1e12
+        peak, unit = MFMA_PEAK_TFLOPS[wl["dtype"]], "TFLOP/s"
+    return {
+        "workload": wl["name"],
+        "ms_per_step": wall_s * 1e3 / steps,
+        "us_per_launch_events": per_launch_s * 1e6,
+        "GBps": wl["bytes"] / per_launch_s / 1e9,
+        "TFLOPs": wl["flops"] / per_launch_s / 1e12,
+        "roofline": {"bound": wl["bound"], "achieved": achieved, "peak": peak, "unit": unit,
+                     "frac": achieved / peak, "traffic": None, "kernel": wl["kernel"],
+                     "alg_bytes_per_launch": wl["bytes"], "alg_flops_per_launch": wl["flops"]},
+    }
+
+
+def cpu_baseline(wl, budget_s: float = 20.0):
+    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    cores = torch.get_num_threads()
+    times = []
+    t_start = time.perf_counter()
+    n = 0
+    while True:
+        t0 = time.perf_counter()
+        wl["cpu"]()
+        dt = time.perf_counter() - t0
+        n += 1
+        if n > 2:
+            times.append(dt)
+        if (n >= 7 or time.perf_counter() - t_start > budget_s) and times:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": wl["bytes"] / med / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "seconds_per_step": med,
+            "sample": f"{len(times)} timed passes (after 2 warm-ups) of the full workload: torch dequant "
+                      f"of the whole weight + fp32 matmul, {wl['name']}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also time the other single-GPU workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; the path has no multi-GPU leg "
+              f"(asked for --gpus {args.gpus}).", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    import mi355x_qlinear  # noqa: F401  (raises if the HIP library is not built)
+    dev = torch.device("cuda:0")
+
+    wl = WORKLOADS[args.workload](dev)
+    wall, ev = run_gpu(wl, args.steps, args.warmup)
+    head = summarize(wl, args.steps, wall, ev)
+    cpu = None if args.no_cpu else cpu_baseline(wl)
+    del wl
+    torch.cuda.empty_cache()
+
+    cases = []
+    if args.all:
+        for name in sorted(WORKLOADS):
+            if name == args.workload:
+                continue
+            w = WORKLOADS[name](dev)
+            wa, e = run_gpu(w, args.steps, args.warmup)
+            c = summarize(w, args.steps, wa, e)
+            c["id"] = name
+            cases.append(c)
+            del w
+            torch.cuda.empty_cache()
+
+    line = {
+        "metric": "HBM GB/s (GEMV) and TFLOP/s (GEMM) as % of MI355X roofline, 1 GPU",
+        "value": wl_value(head),
+        "unit": head["roofline"]["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seeded; weights rotate over >=1 GiB of distinct copies)",
+        "config": {"workload": head["workload"], "id": args.workload,
+                   "timing": "HIP-graph replays of back-to-back launches on one stream"},
+        "roofline": head["roofline"],
+        "cpu_baseline": cpu,
+    }
+    if cases:
+        line["cases"] = cases
+    print(json.dumps(line))
+
+
+def wl_value(head):
+    """Whole-job throughput over the wall-clock timed region."""
+    r = head["roofline"]
+    per_step_s = head["ms_per_step"] * 1e-3
+    if r["bound"] == "hbm":
+        return r["alg_bytes_per_launch"] / per_step_s / 1e9
+    return r["alg_flops_per_launch"] / per_step_s / 1e12
+
+
+if __name__ == "__main__":
+    main()

@@ -28,7 +28,7 @@ __global__ __launch_bounds__(256) void dequant_int4_kernel(const uint32_t* __res
   if constexpr (Act::dt == DT_F16) {
     out[i] = int4x8_to_f16(w[i], (_Float16)s, (_Float16)(1024.0f + z));
   } else {
-    out[i] = int4x8_to_bf16(w[i], s, -z * s);
+    out[i] = int4x8_to_bf16(w[i], s, z);
   }
 }
 

@@ -117,14 +117,16 @@ __device__ __forceinline__ f16x8 int4x8_to_f16(uint32_t w, _Float16 s, _Float16 
   return out;
 }
 
-// bf16: the product (nib - z) * s is exact in fp32 (5 x 11 significant bits) and
-// nib * s - z * s is the same exact value, so one fma then one RNE to bf16.
-__device__ __forceinline__ bf16x8 int4x8_to_bf16(uint32_t w, float s, float neg_zs) {
+// bf16: (nib - z) is an exact small integer and its product with the fp16 scale
+// is exact in fp32 (5 x 11 significant bits), so the only rounding is the RNE to
+// bf16.  Subtract-then-multiply (not an fma with -z*s) keeps the sign of a zero
+// result: (8 - 8) * negative scale is -0.
+__device__ __forceinline__ bf16x8 int4x8_to_bf16(uint32_t w, float s, float z) {
   bf16x8 out;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float nib = (float)((w >> (4 * i)) & 0xFu);
-    out[i] = (__bf16)__builtin_fmaf(nib, s, neg_zs);
+    out[i] = (__bf16)((nib - z) * s);
   }
   return out;
 }

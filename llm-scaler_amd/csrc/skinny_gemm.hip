@@ -129,10 +129,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[u][i], s, z);
           } else {
-            const float s = sc[u];
-            const float nzs = -zz[u] * s;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[u][i], s, nzs);
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[u][i], sc[u], zz[u]);
           }
         } else {
           if constexpr (Act::dt == DT_F16) {
