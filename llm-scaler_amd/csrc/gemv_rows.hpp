@@ -1,0 +1,358 @@
+// Decode GEMV for M <= 4 activation rows: one wavefront per weight row.
+//
+// HBM-bound design.  A wavefront streams whole weight rows with perfectly
+// coalesced 128-bit loads (64 lanes x 16 B = 1 KiB contiguous per instruction),
+// keeps RW rows in flight, and accumulates with v_dot2_f32_{f16,bf16} (two
+// multiply-adds per instruction, fp32 accumulate).  The activations are staged
+// once per workgroup in LDS, already laid out in the order the lanes consume
+// them, so the inner loop touches global memory for weights only.  The K
+// reduction finishes inside the wavefront with cross-lane adds; no LDS
+// reduction, no barrier after the staging one.
+//
+// Per-format arithmetic (x = activation, all sums in fp32):
+//   fp8   : sum x * e4m3(w), exact conversion to 16 bit, scale applied per row
+//           (per-channel / per-tensor) or per lane chunk (128x128 block scale);
+//   int4  : nibbles are planted into the mantissa of a 16-bit constant
+//           (fp16: 0x6400|nib = 1024+nib, and 0x6400|nib<<4 = 1024+16 nib for
+//           odd nibbles, matched by x/16 in LDS; bf16: 0x4300|nib = 128+nib),
+//           the constant's contribution  C1 = sum bias_k x_k  and the
+//           zero-point's  z * C2, C2 = sum x_k  are precomputed per 32-k chunk
+//           at staging time, and the group scale multiplies the corrected
+//           partial:  acc += s * (dot - C1 - z C2);
+//   Q4_K  : same planting; acc += s * (dot - C1) - min * C2.
+// The dequantized weight is therefore never rounded to 16 bit here; against a
+// reference that rounds it the difference is below 2^-9 relative per weight.
+#pragma once
+#include "qlinear_common.hpp"
+
+namespace qlin {
+
+constexpr int kRowsMaxMat = 3;
+
+struct RowsArgs {
+  const void* x;
+  const void* w[kRowsMaxMat];
+  const void* s[kRowsMaxMat];
+  const void* z[kRowsMaxMat];
+  void* out[kRowsMaxMat];
+  int N[kRowsMaxMat];
+  int groups[kRowsMaxMat];     // workgroups per matrix
+  int nmat;
+  int M, K;
+  int nspan;                   // ceil(K / span_k)
+  int scale_f16;
+};
+
+enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2 };
+enum : int { RS_PERN = 0, RS_PERT = 1, RS_BLOCK = 2 };
+
+template <class Act> struct Dot2;
+template <> struct Dot2<ActF16> {
+  static __device__ __forceinline__ float run(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+  }
+};
+template <> struct Dot2<ActBF16> {
+  static __device__ __forceinline__ float run(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+  }
+};
+
+template <class Act>
+__device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_t& p1) {
+  if constexpr (Act::dt == DT_F16) {
+    p0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+    p1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+  } else {
+    p0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+    p1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
+  }
+}
+
+// LDS image: 16-byte pieces.  Piece index for (span s, piece i, lane l) is
+// (s * PPL + i) * 64 + l, PPL = pieces per lane per span (2 for fp8, 4 for the
+// nibble formats), so that the 64 lanes of one ds_read_b128 hit consecutive
+// addresses.  One piece = 8 consecutive k of one activation row.
+template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU>
+__global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
+  constexpr bool kFp8 = FMT == RF_FP8;
+  constexpr bool kNib = !kFp8;
+  constexpr int PPL = kFp8 ? 2 : 4;
+  constexpr int SPAN_K = 64 * PPL * 8;               // k covered by one wave load: 1024 / 2048
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int K = a.K, M = a.M;
+  const int nspan = a.nspan;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int pieces_per_row = nspan * PPL * 64;       // padded to whole spans
+  u32x4* xs = reinterpret_cast<u32x4*>(smem);        // [MR][pieces_per_row]
+  float* c1 = reinterpret_cast<float*>(smem + (size_t)MR * pieces_per_row * 16);   // [MR][nspan*64]
+  float* c2 = c1 + MR * nspan * 64;
+
+  int grp = blockIdx.x, mat = 0;
+#pragma unroll
+  for (int i = 0; i + 1 < kRowsMaxMat; ++i)
+    if (mat == i && i + 1 < a.nmat && grp >= a.groups[i]) { grp -= a.groups[i]; mat = i + 1; }
+  const int N = a.N[mat];
+  const int row0 = (grp * NWV + wave) * RW;
+
+  const uint32_t wrow = kFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
+
+  // ---- first batch of weight loads goes out before the staging barrier ----
+  const _Float16* s16 = (const _Float16*)a.s[mat];
+  const float* s32 = (const float*)a.s[mat];
+  const uint8_t* zp = (const uint8_t*)a.z[mat];
+  const _Float16* qmin = (const _Float16*)a.z[mat];
+
+  u32x4 wreg[RW][SPU];
+  float sreg[RW][SPU];          // per-lane scale of the chunk (int4 group / q4k sub-block / fp8 block)
+  float zreg[RW][SPU];          // int4 zero-point / q4k min
+  auto load_batch = [&](int s0) {
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+      const int nc = (row0 + r) < N ? (row0 + r) : N - 1;
+#pragma unroll
+      for (int sp = 0; sp < SPU; ++sp) {
+        const int s = s0 + sp;
+        const uint32_t kb = (uint32_t)s * (SPAN_K / (kFp8 ? 1 : 2)) + lane * 16u;   // byte in row
+        const bool ok = (row0 + r < N) && (kb < wrow);
+        wreg[r][sp] = buf_load16(wr, ok ? (uint32_t)(row0 + r) * wrow + kb : kOOB);
+        const int chunk = s * 64 + lane;            // 32-k chunk index (nibble formats)
+        if constexpr (FMT == RF_INT4) {
+          const int Kg = K >> 7;
+          int gi = chunk >> 2;
+          gi = gi < Kg ? gi : Kg - 1;
+          sreg[r][sp] = (float)s16[(size_t)nc * Kg + gi];
+          zreg[r][sp] = zp ? (float)zp[(size_t)nc * Kg + gi] : 8.0f;
+        } else if constexpr (FMT == RF_Q4K) {
+          const int Kc = K >> 5;
+          const int ci = chunk < Kc ? chunk : Kc - 1;
+          sreg[r][sp] = (float)s16[(size_t)nc * Kc + ci];
+          zreg[r][sp] = (float)qmin[(size_t)nc * Kc + ci];
+        } else if constexpr (SC == RS_BLOCK) {
+          const int Kb = (K + 127) >> 7;
+          const int kblk = (s * SPAN_K + lane * 16) >> 7;
+          sreg[r][sp] = s32[(size_t)(nc >> 7) * Kb + (kblk < Kb ? kblk : Kb - 1)];
+        }
+      }
+    }
+  };
+  load_batch(0);
+
+  // ---- stage activations ----
+  {
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+    const int total = MR * pieces_per_row;
+    for (int p = threadIdx.x; p < total; p += NWV * 64) {
+      const int m = p / pieces_per_row;
+      const int q = p - m * pieces_per_row;          // (s*PPL + i)*64 + l
+      const int l = q & 63;
+      const int si = q >> 6;
+      const int s = si / PPL, i = si - s * PPL;
+      const int k = s * SPAN_K + (l * PPL + i) * 8;
+      u32x4 v = buf_load16(xr, (m < M && k < K) ? ((uint32_t)m * K + k) * 2u : kOOB);
+      if constexpr (kNib) {
+        // natural pairs (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x4)(x1 x5)(x2 x6)(x3 x7)
+        const uint32_t d0 = v[0], d1 = v[1], d2 = v[2], d3 = v[3];
+        uint32_t e0 = __builtin_amdgcn_perm(d2, d0, 0x05040100u);   // lo(d0), lo(d2)
+        uint32_t e1 = __builtin_amdgcn_perm(d2, d0, 0x07060302u);   // hi(d0), hi(d2)
+        uint32_t e2 = __builtin_amdgcn_perm(d3, d1, 0x05040100u);
+        uint32_t e3 = __builtin_amdgcn_perm(d3, d1, 0x07060302u);
+        if constexpr (Act::dt == DT_F16) {
+          // odd nibbles are planted 4 bits up (1024 + 16 nib): feed them x / 16
+          const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+          e1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, e1) * sixteenth);
+          e3 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, e3) * sixteenth);
+        }
+        v = u32x4{e0, e1, e2, e3};
+      }
+      xs[p] = v;
+    }
+    if constexpr (kNib) {
+      // per 32-k chunk: what the planted constants contribute (c1) and sum x (c2),
+      // summed in a fixed order from the staged image
+      __syncthreads();
+      const int chunks = MR * nspan * 64;
+      for (int c = threadIdx.x; c < chunks; c += NWV * 64) {
+        const int m = c / (nspan * 64);
+        const int sl = c - m * (nspan * 64);
+        const int s = sl >> 6, l = sl & 63;
+        float lo = 0.f, hi = 0.f;
+        auto pair_sum = [](uint32_t bits) -> float {
+          if constexpr (Act::dt == DT_F16) {
+            const f16x2 h = __builtin_bit_cast(f16x2, bits);
+            return (float)h[0] + (float)h[1];
+          } else {
+            const bf16x2 h = __builtin_bit_cast(bf16x2, bits);
+            return (float)h[0] + (float)h[1];
+          }
+        };
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const u32x4 v = xs[m * pieces_per_row + (s * 4 + i) * 64 + l];
+          lo += pair_sum(v[0]);
+          hi += pair_sum(v[1]);
+          lo += pair_sum(v[2]);
+          hi += pair_sum(v[3]);
+        }
+        if constexpr (Act::dt == DT_F16) {
+          c1[c] = 1024.0f * (lo + hi);               // hi already holds x / 16
+          c2[c] = lo + 16.0f * hi;
+        } else {
+          c1[c] = 128.0f * (lo + hi);
+          c2[c] = lo + hi;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  float acc[RW][MR];
+#pragma unroll
+  for (int r = 0; r < RW; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
+
+  for (int s0 = 0; s0 < nspan; s0 += SPU) {
+    if (s0 > 0) load_batch(s0);
+#pragma unroll
+    for (int sp = 0; sp < SPU; ++sp) {
+      const int s = s0 + sp;
+      if (s < nspan) {                                // wave-uniform
+        u32x4 xp[MR][PPL];
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+          for (int i = 0; i < PPL; ++i) xp[m][i] = xs[m * pieces_per_row + (s * PPL + i) * 64 + lane];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+          const u32x4 w = wreg[r][sp];
+          float part[MR];
+#pragma unroll
+          for (int m = 0; m < MR; ++m) part[m] = 0.f;
+          if constexpr (kFp8) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              uint32_t p0, p1;
+              fp8x4_to_pairs<Act>(w[d], p0, p1);
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                part[m] = Dot2<Act>::run(p0, xp[m][d >> 1][(d & 1) * 2], part[m]);
+                part[m] = Dot2<Act>::run(p1, xp[m][d >> 1][(d & 1) * 2 + 1], part[m]);
+              }
+            }
+            if constexpr (SC == RS_BLOCK) {
+#pragma unroll
+              for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * sreg[r][sp];
+            } else {
+#pragma unroll
+              for (int m = 0; m < MR; ++m) acc[r][m] += part[m];
+            }
+          } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              uint32_t t0, t1, t2, t3;
+              if constexpr (Act::dt == DT_F16) {
+                const uint32_t w8 = w[d] >> 8;
+                t0 = (w[d] & 0x000F000Fu) | 0x64006400u;     // 1024 + nib0 , nib4
+                t1 = (w[d] & 0x00F000F0u) | 0x64006400u;     // 1024 + 16 nib1 , nib5
+                t2 = (w8 & 0x000F000Fu) | 0x64006400u;       // nib2 , nib6
+                t3 = (w8 & 0x00F000F0u) | 0x64006400u;       // nib3 , nib7
+              } else {
+                t0 = (w[d] & 0x000F000Fu) | 0x43004300u;     // 128 + nib0 , nib4
+                t1 = ((w[d] >> 4) & 0x000F000Fu) | 0x43004300u;
+                t2 = ((w[d] >> 8) & 0x000F000Fu) | 0x43004300u;
+                t3 = ((w[d] >> 12) & 0x000F000Fu) | 0x43004300u;
+              }
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                part[m] = Dot2<Act>::run(t0, xp[m][d][0], part[m]);
+                part[m] = Dot2<Act>::run(t1, xp[m][d][1], part[m]);
+                part[m] = Dot2<Act>::run(t2, xp[m][d][2], part[m]);
+                part[m] = Dot2<Act>::run(t3, xp[m][d][3], part[m]);
+              }
+            }
+            if constexpr (FMT == RF_INT4) {
+              const float sc = sreg[r][sp];
+              const float z = zreg[r][sp];
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                const float corr = part[m] - c1[(m * nspan + s) * 64 + lane] -
+                                   z * c2[(m * nspan + s) * 64 + lane];
+                acc[r][m] += sc * corr;
+              }
+            } else {
+              const float sc = sreg[r][sp];
+              const float mn = zreg[r][sp];
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                const float corr = part[m] - c1[(m * nspan + s) * 64 + lane];
+                acc[r][m] += sc * corr - mn * c2[(m * nspan + s) * 64 + lane];
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // ---- finish the K reduction inside the wavefront, lane 0 stores ----
+  using Elem = typename Act::elem;
+  Elem* out = (Elem*)a.out[mat];
+#pragma unroll
+  for (int r = 0; r < RW; ++r) {
+    const int n = row0 + r;
+    float os = 1.0f;
+    if constexpr (kFp8 && SC == RS_PERN) {
+      if (n < N) os = a.scale_f16 ? (float)s16[n] : s32[n];
+    }
+    if constexpr (kFp8 && SC == RS_PERT) os = s32[0];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const float v = wave_sum(acc[r][m]);
+      if (lane == 0 && n < N) out[(size_t)m * N + n] = Act::from_f32(v * os);
+    }
+  }
+}
+
+// LDS bytes the kernel needs for a given shape (0 = not applicable).
+static inline size_t rows_lds_bytes(int fmt, int MR, int K) {
+  const int ppl = fmt == RF_FP8 ? 2 : 4;
+  const int span_k = 64 * ppl * 8;
+  const int nspan = (K + span_k - 1) / span_k;
+  size_t b = (size_t)MR * nspan * ppl * 64 * 16;
+  if (fmt != RF_FP8) b += (size_t)2 * MR * nspan * 64 * 4;
+  return b;
+}
+
+template <class Act, int FMT, int SC, int MR>
+static void launch_rows(RowsArgs a, hipStream_t st) {
+  constexpr int NWV = 8;
+  constexpr int RW = FMT == RF_FP8 ? 2 : 4;
+  constexpr int SPU = FMT == RF_FP8 ? 4 : 2;
+  constexpr int ppl = FMT == RF_FP8 ? 2 : 4;
+  constexpr int span_k = 64 * ppl * 8;
+  a.nspan = (a.K + span_k - 1) / span_k;
+  int groups = 0;
+  for (int i = 0; i < a.nmat; ++i) {
+    a.groups[i] = (a.N[i] + NWV * RW - 1) / (NWV * RW);
+    groups += a.groups[i];
+  }
+  if (!groups) return;
+  const size_t lds = rows_lds_bytes(FMT, MR, a.K);
+  hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU>), dim3(groups), dim3(NWV * 64), lds,
+                     st, a);
+}
+
+template <class Act, int FMT, int SC>
+static void launch_rows_m(const RowsArgs& a, hipStream_t st) {
+  switch (a.M) {
+    case 1: launch_rows<Act, FMT, SC, 1>(a, st); break;
+    case 2: launch_rows<Act, FMT, SC, 2>(a, st); break;
+    case 3: launch_rows<Act, FMT, SC, 3>(a, st); break;
+    default: launch_rows<Act, FMT, SC, 4>(a, st); break;
+  }
+}
+
+}  // namespace qlin

@@ -14,6 +14,7 @@
 // holds the 32 consecutive k  [128 gi + 32 g, +32)  of weight row n0 + j and of
 // activation row j.  MFMA i (0..3) consumes the i-th 8-k slice of both.
 #include "qlinear_common.hpp"
+#include "gemv_rows.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -36,7 +37,10 @@ struct SkinnyArgs {
 enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
 
 // ---------------------------------------------------------------- kernel
-template <class Act, int FMT, int SC, int MT, int NW>
+// FMT: 0 = fp8 (SC selects the scale mode), 1 = int4 g128, 2 = Q4_K repacked.
+// MT = 16-row activation tiles (M <= 16 MT), RT = 16-row weight tiles per
+// workgroup, NW = wavefronts splitting K, UN = granules in flight per wave.
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   using V8 = typename Act::v8;
   using Elem = typename Act::elem;
@@ -45,7 +49,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr bool kIsQ4K = (FMT == 2);
   constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
 
-  __shared__ f32x4 red[NW - 1][MT][64];
+  __shared__ f32x4 red[NW - 1][RT][MT][64];
 
   int tile = blockIdx.x;
   int mat = 0;
@@ -58,9 +62,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = lane & 15, g = lane >> 4;
-  const int n0 = tile * 16;
-  const int n = n0 + j;
-  const int nc = n < N ? n : N - 1;                  // clamped row for side loads
+  const int n0 = tile * (16 * RT);
   const int G = (K + 127) >> 7;
 
   const uint32_t wrow = kIsFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
@@ -75,79 +77,91 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   const int Kb32 = K >> 5;                           // q4k sub-blocks per row
   const int Kb = G;                                  // fp8 block columns
 
-  f32x4 acc[MT];
+  f32x4 acc[RT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int UN = MT == 1 ? 4 : (MT == 2 ? 2 : 1);    // granules in flight per wave
+  // Out-of-range granules / lanes / rows load zeros for both operands, so the
+  // loop body needs no branches: a zero weight times a zero activation adds 0.
   for (int gbase = wave; gbase < G; gbase += NW * UN) {
-    u32x4 wa[UN], wb[UN];
+    u32x4 wa[UN][RT], wb[UN][RT];
     u32x4 xa[UN][MT][4];
-    float sc[UN];                                    // int4 / q4k scale, block scale
-    float zz[UN];
+    float sc[UN][RT];                                // int4 / q4k scale, block scale
+    float zz[UN][RT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int gi = gbase + u * NW;
       const int kl = gi * 128 + g * 32;
       const bool ok = (gi < G) && (kl < K);
-      const uint32_t woff = ok ? (uint32_t)n * wrow + (kIsFp8 ? (uint32_t)kl : ((uint32_t)kl >> 1)) : kOOB;
-      wa[u] = buf_load16(wr, woff);
-      if constexpr (kIsFp8) wb[u] = buf_load16(wr, ok ? woff + 16 : kOOB);
+      const int gic = gi < G ? gi : G - 1;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const int n = n0 + t * 16 + j;
+        const int nc = n < N ? n : N - 1;
+        const uint32_t woff =
+            ok ? (uint32_t)n * wrow + (kIsFp8 ? (uint32_t)kl : ((uint32_t)kl >> 1)) : kOOB;
+        wa[u][t] = buf_load16(wr, woff);
+        if constexpr (kIsFp8) wb[u][t] = buf_load16(wr, ok ? woff + 16 : kOOB);
+        if constexpr (kIsInt4) {
+          sc[u][t] = (float)s16[(size_t)nc * Kg + gic];
+          zz[u][t] = zp ? (float)zp[(size_t)nc * Kg + gic] : 8.0f;
+        } else if constexpr (kIsQ4K) {
+          const int sb = gic * 4 + g;
+          const int sbc = sb < Kb32 ? sb : Kb32 - 1;
+          sc[u][t] = (float)s16[(size_t)nc * Kb32 + sbc];
+          zz[u][t] = (float)qmin[(size_t)nc * Kb32 + sbc];
+        } else if constexpr (kBlock) {
+          sc[u][t] = s32[(size_t)((n0 + t * 16) >> 7) * Kb + gic];
+        }
+      }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
 #pragma unroll
         for (int i = 0; i < 4; ++i) xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
       }
-      const int gic = gi < G ? gi : G - 1;
-      if constexpr (kIsInt4) {
-        sc[u] = (float)s16[(size_t)nc * Kg + gic];
-        zz[u] = zp ? (float)zp[(size_t)nc * Kg + gic] : 8.0f;
-      } else if constexpr (kIsQ4K) {
-        const int sb = gic * 4 + g;
-        const int sbc = sb < Kb32 ? sb : Kb32 - 1;
-        sc[u] = (float)s16[(size_t)nc * Kb32 + sbc];
-        zz[u] = (float)qmin[(size_t)nc * Kb32 + sbc];
-      } else if constexpr (kBlock) {
-        sc[u] = s32[(size_t)(n0 >> 7) * Kb + gic];
-      }
     }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int gi = gbase + u * NW;
-      if (gi < G) {                                  // wave-uniform
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
         V8 b[4];
         if constexpr (kIsFp8) {
-          b[0] = fp8x8_to_act<Act>(wa[u][0], wa[u][1]);
-          b[1] = fp8x8_to_act<Act>(wa[u][2], wa[u][3]);
-          b[2] = fp8x8_to_act<Act>(wb[u][0], wb[u][1]);
-          b[3] = fp8x8_to_act<Act>(wb[u][2], wb[u][3]);
+          b[0] = fp8x8_to_act<Act>(wa[u][t][0], wa[u][t][1]);
+          b[1] = fp8x8_to_act<Act>(wa[u][t][2], wa[u][t][3]);
+          b[2] = fp8x8_to_act<Act>(wb[u][t][0], wb[u][t][1]);
+          b[3] = fp8x8_to_act<Act>(wb[u][t][2], wb[u][t][3]);
         } else if constexpr (kIsInt4) {
           if constexpr (Act::dt == DT_F16) {
-            const _Float16 s = (_Float16)sc[u];
-            const _Float16 z = (_Float16)(1024.0f + zz[u]);
+            const _Float16 s = (_Float16)sc[u][t];
+            const _Float16 z = (_Float16)(1024.0f + zz[u][t]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[u][i], s, z);
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[u][t][i], s, z);
           } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[u][i], sc[u], zz[u]);
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[u][t][i], sc[u][t], zz[u][t]);
           }
         } else {
           if constexpr (Act::dt == DT_F16) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = q4kx8_to_f16(wa[u][i], (_Float16)sc[u], (_Float16)zz[u]);
+            for (int i = 0; i < 4; ++i)
+              b[i] = q4kx8_to_f16(wa[u][t][i], (_Float16)sc[u][t], (_Float16)zz[u][t]);
           }
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           if constexpr (kBlock) {
-            f32x4 t = f32x4{0.f, 0.f, 0.f, 0.f};
+            f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < 4; ++i) t = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], t);
-            acc[mt] += t * sc[u];
+            for (int i = 0; i < 4; ++i) tt = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], tt);
+            acc[t][mt] += tt * sc[u][t];
           } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[mt] = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], acc[mt]);
+            for (int i = 0; i < 4; ++i)
+              acc[t][mt] = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], acc[t][mt]);
           }
         }
       }
@@ -157,44 +171,60 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   // ---- reduce the NW partial tiles through LDS ----
   if (wave > 0) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) red[wave - 1][mt][lane] = acc[mt];
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) red[wave - 1][t][mt][lane] = acc[t][mt];
   }
   __syncthreads();
   if (wave != 0) return;
 #pragma unroll
   for (int w = 0; w < NW - 1; ++w)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] += red[w][mt][lane];
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[t][mt] += red[w][t][mt][lane];
 
-  // D layout: lane holds output column n0 + j, rows mt*16 + 4 g + v.
-  float os = 1.0f;
-  if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[nc] : s32[nc];
-  if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
-  if (n < N) {
-    Elem* out = (Elem*)a.out[mat];
+  // D layout: lane holds output column n0 + 16 t + j, rows mt*16 + 4 g + v.
+  Elem* out = (Elem*)a.out[mat];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+  for (int t = 0; t < RT; ++t) {
+    const int n = n0 + t * 16 + j;
+    if (n < N) {
+      float os = 1.0f;
+      if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[n] : s32[n];
+      if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int m = mt * 16 + g * 4 + v;
-        if (m < M) out[(size_t)m * N + n] = Act::from_f32(acc[mt][v] * os);
-      }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = mt * 16 + g * 4 + v;
+          if (m < M) out[(size_t)m * N + n] = Act::from_f32(acc[t][mt][v] * os);
+        }
+    }
   }
+}
+
+template <class Act, int FMT, int SC, int MT, int RT, int UN>
+static void launch_one(SkinnyArgs a, hipStream_t st) {
+  constexpr int NW = 8;
+  int tiles = 0;
+  for (int i = 0; i < a.nmat; ++i) {
+    a.tiles[i] = (a.N[i] + 16 * RT - 1) / (16 * RT);
+    tiles += a.tiles[i];
+  }
+  if (tiles == 0) return;
+  hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, MT, RT, NW, UN>), dim3(tiles), dim3(NW * 64), 0, st, a);
 }
 
 template <class Act, int FMT, int SC>
 static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
-  int tiles = 0;
-  for (int i = 0; i < a.nmat; ++i) tiles += a.tiles[i];
-  if (tiles == 0 || a.M == 0) return MI_OK;
-  constexpr int NW = 8;
-  dim3 grid(tiles), block(NW * 64);
+  if (a.M == 0) return MI_OK;
   if (a.M <= 16)
-    hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, 1, NW>), grid, block, 0, st, a);
+    launch_one<Act, FMT, SC, 1, 1, 4>(a, st);
   else if (a.M <= 32)
-    hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, 2, NW>), grid, block, 0, st, a);
+    launch_one<Act, FMT, SC, 2, 2, 2>(a, st);
   else
-    hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, 4, NW>), grid, block, 0, st, a);
+    launch_one<Act, FMT, SC, 4, 1, 1>(a, st);
   return launch_status();
 }
 
@@ -214,6 +244,20 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     a.tiles[i] = (a.N[i] + 15) / 16;
   }
   if (!a.x) return MI_ERR_ARG;
+  if (a.M == 0) return MI_OK;
+  // decode regime: one wavefront per weight row, activations staged in LDS
+  if (a.M <= 4 && rows_lds_bytes(FMT, a.M, a.K) <= 64 * 1024 && (FMT != 0 || a.K % 16 == 0)) {
+    RowsArgs r{};
+    r.x = a.x; r.nmat = a.nmat; r.M = a.M; r.K = a.K; r.scale_f16 = a.scale_f16;
+    for (int i = 0; i < a.nmat; ++i) {
+      r.w[i] = a.w[i]; r.s[i] = a.s[i]; r.z[i] = a.z[i]; r.out[i] = a.out[i]; r.N[i] = a.N[i];
+    }
+    if (FMT == 2 || act_dtype == DT_F16)
+      launch_rows_m<ActF16, FMT, SC>(r, st);
+    else
+      launch_rows_m<ActBF16, FMT, SC>(r, st);
+    return launch_status();
+  }
   const int M = a.M;
   const size_t esz = 2;
   for (int m0 = 0; m0 < M; m0 += 64) {
