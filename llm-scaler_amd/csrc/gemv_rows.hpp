@@ -36,10 +36,11 @@ struct RowsArgs {
   const void* z[kRowsMaxMat];
   void* out[kRowsMaxMat];
   int N[kRowsMaxMat];
-  int groups[kRowsMaxMat];     // workgroups per matrix
+  int groups[kRowsMaxMat];     // row groups (RW rows each) per matrix
   int nmat;
   int M, K;
   int nspan;                   // ceil(K / span_k)
+  int total_waves;             // persistent grid size in wavefronts
   int scale_f16;
 };
 
@@ -73,102 +74,180 @@ __device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_
 // (s * PPL + i) * 64 + l, PPL = pieces per lane per span (2 for fp8, 4 for the
 // nibble formats), so that the 64 lanes of one ds_read_b128 hit consecutive
 // addresses.  One piece = 8 consecutive k of one activation row.
-template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU>
+//
+// The grid is persistent: `a.total_waves` wavefronts walk the flat list of row
+// groups (RW rows each, all matrices concatenated) with a fixed stride, and the
+// weight loads of the next batch are in flight while the current one is
+// consumed (two register buffers).  Weight loads carry the non-temporal hint:
+// every byte is used exactly once.
+template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI>
 __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   constexpr bool kFp8 = FMT == RF_FP8;
   constexpr bool kNib = !kFp8;
   constexpr int PPL = kFp8 ? 2 : 4;
   constexpr int SPAN_K = 64 * PPL * 8;               // k covered by one wave load: 1024 / 2048
+  constexpr int SPAN_B = kFp8 ? SPAN_K : SPAN_K / 2; // bytes of one weight row per span
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int K = a.K, M = a.M;
   const int nspan = a.nspan;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // provably uniform
   const int pieces_per_row = nspan * PPL * 64;       // padded to whole spans
   u32x4* xs = reinterpret_cast<u32x4*>(smem);        // [MR][pieces_per_row]
   float* c1 = reinterpret_cast<float*>(smem + (size_t)MR * pieces_per_row * 16);   // [MR][nspan*64]
   float* c2 = c1 + MR * nspan * 64;
 
-  int grp = blockIdx.x, mat = 0;
-#pragma unroll
-  for (int i = 0; i + 1 < kRowsMaxMat; ++i)
-    if (mat == i && i + 1 < a.nmat && grp >= a.groups[i]) { grp -= a.groups[i]; mat = i + 1; }
-  const int N = a.N[mat];
-  const int row0 = (grp * NWV + wave) * RW;
-
   const uint32_t wrow = kFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
-  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
+  const int nbatch = (nspan + SPU - 1) / SPU;        // batches per row group
+  const int stride = a.total_waves;
+  const int ngroups = a.groups[0] + a.groups[1] + a.groups[2];
 
-  // ---- first batch of weight loads goes out before the staging barrier ----
-  const _Float16* s16 = (const _Float16*)a.s[mat];
-  const float* s32 = (const float*)a.s[mat];
-  const uint8_t* zp = (const uint8_t*)a.z[mat];
-  const _Float16* qmin = (const _Float16*)a.z[mat];
+  struct Batch {                                     // one batch = RW rows x SPU spans
+    u32x4 w[RW][SPU];
+    float s[RW][SPU];          // per-lane scale of the chunk (int4 group / q4k sub-block / fp8 block)
+    float z[RW][SPU];          // int4 zero-point / q4k min
+    uint16_t os_lo[RW], os_hi[RW];   // fp8 per-channel scale of the row, raw halves (fp32 or fp16)
+  };
 
-  u32x4 wreg[RW][SPU];
-  float sreg[RW][SPU];          // per-lane scale of the chunk (int4 group / q4k sub-block / fp8 block)
-  float zreg[RW][SPU];          // int4 zero-point / q4k min
-  auto load_batch = [&](int s0) {
+  // Kernel arguments are selected with uniform compares, never indexed
+  // dynamically: a dynamic index would turn into memory loads whose waits
+  // serialize behind the weight prefetch.
+#define QLIN_PICK(field, mat) \
+  (MULTI ? ((mat) == 0 ? a.field[0] : ((mat) == 1 ? a.field[1] : a.field[2])) : a.field[0])
+  auto locate = [&](int g, int& mat, int& row0) {
+    mat = 0;
+    if constexpr (MULTI) {
+      if (g >= a.groups[0]) { g -= a.groups[0]; mat = 1; }
+      if (mat == 1 && g >= a.groups[1]) { g -= a.groups[1]; mat = 2; }
+    }
+    row0 = g * RW;
+  };
+
+  // Branch-free: an out-of-range group / row / span turns into out-of-range
+  // buffer offsets (reads zero) and clamped side-table indices.
+  auto load_batch = [&](Batch& b, int g, int sb) {
+    const bool live = g < ngroups;
+    int mat, row0;
+    locate(live ? g : 0, mat, row0);
+    const int N = QLIN_PICK(N, mat);
+    const __amdgpu_buffer_rsrc_t wr = make_rsrc(QLIN_PICK(w, mat), (uint32_t)N * wrow);
+    const _Float16* s16 = (const _Float16*)QLIN_PICK(s, mat);
+    const float* s32 = (const float*)QLIN_PICK(s, mat);
+    const uint8_t* zp = (const uint8_t*)QLIN_PICK(z, mat);
+    const _Float16* qmin = (const _Float16*)QLIN_PICK(z, mat);
+    if constexpr (kFp8 && SC == RS_PERN) {
+#pragma unroll
+      for (int r = 0; r < RW; ++r) {
+        const int nc = (row0 + r) < N ? (row0 + r) : N - 1;
+        // Two 16-bit loads with uniformly selected offsets cover both scale
+        // types without a branch and without converting here: a conversion
+        // would wait on the load, and with it on every weight load in flight.
+        const uint16_t* sraw = reinterpret_cast<const uint16_t*>(s16);
+        const size_t e = a.scale_f16 ? (size_t)nc : (size_t)nc * 2;
+        b.os_lo[r] = sraw[e];
+        b.os_hi[r] = sraw[e + (a.scale_f16 ? 0 : 1)];
+      }
+    }
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
       const int nc = (row0 + r) < N ? (row0 + r) : N - 1;
 #pragma unroll
       for (int sp = 0; sp < SPU; ++sp) {
-        const int s = s0 + sp;
-        const uint32_t kb = (uint32_t)s * (SPAN_K / (kFp8 ? 1 : 2)) + lane * 16u;   // byte in row
-        const bool ok = (row0 + r < N) && (kb < wrow);
-        wreg[r][sp] = buf_load16(wr, ok ? (uint32_t)(row0 + r) * wrow + kb : kOOB);
+        const int s = sb * SPU + sp;
         const int chunk = s * 64 + lane;            // 32-k chunk index (nibble formats)
         if constexpr (FMT == RF_INT4) {
           const int Kg = K >> 7;
           int gi = chunk >> 2;
           gi = gi < Kg ? gi : Kg - 1;
-          sreg[r][sp] = (float)s16[(size_t)nc * Kg + gi];
-          zreg[r][sp] = zp ? (float)zp[(size_t)nc * Kg + gi] : 8.0f;
+          b.s[r][sp] = (float)s16[(size_t)nc * Kg + gi];
+          b.z[r][sp] = zp ? (float)zp[(size_t)nc * Kg + gi] : 8.0f;
         } else if constexpr (FMT == RF_Q4K) {
           const int Kc = K >> 5;
           const int ci = chunk < Kc ? chunk : Kc - 1;
-          sreg[r][sp] = (float)s16[(size_t)nc * Kc + ci];
-          zreg[r][sp] = (float)qmin[(size_t)nc * Kc + ci];
+          b.s[r][sp] = (float)s16[(size_t)nc * Kc + ci];
+          b.z[r][sp] = (float)qmin[(size_t)nc * Kc + ci];
         } else if constexpr (SC == RS_BLOCK) {
           const int Kb = (K + 127) >> 7;
           const int kblk = (s * SPAN_K + lane * 16) >> 7;
-          sreg[r][sp] = s32[(size_t)(nc >> 7) * Kb + (kblk < Kb ? kblk : Kb - 1)];
+          b.s[r][sp] = s32[(size_t)(nc >> 7) * Kb + (kblk < Kb ? kblk : Kb - 1)];
         }
       }
     }
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+      for (int sp = 0; sp < SPU; ++sp) {
+        const uint32_t kb = (uint32_t)(sb * SPU + sp) * SPAN_B + lane * 16u;   // byte in row
+        // in-range offsets stay below 2^31; setting the top bit pushes a dead
+        // lane past the buffer's bound (arithmetic, so no branch is formed)
+        const uint32_t dead = (uint32_t)(!(live && (row0 + r < N) && (kb < wrow))) << 31;
+        b.w[r][sp] = __builtin_amdgcn_raw_buffer_load_b128(
+            wr, ((uint32_t)(row0 + r) * wrow + kb) | dead, 0, 2 /* nt */);
+      }
   };
-  load_batch(0);
 
   // ---- stage activations ----
-  {
-    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
-    const int total = MR * pieces_per_row;
-    for (int p = threadIdx.x; p < total; p += NWV * 64) {
-      const int m = p / pieces_per_row;
-      const int q = p - m * pieces_per_row;          // (s*PPL + i)*64 + l
-      const int l = q & 63;
-      const int si = q >> 6;
-      const int s = si / PPL, i = si - s * PPL;
-      const int k = s * SPAN_K + (l * PPL + i) * 8;
-      u32x4 v = buf_load16(xr, (m < M && k < K) ? ((uint32_t)m * K + k) * 2u : kOOB);
-      if constexpr (kNib) {
-        // natural pairs (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x4)(x1 x5)(x2 x6)(x3 x7)
-        const uint32_t d0 = v[0], d1 = v[1], d2 = v[2], d3 = v[3];
-        uint32_t e0 = __builtin_amdgcn_perm(d2, d0, 0x05040100u);   // lo(d0), lo(d2)
-        uint32_t e1 = __builtin_amdgcn_perm(d2, d0, 0x07060302u);   // hi(d0), hi(d2)
-        uint32_t e2 = __builtin_amdgcn_perm(d3, d1, 0x05040100u);
-        uint32_t e3 = __builtin_amdgcn_perm(d3, d1, 0x07060302u);
-        if constexpr (Act::dt == DT_F16) {
-          // odd nibbles are planted 4 bits up (1024 + 16 nib): feed them x / 16
-          const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-          e1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, e1) * sixteenth);
-          e3 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, e3) * sixteenth);
-        }
-        v = u32x4{e0, e1, e2, e3};
+  // The vector-memory counter retires in order, so the activation loads are
+  // issued BEFORE the weight prefetch: waiting for them then leaves the weight
+  // loads in flight.  XPRE loads per thread go out up front; anything beyond
+  // that (large M x K) is fetched after the prefetch and waits for it.
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+  const int total = MR * pieces_per_row;
+  constexpr int XPRE = 4;
+  auto x_offset = [&](int p) -> uint32_t {
+    const int m = (p >= pieces_per_row) + (p >= 2 * pieces_per_row) + (p >= 3 * pieces_per_row);
+    const int q = p - m * pieces_per_row;          // (s*PPL + i)*64 + l
+    const int l = q & 63;
+    const int si = q >> 6;
+    const int s = si / PPL, i = si - s * PPL;
+    const int k = s * SPAN_K + (l * PPL + i) * 8;
+    const uint32_t dead = (uint32_t)(!(p < total && m < M && k < K)) << 31;
+    return (((uint32_t)m * K + k) * 2u) | dead;
+  };
+  auto x_store = [&](int p, u32x4 v) {
+    if constexpr (kNib) {
+      // natural pairs (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x4)(x1 x5)(x2 x6)(x3 x7)
+      const uint32_t d0 = v[0], d1 = v[1], d2 = v[2], d3 = v[3];
+      uint32_t e0 = __builtin_amdgcn_perm(d2, d0, 0x05040100u);   // lo(d0), lo(d2)
+      uint32_t e1 = __builtin_amdgcn_perm(d2, d0, 0x07060302u);   // hi(d0), hi(d2)
+      uint32_t e2 = __builtin_amdgcn_perm(d3, d1, 0x05040100u);
+      uint32_t e3 = __builtin_amdgcn_perm(d3, d1, 0x07060302u);
+      if constexpr (Act::dt == DT_F16) {
+        // odd nibbles are planted 4 bits up (1024 + 16 nib): feed them x / 16
+        const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+        e1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, e1) * sixteenth);
+        e3 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, e3) * sixteenth);
       }
-      xs[p] = v;
+      v = u32x4{e0, e1, e2, e3};
     }
+    if (p < total) xs[p] = v;
+  };
+  u32x4 xpre[XPRE];
+#pragma unroll
+  for (int t = 0; t < XPRE; ++t) xpre[t] = buf_load16(xr, x_offset(threadIdx.x + t * NWV * 64));
+
+  auto advance = [&](int& g, int& sb) {
+    if (++sb == nbatch) { sb = 0; g += stride; }
+  };
+  // ring of NBUF register buffers: NBUF - 1 batches are in flight while one is consumed
+  Batch buf[NBUF];
+  int gq[NBUF], sq[NBUF];
+  int g_next = blockIdx.x * NWV + wave, sb_next = 0;
+#pragma unroll
+  for (int i = 0; i < NBUF - 1; ++i) {
+    gq[i] = g_next; sq[i] = sb_next;
+    load_batch(buf[i], g_next, sb_next);
+    advance(g_next, sb_next);
+  }
+  float pert_scale = 1.0f;
+  if constexpr (kFp8 && SC == RS_PERT) pert_scale = ((const float*)a.s[0])[0];
+
+  {
+#pragma unroll
+    for (int t = 0; t < XPRE; ++t) x_store(threadIdx.x + t * NWV * 64, xpre[t]);
+    for (int p = threadIdx.x + XPRE * NWV * 64; p < total; p += NWV * 64)
+      x_store(p, buf_load16(xr, x_offset(p)));
     if constexpr (kNib) {
       // per 32-k chunk: what the planted constants contribute (c1) and sum x (c2),
       // summed in a fixed order from the staged image
@@ -214,11 +293,10 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
 
-  for (int s0 = 0; s0 < nspan; s0 += SPU) {
-    if (s0 > 0) load_batch(s0);
+  auto compute = [&](const Batch& b, int sb) {
 #pragma unroll
     for (int sp = 0; sp < SPU; ++sp) {
-      const int s = s0 + sp;
+      const int s = sb * SPU + sp;
       if (s < nspan) {                                // wave-uniform
         u32x4 xp[MR][PPL];
 #pragma unroll
@@ -227,7 +305,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
           for (int i = 0; i < PPL; ++i) xp[m][i] = xs[m * pieces_per_row + (s * PPL + i) * 64 + lane];
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-          const u32x4 w = wreg[r][sp];
+          const u32x4 w = b.w[r][sp];
           float part[MR];
 #pragma unroll
           for (int m = 0; m < MR; ++m) part[m] = 0.f;
@@ -244,7 +322,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
             }
             if constexpr (SC == RS_BLOCK) {
 #pragma unroll
-              for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * sreg[r][sp];
+              for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * b.s[r][sp];
             } else {
 #pragma unroll
               for (int m = 0; m < MR; ++m) acc[r][m] += part[m];
@@ -273,50 +351,66 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
                 part[m] = Dot2<Act>::run(t3, xp[m][d][3], part[m]);
               }
             }
-            if constexpr (FMT == RF_INT4) {
-              const float sc = sreg[r][sp];
-              const float z = zreg[r][sp];
+            const float sc = b.s[r][sp];
+            const float zz = b.z[r][sp];
 #pragma unroll
-              for (int m = 0; m < MR; ++m) {
-                const float corr = part[m] - c1[(m * nspan + s) * 64 + lane] -
-                                   z * c2[(m * nspan + s) * 64 + lane];
-                acc[r][m] += sc * corr;
-              }
-            } else {
-              const float sc = sreg[r][sp];
-              const float mn = zreg[r][sp];
-#pragma unroll
-              for (int m = 0; m < MR; ++m) {
-                const float corr = part[m] - c1[(m * nspan + s) * 64 + lane];
-                acc[r][m] += sc * corr - mn * c2[(m * nspan + s) * 64 + lane];
-              }
+            for (int m = 0; m < MR; ++m) {
+              const float k1 = c1[(m * nspan + s) * 64 + lane];
+              const float k2 = c2[(m * nspan + s) * 64 + lane];
+              if constexpr (FMT == RF_INT4)
+                acc[r][m] += sc * (part[m] - k1 - zz * k2);
+              else
+                acc[r][m] += sc * (part[m] - k1) - zz * k2;
             }
           }
         }
       }
     }
-  }
+  };
 
-  // ---- finish the K reduction inside the wavefront, lane 0 stores ----
+  // finish the K reduction inside the wavefront, lane 0 stores, accumulators reset
   using Elem = typename Act::elem;
-  Elem* out = (Elem*)a.out[mat];
+  auto finish = [&](const Batch& b, int g) {
+    int mat, row0;
+    locate(g, mat, row0);
+    const int N = QLIN_PICK(N, mat);
+    Elem* out = (Elem*)QLIN_PICK(out, mat);
 #pragma unroll
-  for (int r = 0; r < RW; ++r) {
-    const int n = row0 + r;
-    float os = 1.0f;
-    if constexpr (kFp8 && SC == RS_PERN) {
-      if (n < N) os = a.scale_f16 ? (float)s16[n] : s32[n];
+    for (int r = 0; r < RW; ++r) {
+      const int n = row0 + r;
+      float os = 1.0f;
+      if constexpr (kFp8 && SC == RS_PERN)
+        os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, b.os_lo[r])
+                         : __builtin_bit_cast(float, (uint32_t)b.os_lo[r] | ((uint32_t)b.os_hi[r] << 16));
+      if constexpr (kFp8 && SC == RS_PERT) os = pert_scale;
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        const float v = wave_sum(acc[r][m]);
+        acc[r][m] = 0.f;
+        if (lane == 0 && n < N && m < M) out[(size_t)m * N + n] = Act::from_f32(v * os);
+      }
     }
-    if constexpr (kFp8 && SC == RS_PERT) os = s32[0];
+  };
+
+  // ---- walk the wave's batches; buffer indices are static after unrolling ----
+  bool more = true;
+  while (more) {
 #pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      const float v = wave_sum(acc[r][m]);
-      if (lane == 0 && n < N) out[(size_t)m * N + n] = Act::from_f32(v * os);
+    for (int i = 0; i < NBUF; ++i) {
+      constexpr int dummy = 0; (void)dummy;
+      const int j = (i + NBUF - 1) % NBUF;
+      gq[j] = g_next; sq[j] = sb_next;
+      load_batch(buf[j], g_next, sb_next);
+      advance(g_next, sb_next);
+      if (gq[i] >= ngroups) { more = false; break; }
+      compute(buf[i], sq[i]);
+      if (sq[i] == nbatch - 1) finish(buf[i], gq[i]);
     }
   }
+#undef QLIN_PICK
 }
 
-// LDS bytes the kernel needs for a given shape (0 = not applicable).
+// LDS bytes the kernel needs for a given shape.
 static inline size_t rows_lds_bytes(int fmt, int MR, int K) {
   const int ppl = fmt == RF_FP8 ? 2 : 4;
   const int span_k = 64 * ppl * 8;
@@ -326,23 +420,64 @@ static inline size_t rows_lds_bytes(int fmt, int MR, int K) {
   return b;
 }
 
-template <class Act, int FMT, int SC, int MR>
-static void launch_rows(RowsArgs a, hipStream_t st) {
+static inline int device_cu_count() {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+template <class Act, int FMT, int SC, int MR, int RW>
+static void launch_rows_rw(RowsArgs a, hipStream_t st) {
   constexpr int NWV = 8;
-  constexpr int RW = FMT == RF_FP8 ? 2 : 4;
+  constexpr int NBUF = 2;
   constexpr int SPU = FMT == RF_FP8 ? 4 : 2;
-  constexpr int ppl = FMT == RF_FP8 ? 2 : 4;
-  constexpr int span_k = 64 * ppl * 8;
-  a.nspan = (a.K + span_k - 1) / span_k;
   int groups = 0;
-  for (int i = 0; i < a.nmat; ++i) {
-    a.groups[i] = (a.N[i] + NWV * RW - 1) / (NWV * RW);
+  for (int i = 0; i < kRowsMaxMat; ++i) {
+    a.groups[i] = i < a.nmat ? (a.N[i] + RW - 1) / RW : 0;
     groups += a.groups[i];
   }
   if (!groups) return;
+  // persistent grid: the workgroup count (per CU) that wastes the fewest wave slots
+  const int cus = device_cu_count();
+  int best_wgs = 0;
+  double best_eff = -1.0;
+  for (int per_cu = 1; per_cu <= 4; ++per_cu) {
+    const long waves = (long)cus * per_cu * NWV;
+    const long iters = (groups + waves - 1) / waves;
+    const double eff = (double)groups / (double)(iters * waves);
+    if (eff > best_eff + 1e-9) { best_eff = eff; best_wgs = cus * per_cu; }
+  }
+  const int needed = (groups + NWV - 1) / NWV;
+  const int wgs = needed < best_wgs ? needed : best_wgs;
+  a.total_waves = wgs * NWV;
   const size_t lds = rows_lds_bytes(FMT, MR, a.K);
-  hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU>), dim3(groups), dim3(NWV * 64), lds,
-                     st, a);
+  if (a.nmat == 1)
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false>), dim3(wgs), dim3(NWV * 64),
+                       lds, st, a);
+  else
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true>), dim3(wgs), dim3(NWV * 64),
+                       lds, st, a);
+}
+
+template <class Act, int FMT, int SC, int MR>
+static void launch_rows(RowsArgs a, hipStream_t st) {
+  constexpr int ppl = FMT == RF_FP8 ? 2 : 4;
+  constexpr int span_k = 64 * ppl * 8;
+  constexpr int SPU = FMT == RF_FP8 ? 4 : 2;
+  a.nspan = (a.K + span_k - 1) / span_k;
+  const int per_batch = a.nspan < SPU ? a.nspan : SPU;     // loads per row per batch
+  if (per_batch >= 4)
+    launch_rows_rw<Act, FMT, SC, MR, 1>(a, st);
+  else if (per_batch >= 2)
+    launch_rows_rw<Act, FMT, SC, MR, 2>(a, st);
+  else
+    launch_rows_rw<Act, FMT, SC, MR, 4>(a, st);
 }
 
 template <class Act, int FMT, int SC>
@@ -350,7 +485,6 @@ static void launch_rows_m(const RowsArgs& a, hipStream_t st) {
   switch (a.M) {
     case 1: launch_rows<Act, FMT, SC, 1>(a, st); break;
     case 2: launch_rows<Act, FMT, SC, 2>(a, st); break;
-    case 3: launch_rows<Act, FMT, SC, 3>(a, st); break;
     default: launch_rows<Act, FMT, SC, 4>(a, st); break;
   }
 }
