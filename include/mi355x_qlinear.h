@@ -104,6 +104,62 @@ int mi_dequant_q4k(const void* ql, const void* scale, const void* qmin, void* ou
                    void* stream);
 int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int K, void* stream);
 
+/* ---- MoE routing and permutation --------------------------------------------
+ * mi_moe_topk: fp32 softmax over E experts -> top-K (lowest index wins ties,
+ *   descending probability) -> optional renormalisation; top_w in the activation
+ *   dtype, top_ids int32.  E <= 1024, K <= 64.  Replaces esimd_moe_topk /
+ *   moe_ops::moe_topk (V/csrc/xpu/esimd_kernels/moe_ops.h:106-231,
+ *   V/csrc/xpu/esimd_kernel_moe.sycl:71-84).
+ * mi_moe_sort: stable counting sort of the T*K (token, route) pairs by expert:
+ *   sorted_pairs[pos] = t*K + j, expert_start[E+1] (exclusive prefix of counts),
+ *   inv[t*K + j] = pos, optional sorted_token[pos] = t and max_count[0] = largest
+ *   expert load.  Deterministic; the K experts of a token must be distinct.
+ *   Same result as build_sorted_token_ids / build_topk_ids
+ *   (V/csrc/xpu/esimd_kernels/moe_ops.h:238-271); replaces the scatter
+ *   init/prefix kernels (:437-520) and moe_prefill_gather_forward_kernel_fp8
+ *   (S/csrc/moe_prefill/moe_prefill_fp8.sycl:105-161), whose in-expert order is
+ *   atomic-arrival order. */
+int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
+                int act_dtype, void* stream);
+int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
+                int32_t* sorted_token, int32_t* max_count, int T, int K, int E, void* stream);
+
+/* ---- MoE elementwise helpers -------------------------------------------------
+ * mi_act_quant_fp8: per row, per 128-wide K group: s = max|x|/448 (>= 1e-12/448),
+ *   q = e4m3(x / s).  No counterpart in the reference's kernels (they are w8a16,
+ *   V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:5-7).
+ * mi_moe_silu_mul: out[r, c] = silu(in[r, c]) * in[r, n_half + c]
+ *   (esimd_moe_silu_mul, V/csrc/xpu/esimd_kernels/moe_ops.h:576-621).
+ * mi_moe_scatter: scattered[pos] = hidden[sorted_pairs[pos] / topk], optional
+ *   scattered_w[pos] = top_w[sorted_pairs[pos]]   (esimd_moe_scatter, moe_ops.h:522-569).
+ * mi_moe_combine: out[t] = sum_j w * y[inv[t*topk + j]], weights indexed by sorted
+ *   position (weights_by_position = 1, esimd_moe_gather, moe_ops.h:627-676) or by
+ *   pair; y is in the activation dtype, or fp32 when y_f32 = 1. */
+int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K, int act_dtype,
+                     void* stream);
+int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
+                    void* stream);
+int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_pairs, void* scattered,
+                   void* scattered_w, int K, int topk, int total, void* stream);
+int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
+                   int weights_by_position, int act_dtype, int y_f32, void* stream);
+
+/* ---- MoE grouped FP8 block-scaled GEMM ----------------------------------------
+ * out[r, :] = a[src(r), :] @ dequant(w[e])^T for the rows r of expert e,
+ * expert_start[e] <= r < expert_start[e+1]; src(r) = row_map[r] if row_map else r.
+ * w [E, N, K] e4m3, w_scale [E, ceil(N/128), K/128] fp32, K % 128 == 0.
+ * a_scale == NULL: a is fp16/bf16 (w8a16) — replaces esimd_moe_gemm_fp8_blockscale
+ *   (V/csrc/xpu/esimd_kernel_moe.sycl:201-269,
+ *   V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:123-334).
+ * a_scale != NULL: a is e4m3 with per-row per-128 scales [a_rows, K/128]; native
+ *   fp8 MFMA.  fuse_silu_mul: weight rows [0, N/2) are gate, [N/2, N) up; out is
+ *   [total_rows, N/2] = silu(gate) * up.  Both have no reference counterpart.
+ * out is in the activation dtype (act_dtype), or fp32 when out_f32 = 1. */
+int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
+                          const float* w_scale, const int32_t* expert_start, void* out, int a_rows,
+                          int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,
+                          int out_f32, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,361 @@
+// MoE auxiliary kernels: routing (softmax + top-k), the expert-sorted token
+// permutation, dynamic activation quantisation, SiLU*mul, row scatter and the
+// weighted top-k combine.  All are small, HBM- or latency-bound integer / byte /
+// elementwise kernels; none of them is reshaped into a GEMM.
+#include "qlinear_common.hpp"
+#include "../../include/mi355x_qlinear.h"
+
+namespace qlin {
+
+// ---------------------------------------------------------------- top-k
+// One wavefront per token.  Expert e lives in lane e % 64, slot e / 64.  The
+// selection runs on the logits (softmax is monotone): K rounds of wave-wide
+// argmax where the LOWEST index wins ties, then the selected probabilities are
+// renormalised.
+constexpr int kTopkSlots = 16;                       // up to 1024 experts
+
+template <class Act>
+__global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,
+                                                       typename Act::elem* __restrict__ top_w,
+                                                       int32_t* __restrict__ top_ids, int T, int E,
+                                                       int K, int renorm) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const typename Act::elem* row = logits + (size_t)t * E;
+  float v[kTopkSlots];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < kTopkSlots; ++s) {
+    const int e = s * 64 + lane;
+    v[s] = e < E ? Act::to_f32(row[e]) : -INFINITY;
+    mx = fmaxf(mx, v[s]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int s = 0; s < kTopkSlots; ++s) sum += (s * 64 + lane < E) ? __expf(v[s] - mx) : 0.f;
+  sum = wave_sum(sum);
+
+  float my_w = 0.f;                                  // lane r keeps the r-th pick
+  int my_id = 0;
+  float sel_sum = 0.f;
+  for (int r = 0; r < K; ++r) {
+    float best = -INFINITY;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int s = 0; s < kTopkSlots; ++s) {
+      if (v[s] > best) { best = v[s]; best_e = s * 64 + lane; }   // strict: lowest slot kept
+    }
+    const float wbest = wave_max(best);
+    int cand = (best == wbest) ? best_e : 0x7fffffff;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+    // remove the winner from its owner lane
+#pragma unroll
+    for (int s = 0; s < kTopkSlots; ++s)
+      if (s * 64 + lane == cand) v[s] = -INFINITY;
+    const float p = __expf(wbest - mx) / sum;
+    sel_sum += p;
+    if (lane == r) { my_w = p; my_id = cand; }
+  }
+  if (lane < K) {
+    const float w = renorm ? my_w / sel_sum : my_w;
+    top_w[(size_t)t * K + lane] = Act::from_f32(w);
+    top_ids[(size_t)t * K + lane] = my_id;
+  }
+}
+
+// ---------------------------------------------------------------- sort
+// Stable counting sort of the flattened (token, route) pairs by expert, in one
+// workgroup, deterministic.  Inside an expert the pairs keep their pair-index
+// order.  Because a token's K experts are distinct, the rank of pair (t, j) in
+// expert e equals the number of tokens t' < t that selected e: a per-expert
+// bitmap over tokens (built with order-independent LDS atomic ORs) plus popcounts
+// gives the rank without any ordered atomics.  Tokens are processed in chunks
+// that fit the LDS bitmap.
+constexpr int kSortThreads = 1024;
+constexpr int kSortWords = 4096;                     // bitmap words in LDS
+
+__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
+    const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
+    int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
+    int32_t* __restrict__ max_count, int T, int K, int E) {
+  __shared__ uint32_t bitmap[kSortWords];
+  __shared__ uint32_t wordpre[kSortWords];
+  __shared__ int32_t count[1024];
+  __shared__ int32_t start[1025];
+  __shared__ int32_t base[1024];
+  const int tid = threadIdx.x;
+  const int P = T * K;
+  const int wpe = kSortWords / E;                     // words per expert in one chunk
+  const int Tc = wpe * 32;                            // tokens per chunk
+
+  if (tid < E) { count[tid] = 0; base[tid] = 0; }
+  __syncthreads();
+  for (int p = tid; p < P; p += kSortThreads) atomicAdd(&count[top_ids[p]], 1);
+  __syncthreads();
+  // exclusive prefix over experts (Hillis-Steele on up to 1024 entries)
+  if (tid < E) start[tid + 1] = count[tid];
+  if (tid == 0) start[0] = 0;
+  __syncthreads();
+  for (int off = 1; off < E; off <<= 1) {
+    int add = 0;
+    if (tid < E && tid >= off) add = start[tid + 1 - off];
+    __syncthreads();
+    if (tid < E) start[tid + 1] += add;
+    __syncthreads();
+  }
+  for (int i = tid; i <= E; i += kSortThreads) expert_start[i] = start[i];
+  if (max_count) {
+    __shared__ int32_t mx;
+    if (tid == 0) mx = 0;
+    __syncthreads();
+    if (tid < E) atomicMax(&mx, count[tid]);
+    __syncthreads();
+    if (tid == 0) max_count[0] = mx;
+  }
+
+  for (int t0 = 0; t0 < T; t0 += Tc) {
+    const int tn = min(Tc, T - t0);
+    for (int i = tid; i < E * wpe; i += kSortThreads) bitmap[i] = 0;
+    __syncthreads();
+    for (int q = tid; q < tn * K; q += kSortThreads) {
+      const int tl = q / K;
+      const int e = top_ids[(size_t)t0 * K + q];
+      atomicOr(&bitmap[e * wpe + (tl >> 5)], 1u << (tl & 31));
+    }
+    __syncthreads();
+    if (tid < E) {
+      uint32_t run = 0;
+      for (int w = 0; w < wpe; ++w) {
+        wordpre[tid * wpe + w] = run;
+        run += __popc(bitmap[tid * wpe + w]);
+      }
+      count[tid] = (int32_t)run;                      // pairs of this expert in the chunk
+    }
+    __syncthreads();
+    for (int q = tid; q < tn * K; q += kSortThreads) {
+      const int tl = q / K;
+      const int p = t0 * K + q;
+      const int e = top_ids[p];
+      const uint32_t word = bitmap[e * wpe + (tl >> 5)];
+      const int rank = base[e] + (int)wordpre[e * wpe + (tl >> 5)] +
+                       __popc(word & ((1u << (tl & 31)) - 1u));
+      const int pos = start[e] + rank;
+      sorted_pairs[pos] = p;
+      inv[p] = pos;
+      if (sorted_token) sorted_token[pos] = t0 + tl;
+    }
+    __syncthreads();
+    if (tid < E) base[tid] += count[tid];
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------- activation quant
+// Per row, per 128-wide group: s = max|x| / 448 (clamped at 1e-12), q = e4m3(x / s).
+// 16 lanes own one group (8 elements each); the group maximum is a DPP butterfly
+// inside the 16-lane row.
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+  return fmaxf(v, __builtin_bit_cast(float, moved));
+}
+
+template <class Act>
+__global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* __restrict__ x,
+                                                        u32x2* __restrict__ q, float* __restrict__ s,
+                                                        size_t groups16) {   // 16-lane groups in total
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;     // one lane = 8 elements
+  const bool live = (i >> 4) < groups16;
+  typename Act::v8 v;
+  if (live) v = x[i];
+  float f[8];
+  float amax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    f[e] = live ? Act::to_f32(v[e]) : 0.f;
+    amax = fmaxf(amax, fabsf(f[e]));
+  }
+  amax = dpp_max<0xB1>(amax);
+  amax = dpp_max<0x4E>(amax);
+  amax = dpp_max<0x141>(amax);
+  amax = dpp_max<0x140>(amax);
+  const float scale = fmaxf(amax, 1e-12f) / 448.0f;
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] / scale, f[1] / scale, lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] / scale, f[3] / scale, lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4] / scale, f[5] / scale, hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6] / scale, f[7] / scale, hi, true);
+  if (live) {
+    q[i] = u32x2{(uint32_t)lo, (uint32_t)hi};
+    if ((threadIdx.x & 15) == 0) s[i >> 4] = scale;
+  }
+}
+
+// ---------------------------------------------------------------- elementwise
+template <class Act>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const typename Act::elem* __restrict__ in,
+                                                       typename Act::elem* __restrict__ out, int n_gate_up,
+                                                       int n_half, int rows) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)rows * n_half) return;
+  const int r = (int)(i / n_half), c = (int)(i % n_half);
+  const float g = Act::to_f32(in[(size_t)r * n_gate_up + c]);
+  const float u = Act::to_f32(in[(size_t)r * n_gate_up + n_half + c]);
+  out[i] = Act::from_f32(g / (1.0f + expf(-g)) * u);
+}
+
+// scattered[pos] = hidden[pair / topk], weights[pos] = top_w[pair]   (pos -> pair = sorted_pairs[pos])
+__global__ __launch_bounds__(256) void scatter_rows_kernel(const u32x4* __restrict__ hidden,
+                                                           const uint16_t* __restrict__ top_w,
+                                                           const int32_t* __restrict__ sorted_pairs,
+                                                           u32x4* __restrict__ scattered,
+                                                           uint16_t* __restrict__ weights, int K8, int topk,
+                                                           int total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)total * K8) return;
+  const int pos = (int)(i / K8), c = (int)(i % K8);
+  const int pair = sorted_pairs[pos];
+  scattered[i] = hidden[(size_t)(pair / topk) * K8 + c];
+  if (c == 0 && weights) weights[pos] = top_w[pair];
+}
+
+// final[t] = sum_j w_j * y[pos(t, j)]; weights either per sorted position
+// (by_pos = 1, the reference's scattered_weights) or per pair (top_w).
+template <class Act, bool Y32>
+__global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ yv,
+                                                      const int32_t* __restrict__ inv,
+                                                      const typename Act::elem* __restrict__ w,
+                                                      typename Act::v8* __restrict__ out, int H8, int topk,
+                                                      int T, int by_pos) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)T * H8) return;
+  const int t = (int)(i / H8), c = (int)(i % H8);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < topk; ++j) {
+    const int pos = inv[(size_t)t * topk + j];
+    const float wj = Act::to_f32(w[by_pos ? pos : t * topk + j]);
+    if constexpr (Y32) {
+      const f32x4* y = (const f32x4*)yv;
+      const f32x4 a = y[((size_t)pos * H8 + c) * 2], b = y[((size_t)pos * H8 + c) * 2 + 1];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { acc[e] += wj * a[e]; acc[4 + e] += wj * b[e]; }
+    } else {
+      const typename Act::v8 v = ((const typename Act::v8*)yv)[(size_t)pos * H8 + c];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += wj * Act::to_f32(v[e]);
+    }
+  }
+  typename Act::v8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = Act::from_f32(acc[e]);
+  out[i] = o;
+}
+
+static inline dim3 grid1d(size_t n, int bs = 256) { return dim3((unsigned)((n + bs - 1) / bs)); }
+
+}  // namespace qlin
+
+using namespace qlin;
+
+extern "C" {
+
+int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
+                int act_dtype, void* stream) {
+  if (!logits || !top_w || !top_ids) return MI_ERR_ARG;
+  if (T < 0 || E < 1 || E > 64 * kTopkSlots || K < 1 || K > 64 || K > E) return MI_ERR_SHAPE;
+  if (!T) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(moe_topk_kernel<ActF16>, dim3((T + 3) / 4), dim3(256), 0, st, (const _Float16*)logits,
+                       (_Float16*)top_w, top_ids, T, E, K, renorm);
+  else if (act_dtype == DT_BF16)
+    hipLaunchKernelGGL(moe_topk_kernel<ActBF16>, dim3((T + 3) / 4), dim3(256), 0, st, (const __bf16*)logits,
+                       (__bf16*)top_w, top_ids, T, E, K, renorm);
+  else
+    return MI_ERR_ARG;
+  return launch_status();
+}
+
+int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
+                int32_t* sorted_token, int32_t* max_count, int T, int K, int E, void* stream) {
+  if (!expert_start) return MI_ERR_ARG;
+  if (T < 0 || K < 1 || E < 1 || E > 1024) return MI_ERR_SHAPE;
+  if (T > 0 && (!top_ids || !sorted_pairs || !inv)) return MI_ERR_ARG;   // T == 0 only fills expert_start
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(kSortThreads), 0, (hipStream_t)stream, top_ids,
+                     sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+  return launch_status();
+}
+
+int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K, int act_dtype,
+                     void* stream) {
+  if (!x || !q || !scale) return MI_ERR_ARG;
+  if (rows < 0 || K <= 0 || (K % 128)) return MI_ERR_SHAPE;
+  const size_t groups16 = (size_t)rows * (K / 128);
+  if (!groups16) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid = grid1d(groups16 * 16);
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(act_quant_kernel<ActF16>, grid, dim3(256), 0, st, (const f16x8*)x, (u32x2*)q, scale,
+                       groups16);
+  else if (act_dtype == DT_BF16)
+    hipLaunchKernelGGL(act_quant_kernel<ActBF16>, grid, dim3(256), 0, st, (const bf16x8*)x, (u32x2*)q, scale,
+                       groups16);
+  else
+    return MI_ERR_ARG;
+  return launch_status();
+}
+
+int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
+                    void* stream) {
+  if (!in || !out) return MI_ERR_ARG;
+  if (rows < 0 || n_half <= 0 || n_gate_up != 2 * n_half) return MI_ERR_SHAPE;
+  if (!rows) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid = grid1d((size_t)rows * n_half);
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(silu_mul_kernel<ActF16>, grid, dim3(256), 0, st, (const _Float16*)in, (_Float16*)out,
+                       n_gate_up, n_half, rows);
+  else if (act_dtype == DT_BF16)
+    hipLaunchKernelGGL(silu_mul_kernel<ActBF16>, grid, dim3(256), 0, st, (const __bf16*)in, (__bf16*)out,
+                       n_gate_up, n_half, rows);
+  else
+    return MI_ERR_ARG;
+  return launch_status();
+}
+
+int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_pairs, void* scattered,
+                   void* scattered_w, int K, int topk, int total, void* stream) {
+  if (!hidden || !sorted_pairs || !scattered) return MI_ERR_ARG;
+  if (K <= 0 || (K % 8) || topk < 1 || total < 0) return MI_ERR_SHAPE;
+  if (scattered_w && !top_w) return MI_ERR_ARG;
+  if (!total) return MI_OK;
+  hipLaunchKernelGGL(scatter_rows_kernel, grid1d((size_t)total * (K / 8)), dim3(256), 0, (hipStream_t)stream,
+                     (const u32x4*)hidden, (const uint16_t*)top_w, sorted_pairs, (u32x4*)scattered,
+                     (uint16_t*)scattered_w, K / 8, topk, total);
+  return launch_status();
+}
+
+int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
+                   int weights_by_position, int act_dtype, int y_f32, void* stream) {
+  if (!y || !inv || !w || !out) return MI_ERR_ARG;
+  if (H <= 0 || (H % 8) || topk < 1 || T < 0) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (!T) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid = grid1d((size_t)T * (H / 8));
+#define QLIN_COMBINE(ACT, Y32, WT, OT)                                                                   \
+  hipLaunchKernelGGL((combine_kernel<ACT, Y32>), grid, dim3(256), 0, st, y, inv, (const WT*)w, (OT*)out, \
+                     H / 8, topk, T, weights_by_position)
+  if (act_dtype == DT_F16) {
+    if (y_f32) QLIN_COMBINE(ActF16, true, _Float16, f16x8); else QLIN_COMBINE(ActF16, false, _Float16, f16x8);
+  } else {
+    if (y_f32) QLIN_COMBINE(ActBF16, true, __bf16, bf16x8); else QLIN_COMBINE(ActBF16, false, __bf16, bf16x8);
+  }
+#undef QLIN_COMBINE
+  return launch_status();
+}
+
+}  // extern "C"

@@ -70,3 +70,85 @@ def fp8_dequant(weight, weight_scale, output, mode):
 
 def e4m3_decode(codes, output):
     return _ops.e4m3_decode(codes, output)
+
+
+# ---- MoE ----
+_moe = torch.ops.moe_ops
+
+
+def esimd_moe_topk(router_logits, top_values, top_indices, T):
+    """router_logits [T, E], top_values [T, K] (output, logits dtype), top_indices [T, K] int32 (output)."""
+    return _ops.esimd_moe_topk(router_logits, top_values, top_indices, T)
+
+
+def esimd_moe_scatter(hidden_states, router_top_value, sorted_token_ids, scattered_hidden, scattered_weights,
+                      K, topk, total_expanded):
+    return _ops.esimd_moe_scatter(hidden_states, router_top_value, sorted_token_ids, scattered_hidden,
+                                  scattered_weights, K, topk, total_expanded)
+
+
+def esimd_moe_scatter_fused(hidden_states, top_values, top_indices, scattered_hidden, scattered_weights,
+                            topk_ids, expert_start, max_tokens_out, K, topk, T, num_experts):
+    return _ops.esimd_moe_scatter_fused(hidden_states, top_values, top_indices, scattered_hidden,
+                                        scattered_weights, topk_ids, expert_start, max_tokens_out,
+                                        K, topk, T, num_experts)
+
+
+def esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows):
+    return _ops.esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows)
+
+
+def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T):
+    return _ops.esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T)
+
+
+def esimd_moe_gemm_fp8_blockscale(input, weight, weight_scale, output, expert_idx, N, K, num_experts,
+                                  block_n=128, block_k=128):
+    """input [total_tokens, K] (expert-grouped rows), weight [E, N, K] e4m3, weight_scale
+    [E, ceil(N/128), K/128] fp32, expert_idx [E+1] start offsets; activations stay 16 bit."""
+    return _ops.esimd_moe_gemm_fp8_blockscale(input, weight, weight_scale, output, expert_idx,
+                                              N, K, num_experts, block_n, block_k)
+
+
+def moe_topk(logits, top_k, norm=True):
+    return _moe.moe_topk(logits, top_k, norm)
+
+
+def moe_sort(top_ids, num_experts, sorted_pairs, expert_start, inv, sorted_token=None, max_count=None):
+    return _ops.moe_sort(top_ids, num_experts, sorted_pairs, expert_start, inv, sorted_token, max_count)
+
+
+def act_quant_fp8(x, q, scale):
+    return _ops.act_quant_fp8(x, q, scale)
+
+
+def moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, output, N, K,
+                       num_experts, fuse_silu_mul=False):
+    """Grouped block-FP8 GEMM; a_scale None -> 16-bit activations (w8a16), else e4m3 activations
+    with per-row per-128 scales.  Optional row gather, fused SiLU*mul, fp32 output."""
+    return _ops.moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, output,
+                                   N, K, num_experts, fuse_silu_mul)
+
+
+def moe_combine(y, inv, top_w, output, top_k):
+    return _ops.moe_combine(y, inv, top_w, output, top_k)
+
+
+def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale, output,
+                          top_k, act_quant=True):
+    return _ops.moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                                      output, top_k, act_quant)
+
+
+def precompute_moe_route(topk_weights, topk_ids, num_experts):
+    """Same contract as the reference helper: (sorted_rows, sorted_weights, rows_per_expert),
+    stable by expert; computed on the device by the sort kernel."""
+    T, k = topk_ids.shape
+    dev = topk_ids.device
+    ids = topk_ids.to(torch.int32).contiguous()
+    pairs = torch.empty(T * k, dtype=torch.int32, device=dev)
+    start = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(T * k, dtype=torch.int32, device=dev)
+    tok = torch.empty(T * k, dtype=torch.int32, device=dev)
+    moe_sort(ids, num_experts, pairs, start, inv, tok, None)
+    return tok.to(torch.int64), topk_weights.reshape(-1)[pairs.long()].contiguous(), (start[1:] - start[:-1]).contiguous()

@@ -320,6 +320,260 @@ def e4m3_decode(codes, output):
     return output
 
 
+
+# --------------------------------------------------------------------------
+# MoE: routing, permutation, grouped GEMM, combine
+# --------------------------------------------------------------------------
+def esimd_moe_topk(router_logits, top_values, top_indices, T):
+    who = "esimd_moe_topk"
+    _chk(router_logits.dim() == 2 and router_logits.is_contiguous(), f"{who}: router_logits must be contiguous [T, E]")
+    T = int(T)
+    _chk(router_logits.shape[0] >= T, f"{who}: T={T} exceeds router_logits rows")
+    E = router_logits.shape[1]
+    _chk(top_values.dim() == 2 and top_values.dtype == router_logits.dtype and top_values.is_contiguous(),
+         f"{who}: top_values must be contiguous [T, K] in the logits dtype")
+    K = top_values.shape[1]
+    _chk(top_indices.dtype == torch.int32 and top_indices.is_contiguous() and top_indices.numel() >= T * K,
+         f"{who}: top_indices must be contiguous int32 [T, K]")
+    _chk(E <= 1024 and 1 <= K <= min(64, E), f"{who}: needs E <= 1024 and 1 <= K <= min(64, E)")
+    capi.call("mi_moe_topk", router_logits, capi.ptr(router_logits), capi.ptr(top_values),
+              capi.ptr(top_indices), T, E, K, 1, capi.act_dtype(router_logits))
+    return top_values
+
+
+def moe_topk(logits, top_k, norm):
+    """moe_ops::moe_topk(logits, top_k, norm) -> (weights, ids); outputs are allocated here."""
+    _chk(logits.dim() == 2 and logits.is_contiguous(), "moe_topk: logits must be contiguous [T, E]")
+    T, E = logits.shape
+    w = torch.empty(T, int(top_k), dtype=logits.dtype, device=logits.device)
+    ids = torch.empty(T, int(top_k), dtype=torch.int32, device=logits.device)
+    _chk(E <= 1024 and 1 <= int(top_k) <= min(64, E), "moe_topk: needs E <= 1024 and 1 <= top_k <= min(64, E)")
+    capi.call("mi_moe_topk", logits, capi.ptr(logits), capi.ptr(w), capi.ptr(ids), T, E, int(top_k),
+              1 if norm else 0, capi.act_dtype(logits))
+    return w, ids
+
+
+def moe_sort(top_ids, num_experts, sorted_pairs, expert_start, inv, sorted_token=None, max_count=None):
+    """Stable expert sort of the flattened (token, route) pairs; all outputs int32, written in place."""
+    who = "moe_sort"
+    _chk(top_ids.dim() == 2 and top_ids.dtype == torch.int32 and top_ids.is_contiguous(),
+         f"{who}: top_ids must be contiguous int32 [T, K]")
+    T, K = top_ids.shape
+    E = int(num_experts)
+    _chk(1 <= E <= 1024, f"{who}: num_experts must be in 1..1024")
+    for t, n, nm in ((sorted_pairs, T * K, "sorted_pairs"), (expert_start, E + 1, "expert_start"), (inv, T * K, "inv")):
+        _chk(t.dtype in (torch.int32, torch.uint32) and t.is_contiguous() and t.numel() >= n,
+             f"{who}: {nm} must be contiguous int32 with >= {n} entries")
+    if sorted_token is not None:
+        _chk(sorted_token.dtype == torch.int32 and sorted_token.numel() >= T * K, f"{who}: sorted_token must be int32 [T*K]")
+    if max_count is not None:
+        _chk(max_count.dtype == torch.int32 and max_count.numel() >= 1, f"{who}: max_count must be int32 [1]")
+    capi.call("mi_moe_sort", top_ids, capi.ptr(top_ids), capi.ptr(sorted_pairs), capi.ptr(expert_start),
+              capi.ptr(inv), capi.ptr(sorted_token), capi.ptr(max_count), T, K, E)
+    return sorted_pairs
+
+
+def act_quant_fp8(x, q, scale):
+    who = "act_quant_fp8"
+    _chk(x.dim() == 2 and x.is_contiguous() and x.dtype in (torch.float16, torch.bfloat16), f"{who}: x must be contiguous fp16/bf16 [rows, K]")
+    rows, K = x.shape
+    _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+    _chk(q.dtype in _FP8_TYPES and q.is_contiguous() and q.numel() == rows * K, f"{who}: q must be e4m3/uint8 [rows, K]")
+    _chk(scale.dtype == torch.float32 and scale.is_contiguous() and scale.numel() == rows * (K // 128),
+         f"{who}: scale must be fp32 [rows, K/128]")
+    capi.call("mi_act_quant_fp8", x, capi.ptr(x), capi.ptr(q), capi.ptr(scale), rows, K, capi.act_dtype(x))
+    return q
+
+
+def esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows):
+    who = "esimd_moe_silu_mul"
+    _chk_act(input, output, who)
+    _chk(int(N_gate_up) == 2 * int(N_half), f"{who}: N_gate_up must be 2 * N_half")
+    _chk(input.numel() >= int(total_rows) * int(N_gate_up) and output.numel() >= int(total_rows) * int(N_half),
+         f"{who}: tensors too small for total_rows")
+    capi.call("mi_moe_silu_mul", input, capi.ptr(input), capi.ptr(output), int(N_gate_up), int(N_half),
+              int(total_rows), capi.act_dtype(input))
+    return output
+
+
+def esimd_moe_scatter(hidden_states, router_top_value, sorted_token_ids, scattered_hidden, scattered_weights,
+                      K, topk, total_expanded):
+    who = "esimd_moe_scatter"
+    _chk_act(hidden_states, scattered_hidden, who)
+    _chk(int(K) % 8 == 0, f"{who}: K must be a multiple of 8")
+    _chk(sorted_token_ids.dtype == torch.int32 and sorted_token_ids.numel() >= int(total_expanded), f"{who}: sorted_token_ids must be int32")
+    _chk(router_top_value.dtype == hidden_states.dtype and scattered_weights.dtype == hidden_states.dtype,
+         f"{who}: weights must share the activation dtype")
+    capi.call("mi_moe_scatter", hidden_states, capi.ptr(hidden_states), capi.ptr(router_top_value),
+              capi.ptr(sorted_token_ids), capi.ptr(scattered_hidden), capi.ptr(scattered_weights), int(K),
+              int(topk), int(total_expanded))
+    return scattered_hidden
+
+
+def esimd_moe_scatter_fused(hidden_states, top_values, top_indices, scattered_hidden, scattered_weights,
+                            topk_ids, expert_start, max_tokens_out, K, topk, T, num_experts):
+    """Device-side expert sort + row scatter.  topk_ids receives the reverse map
+    (pair -> scattered row), expert_start the E+1 start offsets."""
+    who = "esimd_moe_scatter_fused"
+    T, topk, K, E = int(T), int(topk), int(K), int(num_experts)
+    _chk_act(hidden_states, scattered_hidden, who)
+    _chk(top_indices.dtype == torch.int32 and top_indices.is_contiguous() and top_indices.numel() >= T * topk,
+         f"{who}: top_indices must be contiguous int32 [T, topk]")
+    _chk(expert_start.dtype in (torch.int32, torch.uint32) and expert_start.numel() >= E + 1,
+         f"{who}: expert_start must be int32/uint32 [num_experts+1]")
+    _chk(topk_ids.dtype == torch.int32 and topk_ids.numel() >= T * topk, f"{who}: topk_ids must be int32 [T*topk]")
+    sorted_pairs = torch.empty(T * topk, dtype=torch.int32, device=hidden_states.device)
+    ids2d = top_indices.reshape(-1)[:T * topk].reshape(T, topk)
+    moe_sort(ids2d, E, sorted_pairs, expert_start, topk_ids, None, max_tokens_out)
+    esimd_moe_scatter(hidden_states, top_values, sorted_pairs, scattered_hidden, scattered_weights, K, topk, T * topk)
+    return scattered_hidden
+
+
+def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T):
+    who = "esimd_moe_gather"
+    _chk_act(moe_output, final_hidden, who)
+    _chk(int(K) % 8 == 0, f"{who}: K must be a multiple of 8")
+    _chk(topk_ids.dtype == torch.int32 and topk_ids.numel() >= int(T) * int(topk), f"{who}: topk_ids must be int32 [T, topk]")
+    _chk(scattered_weights.dtype == moe_output.dtype, f"{who}: scattered_weights must share the activation dtype")
+    capi.call("mi_moe_combine", moe_output, capi.ptr(moe_output), capi.ptr(topk_ids), capi.ptr(scattered_weights),
+              capi.ptr(final_hidden), int(K), int(topk), int(T), 1, capi.act_dtype(moe_output), 0)
+    return final_hidden
+
+
+def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse, who):
+    _chk_fp8(w, who)
+    _chk(w.numel() == E * N * K, f"{who}: weight must be [num_experts, N, K]")
+    _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+    _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and
+         w_scale.numel() == E * ((N + 127) // 128) * (K // 128),
+         f"{who}: weight_scale must be contiguous fp32 [E, ceil(N/128), K/128]")
+    _chk(expert_start.dtype in (torch.int32, torch.uint32) and expert_start.numel() >= E + 1,
+         f"{who}: expert_idx must be int32/uint32 [num_experts+1]")
+    _chk(out.dtype in (torch.float16, torch.bfloat16, torch.float32) and out.is_contiguous(),
+         f"{who}: output must be contiguous fp16/bf16/fp32")
+    n_out = N // 2 if fuse else N
+    total = out.numel() // n_out
+    a_rows = a.numel() // K
+    if a_scale is None:
+        adt = capi.act_dtype(a)
+        _chk(out.dtype in (a.dtype, torch.float32), f"{who}: output must be fp32 or share the activation dtype")
+    else:
+        adt = capi.act_dtype(out) if out.dtype != torch.float32 else capi.DT_BF16
+    capi.call("mi_moe_gemm_fp8_block", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), capi.ptr(w),
+              capi.ptr(w_scale), capi.ptr(expert_start), capi.ptr(out), a_rows, total, E, N, K,
+              1 if fuse else 0, adt, 1 if out.dtype == torch.float32 else 0)
+    return out
+
+
+def esimd_moe_gemm_fp8_blockscale(input, weight, weight_scale, output, expert_idx, N, K, num_experts,
+                                  block_n, block_k):
+    who = "esimd_moe_gemm_fp8_blockscale"
+    _chk(int(block_n) == 128 and int(block_k) == 128, f"{who}: only block_n == block_k == 128 is supported")
+    _chk_act(input, output, who)
+    N, K, E = int(N), int(K), int(num_experts)
+    _chk(input.numel() % K == 0 and output.numel() == (input.numel() // K) * N, f"{who}: output must be [total_tokens, N]")
+    return _moe_gemm(input, None, None, weight, weight_scale, expert_idx, output, E, N, K, False, who)
+
+
+def moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, output, N, K, num_experts,
+                       fuse_silu_mul):
+    """Grouped block-FP8 GEMM.  a_scale given: `a` is e4m3 with per-row per-128 fp32 scales
+    (native fp8 MFMA); a_scale None: `a` is fp16/bf16 (w8a16).  row_map (int32, optional)
+    gathers source rows; fuse_silu_mul writes silu(gate) * up ([rows, N/2]); output may be fp32."""
+    who = "moe_gemm_fp8_block"
+    K = int(K)
+    if a_scale is not None:
+        _chk(a.dtype in _FP8_TYPES and a.is_contiguous(), f"{who}: quantised activations must be contiguous e4m3/uint8")
+        _chk(a_scale.dtype == torch.float32 and a_scale.is_contiguous() and a_scale.numel() == (a.numel() // K) * (K // 128),
+             f"{who}: a_scale must be fp32 [rows, K/128]")
+    else:
+        _chk(a.dtype in (torch.float16, torch.bfloat16) and a.is_contiguous(), f"{who}: activations must be contiguous fp16/bf16")
+    if row_map is not None:
+        _chk(row_map.dtype == torch.int32 and row_map.is_contiguous(), f"{who}: row_map must be int32")
+    return _moe_gemm(a, a_scale, row_map, weight, weight_scale, expert_start, output, int(num_experts), int(N),
+                     K, bool(fuse_silu_mul), who)
+
+
+def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale, output, top_k,
+                          act_quant):
+    """Routed-experts MoE forward for 128x128 block-FP8 weights (no shared expert).
+
+    x [T, H], logits [T, E] fp16/bf16; gate_up_weight [E, 2I, H], down_weight [E, H, I]
+    e4m3 with fp32 block scales [E, 2I/128, H/128] / [E, H/128, I/128]; output [T, H].
+    act_quant=True quantises the activations entering both GEMMs per token per
+    128-group to e4m3 (native fp8 MFMA); False keeps them 16 bit (w8a16).
+    Pipeline: top-k -> stable expert sort -> [quantise x] -> grouped gate_up GEMM
+    with fused SiLU*mul -> [quantise] -> grouped down GEMM -> weighted combine.
+    """
+    who = "moe_forward_fp8_block"
+    _chk(x.dim() == 2 and logits.dim() == 2 and x.shape[0] == logits.shape[0], f"{who}: x [T,H], logits [T,E]")
+    _chk_act(x, output, who)
+    _chk(logits.dtype == x.dtype and logits.is_contiguous(), f"{who}: logits must share x's dtype")
+    _chk(output.data_ptr() != x.data_ptr(), f"{who}: output must not alias x")
+    T, H = x.shape
+    E = logits.shape[1]
+    _chk(gate_up_weight.dim() == 3 and down_weight.dim() == 3, f"{who}: weights must be [E, N, K]")
+    I = down_weight.shape[2]
+    _chk(tuple(gate_up_weight.shape) == (E, 2 * I, H) and tuple(down_weight.shape) == (E, H, I),
+         f"{who}: expected gate_up [E, 2I, H] and down [E, H, I]")
+    _chk(H % 128 == 0 and I % 128 == 0, f"{who}: H and I must be multiples of 128")
+    k = int(top_k)
+    P = T * k
+    dev = x.device
+    top_w = torch.empty(T, k, dtype=x.dtype, device=dev)
+    top_ids = torch.empty(T, k, dtype=torch.int32, device=dev)
+    esimd_moe_topk(logits, top_w, top_ids, T)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    start = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
+    moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
+    inter = torch.empty(P, I, dtype=x.dtype, device=dev)
+    y = torch.empty(P, H, dtype=torch.float32, device=dev)      # fp32: the combine adds K rounded terms otherwise
+    if act_quant:
+        xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
+        xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)
+        act_quant_fp8(x, xq, xs)
+        moe_gemm_fp8_block(xq, xs, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
+        iq = torch.empty(P, I, dtype=torch.uint8, device=dev)
+        isc = torch.empty(P, I // 128, dtype=torch.float32, device=dev)
+        act_quant_fp8(inter, iq, isc)
+        moe_gemm_fp8_block(iq, isc, None, down_weight, down_scale, start, y, H, I, E, False)
+    else:
+        moe_gemm_fp8_block(x, None, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
+        moe_gemm_fp8_block(inter, None, None, down_weight, down_scale, start, y, H, I, E, False)
+    moe_combine(y, inv, top_w, output, k)
+    return output
+
+
+def moe_combine(y, inv, top_w, output, top_k):
+    """output[t] = sum_j top_w[t, j] * y[inv[t * top_k + j]]; y fp32 or the activation dtype."""
+    who = "moe_combine"
+    T, H = output.shape
+    _chk(output.dtype in (torch.float16, torch.bfloat16) and output.is_contiguous(), f"{who}: output must be contiguous fp16/bf16 [T, H]")
+    _chk(y.dtype in (output.dtype, torch.float32) and y.is_contiguous() and y.shape[-1] == H, f"{who}: y must be [T*k, H] fp32 or activation dtype")
+    _chk(inv.dtype == torch.int32 and inv.numel() >= T * int(top_k), f"{who}: inv must be int32 [T*k]")
+    _chk(top_w.dtype == output.dtype and top_w.is_contiguous(), f"{who}: top_w must share the output dtype")
+    _chk(H % 8 == 0, f"{who}: H must be a multiple of 8")
+    capi.call("mi_moe_combine", y, capi.ptr(y), capi.ptr(inv), capi.ptr(top_w), capi.ptr(output), H, int(top_k), T, 0,
+              capi.act_dtype(output), 1 if y.dtype == torch.float32 else 0)
+    return output
+
+
+def moe_prefill_gather_forward_fp8(selected_experts, num_experts):
+    """-> [expert_offsets [E], expert_tokens [T*k] (sorted position -> pair index),
+    pair_to_perm [T*k], rows_for_experts [E]], with the stable in-expert order."""
+    _chk(selected_experts.dim() == 2 and selected_experts.dtype == torch.int32, "moe_prefill_gather_forward_fp8: selected_experts must be int32 [T, k]")
+    sel = selected_experts.contiguous()
+    T, k = sel.shape
+    E = int(num_experts)
+    dev = sel.device
+    start = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    tokens = torch.empty(T * k, dtype=torch.int32, device=dev)
+    perm = torch.empty(T * k, dtype=torch.int32, device=dev)
+    moe_sort(sel, E, tokens, start, perm, None, None)
+    return [start[:E], tokens, perm, start[1:] - start[:E]]
+
 # --------------------------------------------------------------------------
 # registration
 # --------------------------------------------------------------------------
@@ -382,6 +636,42 @@ def register():
     _define(_V, "fp8_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output, str mode) -> Tensor(a!)",
             fp8_dequant, _ret(2))
     _define(_V, "e4m3_decode(Tensor codes, Tensor(a!) output) -> Tensor(a!)", e4m3_decode, _ret(1))
+
+    # ---- MoE (reference fragment torch_extension_moe.cc + moe_ops + sglang prefill ops)
+    for ns in (_V, _S):
+        _define(ns, "esimd_moe_topk(Tensor router_logits, Tensor top_values, Tensor top_indices, int T) -> Tensor",
+                esimd_moe_topk, _ret(1))
+        _define(ns, "esimd_moe_scatter(Tensor hidden_states, Tensor router_top_value, Tensor sorted_token_ids, "
+                    "Tensor scattered_hidden, Tensor scattered_weights, int K, int topk, int total_expanded) -> Tensor",
+                esimd_moe_scatter, _ret(3))
+        _define(ns, "esimd_moe_scatter_fused(Tensor hidden_states, Tensor top_values, Tensor top_indices, "
+                    "Tensor scattered_hidden, Tensor scattered_weights, Tensor topk_ids, Tensor expert_start, "
+                    "Tensor max_tokens_out, int K, int topk, int T, int num_experts) -> Tensor",
+                esimd_moe_scatter_fused, _ret(3))
+        _define(ns, "esimd_moe_silu_mul(Tensor input, Tensor output, int N_gate_up, int N_half, int total_rows) -> Tensor",
+                esimd_moe_silu_mul, _ret(1))
+        _define(ns, "esimd_moe_gather(Tensor moe_output, Tensor topk_ids, Tensor scattered_weights, "
+                    "Tensor final_hidden, int K, int topk, int T) -> Tensor", esimd_moe_gather, _ret(3))
+    _define(_V, "esimd_moe_gemm_fp8_blockscale(Tensor input, Tensor weight, Tensor weight_scale, Tensor(a!) output, "
+                "Tensor expert_idx, int N, int K, int num_experts, int block_n, int block_k) -> Tensor(a!)",
+            esimd_moe_gemm_fp8_blockscale, _ret(3))
+    _define("moe_ops", "moe_topk(Tensor logits, int top_k, bool norm) -> (Tensor, Tensor)", moe_topk,
+            lambda logits, top_k, norm: (logits.new_empty(logits.shape[0], top_k),
+                                         logits.new_empty(logits.shape[0], top_k, dtype=torch.int32)))
+    _define("moe_fp8_prefill_ops", "moe_prefill_gather_forward_fp8(Tensor selected_experts, int num_experts) -> Tensor[]",
+            moe_prefill_gather_forward_fp8)
+    # siblings without a reference counterpart
+    _define(_V, "moe_sort(Tensor top_ids, int num_experts, Tensor(a!) sorted_pairs, Tensor(b!) expert_start, "
+                "Tensor(c!) inv, Tensor(d!)? sorted_token, Tensor(e!)? max_count) -> Tensor(a!)", moe_sort, _ret(2))
+    _define(_V, "act_quant_fp8(Tensor x, Tensor(a!) q, Tensor(b!) scale) -> Tensor(a!)", act_quant_fp8, _ret(1))
+    _define(_V, "moe_gemm_fp8_block(Tensor a, Tensor? a_scale, Tensor? row_map, Tensor weight, Tensor weight_scale, "
+                "Tensor expert_start, Tensor(a!) output, int N, int K, int num_experts, bool fuse_silu_mul) -> Tensor(a!)",
+            moe_gemm_fp8_block, _ret(6))
+    _define(_V, "moe_combine(Tensor y, Tensor inv, Tensor top_w, Tensor(a!) output, int top_k) -> Tensor(a!)",
+            moe_combine, _ret(3))
+    _define(_V, "moe_forward_fp8_block(Tensor x, Tensor logits, Tensor gate_up_weight, Tensor gate_up_scale, "
+                "Tensor down_weight, Tensor down_scale, Tensor(a!) output, int top_k, bool act_quant) -> Tensor(a!)",
+            moe_forward_fp8_block, _ret(6))
 
 
 register()

@@ -415,9 +415,17 @@ def moe_forward(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, *, act_quant: bool,
 
 
 def moe_forward_grouped(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, num_experts, *,
-                        act_quant: bool, act_dtype=torch.bfloat16):
+                        act_quant: bool, act_dtype=torch.bfloat16, inter_q=None, return_parts=False):
     """Same result as moe_forward, computed expert by expert on the sorted rows
-    (V/tests/test_fp8_blockscale_moe_prefill.py:113-118).  Fast enough for cfg3."""
+    (V/tests/test_fp8_blockscale_moe_prefill.py:113-118).  Fast enough for cfg3.
+
+    inter_q = (codes uint8 [T*k, I], scale fp32 [T*k, I/128]) in SORTED row order
+    replaces this function's own quantisation of the intermediate: re-quantising
+    is discontinuous (a 1-ulp change of a group's largest element moves the whole
+    group's grid), so a check of the down GEMM and of the combine has to start
+    from the very codes the kernel under test produced.
+    return_parts -> (out, inter [T*k, I] in act_dtype, y [T*k, H] fp32), sorted order.
+    """
     T, H = x.shape
     k = top_ids.shape[1]
     order, start, _ = moe_sort(top_ids, num_experts)
@@ -429,6 +437,9 @@ def moe_forward_grouped(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, num_experts
         x32 = x.to(torch.float32)
     out = torch.zeros(T, H, dtype=torch.float32)
     wflat = top_w.reshape(-1).to(torch.float32)
+    I = w2_q.shape[-1]
+    inter_all = torch.zeros(T * k, I, dtype=act_dtype)
+    y_all = torch.zeros(T * k, H, dtype=torch.float32)
     for e in range(num_experts):
         lo, hi = int(start[e]), int(start[e + 1])
         if hi == lo:
@@ -437,13 +448,19 @@ def moe_forward_grouped(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, num_experts
         dw13 = fp8_dequant_block(w13_q[e], w13_s[e])
         dw2 = fp8_dequant_block(w2_q[e], w2_s[e])
         inter = silu_mul(x32[rows] @ dw13.t()).to(act_dtype)
-        if act_quant:
+        inter_all[lo:hi] = inter
+        if inter_q is not None:
+            inter32 = act_dequant_per_token_group(inter_q[0][lo:hi], inter_q[1][lo:hi])
+        elif act_quant:
             iq, isc = act_quant_per_token_group(inter)
             inter32 = act_dequant_per_token_group(iq, isc)
         else:
             inter32 = inter.to(torch.float32)
         y = inter32 @ dw2.t()
+        y_all[lo:hi] = y
         out.index_add_(0, rows, y * wflat[order[lo:hi].long()][:, None])
+    if return_parts:
+        return out, inter_all, y_all
     return out
 
 

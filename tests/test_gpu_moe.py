@@ -1,0 +1,281 @@
+"""GPU parity for the MoE path: routing ids and the expert-sorted permutation are
+bit-exact against the oracle; activation quantisation codes and scales are
+bit-exact; grouped GEMMs and the full forward are within max relative error
+1e-2 (denominator floored at the mean magnitude) of the oracle that quantises
+the same activations."""
+import pytest
+import torch
+
+from oracle import qlinear_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def v(dev):
+    import custom_esimd_kernels_vllm as mod
+    return mod
+
+
+# ------------------------------------------------------------------ routing
+@pytest.mark.parametrize("T,E,K,dt", [(512, 128, 8, torch.bfloat16), (7, 16, 4, torch.float16),
+                                      (33, 64, 6, torch.float16), (5, 256, 8, torch.bfloat16),
+                                      (3, 8, 8, torch.float16), (1, 1024, 2, torch.float16)])
+def test_topk_ids_exact_weights_close(v, dev, T, E, K, dt):
+    g = torch.Generator().manual_seed(T * 131 + E)
+    logits = torch.randn(T, E, generator=g).to(dt)
+    if T > 2 and E >= 8:
+        logits[1, 5] = logits[1, 2]                 # a tie inside the top range
+        logits[1, 2] = logits[1].max()
+        logits[1, 5] = logits[1, 2]
+        logits[2, :] = 0.5                          # all equal: ids 0..K-1
+    tw = torch.empty(T, K, dtype=dt, device=dev)
+    ti = torch.empty(T, K, dtype=torch.int32, device=dev)
+    r = v.esimd_moe_topk(logits.to(dev), tw, ti, T)
+    assert r.data_ptr() == tw.data_ptr()
+    rw, ri = O.moe_topk(logits, K)
+    assert torch.equal(ti.cpu(), ri)
+    ulp = 2.0 ** -8 if dt == torch.bfloat16 else 2.0 ** -11
+    assert ((tw.cpu().float() - rw.float()).abs() <= 2 * ulp * rw.float().abs() + 1e-7).all()
+    w2, i2 = v.moe_topk(logits.to(dev), K, True)
+    assert torch.equal(i2.cpu(), ri) and torch.equal(w2, tw)
+
+
+@pytest.mark.parametrize("T,E,K", [(512, 128, 8), (1, 8, 2), (37, 16, 4), (4096, 128, 8), (300, 1000, 6),
+                                   (2500, 64, 2), (0, 8, 2)])
+def test_sort_bit_exact(v, dev, T, E, K):
+    g = torch.Generator().manual_seed(T + E + K)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(max(T, 1))])[:T].to(torch.int32).reshape(T, K)
+    if T >= 20:
+        for t in range(T // 2):                     # skew: half the tokens route to expert 3
+            if 3 not in ids[t].tolist():
+                ids[t, 0] = 3
+        assert all(len(set(ids[t].tolist())) == K for t in range(min(T, 50)))
+    P = T * K
+    sp = torch.full((max(P, 1),), -1, dtype=torch.int32, device=dev)
+    st = torch.full((E + 1,), -1, dtype=torch.int32, device=dev)
+    inv = torch.full((max(P, 1),), -1, dtype=torch.int32, device=dev)
+    tok = torch.full((max(P, 1),), -1, dtype=torch.int32, device=dev)
+    mx = torch.full((1,), -1, dtype=torch.int32, device=dev)
+    v.moe_sort(ids.to(dev), E, sp, st, inv, tok, mx)
+    ro, rs, ri = O.moe_sort(ids, E)
+    assert torch.equal(st.cpu(), rs)
+    assert torch.equal(sp.cpu()[:P], ro)
+    assert torch.equal(inv.cpu()[:P], ri)
+    assert torch.equal(tok.cpu()[:P], ro // K)
+    assert int(mx.cpu()) == int((rs[1:] - rs[:-1]).max())
+
+
+def test_sort_golden_fixture(v, dev):
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "routing_4tok_8exp.json")) as f:
+        fx = json.load(f)
+    ids = torch.tensor(fx["top_ids"], dtype=torch.int32)
+    sp = torch.empty(8, dtype=torch.int32, device=dev)
+    st = torch.empty(9, dtype=torch.int32, device=dev)
+    inv = torch.empty(8, dtype=torch.int32, device=dev)
+    v.moe_sort(ids.to(dev), 8, sp, st, inv)
+    assert sp.cpu().tolist() == fx["sorted_pairs"]
+    assert st.cpu().tolist() == fx["expert_start"]
+    assert inv.cpu().tolist() == fx["inv"]
+
+
+def test_scatter_fused_and_gather_roundtrip(v, dev):
+    # scatter rows by expert, then gather with weights: final[t] = sum_j w[t,j] * x[t] = x[t] (weights sum to 1)
+    T, E, K, H = 50, 16, 4, 256
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(T, H, generator=g).to(torch.float16)
+    logits = torch.randn(T, E, generator=g).to(torch.float16)
+    tw, ti = O.moe_topk(logits, K)
+    sh = torch.empty(T * K, H, dtype=torch.float16, device=dev)
+    sw = torch.empty(T * K, dtype=torch.float16, device=dev)
+    topk_ids = torch.empty(T * K, dtype=torch.int32, device=dev)
+    est = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    mx = torch.empty(1, dtype=torch.int32, device=dev)
+    v.esimd_moe_scatter_fused(x.to(dev), tw.to(dev), ti.to(dev), sh, sw, topk_ids, est, mx, H, K, T, E)
+    order, start, inv = O.moe_sort(ti, E)
+    assert torch.equal(est.cpu(), start) and torch.equal(topk_ids.cpu(), inv)
+    assert torch.equal(sh.cpu(), x[(order // K).long()])
+    assert torch.equal(sw.cpu(), tw.reshape(-1)[order.long()])
+    out = torch.empty(T, H, dtype=torch.float16, device=dev)
+    v.esimd_moe_gather(sh, topk_ids.reshape(T, K), sw, out, H, K, T)
+    ref = (tw.float().sum(-1, keepdim=True) * x.float())
+    assert O.max_rel_err(out.cpu(), ref) < 5e-3
+
+
+# ------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_act_quant_bit_exact(v, dev, dt):
+    g = torch.Generator().manual_seed(13)
+    x = (torch.randn(77, 768, generator=g) * torch.rand(77, 1, generator=g) * 3).to(dt)
+    x[3, :128] = 0                                   # an all-zero group
+    x[4, 5] = 1e-30 if dt == torch.bfloat16 else 6e-8
+    q = torch.empty(77, 768, dtype=torch.uint8, device=dev)
+    s = torch.empty(77, 6, dtype=torch.float32, device=dev)
+    v.act_quant_fp8(x.to(dev), q, s)
+    rq, rs = O.act_quant_per_token_group(x)
+    assert torch.equal(s.cpu(), rs)
+    assert torch.equal(q.cpu(), rq)
+
+
+def test_silu_mul(v, dev):
+    g = torch.Generator().manual_seed(14)
+    x = (torch.randn(37, 512, generator=g) * 3).to(torch.bfloat16)
+    out = torch.empty(37, 256, dtype=torch.bfloat16, device=dev)
+    v.esimd_moe_silu_mul(x.to(dev), out, 512, 256, 37)
+    ref = O.silu_mul(x)
+    assert O.max_rel_err(out.cpu(), ref) < 8e-3     # bf16 output rounding is 2^-9
+
+
+# ------------------------------------------------------------------ grouped GEMM
+def _grouped_ref(x, dw, counts):
+    ref = torch.empty(x.shape[0], dw.shape[1], dtype=torch.float32)
+    s = 0
+    for e, c in enumerate(counts):
+        ref[s:s + c] = x[s:s + c].float() @ dw[e].t()
+        s += c
+    return ref
+
+
+def test_moe_gemm_w8a16_reference_case(v, dev):
+    # V/tests/test_fp8_blockscale_moe_prefill.py:93-144: 4 experts, counts 33/40/27/36, n = k = 256
+    torch.manual_seed(20260713)
+    experts, n, k = 4, 256, 256
+    counts = [33, 40, 27, 36]
+    offsets = torch.tensor([0, 33, 73, 100, 136], dtype=torch.int32)
+    x = (torch.randn(136, k) * 0.2).half()
+    w8, ws = O.fp8_quantize_block(torch.randn(experts, n, k) * 0.15)
+    out = torch.empty(136, n, dtype=torch.float16, device=dev)
+    v.esimd_moe_gemm_fp8_blockscale(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), ws.to(dev), out,
+                                    offsets.to(dev), n, k, experts)
+    ref = _grouped_ref(x, O.fp8_dequant_block(w8, ws), counts)
+    o = out.cpu().float()
+    assert O.max_rel_err(o, ref) < TOL
+    mean_rel = ((o - ref).abs().mean() / ref.abs().mean()).item()
+    assert mean_rel < 3e-3                           # the reference's own bar
+
+
+@pytest.mark.parametrize("total", [1, 128])
+def test_moe_gemm_all_e4m3_codes_exact(v, dev, total):
+    # V/tests/test_fp8_blockscale_moe_prefill.py:54-90
+    raw = torch.arange(256, dtype=torch.uint8).view(1, 256, 1).expand(1, 256, 128).contiguous()
+    reference = raw[0, :, 0].view(torch.float8_e4m3fn).float() * 128
+    finite = torch.isfinite(reference)
+    scale = torch.ones(1, 2, 1)
+    x = torch.ones(total, 128, dtype=torch.float16)
+    out = torch.empty(total, 256, dtype=torch.float16, device=dev)
+    offsets = torch.tensor([0, total], dtype=torch.int32)
+    v.esimd_moe_gemm_fp8_blockscale(x.to(dev), raw.to(dev), scale.to(dev), out, offsets.to(dev), 256, 128, 1, 128, 128)
+    for row in (0, total - 1):
+        actual = out[row].cpu().float()
+        assert torch.equal(actual[finite], reference[finite])
+        assert actual[0x80].item() == 0.0
+
+
+@pytest.mark.parametrize("counts", [[0, 5, 0, 70, 1, 16, 17, 0], [130, 0, 0, 3]])
+@pytest.mark.parametrize("a8", [False, True])
+def test_moe_gemm_skewed_experts(v, dev, counts, a8):
+    E, N, K = len(counts), 272, 384                  # N not a multiple of 128: ragged scale rows
+    g = torch.Generator().manual_seed(sum(counts) + a8)
+    total = sum(counts)
+    st = torch.zeros(E + 1, dtype=torch.int32)
+    st[1:] = torch.tensor(counts).cumsum(0)
+    x = torch.randn(total, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(E, 384, K, generator=g) * 0.05
+    w8, ws = O.fp8_quantize_block(w)
+    w8 = w8[:, :N].contiguous()
+    dw = O.fp8_dequant_block(w8, ws)
+    out = torch.empty(total, N, dtype=torch.bfloat16, device=dev)
+    if a8:
+        xq, xs = O.act_quant_per_token_group(x)
+        v.moe_gemm_fp8_block(xq.to(dev), xs.to(dev), None, w8.to(dev), ws.to(dev), st.to(dev), out, N, K, E, False)
+        ref = _grouped_ref(O.act_dequant_per_token_group(xq, xs), dw, counts)
+    else:
+        v.esimd_moe_gemm_fp8_blockscale(x.to(dev), w8.to(dev), ws.to(dev), out, st.to(dev), N, K, E)
+        ref = _grouped_ref(x, dw, counts)
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
+# ------------------------------------------------------------------ full forward
+def _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq):
+    """The fused op's own pipeline, run stage by stage through the same ops, so that the
+    quantised intermediate is visible."""
+    T, H = x.shape
+    I = w2q.shape[-1]
+    P = T * K
+    dt = x.dtype
+    xd = x.to(dev)
+    tw = torch.empty(T, K, dtype=dt, device=dev)
+    ti = torch.empty(T, K, dtype=torch.int32, device=dev)
+    v.esimd_moe_topk(logits.to(dev), tw, ti, T)
+    sp = torch.empty(P, dtype=torch.int32, device=dev)
+    st = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    tok = torch.empty(P, dtype=torch.int32, device=dev)
+    v.moe_sort(ti, E, sp, st, inv, tok)
+    inter = torch.empty(P, I, dtype=dt, device=dev)
+    y = torch.empty(P, H, dtype=torch.float32, device=dev)
+    w13d, s13d, w2d, s2d = w13q.to(dev), w13s.to(dev), w2q.to(dev), w2s.to(dev)
+    iq = isc = None
+    if aq:
+        xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
+        xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)
+        v.act_quant_fp8(xd, xq, xs)
+        v.moe_gemm_fp8_block(xq, xs, tok, w13d, s13d, st, inter, 2 * I, H, E, True)
+        iq = torch.empty(P, I, dtype=torch.uint8, device=dev)
+        isc = torch.empty(P, I // 128, dtype=torch.float32, device=dev)
+        v.act_quant_fp8(inter, iq, isc)
+        v.moe_gemm_fp8_block(iq, isc, None, w2d, s2d, st, y, H, I, E, False)
+    else:
+        v.moe_gemm_fp8_block(xd, None, tok, w13d, s13d, st, inter, 2 * I, H, E, True)
+        v.moe_gemm_fp8_block(inter, None, None, w2d, s2d, st, y, H, I, E, False)
+    out = torch.empty(T, H, dtype=dt, device=dev)
+    v.moe_combine(y, inv, tw, out, K)
+    return dict(tw=tw, ti=ti, inter=inter, iq=iq, isc=isc, y=y, out=out)
+
+
+def _check_forward(v, dev, T, E, K, H, I, aq, seed):
+    x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I, seed=seed)
+    g = _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq)
+    rtw, rti = O.moe_topk(logits, K)
+    assert torch.equal(g["ti"].cpu(), rti)
+    # oracle forward that starts the down GEMM from the kernel's own quantised intermediate
+    iq_override = (g["iq"].cpu(), g["isc"].cpu()) if aq else None
+    ref, ref_inter, ref_y = O.moe_forward_grouped(x, g["tw"].cpu(), rti, w13q, w13s, w2q, w2s, E, act_quant=aq,
+                                                  inter_q=iq_override, return_parts=True)
+    if aq:
+        # stage 1: gate_up GEMM + SiLU*mul from the same quantised x
+        assert O.max_rel_err(g["inter"].cpu(), ref_inter.float()) < TOL
+        # stage 2: the kernel's quantisation of its own intermediate is bit-exact
+        rq, rs = O.act_quant_per_token_group(g["inter"].cpu())
+        assert torch.equal(g["iq"].cpu(), rq) and torch.equal(g["isc"].cpu(), rs)
+    # stage 3: down GEMM, stage 4: weighted combine
+    assert O.max_rel_err(g["y"].cpu(), ref_y) < TOL
+    assert O.max_rel_err(g["out"].cpu(), ref) < TOL
+    # the fused op runs the same kernels; with fused SiLU (act-quant mode) it is bit-identical
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    r = v.moe_forward_fp8_block(x.to(dev), logits.to(dev), w13q.view(torch.float8_e4m3fn).to(dev), w13s.to(dev),
+                                w2q.view(torch.float8_e4m3fn).to(dev), w2s.to(dev), out, K, aq)
+    assert r.data_ptr() == out.data_ptr()
+    assert torch.equal(out, g["out"])
+    # free-running oracle (quantises its own intermediate): the reference's looser, mean-based bar
+    free = O.moe_forward_grouped(x, rtw, rti, w13q, w13s, w2q, w2s, E, act_quant=aq)
+    o = out.cpu().float()
+    mean_rel = ((o - free).abs().mean() / free.abs().mean()).item()
+    cos = torch.nn.functional.cosine_similarity(o.flatten(), free.flatten(), dim=0).item()
+    assert mean_rel < 1e-2 and cos > 0.9995, (mean_rel, cos)
+    return out
+
+
+@pytest.mark.parametrize("T,E,K,H,I,aq", [(5, 8, 2, 256, 128, True), (5, 8, 2, 256, 128, False),
+                                          (12, 16, 4, 256, 128, True), (40, 16, 4, 512, 256, True),
+                                          (12, 16, 4, 256, 128, False), (1, 16, 4, 256, 128, True)])
+def test_moe_forward_small(v, dev, T, E, K, H, I, aq):
+    _check_forward(v, dev, T, E, K, H, I, aq, seed=T + E)
+
+
+def test_cfg3_moe_forward(v, dev):
+    out = _check_forward(v, dev, 512, 128, 8, 2048, 768, True, seed=1237)
+    assert torch.isfinite(out.float()).all()
