@@ -125,11 +125,67 @@ def wl_q4k(M: int, dev):
                 kernel="skinny_kernel", cpu=cpu)
 
 
+def wl_gemm_w4a16(dev):
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    M, K, N = 2048, 4096, 14336
+    x, packed, scale, zp = O.make_int4_case(M, K, N, seed=1236, act_dtype=torch.bfloat16, asym=True)
+    xd, wd, sd, zd = x.to(dev), packed.to(dev), scale.to(dev), zp.to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+    def launch(i):
+        v.esimd_gemm_int4_pgrp_zp(xd, wd, sd, zd, out)
+
+    def cpu():
+        # bounded sample: 256 of the 2048 rows (the dequant of the whole weight is in every pass)
+        return O.matmul_ref(x[:256], O.int4_dequant(packed, scale, out_dtype=torch.bfloat16, zp=zp)).to(torch.bfloat16)
+
+    alg_bytes = N * K // 2 + N * (K // 128) * 3 + 2 * M * K + 2 * M * N
+    return dict(launch=launch, R=1, bytes=alg_bytes, flops=2 * M * N * K, bound="mfma", dtype="bf16",
+                name=f"cfg2 W4A16 asymmetric group-128 prefill GEMM M={M} K={K} N={N} bf16",
+                kernel="gemm_w4a16_kernel", cpu=cpu, cpu_scale=256 / M)
+
+
+def wl_moe(dev):
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    T, E, K, H, I = 512, 128, 8, 2048, 768
+    x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I)
+    wbytes = E * (2 * I * H + H * I)
+    R = _copies(wbytes)
+    g = torch.Generator().manual_seed(96)
+    W = [(w13q.to(dev), w13s.to(dev), w2q.to(dev), w2s.to(dev))]
+    for _ in range(R - 1):                      # permute the experts: distinct bytes, same distribution
+        p = torch.randperm(E, generator=g)
+        W.append((w13q[p].to(dev), w13s[p].to(dev), w2q[p].to(dev), w2s[p].to(dev)))
+    xd, ld = x.to(dev), logits.to(dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+
+    def launch(i):
+        a, b, c, d = W[i % R]
+        v.moe_forward_fp8_block(xd, ld, a, b, c, d, out, K, True)
+
+    def cpu():
+        tw, ti = O.moe_topk(logits, K)
+        return O.moe_forward_grouped(x, tw, ti, w13q, w13s, w2q, w2s, E, act_quant=True).to(torch.bfloat16)
+
+    P = T * K
+    # algorithmic bytes: every expert's weights + block scales once, x and logits in, output out
+    alg_bytes = wbytes + 4 * E * ((2 * I // 128) * (H // 128) + (H // 128) * (I // 128)) + 2 * T * H + 2 * T * E + 2 * T * H
+    flops = 2 * P * (2 * I * H + H * I)
+    return dict(launch=launch, R=R, bytes=alg_bytes, flops=flops, bound="hbm", dtype="fp8",
+                name=f"cfg3 FP8 128x128-block MoE forward (topk+sort+quant+gate_up/SiLU+quant+down+combine) "
+                     f"T={T} E={E} top{K} H={H} I={I} bf16, fp8 activations",
+                kernel="moe_gemm_kernel", cpu=cpu)
+
+
 WORKLOADS = {
     "cfg1_m1": lambda dev: wl_fp8_pern(1, dev),
     "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
     "cfg1_m32": lambda dev: wl_fp8_pern(32, dev),
     "cfg0": wl_int4_gemv,
+    "cfg2": wl_gemm_w4a16,
+    "cfg3": wl_moe,
     "cfg4_m1": lambda dev: wl_q4k(1, dev),
     "cfg4_m64": lambda dev: wl_q4k(64, dev),
 }

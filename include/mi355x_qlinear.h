@@ -74,6 +74,16 @@ int mi_gemv_int4_multi(const void* x, int nmat, const void* const* w, const void
                        const void* const* zp, void* const* out, const int* N, int M, int K,
                        int act_dtype, void* stream);
 
+/* ---- INT4 group-128 GEMM, any M (prefill) --------------------------------------
+ * Same operands as mi_gemv_int4.  M <= 64 runs the weight-streaming kernel; larger
+ * M runs the LDS-tiled MFMA GEMM (weights dequantized to the activation dtype,
+ * bit-exact, while they are staged into LDS).  Replaces esimd_gemm_int4_pgrp
+ * (V/csrc/xpu/esimd_kernel_gemm.sycl:55-91, V/csrc/xpu/esimd_kernels/int4_GEMM.h:291-320),
+ * without its 64-row limit; the zero-point operand (cfg2's asymmetric weights) has
+ * no counterpart in the reference's kernels. */
+int mi_gemm_int4(const void* x, const void* w, const void* scale, const void* zp, void* out, int M, int N,
+                 int K, int act_dtype, void* stream);
+
 /* ---- GGUF Q4_K on the repacked representation, fp16 -------------------------
  * ql [N, K/2] uint8 interleaved nibbles, scale/qmin [N, K/32] fp16;
  * w = fp16(fp16(nib * scale) - qmin);  out = x @ w^T.  K % 32 == 0.

@@ -40,9 +40,115 @@ struct MoeGemmArgs {
   int total_rows;             // rows in `out`
 };
 
+// One pass over K for a chunk of MTC 16-row activation tiles.  The weights are the
+// MFMA A operand and the activations the B operand, so a lane ends up holding
+// ONE activation row (mt*16 + j) and four consecutive weight rows (4 g + v): the
+// per-row activation scale is then a single value per lane, tile and granule.
+// Granules are software-pipelined through two register buffers; loads of a
+// granule (weights first, then activations, then scales) are issued together so
+// that the in-order memory counter lets granule i be consumed while granule
+// i + 1 is still in flight.
+template <class Act, bool A8, int RT, int NW, int MTC>
+__device__ __forceinline__ void moe_chunk(const MoeGemmArgs& p, f32x4 (&acc)[RT][4],
+                                          __amdgpu_buffer_rsrc_t wr, __amdgpu_buffer_rsrc_t ar,
+                                          const float* wsc, const int (&nbase)[RT],
+                                          const uint32_t (&wdead)[RT], const uint32_t (&arow)[4],
+                                          const uint32_t (&adead)[4], int wave, int j, int g) {
+  using V8 = typename Act::v8;
+  constexpr int NA = A8 ? 2 : 4;                      // 16-byte loads per activation row per granule
+  const int K = p.K;
+  const int G = K >> 7;
+  const int Kb = G;
+  const int Nb = (p.N + 127) >> 7;
+  const uint32_t a_esz = A8 ? 1u : 2u;
+
+  struct Frag {
+    u32x4 wa[RT], wb[RT];
+    u32x4 af[MTC][NA];
+    float ws[RT];
+    float xs[MTC];
+  };
+  auto load_frag = [&](Frag& f, int gi) {
+    const uint32_t gdead = (uint32_t)(gi >= G) << 31;
+    const int gic = gi < G ? gi : G - 1;
+    const uint32_t kl = (uint32_t)gic * 128u + (uint32_t)g * 32u;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const uint32_t off = ((uint32_t)(nbase[t] + j) * (uint32_t)K + kl) | wdead[t] | gdead;
+      f.wa[t] = __builtin_amdgcn_raw_buffer_load_b128(wr, off, 0, 2);
+      f.wb[t] = __builtin_amdgcn_raw_buffer_load_b128(wr, off + 16u, 0, 2);
+    }
+#pragma unroll
+    for (int mt = 0; mt < MTC; ++mt) {
+      const uint32_t off = ((arow[mt] * (uint32_t)K + kl) * a_esz) | adead[mt] | gdead;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) f.af[mt][i] = buf_load16(ar, off + 16u * i);
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const int nb = min(nbase[t] >> 7, Nb - 1);
+      f.ws[t] = wsc[(size_t)nb * Kb + gic];
+    }
+    if constexpr (A8) {
+#pragma unroll
+      for (int mt = 0; mt < MTC; ++mt) f.xs[mt] = p.a_scale[(size_t)arow[mt] * Kb + gic];
+    }
+  };
+  auto compute = [&](const Frag& f) {
+    V8 w16[RT][4];
+    if constexpr (!A8) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        w16[t][0] = fp8x8_to_act<Act>(f.wa[t][0], f.wa[t][1]);
+        w16[t][1] = fp8x8_to_act<Act>(f.wa[t][2], f.wa[t][3]);
+        w16[t][2] = fp8x8_to_act<Act>(f.wb[t][0], f.wb[t][1]);
+        w16[t][3] = fp8x8_to_act<Act>(f.wb[t][2], f.wb[t][3]);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MTC; ++mt) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (A8) {
+          const long x0 = (long)(((uint64_t)f.af[mt][0][1] << 32) | f.af[mt][0][0]);
+          const long x1 = (long)(((uint64_t)f.af[mt][0][3] << 32) | f.af[mt][0][2]);
+          const long x2 = (long)(((uint64_t)f.af[mt][1][1] << 32) | f.af[mt][1][0]);
+          const long x3 = (long)(((uint64_t)f.af[mt][1][3] << 32) | f.af[mt][1][2]);
+          const long w0 = (long)(((uint64_t)f.wa[t][1] << 32) | f.wa[t][0]);
+          const long w1 = (long)(((uint64_t)f.wa[t][3] << 32) | f.wa[t][2]);
+          const long w2 = (long)(((uint64_t)f.wb[t][1] << 32) | f.wb[t][0]);
+          const long w3 = (long)(((uint64_t)f.wb[t][3] << 32) | f.wb[t][2]);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, x0, tt, 0, 0, 0);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, x1, tt, 0, 0, 0);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, x2, tt, 0, 0, 0);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, x3, tt, 0, 0, 0);
+          acc[t][mt] += tt * (f.xs[mt] * f.ws[t]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) tt = Act::mfma(w16[t][i], as_v8<V8>(f.af[mt][i]), tt);
+          acc[t][mt] += tt * f.ws[t];
+        }
+      }
+    }
+  };
+
+  Frag fa, fb;
+  int gi = wave;
+  load_frag(fa, gi);
+  while (gi < G) {
+    load_frag(fb, gi + NW);
+    compute(fa);
+    gi += NW;
+    if (gi >= G) break;
+    load_frag(fa, gi + NW);
+    compute(fb);
+    gi += NW;
+  }
+}
+
 template <class Act, bool A8, bool SILU, int RT, int NW>
 __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) {
-  using V8 = typename Act::v8;
   using Elem = typename Act::elem;
   constexpr int MT = 4;                               // up to 64 rows per pass
   __shared__ f32x4 red[NW > 1 ? NW - 1 : 1][RT][MT][64];
@@ -57,51 +163,41 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int j = lane & 15, g = lane >> 4;
   const int K = p.K, N = p.N;
-  const int G = K >> 7;
   const int half = N >> 1;
   // weight rows of this workgroup: tile t covers rows nbase[t] .. +16
   int nbase[RT];
+  uint32_t wdead[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
-    if constexpr (SILU)
-      nbase[t] = (t & 1) * half + (tile * (RT / 2) + (t >> 1)) * 16;   // (gate, up) pairs
-    else
+    if constexpr (SILU) {
+      const int col = (tile * (RT / 2) + (t >> 1)) * 16;       // (gate, up) pairs share a column
+      nbase[t] = (t & 1) * half + col;
+      wdead[t] = (uint32_t)(!(col + j < half)) << 31;
+    } else {
       nbase[t] = (tile * RT + t) * 16;
+      wdead[t] = (uint32_t)(!(nbase[t] + j < N)) << 31;
+    }
   }
-  const int nlimit = SILU ? half : N;                 // valid column range per tile family
 
   const uint8_t* wexp = (const uint8_t*)p.w + (size_t)e * N * K;
   const __amdgpu_buffer_rsrc_t wr = make_rsrc(wexp, (uint32_t)N * (uint32_t)K);
   const uint32_t a_esz = A8 ? 1u : 2u;
   const __amdgpu_buffer_rsrc_t ar = make_rsrc(p.a, (uint32_t)p.a_rows * (uint32_t)K * a_esz);
-  const int Kb = G;
   const int Nb = (N + 127) >> 7;
-  const float* wsc = p.w_scale + (size_t)e * Nb * Kb;
+  const float* wsc = p.w_scale + (size_t)e * Nb * (K >> 7);
 
   for (int mc = 0; mc < cnt; mc += 16 * MT) {
     const int rows_here = min(16 * MT, cnt - mc);
     const int mtiles = (rows_here + 15) >> 4;
-    // source row of this lane's A fragment, per m-tile
-    uint32_t arow[MT];
-    bool avalid[MT];
+    // source row of this lane's activation fragment, per m-tile
+    uint32_t arow[MT], adead[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = mc + mt * 16 + j;
-      avalid[mt] = m < cnt;
-      const int pos = r0 + (avalid[mt] ? m : 0);
+      const bool ok = m < cnt;
+      adead[mt] = (uint32_t)(!ok) << 31;
+      const int pos = r0 + (ok ? m : 0);
       arow[mt] = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
-    }
-    // rows whose activation scale this lane needs in the D layout: mt*16 + 4g + v
-    uint32_t srow[MT][4];
-    if constexpr (A8) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int m = mc + mt * 16 + g * 4 + v;
-          const int pos = r0 + (m < cnt ? m : 0);
-          srow[mt][v] = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
-        }
     }
 
     f32x4 acc[RT][MT];
@@ -110,75 +206,11 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int gi = wave; gi < G; gi += NW) {
-      const uint32_t kl = (uint32_t)gi * 128u + (uint32_t)g * 32u;
-      u32x4 wa[RT], wb[RT];
-      float ws[RT];
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const uint32_t n = (uint32_t)(nbase[t] + j);
-        const uint32_t dead = (uint32_t)(!((nbase[t] + j - (SILU ? (t & 1) * half : 0)) < nlimit)) << 31;
-        const uint32_t off = (n * (uint32_t)K + kl) | dead;
-        wa[t] = __builtin_amdgcn_raw_buffer_load_b128(wr, off, 0, 2);
-        wb[t] = __builtin_amdgcn_raw_buffer_load_b128(wr, off + 16u, 0, 2);
-        const int nb = min(nbase[t] >> 7, Nb - 1);
-        ws[t] = wsc[(size_t)nb * Kb + gi];
-      }
-      // A fragments
-      u32x4 af[MT][A8 ? 2 : 4];
-      float xs[MT][4];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if (mt < mtiles) {                             // wave-uniform
-          const uint32_t dead = (uint32_t)(!avalid[mt]) << 31;
-          const uint32_t off = ((arow[mt] * (uint32_t)K + kl) * a_esz) | dead;
-#pragma unroll
-          for (int i = 0; i < (A8 ? 2 : 4); ++i) af[mt][i] = buf_load16(ar, off + 16u * i);
-          if constexpr (A8) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) xs[mt][v] = p.a_scale[(size_t)srow[mt][v] * Kb + gi];
-          }
-        }
-      }
-      V8 b16[RT][4];
-      if constexpr (!A8) {
-#pragma unroll
-        for (int t = 0; t < RT; ++t) {
-          b16[t][0] = fp8x8_to_act<Act>(wa[t][0], wa[t][1]);
-          b16[t][1] = fp8x8_to_act<Act>(wa[t][2], wa[t][3]);
-          b16[t][2] = fp8x8_to_act<Act>(wb[t][0], wb[t][1]);
-          b16[t][3] = fp8x8_to_act<Act>(wb[t][2], wb[t][3]);
-        }
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if (mt < mtiles) {
-#pragma unroll
-          for (int t = 0; t < RT; ++t) {
-            f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-            if constexpr (A8) {
-              const long a0 = (long)(((uint64_t)af[mt][0][1] << 32) | af[mt][0][0]);
-              const long a1 = (long)(((uint64_t)af[mt][0][3] << 32) | af[mt][0][2]);
-              const long a2 = (long)(((uint64_t)af[mt][1][1] << 32) | af[mt][1][0]);
-              const long a3 = (long)(((uint64_t)af[mt][1][3] << 32) | af[mt][1][2]);
-              const long b0 = (long)(((uint64_t)wa[t][1] << 32) | wa[t][0]);
-              const long b1 = (long)(((uint64_t)wa[t][3] << 32) | wa[t][2]);
-              const long b2 = (long)(((uint64_t)wb[t][1] << 32) | wb[t][0]);
-              const long b3 = (long)(((uint64_t)wb[t][3] << 32) | wb[t][2]);
-              tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, tt, 0, 0, 0);
-              tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, tt, 0, 0, 0);
-              tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a2, b2, tt, 0, 0, 0);
-              tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a3, b3, tt, 0, 0, 0);
-#pragma unroll
-              for (int v = 0; v < 4; ++v) acc[t][mt][v] += tt[v] * (xs[mt][v] * ws[t]);
-            } else {
-#pragma unroll
-              for (int i = 0; i < 4; ++i) tt = Act::mfma(as_v8<V8>(af[mt][i]), b16[t][i], tt);
-              acc[t][mt] += tt * ws[t];
-            }
-          }
-        }
-      }
+    switch (mtiles) {                                  // wave-uniform
+      case 1: moe_chunk<Act, A8, RT, NW, 1>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
+      case 2: moe_chunk<Act, A8, RT, NW, 2>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
+      case 3: moe_chunk<Act, A8, RT, NW, 3>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
+      default: moe_chunk<Act, A8, RT, NW, 4>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
     }
 
     // ---- reduce across the NW wavefronts ----
@@ -199,20 +231,21 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
             for (int mt = 0; mt < MT; ++mt) acc[t][mt] += red[w][t][mt][lane];
       }
     }
+    // D layout: lane holds activation row mt*16 + j and weight rows nbase + 4 g + v
     if (wave == 0) {
       Elem* out = (Elem*)p.out;
       float* out32 = (float*)p.out;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = mc + mt * 16 + j;
+        if (m < cnt) {
+          const size_t orow = (size_t)(r0 + m) * p.n_out;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int m = mc + mt * 16 + g * 4 + v;
-          if (m < cnt) {
-            const size_t orow = (size_t)(r0 + m) * p.n_out;
+          for (int v = 0; v < 4; ++v) {
             if constexpr (SILU) {
 #pragma unroll
               for (int t = 0; t < RT; t += 2) {
-                const int n = nbase[t] + j;            // gate row == output column
+                const int n = nbase[t] + g * 4 + v;      // gate row == output column
                 if (n < half) {
                   const float gate = acc[t][mt][v], up = acc[t + 1][mt][v];
                   const float r = gate / (1.0f + expf(-gate)) * up;
@@ -222,7 +255,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
             } else {
 #pragma unroll
               for (int t = 0; t < RT; ++t) {
-                const int n = nbase[t] + j;
+                const int n = nbase[t] + g * 4 + v;
                 if (n < N) {
                   if (p.out_f32) out32[orow + n] = acc[t][mt][v]; else out[orow + n] = Act::from_f32(acc[t][mt][v]);
                 }
@@ -230,6 +263,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
             }
           }
         }
+      }
     }
     if constexpr (NW > 1) __syncthreads();            // red[] is reused by the next pass
   }

@@ -38,3 +38,7 @@ def esimd_gemv_int4_fused2(input, w0, s0, o0, w1, s1, o1):
 
 def esimd_gemm_fp8_pert(input, weight, weight_scale, output):
     return _ops_gemm.esimd_gemm_fp8_pert(input, weight, weight_scale, output)
+
+
+def esimd_gemm_int4_pgrp(input, weight, weight_scale, output):
+    return _ops_gemm.esimd_gemm_int4_pgrp(input, weight, weight_scale, output)

@@ -60,6 +60,17 @@ def esimd_gemv_int4_fused2(input, w0, s0, o0, w1, s1, o1):
     return _ops.esimd_gemv_int4_fused2(input, w0, s0, o0, w1, s1, o1)
 
 
+def esimd_gemm_int4_pgrp(input, weight, weight_scale, output):
+    """input [M, K], weight [N, K/2] uint8 (low nibble = even k, value + 8), weight_scale [N, K/128]
+    fp16, output [M, N]; any M (the reference's kernel stops at 64 rows)."""
+    return _ops.esimd_gemm_int4_pgrp(input, weight, weight_scale, output)
+
+
+def esimd_gemm_int4_pgrp_zp(input, weight, weight_scale, weight_zp, output):
+    """Asymmetric sibling: weight_zp [N, K/128] uint8 in 0..15."""
+    return _ops.esimd_gemm_int4_pgrp_zp(input, weight, weight_scale, weight_zp, output)
+
+
 def int4_dequant(weight, weight_scale, weight_zp, output):
     return _ops.int4_dequant(weight, weight_scale, weight_zp, output)
 

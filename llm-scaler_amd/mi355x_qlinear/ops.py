@@ -217,6 +217,23 @@ def esimd_gemv_int4_fused2(input, w0, s0, o0, w1, s1, o1):
     return _int4_multi(input, [w0, w1], [s0, s1], [None, None], [o0, o1], "esimd_gemv_int4_fused2")
 
 
+def _gemm_int4(x, w, s, zp, o, who):
+    M, N, K = _chk_int4(x, w, s, zp, o, who)
+    capi.call("mi_gemm_int4", x, capi.ptr(x), capi.ptr(w), capi.ptr(s), capi.ptr(zp), capi.ptr(o), M, N, K,
+              capi.act_dtype(x))
+    return o
+
+
+def esimd_gemm_int4_pgrp(input, weight, weight_scale, output):
+    """Symmetric (implicit zero-point 8) group-128 int4 GEMM for any M."""
+    return _gemm_int4(input, weight, weight_scale, None, output, "esimd_gemm_int4_pgrp")
+
+
+def esimd_gemm_int4_pgrp_zp(input, weight, weight_scale, weight_zp, output):
+    """Asymmetric sibling: weight_zp [N, K/128] uint8 with values 0..15; w = (nibble - zp) * scale."""
+    return _gemm_int4(input, weight, weight_scale, weight_zp, output, "esimd_gemm_int4_pgrp_zp")
+
+
 # --------------------------------------------------------------------------
 # GGUF Q4_K  (esimd_gemv_q4_k + siblings)
 # --------------------------------------------------------------------------
@@ -617,6 +634,10 @@ def register():
     # the reference registers its GEMM fragment under the vllm namespace, and in the
     # sglang fork under `custom_esimd_kernels`
     for ns in (_V, "custom_esimd_kernels"):
+        _define(ns, "esimd_gemm_int4_pgrp(Tensor input, Tensor weight, Tensor weight_scale, "
+                    "Tensor output) -> Tensor", esimd_gemm_int4_pgrp, _ret(3))
+        _define(ns, "esimd_gemm_int4_pgrp_zp(Tensor input, Tensor weight, Tensor weight_scale, Tensor weight_zp, "
+                    "Tensor(a!) output) -> Tensor(a!)", esimd_gemm_int4_pgrp_zp, _ret(4))
         _define(ns, "esimd_gemm_fp8_pert(Tensor input, Tensor weight, Tensor weight_scale, "
                     "Tensor output) -> Tensor", esimd_gemm_fp8_pert, _ret(3))
         _define(ns, "esimd_gemm_fp8_blockscale(Tensor input, Tensor weight, Tensor weight_scale, "

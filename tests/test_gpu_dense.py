@@ -309,3 +309,46 @@ def test_argument_errors_raise(ops, dev):
     with pytest.raises(RuntimeError):
         v.esimd_gemm_fp8_blockscale(x, torch.zeros(16, 256, dtype=torch.uint8, device=dev),
                                     torch.zeros(1, 2, device=dev), out, 64, 128)   # block size
+
+
+# ----------------------------------------------------------------- prefill W4A16 GEMM
+def _run_gemm_int4(v, dev, M, K, N, dt, asym, seed):
+    x, packed, scale, zp = O.make_int4_case(M, K, N, seed=seed, act_dtype=dt, asym=asym)
+    out = torch.empty(M, N, dtype=dt, device=dev)
+    if asym:
+        r = v.esimd_gemm_int4_pgrp_zp(x.to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out)
+    else:
+        r = v.esimd_gemm_int4_pgrp(x.to(dev), packed.to(dev), scale.to(dev), out)
+    assert r.data_ptr() == out.data_ptr()
+    ref = O.matmul_ref(x, O.int4_dequant(packed, scale, out_dtype=dt, zp=zp))
+    return O.max_rel_err(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("M,K,N,dt,asym", [
+    (65, 256, 64, torch.float16, False), (128, 512, 128, torch.bfloat16, True),
+    (200, 1024, 272, torch.bfloat16, True), (257, 384, 520, torch.float16, True),
+    (300, 128, 16, torch.bfloat16, False), (1000, 2048, 1000, torch.bfloat16, True),
+    (4096, 512, 4096, torch.bfloat16, True), (4100, 256, 4100, torch.float16, False)])
+def test_gemm_int4_shapes(ops, dev, M, K, N, dt, asym):
+    v, _ = ops
+    assert _run_gemm_int4(v, dev, M, K, N, dt, asym, seed=M + N) < TOL
+
+
+def test_cfg2_w4a16_prefill_gemm(ops, dev):
+    v, _ = ops
+    M, K, N = 2048, 4096, 14336
+    x, packed, scale, zp = O.make_int4_case(M, K, N, seed=1236, act_dtype=torch.bfloat16, asym=True)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    v.esimd_gemm_int4_pgrp_zp(x.to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out)
+    o = out.cpu()
+    wd = O.int4_dequant(packed, scale, out_dtype=torch.bfloat16, zp=zp)
+    # full-size check on a strided sample of rows and columns (the oracle matmul of the whole
+    # problem is 240 GFLOP on the CPU); every 256x256 tile contributes rows and columns
+    rows = torch.arange(0, M, 37)
+    cols = torch.arange(0, N, 29)
+    ref = O.matmul_ref(x[rows], wd[cols])
+    assert O.max_rel_err(o[rows][:, cols], ref) < TOL
+    # size-independent property: linearity in x.  out(2x) == 2 out(x) exactly (power of two)
+    out2 = torch.empty_like(out)
+    v.esimd_gemm_int4_pgrp_zp((x * 2).to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out2)
+    assert torch.equal(out2.cpu().float(), 2 * o.float())
