@@ -66,7 +66,7 @@ def wl_fp8_pern(M: int, dev):
     alg_bytes = N * K + 4 * N + 2 * M * K + 2 * M * N
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="bf16",
                 name=f"cfg1 FP8 e4m3 per-channel weight-only GEMV M={M} K={K} N={N} bf16",
-                kernel="skinny_kernel", cpu=cpu)
+                kernel="gemv_rows_kernel" if M <= 4 else "skinny_kernel", cpu=cpu)
 
 
 def wl_int4_gemv(dev):
@@ -92,7 +92,7 @@ def wl_int4_gemv(dev):
 
     alg_bytes = N * K // 2 + N * (K // 128) * 2 + K * 2 + N * 2
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="f16",
-                name=f"cfg0 W4A16 group-128 GEMV M={M} K={K} N={N} fp16", kernel="skinny_kernel", cpu=cpu)
+                name=f"cfg0 W4A16 group-128 GEMV M={M} K={K} N={N} fp16", kernel="gemv_rows_kernel", cpu=cpu)
 
 
 def wl_q4k(M: int, dev):
@@ -122,7 +122,7 @@ def wl_q4k(M: int, dev):
     alg_bytes = per + 2 * M * K + 2 * M * N
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="f16",
                 name=f"cfg4 GGUF Q4_K (repacked) dequant-matmul M={M} K={K} N={N} fp16",
-                kernel="skinny_kernel", cpu=cpu)
+                kernel="gemv_rows_kernel" if M <= 4 else "skinny_kernel", cpu=cpu)
 
 
 def wl_gemm_w4a16(dev):
@@ -144,6 +144,19 @@ def wl_gemm_w4a16(dev):
     return dict(launch=launch, R=1, bytes=alg_bytes, flops=2 * M * N * K, bound="mfma", dtype="bf16",
                 name=f"cfg2 W4A16 asymmetric group-128 prefill GEMM M={M} K={K} N={N} bf16",
                 kernel="gemm_w4a16_kernel", cpu=cpu, cpu_scale=256 / M)
+
+
+def wl_copy(dev):
+    """Plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    n = 256 << 20
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+
+    def launch(i):
+        dst.copy_(src)
+
+    return dict(launch=launch, R=1, bytes=2 * n, flops=0, bound="hbm", dtype="u8",
+                name="plain device copy, 256 MiB read + 256 MiB written", kernel="copy", cpu=lambda: None)
 
 
 def wl_moe(dev):
@@ -184,6 +197,7 @@ WORKLOADS = {
     "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
     "cfg1_m32": lambda dev: wl_fp8_pern(32, dev),
     "cfg0": wl_int4_gemv,
+    "copy": wl_copy,
     "cfg2": wl_gemm_w4a16,
     "cfg3": wl_moe,
     "cfg4_m1": lambda dev: wl_q4k(1, dev),
@@ -224,6 +238,15 @@ def run_gpu(wl, steps: int, warmup: int):
     return t1 - t0, e0.elapsed_time(e1)
 
 
+def measured_traffic(workload_id):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary, or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(workload_id, {}).get("bytes")
+    except (OSError, ValueError):
+        return None
+
+
 def summarize(wl, steps, wall_s, ev_ms):
     per_launch_s = ev_ms * 1e-3 / steps
     if wl["bound"] == "hbm":
@@ -261,10 +284,16 @@ def cpu_baseline(wl, budget_s: float = 20.0):
             break
     times.sort()
     med = times[len(times) // 2]
-    return {"value": wl["bytes"] / med / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "seconds_per_step": med,
-            "sample": f"{len(times)} timed passes (after 2 warm-ups) of the full workload: torch dequant "
-                      f"of the whole weight + fp32 matmul, {wl['name']}"}
+    frac = wl.get("cpu_scale", 1.0)                 # share of the workload one CPU pass covers
+    if wl["bound"] == "hbm":
+        value, unit = wl["bytes"] * frac / med / 1e9, "GB/s"
+    else:
+        value, unit = wl["flops"] * frac / med / 1e12, "TFLOP/s"
+    what = "the full workload" if frac == 1.0 else f"{frac:.3f} of the workload's rows"
+    return {"value": value, "unit": unit, "cores": cores, "kind": "port",
+            "seconds_per_pass": med,
+            "sample": f"{len(times)} timed passes (after 2 warm-ups) over {what}: torch dequant of the "
+                      f"whole weight + fp32 matmul, {wl['name']}"}
 
 
 def main():
@@ -289,6 +318,7 @@ def main():
     wl = WORKLOADS[args.workload](dev)
     wall, ev = run_gpu(wl, args.steps, args.warmup)
     head = summarize(wl, args.steps, wall, ev)
+    head["roofline"]["traffic"] = measured_traffic(args.workload)
     cpu = None if args.no_cpu else cpu_baseline(wl)
     del wl
     torch.cuda.empty_cache()
