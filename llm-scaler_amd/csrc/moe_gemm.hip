@@ -40,109 +40,170 @@ struct MoeGemmArgs {
   int total_rows;             // rows in `out`
 };
 
+// LDS staging geometry.  A wavefront stages one K granule (128 k) of its weight
+// tiles and of the expert's activation rows in a private LDS region: global
+// loads are row-coalesced (8 or 16 consecutive lanes read one row's contiguous
+// 128 / 256 bytes — loading the MFMA operand layout directly, where consecutive
+// lanes hit different rows, halves the L1 rate once the activation stream from
+// L2 is added to the weight stream), and the operands are then read back in MFMA
+// layout.  Rows are padded by 16 bytes so that the 16 lanes of an operand read
+// (row stride 144 / 272 bytes) fall into distinct banks.
+constexpr int kWPitch = 128 + 16;                    // fp8 weight / activation row of one granule
+constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of one granule
+
+template <bool A8, int RT>
+__host__ __device__ constexpr int moe_stage_bytes() {
+  return RT * 16 * kWPitch + 64 * (A8 ? kWPitch : kA16Pitch);
+}
+
 // One pass over K for a chunk of MTC 16-row activation tiles.  The weights are the
 // MFMA A operand and the activations the B operand, so a lane ends up holding
 // ONE activation row (mt*16 + j) and four consecutive weight rows (4 g + v): the
 // per-row activation scale is then a single value per lane, tile and granule.
-// Granules are software-pipelined through two register buffers; loads of a
-// granule (weights first, then activations, then scales) are issued together so
-// that the in-order memory counter lets granule i be consumed while granule
-// i + 1 is still in flight.
+// The global loads of granule i+1 are issued right after granule i has been
+// written to LDS, so they are in flight while granule i is multiplied.
 template <class Act, bool A8, int RT, int NW, int MTC>
 __device__ __forceinline__ void moe_chunk(const MoeGemmArgs& p, f32x4 (&acc)[RT][4],
                                           __amdgpu_buffer_rsrc_t wr, __amdgpu_buffer_rsrc_t ar,
                                           const float* wsc, const int (&nbase)[RT],
-                                          const uint32_t (&wdead)[RT], const uint32_t (&arow)[4],
-                                          const uint32_t (&adead)[4], int wave, int j, int g) {
+                                          const uint32_t (&woff)[RT][2], const uint32_t (&aoff)[16],
+                                          const uint32_t (&arow)[4], unsigned char* stage, int wave,
+                                          int lane) {
+  static_assert(MTC >= 1 && MTC <= 4, "one to four activation tiles");
   using V8 = typename Act::v8;
-  constexpr int NA = A8 ? 2 : 4;                      // 16-byte loads per activation row per granule
+  constexpr int NAI = A8 ? 2 * MTC : 4 * MTC;         // activation staging loads per granule
+  constexpr int APitch = A8 ? kWPitch : kA16Pitch;
+  constexpr uint32_t AGran = A8 ? 128u : 256u;        // activation bytes per row per granule
+  const int j = lane & 15, g = lane >> 4;
   const int K = p.K;
   const int G = K >> 7;
   const int Kb = G;
   const int Nb = (p.N + 127) >> 7;
-  const uint32_t a_esz = A8 ? 1u : 2u;
+  unsigned char* wl = stage;
+  unsigned char* al = stage + RT * 16 * kWPitch;
+  // staging slots of this lane
+  const int wrow = lane >> 3, wch = lane & 7;          // weights and fp8 activations: 8 lanes per row
+  const int a16row = lane >> 4, a16ch = lane & 15;     // 16-bit activations: 16 lanes per row
 
-  struct Frag {
-    u32x4 wa[RT], wb[RT];
-    u32x4 af[MTC][NA];
-    float ws[RT];
-    float xs[MTC];
+  struct Regs {                                       // one granule in flight
+    u32x4 w[RT][2];
+    u32x4 a[NAI];
+    float ws[RT], xs[MTC];
   };
-  auto load_frag = [&](Frag& f, int gi) {
-    const uint32_t gdead = (uint32_t)(gi >= G) << 31;
+  // The granule index enters every address as a scalar offset, so a load costs no
+  // vector ALU work.  A prefetch past the last granule re-reads the last one
+  // (clamped index); its data is never staged.
+  const __amdgpu_buffer_rsrc_t xsr = make_rsrc(p.a_scale, A8 ? (uint32_t)p.a_rows * (uint32_t)Kb * 4u : 0u);
+  uint32_t xsoff[MTC];
+#pragma unroll
+  for (int mt = 0; mt < MTC; ++mt) xsoff[mt] = arow[mt] * (uint32_t)Kb * 4u;
+  auto load_granule = [&](Regs& r, int gi) {
     const int gic = gi < G ? gi : G - 1;
-    const uint32_t kl = (uint32_t)gic * 128u + (uint32_t)g * 32u;
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
-      const uint32_t off = ((uint32_t)(nbase[t] + j) * (uint32_t)K + kl) | wdead[t] | gdead;
-      f.wa[t] = __builtin_amdgcn_raw_buffer_load_b128(wr, off, 0, 2);
-      f.wb[t] = __builtin_amdgcn_raw_buffer_load_b128(wr, off + 16u, 0, 2);
-    }
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-    for (int mt = 0; mt < MTC; ++mt) {
-      const uint32_t off = ((arow[mt] * (uint32_t)K + kl) * a_esz) | adead[mt] | gdead;
+      for (int i = 0; i < 2; ++i)
+        r.w[t][i] = __builtin_amdgcn_raw_buffer_load_b128(wr, woff[t][i], (uint32_t)gic * 128u, 2);
 #pragma unroll
-      for (int i = 0; i < NA; ++i) f.af[mt][i] = buf_load16(ar, off + 16u * i);
-    }
+    for (int i = 0; i < NAI; ++i)
+      r.a[i] = __builtin_amdgcn_raw_buffer_load_b128(ar, aoff[i], (uint32_t)gic * AGran, 0);
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       const int nb = min(nbase[t] >> 7, Nb - 1);
-      f.ws[t] = wsc[(size_t)nb * Kb + gic];
+      r.ws[t] = wsc[(size_t)nb * Kb + gic];
     }
     if constexpr (A8) {
 #pragma unroll
-      for (int mt = 0; mt < MTC; ++mt) f.xs[mt] = p.a_scale[(size_t)arow[mt] * Kb + gic];
+      for (int mt = 0; mt < MTC; ++mt)
+        r.xs[mt] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xsr, xsoff[mt], (uint32_t)gic * 4u, 0));
     }
   };
-  auto compute = [&](const Frag& f) {
+  // stage granule `r` into LDS, start the load of granule `next` into the same
+  // registers, then multiply out of LDS
+  auto step = [&](Regs& r, int next) {
+    float wsc_cur[RT], xsc_cur[MTC];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) wsc_cur[t] = r.ws[t];
+#pragma unroll
+    for (int mt = 0; mt < MTC; ++mt) xsc_cur[mt] = A8 ? r.xs[mt] : 1.0f;
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        *reinterpret_cast<u32x4*>(wl + (t * 16 + wrow + 8 * i) * kWPitch + wch * 16) = r.w[t][i];
+#pragma unroll
+    for (int i = 0; i < NAI; ++i) {
+      if constexpr (A8)
+        *reinterpret_cast<u32x4*>(al + (wrow + 8 * i) * APitch + wch * 16) = r.a[i];
+      else
+        *reinterpret_cast<u32x4*>(al + (a16row + 4 * i) * APitch + a16ch * 16) = r.a[i];
+    }
+    load_granule(r, next);                            // prefetch; dead beyond the last granule
+    // operands back in MFMA layout
+    u32x4 wf[RT][2];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        wf[t][i] = *reinterpret_cast<const u32x4*>(wl + (t * 16 + j) * kWPitch + g * 32 + i * 16);
     V8 w16[RT][4];
     if constexpr (!A8) {
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
-        w16[t][0] = fp8x8_to_act<Act>(f.wa[t][0], f.wa[t][1]);
-        w16[t][1] = fp8x8_to_act<Act>(f.wa[t][2], f.wa[t][3]);
-        w16[t][2] = fp8x8_to_act<Act>(f.wb[t][0], f.wb[t][1]);
-        w16[t][3] = fp8x8_to_act<Act>(f.wb[t][2], f.wb[t][3]);
+        w16[t][0] = fp8x8_to_act<Act>(wf[t][0][0], wf[t][0][1]);
+        w16[t][1] = fp8x8_to_act<Act>(wf[t][0][2], wf[t][0][3]);
+        w16[t][2] = fp8x8_to_act<Act>(wf[t][1][0], wf[t][1][1]);
+        w16[t][3] = fp8x8_to_act<Act>(wf[t][1][2], wf[t][1][3]);
       }
     }
 #pragma unroll
     for (int mt = 0; mt < MTC; ++mt) {
+      if constexpr (A8) {
+        const u32x4 x0 = *reinterpret_cast<const u32x4*>(al + (mt * 16 + j) * APitch + g * 32);
+        const u32x4 x1 = *reinterpret_cast<const u32x4*>(al + (mt * 16 + j) * APitch + g * 32 + 16);
+        const long xa = (long)(((uint64_t)x0[1] << 32) | x0[0]);
+        const long xb = (long)(((uint64_t)x0[3] << 32) | x0[2]);
+        const long xc = (long)(((uint64_t)x1[1] << 32) | x1[0]);
+        const long xd = (long)(((uint64_t)x1[3] << 32) | x1[2]);
 #pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-        if constexpr (A8) {
-          const long x0 = (long)(((uint64_t)f.af[mt][0][1] << 32) | f.af[mt][0][0]);
-          const long x1 = (long)(((uint64_t)f.af[mt][0][3] << 32) | f.af[mt][0][2]);
-          const long x2 = (long)(((uint64_t)f.af[mt][1][1] << 32) | f.af[mt][1][0]);
-          const long x3 = (long)(((uint64_t)f.af[mt][1][3] << 32) | f.af[mt][1][2]);
-          const long w0 = (long)(((uint64_t)f.wa[t][1] << 32) | f.wa[t][0]);
-          const long w1 = (long)(((uint64_t)f.wa[t][3] << 32) | f.wa[t][2]);
-          const long w2 = (long)(((uint64_t)f.wb[t][1] << 32) | f.wb[t][0]);
-          const long w3 = (long)(((uint64_t)f.wb[t][3] << 32) | f.wb[t][2]);
-          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, x0, tt, 0, 0, 0);
-          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, x1, tt, 0, 0, 0);
-          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, x2, tt, 0, 0, 0);
-          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, x3, tt, 0, 0, 0);
-          acc[t][mt] += tt * (f.xs[mt] * f.ws[t]);
-        } else {
+        for (int t = 0; t < RT; ++t) {
+          const long w0 = (long)(((uint64_t)wf[t][0][1] << 32) | wf[t][0][0]);
+          const long w1 = (long)(((uint64_t)wf[t][0][3] << 32) | wf[t][0][2]);
+          const long w2 = (long)(((uint64_t)wf[t][1][1] << 32) | wf[t][1][0]);
+          const long w3 = (long)(((uint64_t)wf[t][1][3] << 32) | wf[t][1][2]);
+          f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, xa, tt, 0, 0, 0);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, xb, tt, 0, 0, 0);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, xc, tt, 0, 0, 0);
+          tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, xd, tt, 0, 0, 0);
+          acc[t][mt] += tt * (xsc_cur[mt] * wsc_cur[t]);
+        }
+      } else {
+        V8 xf[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) tt = Act::mfma(w16[t][i], as_v8<V8>(f.af[mt][i]), tt);
-          acc[t][mt] += tt * f.ws[t];
+        for (int i = 0; i < 4; ++i)
+          xf[i] = *reinterpret_cast<const V8*>(al + (mt * 16 + j) * APitch + g * 64 + i * 16);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+          f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) tt = Act::mfma(w16[t][i], xf[i], tt);
+          acc[t][mt] += tt * wsc_cur[t];
         }
       }
     }
   };
 
-  Frag fa, fb;
+  // two granules in flight per wavefront
+  Regs r0, r1;
   int gi = wave;
-  load_frag(fa, gi);
+  load_granule(r0, gi);
+  load_granule(r1, gi + NW);
   while (gi < G) {
-    load_frag(fb, gi + NW);
-    compute(fa);
+    step(r0, gi + 2 * NW);
     gi += NW;
     if (gi >= G) break;
-    load_frag(fa, gi + NW);
-    compute(fb);
+    step(r1, gi + 2 * NW);
     gi += NW;
   }
 }
@@ -151,7 +212,12 @@ template <class Act, bool A8, bool SILU, int RT, int NW>
 __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) {
   using Elem = typename Act::elem;
   constexpr int MT = 4;                               // up to 64 rows per pass
-  __shared__ f32x4 red[NW > 1 ? NW - 1 : 1][RT][MT][64];
+  constexpr int kStage = moe_stage_bytes<A8, RT>();
+  constexpr int kRed = NW * RT * MT * 64 * 16;
+  constexpr int kLds = NW * kStage > kRed ? NW * kStage : kRed;
+  // the cross-wave reduction buffer overlays the staging regions (used after a barrier)
+  __shared__ __attribute__((aligned(16))) unsigned char smem[kLds];
+  f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
 
   const int e = blockIdx.x / p.tiles_per_expert;
   const int tile = blockIdx.x - e * p.tiles_per_expert;
@@ -166,16 +232,22 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
   const int half = N >> 1;
   // weight rows of this workgroup: tile t covers rows nbase[t] .. +16
   int nbase[RT];
-  uint32_t wdead[RT];
+  uint32_t woff[RT][2];                               // staging offsets (granule 0), dead bit for ragged N
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
+    int col;
     if constexpr (SILU) {
-      const int col = (tile * (RT / 2) + (t >> 1)) * 16;       // (gate, up) pairs share a column
+      col = (tile * (RT / 2) + (t >> 1)) * 16;        // (gate, up) pairs share a column
       nbase[t] = (t & 1) * half + col;
-      wdead[t] = (uint32_t)(!(col + j < half)) << 31;
     } else {
-      nbase[t] = (tile * RT + t) * 16;
-      wdead[t] = (uint32_t)(!(nbase[t] + j < N)) << 31;
+      col = (tile * RT + t) * 16;
+      nbase[t] = col;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = (lane >> 3) + 8 * i;
+      const bool ok = col + row < (SILU ? half : N);
+      woff[t][i] = ((uint32_t)(nbase[t] + row) * (uint32_t)K + (uint32_t)(lane & 7) * 16u) | ((uint32_t)(!ok) << 31);
     }
   }
 
@@ -185,19 +257,29 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
   const __amdgpu_buffer_rsrc_t ar = make_rsrc(p.a, (uint32_t)p.a_rows * (uint32_t)K * a_esz);
   const int Nb = (N + 127) >> 7;
   const float* wsc = p.w_scale + (size_t)e * Nb * (K >> 7);
+  unsigned char* stage = smem + wave * kStage;
 
   for (int mc = 0; mc < cnt; mc += 16 * MT) {
     const int rows_here = min(16 * MT, cnt - mc);
     const int mtiles = (rows_here + 15) >> 4;
-    // source row of this lane's activation fragment, per m-tile
-    uint32_t arow[MT], adead[MT];
+    // source rows: in MFMA layout (for the activation scales) and in staging layout
+    uint32_t arow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = mc + mt * 16 + j;
-      const bool ok = m < cnt;
-      adead[mt] = (uint32_t)(!ok) << 31;
-      const int pos = r0 + (ok ? m : 0);
+      const int pos = r0 + (m < cnt ? m : 0);
       arow[mt] = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
+    }
+    uint32_t aoff[16];
+#pragma unroll
+    for (int i = 0; i < (A8 ? 8 : 16); ++i) {
+      const int row = A8 ? (lane >> 3) + 8 * i : (lane >> 4) + 4 * i;
+      const int m = mc + row;
+      const bool ok = m < cnt;
+      const int pos = r0 + (ok ? m : 0);
+      const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
+      const uint32_t ch = A8 ? (uint32_t)(lane & 7) : (uint32_t)(lane & 15);
+      aoff[i] = (src * (uint32_t)K * a_esz + ch * 16u) | ((uint32_t)(!ok) << 31);
     }
 
     f32x4 acc[RT][MT];
@@ -207,57 +289,66 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
       for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     switch (mtiles) {                                  // wave-uniform
-      case 1: moe_chunk<Act, A8, RT, NW, 1>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
-      case 2: moe_chunk<Act, A8, RT, NW, 2>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
-      case 3: moe_chunk<Act, A8, RT, NW, 3>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
-      default: moe_chunk<Act, A8, RT, NW, 4>(p, acc, wr, ar, wsc, nbase, wdead, arow, adead, wave, j, g); break;
+      case 1: moe_chunk<Act, A8, RT, NW, 1>(p, acc, wr, ar, wsc, nbase, woff, aoff, arow, stage, wave, lane); break;
+      case 2: moe_chunk<Act, A8, RT, NW, 2>(p, acc, wr, ar, wsc, nbase, woff, aoff, arow, stage, wave, lane); break;
+      case 3: moe_chunk<Act, A8, RT, NW, 3>(p, acc, wr, ar, wsc, nbase, woff, aoff, arow, stage, wave, lane); break;
+      default: moe_chunk<Act, A8, RT, NW, 4>(p, acc, wr, ar, wsc, nbase, woff, aoff, arow, stage, wave, lane); break;
     }
 
-    // ---- reduce across the NW wavefronts ----
+    // ---- reduce across the NW wavefronts (buffer overlays the staging regions) ----
+    // Every wave deposits its partial tiles; wave w then sums and stores the
+    // activation tiles mt = w, w + NW, ... so the epilogue is spread over the
+    // whole workgroup instead of serialising on one wave.
     if constexpr (NW > 1) {
-      if (wave > 0) {
-#pragma unroll
-        for (int t = 0; t < RT; ++t)
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) red[wave - 1][t][mt][lane] = acc[t][mt];
-      }
       __syncthreads();
-      if (wave == 0) {
 #pragma unroll
-        for (int w = 0; w < NW - 1; ++w)
+      for (int t = 0; t < RT; ++t)
 #pragma unroll
-          for (int t = 0; t < RT; ++t)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[t][mt] += red[w][t][mt][lane];
-      }
+        for (int mt = 0; mt < MT; ++mt)
+          if (mt < mtiles) red[wave][t][mt][lane] = acc[t][mt];
+      __syncthreads();
     }
     // D layout: lane holds activation row mt*16 + j and weight rows nbase + 4 g + v
-    if (wave == 0) {
+    {
       Elem* out = (Elem*)p.out;
       float* out32 = (float*)p.out;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const int m = mc + mt * 16 + j;
-        if (m < cnt) {
-          const size_t orow = (size_t)(r0 + m) * p.n_out;
+        const bool mine = (NW == 1) || ((mt % NW) == wave);
+        if (mine && mt < mtiles) {
+          f32x4 sum[RT];
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            if constexpr (SILU) {
+          for (int t = 0; t < RT; ++t) {
+            if constexpr (NW > 1) {
+              sum[t] = red[0][t][mt][lane];
 #pragma unroll
-              for (int t = 0; t < RT; t += 2) {
-                const int n = nbase[t] + g * 4 + v;      // gate row == output column
-                if (n < half) {
-                  const float gate = acc[t][mt][v], up = acc[t + 1][mt][v];
-                  const float r = gate / (1.0f + expf(-gate)) * up;
-                  if (p.out_f32) out32[orow + n] = r; else out[orow + n] = Act::from_f32(r);
-                }
-              }
+              for (int w = 1; w < NW; ++w) sum[t] += red[w][t][mt][lane];
             } else {
+              sum[t] = acc[t][mt];
+            }
+          }
+          if (m < cnt) {
+            const size_t orow = (size_t)(r0 + m) * p.n_out;
 #pragma unroll
-              for (int t = 0; t < RT; ++t) {
-                const int n = nbase[t] + g * 4 + v;
-                if (n < N) {
-                  if (p.out_f32) out32[orow + n] = acc[t][mt][v]; else out[orow + n] = Act::from_f32(acc[t][mt][v]);
+            for (int v = 0; v < 4; ++v) {
+              if constexpr (SILU) {
+#pragma unroll
+                for (int t = 0; t < RT; t += 2) {
+                  const int n = nbase[t] + g * 4 + v;      // gate row == output column
+                  if (n < half) {
+                    const float gate = sum[t][v], up = sum[t + 1][v];
+                    const float r = gate / (1.0f + __expf(-gate)) * up;
+                    if (p.out_f32) out32[orow + n] = r; else out[orow + n] = Act::from_f32(r);
+                  }
+                }
+              } else {
+#pragma unroll
+                for (int t = 0; t < RT; ++t) {
+                  const int n = nbase[t] + g * 4 + v;
+                  if (n < N) {
+                    if (p.out_f32) out32[orow + n] = sum[t][v]; else out[orow + n] = Act::from_f32(sum[t][v]);
+                  }
                 }
               }
             }
@@ -265,7 +356,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_kernel(const MoeGemmArgs p) 
         }
       }
     }
-    if constexpr (NW > 1) __syncthreads();            // red[] is reused by the next pass
+    if constexpr (NW > 1) __syncthreads();            // the overlay is reused by the next pass
   }
 }
 
