@@ -11,10 +11,44 @@ namespace qlin {
 // One wavefront per token.  Expert e lives in lane e % 64, slot e / 64.  The
 // selection runs on the logits (softmax is monotone): K rounds of wave-wide
 // argmax where the LOWEST index wins ties, then the selected probabilities are
-// renormalised.
+// renormalised.  A round is one 64-bit wave maximum over keys
+// (order-preserving logit bits, ~index), reduced with DPP inside rows of 16
+// lanes and v_readlane across the four rows.
 constexpr int kTopkSlots = 16;                       // up to 1024 experts
 
-template <class Act>
+template <int CTRL>
+__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, 0xF, 0xF, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, 0xF, 0xF, true);
+  const uint64_t o = ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo;
+  return o > v ? o : v;
+}
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+  v = dpp_max_u64<0xB1>(v);
+  v = dpp_max_u64<0x4E>(v);
+  v = dpp_max_u64<0x141>(v);
+  v = dpp_max_u64<0x140>(v);
+  uint64_t r = 0;
+#pragma unroll
+  for (int row = 0; row < 4; ++row) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, row * 16);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), row * 16);
+    const uint64_t o = ((uint64_t)hi << 32) | lo;
+    r = o > r ? o : r;
+  }
+  return r;
+}
+// float -> unsigned, monotone (NaN-free inputs; -inf maps below every finite value)
+__device__ __forceinline__ uint32_t f32_order(float f) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float f32_unorder(uint32_t u) {
+  const uint32_t b = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
+  return __builtin_bit_cast(float, b);
+}
+
+template <class Act, int SLOTS>
 __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,
                                                        typename Act::elem* __restrict__ top_w,
                                                        int32_t* __restrict__ top_ids, int T, int E,
@@ -23,10 +57,10 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   const typename Act::elem* row = logits + (size_t)t * E;
-  float v[kTopkSlots];
+  float v[SLOTS];
   float mx = -INFINITY;
 #pragma unroll
-  for (int s = 0; s < kTopkSlots; ++s) {
+  for (int s = 0; s < SLOTS; ++s) {
     const int e = s * 64 + lane;
     v[s] = e < E ? Act::to_f32(row[e]) : -INFINITY;
     mx = fmaxf(mx, v[s]);
@@ -34,26 +68,25 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
   mx = wave_max(mx);
   float sum = 0.f;
 #pragma unroll
-  for (int s = 0; s < kTopkSlots; ++s) sum += (s * 64 + lane < E) ? __expf(v[s] - mx) : 0.f;
+  for (int s = 0; s < SLOTS; ++s) sum += (s * 64 + lane < E) ? __expf(v[s] - mx) : 0.f;
   sum = wave_sum(sum);
 
   float my_w = 0.f;                                  // lane r keeps the r-th pick
   int my_id = 0;
   float sel_sum = 0.f;
   for (int r = 0; r < K; ++r) {
-    float best = -INFINITY;
-    int best_e = 0x7fffffff;
+    uint64_t key = 0;
 #pragma unroll
-    for (int s = 0; s < kTopkSlots; ++s) {
-      if (v[s] > best) { best = v[s]; best_e = s * 64 + lane; }   // strict: lowest slot kept
+    for (int s = 0; s < SLOTS; ++s) {
+      const uint64_t k = ((uint64_t)f32_order(v[s]) << 32) | (uint32_t)~(uint32_t)(s * 64 + lane);
+      key = k > key ? k : key;
     }
-    const float wbest = wave_max(best);
-    int cand = (best == wbest) ? best_e : 0x7fffffff;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+    key = wave_max_u64(key);
+    const int cand = (int)~(uint32_t)key;
+    const float wbest = f32_unorder((uint32_t)(key >> 32));
     // remove the winner from its owner lane
 #pragma unroll
-    for (int s = 0; s < kTopkSlots; ++s)
+    for (int s = 0; s < SLOTS; ++s)
       if (s * 64 + lane == cand) v[s] = -INFINITY;
     const float p = __expf(wbest - mx) / sum;
     sel_sum += p;
@@ -72,25 +105,116 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
 // order.  Because a token's K experts are distinct, the rank of pair (t, j) in
 // expert e equals the number of tokens t' < t that selected e: a per-expert
 // bitmap over tokens (built with order-independent LDS atomic ORs) plus popcounts
-// gives the rank without any ordered atomics.  Tokens are processed in chunks
-// that fit the LDS bitmap.
+// gives the rank without any ordered atomics.
+//
+// When all tokens fit the LDS bitmap (the serving case) a single exclusive scan
+// of the popcounts over the expert-major words yields, for every word, the final
+// output position of its first pair — expert offsets included — so the kernel is
+// clear, OR, scan, write.  Longer inputs run the chunked path: count, prefix,
+// then one bitmap pass per chunk of tokens.
 constexpr int kSortThreads = 1024;
 constexpr int kSortWords = 4096;                     // bitmap words in LDS
+
+// inclusive scan of one value per thread over the 1024-thread workgroup
+__device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* wave_tot, int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t o = __shfl_up(v, off, 64);
+    if (lane >= off) v += o;
+  }
+  if (lane == 63) wave_tot[wave] = v;
+  __syncthreads();
+  if (tid < 64) {
+    uint32_t w = tid < 16 ? wave_tot[tid] : 0;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      const uint32_t o = __shfl_up(w, off, 64);
+      if (tid >= off) w += o;
+    }
+    if (tid < 16) wave_tot[tid] = w;                  // inclusive totals of waves 0..tid
+  }
+  __syncthreads();
+  return v + (wave ? wave_tot[wave - 1] : 0u);
+}
 
 __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
     int32_t* __restrict__ max_count, int T, int K, int E) {
   __shared__ uint32_t bitmap[kSortWords];
-  __shared__ uint32_t wordpre[kSortWords];
+  __shared__ uint32_t wordpre[kSortWords + 4];
   __shared__ int32_t count[1024];
   __shared__ int32_t start[1025];
   __shared__ int32_t base[1024];
+  __shared__ uint32_t wave_tot[16];
+  __shared__ int32_t mx;
   const int tid = threadIdx.x;
   const int P = T * K;
   const int wpe = kSortWords / E;                     // words per expert in one chunk
   const int Tc = wpe * 32;                            // tokens per chunk
 
+  if (T <= Tc) {
+    // ---- single pass ----
+    constexpr int WPT = kSortWords / kSortThreads;    // consecutive words per thread
+#pragma unroll
+    for (int i = 0; i < WPT; ++i) bitmap[tid + i * kSortThreads] = 0;
+    if (tid == 0) mx = 0;
+    constexpr int kCache = 8;                         // pairs per thread kept in registers
+    int ecache[kCache];
+#pragma unroll
+    for (int i = 0; i < kCache; ++i) {
+      const int q = tid + i * kSortThreads;
+      ecache[i] = q < P ? top_ids[q] : -1;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kCache; ++i) {
+      const int q = tid + i * kSortThreads;
+      if (q < P) { const int tl = q / K; atomicOr(&bitmap[ecache[i] * wpe + (tl >> 5)], 1u << (tl & 31)); }
+    }
+    for (int q = tid + kCache * kSortThreads; q < P; q += kSortThreads) {
+      const int tl = q / K;
+      atomicOr(&bitmap[top_ids[q] * wpe + (tl >> 5)], 1u << (tl & 31));
+    }
+    __syncthreads();
+    uint32_t pc[WPT], tot = 0;
+#pragma unroll
+    for (int i = 0; i < WPT; ++i) { pc[i] = __popc(bitmap[tid * WPT + i]); tot += pc[i]; }
+    const uint32_t incl = block_scan_1024(tot, wave_tot, tid);
+    uint32_t run = incl - tot;
+#pragma unroll
+    for (int i = 0; i < WPT; ++i) { wordpre[tid * WPT + i] = run; run += pc[i]; }
+    if (tid == kSortThreads - 1) wordpre[kSortWords] = run;
+    __syncthreads();
+    // words of expert e: [e * wpe, (e + 1) * wpe); words past E * wpe are empty
+    for (int e = tid; e <= E; e += kSortThreads) {
+      const int s0 = (int)wordpre[min(e * wpe, kSortWords)];
+      expert_start[e] = s0;
+      if (max_count && e < E) atomicMax(&mx, (int)wordpre[min((e + 1) * wpe, kSortWords)] - s0);
+    }
+    auto place = [&](int q, int e) {
+      const int tl = q / K;
+      const int wi = e * wpe + (tl >> 5);
+      const int pos = (int)wordpre[wi] + __popc(bitmap[wi] & ((1u << (tl & 31)) - 1u));
+      sorted_pairs[pos] = q;
+      inv[q] = pos;
+      if (sorted_token) sorted_token[pos] = tl;
+    };
+#pragma unroll
+    for (int i = 0; i < kCache; ++i) {
+      const int q = tid + i * kSortThreads;
+      if (q < P) place(q, ecache[i]);
+    }
+    for (int q = tid + kCache * kSortThreads; q < P; q += kSortThreads) place(q, top_ids[q]);
+    if (max_count) {
+      __syncthreads();
+      if (tid == 0) max_count[0] = mx;
+    }
+    return;
+  }
+
+  // ---- chunked path ----
   if (tid < E) { count[tid] = 0; base[tid] = 0; }
   __syncthreads();
   for (int p = tid; p < P; p += kSortThreads) atomicAdd(&count[top_ids[p]], 1);
@@ -108,7 +232,6 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
   }
   for (int i = tid; i <= E; i += kSortThreads) expert_start[i] = start[i];
   if (max_count) {
-    __shared__ int32_t mx;
     if (tid == 0) mx = 0;
     __syncthreads();
     if (tid < E) atomicMax(&mx, count[tid]);
@@ -268,14 +391,22 @@ int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E,
   if (T < 0 || E < 1 || E > 64 * kTopkSlots || K < 1 || K > 64 || K > E) return MI_ERR_SHAPE;
   if (!T) return MI_OK;
   hipStream_t st = (hipStream_t)stream;
-  if (act_dtype == DT_F16)
-    hipLaunchKernelGGL(moe_topk_kernel<ActF16>, dim3((T + 3) / 4), dim3(256), 0, st, (const _Float16*)logits,
-                       (_Float16*)top_w, top_ids, T, E, K, renorm);
-  else if (act_dtype == DT_BF16)
-    hipLaunchKernelGGL(moe_topk_kernel<ActBF16>, dim3((T + 3) / 4), dim3(256), 0, st, (const __bf16*)logits,
-                       (__bf16*)top_w, top_ids, T, E, K, renorm);
-  else
-    return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  const dim3 grid((T + 3) / 4), block(256);
+#define QLIN_TOPK(SLOTS)                                                                            \
+  do {                                                                                              \
+    if (act_dtype == DT_F16)                                                                        \
+      hipLaunchKernelGGL((moe_topk_kernel<ActF16, SLOTS>), grid, block, 0, st, (const _Float16*)logits, \
+                         (_Float16*)top_w, top_ids, T, E, K, renorm);                               \
+    else                                                                                            \
+      hipLaunchKernelGGL((moe_topk_kernel<ActBF16, SLOTS>), grid, block, 0, st, (const __bf16*)logits,  \
+                         (__bf16*)top_w, top_ids, T, E, K, renorm);                                 \
+  } while (0)
+  if (E <= 128) QLIN_TOPK(2);
+  else if (E <= 256) QLIN_TOPK(4);
+  else if (E <= 512) QLIN_TOPK(8);
+  else QLIN_TOPK(16);
+#undef QLIN_TOPK
   return launch_status();
 }
 
