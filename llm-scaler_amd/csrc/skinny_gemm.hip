@@ -2,8 +2,8 @@
 //
 // Regime: M <= 64 rows of activations against an [N, K] quantized weight.  The
 // weight is read exactly once at full HBM rate; everything else (activations,
-// scales) comes out of L2.  One workgroup owns 16 output columns (weight rows)
-// and all of K; its NW wavefronts interleave 128-wide K granules so that the
+// scales) comes out of L2.  One workgroup owns up to 64 output columns (weight
+// rows, in 16-row tiles) and all of K; its NW wavefronts interleave 128-wide K granules so that the
 // workgroup as a whole walks each weight row front to back, and every lane
 // issues 128-bit loads.  Weights are dequantized in registers to the activation
 // type and fed to v_mfma_f32_16x16x32_{f16,bf16} with the activations as the A
@@ -31,6 +31,7 @@ struct SkinnyArgs {
   int tiles[kMaxMat];         // 16-row tiles per matrix
   int nmat;
   int M, K;
+  int rpw;                    // weight rows owned by one workgroup (<= 16 RT)
   int scale_f16;              // fp8 per-channel: scale is fp16 instead of fp32
 };
 
@@ -62,7 +63,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = lane & 15, g = lane >> 4;
-  const int n0 = tile * (16 * RT);
+  const int n0 = tile * a.rpw;
+  const int nend = min(N, n0 + a.rpw);                // rows past it belong to the next workgroup
   const int G = (K + 127) >> 7;
 
   const uint32_t wrow = kIsFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
@@ -101,9 +103,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
         const int n = n0 + t * 16 + j;
         const int nc = n < N ? n : N - 1;
         const uint32_t woff =
-            ok ? (uint32_t)n * wrow + (kIsFp8 ? (uint32_t)kl : ((uint32_t)kl >> 1)) : kOOB;
+            (ok && n < nend) ? (uint32_t)n * wrow + (kIsFp8 ? (uint32_t)kl : ((uint32_t)kl >> 1)) : kOOB;
         wa[u][t] = buf_load16(wr, woff);
-        if constexpr (kIsFp8) wb[u][t] = buf_load16(wr, ok ? woff + 16 : kOOB);
+        if constexpr (kIsFp8) wb[u][t] = buf_load16(wr, (ok && n < nend) ? woff + 16 : kOOB);
         if constexpr (kIsInt4) {
           sc[u][t] = (float)s16[(size_t)nc * Kg + gic];
           zz[u][t] = zp ? (float)zp[(size_t)nc * Kg + gic] : 8.0f;
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
           sc[u][t] = (float)s16[(size_t)nc * Kb32 + sbc];
           zz[u][t] = (float)qmin[(size_t)nc * Kb32 + sbc];
         } else if constexpr (kBlock) {
-          sc[u][t] = s32[(size_t)((n0 + t * 16) >> 7) * Kb + gic];
+          sc[u][t] = s32[(size_t)(min(n0 + t * 16, N - 1) >> 7) * Kb + gic];
         }
       }
 #pragma unroll
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     const int n = n0 + t * 16 + j;
-    if (n < N) {
+    if (n < nend) {
       float os = 1.0f;
       if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[n] : s32[n];
       if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
@@ -204,12 +206,12 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   }
 }
 
-template <class Act, int FMT, int SC, int MT, int RT, int UN>
-static void launch_one(SkinnyArgs a, hipStream_t st) {
-  constexpr int NW = 8;
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
+static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
   int tiles = 0;
+  a.rpw = rpw;
   for (int i = 0; i < a.nmat; ++i) {
-    a.tiles[i] = (a.N[i] + 16 * RT - 1) / (16 * RT);
+    a.tiles[i] = (a.N[i] + rpw - 1) / rpw;
     tiles += a.tiles[i];
   }
   if (tiles == 0) return;
@@ -219,12 +221,34 @@ static void launch_one(SkinnyArgs a, hipStream_t st) {
 template <class Act, int FMT, int SC>
 static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
   if (a.M == 0) return MI_OK;
-  if (a.M <= 16)
-    launch_one<Act, FMT, SC, 1, 1, 4>(a, st);
-  else if (a.M <= 32)
-    launch_one<Act, FMT, SC, 2, 2, 2>(a, st);
-  else
-    launch_one<Act, FMT, SC, 4, 1, 1>(a, st);
+  {
+    // One workgroup per CU and round, R weight rows each (a multiple of 8, at most
+    // 64): wide workgroups re-read the activations from L2 least often, and an
+    // exact multiple of the CU count leaves no partial last round.  Rows of a
+    // workgroup's last 16-row tile beyond R are dead lanes that load nothing.
+    long ntot = 0;
+    for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
+    const int cus = device_cu_count();
+    int rounds = (int)((ntot + (long)cus * 64 - 1) / ((long)cus * 64));
+    if (rounds < 1) rounds = 1;
+    int rpw = (int)((ntot + (long)cus * rounds - 1) / ((long)cus * rounds));
+    // block scales: tiles must not straddle a 128-row scale block
+    rpw = (FMT == 0 && SC == SC_BLOCK) ? ((rpw + 15) & ~15) : ((rpw + 7) & ~7);
+    if (rpw > 64) rpw = 64;
+    if (rpw <= 16) {
+      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 1, 8, 4>(a, rpw, st);
+      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 1, 8, 2>(a, rpw, st);
+      else launch_one<Act, FMT, SC, 4, 1, 8, 1>(a, rpw, st);
+    } else if (rpw <= 32) {
+      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
+      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
+      else launch_one<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
+    } else {
+      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
+      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 4, 4, 1>(a, rpw, st);
+      else launch_one<Act, FMT, SC, 4, 4, 4, 1>(a, rpw, st);
+    }
+  }
   return launch_status();
 }
 
