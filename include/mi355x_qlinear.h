@@ -76,13 +76,22 @@ int mi_gemv_int4_multi(const void* x, int nmat, const void* const* w, const void
 
 /* ---- INT4 group-128 GEMM, any M (prefill) --------------------------------------
  * Same operands as mi_gemv_int4.  M <= 64 runs the weight-streaming kernel; larger
- * M runs the LDS-tiled MFMA GEMM (weights dequantized to the activation dtype,
- * bit-exact, while they are staged into LDS).  Replaces esimd_gemm_int4_pgrp
+ * M runs the MFMA GEMM (weights dequantized to the activation dtype while they are
+ * staged into LDS; activations re-tiled into MFMA operand order by a pre-pass and
+ * read straight into registers).  Replaces esimd_gemm_int4_pgrp
  * (V/csrc/xpu/esimd_kernel_gemm.sycl:55-91, V/csrc/xpu/esimd_kernels/int4_GEMM.h:291-320),
  * without its 64-row limit; the zero-point operand (cfg2's asymmetric weights) has
- * no counterpart in the reference's kernels. */
+ * no counterpart in the reference's kernels.
+ * mi_gemm_int4 takes its scratch for the re-tiled activations from the stream-
+ * ordered allocator; mi_gemm_int4_ws uses a caller-provided workspace of at least
+ * mi_gemm_int4_workspace() bytes (0 when no workspace is needed), 16-byte aligned,
+ * which must stay untouched until the stream has passed the call. */
 int mi_gemm_int4(const void* x, const void* w, const void* scale, const void* zp, void* out, int M, int N,
                  int K, int act_dtype, void* stream);
+int mi_gemm_int4_workspace(int M, int N, int K, long long* bytes);
+int mi_gemm_int4_ws(const void* x, const void* w, const void* scale, const void* zp, void* out,
+                    void* workspace, long long workspace_bytes, int M, int N, int K, int act_dtype,
+                    void* stream);
 
 /* ---- GGUF Q4_K on the repacked representation, fp16 -------------------------
  * ql [N, K/2] uint8 interleaved nibbles, scale/qmin [N, K/32] fp16;

@@ -17,6 +17,8 @@ exact signatures.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import capi
@@ -219,8 +221,15 @@ def esimd_gemv_int4_fused2(input, w0, s0, o0, w1, s1, o1):
 
 def _gemm_int4(x, w, s, zp, o, who):
     M, N, K = _chk_int4(x, w, s, zp, o, who)
-    capi.call("mi_gemm_int4", x, capi.ptr(x), capi.ptr(w), capi.ptr(s), capi.ptr(zp), capi.ptr(o), M, N, K,
-              capi.act_dtype(x))
+    # the prefill kernel re-tiles the activations into a workspace; it comes from torch's
+    # caching allocator so that the op stays capturable in a HIP graph
+    need = ctypes.c_longlong(0)
+    rc = capi.lib().mi_gemm_int4_workspace(M, N, K, ctypes.byref(need))
+    if rc != 0:
+        raise RuntimeError(f"{who}: {capi.MI_ERRORS.get(rc, rc)}")
+    ws = torch.empty(need.value, dtype=torch.uint8, device=x.device) if need.value else None
+    capi.call("mi_gemm_int4_ws", x, capi.ptr(x), capi.ptr(w), capi.ptr(s), capi.ptr(zp), capi.ptr(o),
+              capi.ptr(ws), need.value, M, N, K, capi.act_dtype(x))
     return o
 
 

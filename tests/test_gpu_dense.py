@@ -334,6 +334,33 @@ def test_gemm_int4_shapes(ops, dev, M, K, N, dt, asym):
     assert _run_gemm_int4(v, dev, M, K, N, dt, asym, seed=M + N) < TOL
 
 
+def test_gemm_int4_c_abi_without_workspace(ops, dev):
+    """mi_gemm_int4 (no workspace argument) takes its scratch from the stream-ordered allocator
+    and must agree bit for bit with the workspace entry point the torch op uses."""
+    import ctypes
+    from mi355x_qlinear import capi
+    v, _ = ops
+    M, K, N = 300, 512, 272
+    x, packed, scale, zp = O.make_int4_case(M, K, N, seed=77, act_dtype=torch.bfloat16, asym=True)
+    xd, wd, sd, zd = x.to(dev), packed.to(dev), scale.to(dev), zp.to(dev)
+    a = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    b = torch.full_like(a, float("nan"))
+    v.esimd_gemm_int4_pgrp_zp(xd, wd, sd, zd, a)
+    capi.call("mi_gemm_int4", xd, capi.ptr(xd), capi.ptr(wd), capi.ptr(sd), capi.ptr(zd), capi.ptr(b), M, N, K,
+              capi.act_dtype(xd))
+    torch.cuda.synchronize()
+    assert torch.equal(a.cpu().view(torch.int16), b.cpu().view(torch.int16))
+    need = ctypes.c_longlong(-1)
+    assert capi.lib().mi_gemm_int4_workspace(M, N, K, ctypes.byref(need)) == 0
+    assert need.value == 304 * K * 2
+    assert capi.lib().mi_gemm_int4_workspace(64, N, K, ctypes.byref(need)) == 0 and need.value == 0
+    # too small a workspace is rejected, nothing is launched
+    ws = torch.empty(16, dtype=torch.uint8, device=dev)
+    with pytest.raises(RuntimeError):
+        capi.call("mi_gemm_int4_ws", xd, capi.ptr(xd), capi.ptr(wd), capi.ptr(sd), capi.ptr(zd), capi.ptr(b),
+                  capi.ptr(ws), 16, M, N, K, capi.act_dtype(xd))
+
+
 def test_cfg2_w4a16_prefill_gemm(ops, dev):
     v, _ = ops
     M, K, N = 2048, 4096, 14336
