@@ -28,6 +28,18 @@
 #include "qlinear_common.hpp"
 #include "../../include/mi355x_qlinear.h"
 
+#ifndef QLIN_EXP_NODQ
+#define QLIN_EXP_NODQ 0
+#endif
+#ifndef QLIN_EXP_NOX
+#define QLIN_EXP_NOX 0
+#endif
+#ifndef QLIN_EXP_TIME
+#define QLIN_EXP_TIME 0
+#endif
+#ifndef QLIN_EXP_NOBAR
+#define QLIN_EXP_NOBAR 0
+#endif
 namespace qlin {
 
 struct GemmArgs {
@@ -105,13 +117,14 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
   const uint32_t xtile0 = (uint32_t)((m0 + wm0) >> 4);
   const uint32_t xtiles = (uint32_t)(Mp >> 4);
   u32x4 xring[4][TM];
-  auto load_x = [&](int slot, int q) {                // a step beyond the last re-reads the last (never used)
+  auto load_x1 = [&](int slot, int b, int q) {        // a step beyond the last re-reads the last (never used)
     const uint32_t qc = (uint32_t)(q < Q ? q : Q - 1);
+    const uint32_t t = xtile0 + b < xtiles ? xtile0 + b : xtiles - 1;     // tiles past M: any valid block
+    xring[slot][b] = __builtin_amdgcn_raw_buffer_load_b128(xr, xlane, (t * (uint32_t)Q + qc) * 1024u, 0);
+  };
+  auto load_x = [&](int slot, int q) {
 #pragma unroll
-    for (int b = 0; b < TM; ++b) {
-      const uint32_t t = xtile0 + b < xtiles ? xtile0 + b : xtiles - 1;   // tiles past M: any valid block
-      xring[slot][b] = __builtin_amdgcn_raw_buffer_load_b128(xr, xlane, (t * (uint32_t)Q + qc) * 1024u, 0);
-    }
+    for (int b = 0; b < TM; ++b) load_x1(slot, b, q);
   };
 
   // ---- weights: per-thread chunk addresses at k = 0
@@ -132,64 +145,91 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
     uint16_t s[B_CH];
     uint8_t z[B_CH];
   };
-  auto load_b = [&](StageB& st, int kt) {
+  // One of the 3 B_CH loads of a stage (idx = 3 i + kind), so that the main loop can
+  // issue them one at a time between MFMAs: a wavefront that issues vector-memory
+  // instructions back to back stalls ~35 cycles on each.
+  auto load_b1 = [&](StageB& st, int kt, int idx) {
     const uint32_t dead = kt < KT ? 0u : 0x80000000u;
     const uint32_t k0 = (uint32_t)kt * kBK;
-#pragma unroll
-    for (int i = 0; i < B_CH; ++i) {
+    const int i = idx / 3, kind = idx % 3;
+    if (kind == 0)
       st.b[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, boff[i] | dead, k0 >> 1, 0);
+    else if (kind == 1)
       st.s[i] = __builtin_amdgcn_raw_buffer_load_b16(sr, ((soff[i] & 0x7fffffffu) * 2u) | (soff[i] & 0x80000000u) | dead,
                                                      (k0 >> 7) * 2u, 0);
-      // without zero-points the resource is empty and the load returns 0
-      const uint8_t zraw = __builtin_amdgcn_raw_buffer_load_b8(zr, soff[i] | dead, k0 >> 7, 0);
-      st.z[i] = has_zp ? zraw : (uint8_t)8;
-    }
+    else          // without zero-points the resource is empty and the load returns 0
+      st.z[i] = __builtin_amdgcn_raw_buffer_load_b8(zr, soff[i] | dead, k0 >> 7, 0);
+  };
+  auto load_b = [&](StageB& st, int kt) {
+#pragma unroll
+    for (int idx = 0; idx < 3 * B_CH; ++idx) load_b1(st, kt, idx);
   };
 
-  // Dequantization of one stage in kPieces pieces (one nibble pair = two halves).
+  // Dequantization of one stage in kPieces pieces of at most 4 vector-ALU
+  // instructions (8 pieces per packed dword of 8 nibbles).
   //   fp16: d = (0x6400 | nib) - (1024 + z) exactly, one packed multiply rounds d * s once.
-  //   bf16: fma(float(nib), s, -z * s) in fp32 is exact ((nib - z) * s has at most
-  //         16 significant bits), then one RNE to bf16.
+  //   bf16: a nibble 0..15 read as an E4M3 code is nib * 2^-9 (codes below 16 are the
+  //         subnormals and the first binade, same spacing), so one v_cvt_pk_f32_fp8
+  //         turns two nibbles into floats; fma(nib * 2^-9, 512 s, -z s) in fp32 is exact
+  //         ((nib - z) * s has at most 16 significant bits), then one RNE to bf16.
   // Both give the same value as rne((nib - z) * s); only the sign of a zero can
   // differ from the subtract-then-multiply form, which no product notices.
-  constexpr int kPieces = B_CH * 4 * 4 * 2;
+  constexpr int kPieces = B_CH * 4 * 8;
   struct DqState {
     uint32_t e, o;
-    uint32_t t0, t1;
+    f32x2 fe, fo;
     u32x4 outv;
+    float sf[B_CH], nzs[B_CH];                        // bf16: 512 * scale and -z * scale (exact)
+    f16x2 sv[B_CH], zv[B_CH];                         // fp16: packed scale and 1024 + z
+  };
+  auto dq_begin = [&](const StageB& st, DqState& q) {
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) {
+      const _Float16 sc = __builtin_bit_cast(_Float16, st.s[i]);
+      const float z = has_zp ? (float)st.z[i] : 8.0f;
+      if constexpr (Act::dt == DT_F16) {
+        const _Float16 z1024 = (_Float16)(1024.0f + z);
+        q.sv[i] = f16x2{sc, sc};
+        q.zv[i] = f16x2{z1024, z1024};
+      } else {
+        q.sf[i] = (float)sc * 512.0f;
+        q.nzs[i] = -z * (float)sc;
+      }
+    }
   };
   constexpr size_t kBufBytes = (size_t)BNP * kPitch * 2;
   auto dq_piece = [&](const StageB& st, int buf, int I, DqState& q) {
-    const int pair = I >> 1, half = I & 1;
-    const int i = pair / 16, dw = (pair / 4) % 4, pp = pair % 4;
-    const _Float16 sc = __builtin_bit_cast(_Float16, st.s[i]);
-    if (half == 0) {
-      if (pp == 0) {
-        const uint32_t w = st.b[i][dw];
-        q.e = w & 0x0F0F0F0Fu;
-        q.o = (w >> 4) & 0x0F0F0F0Fu;
-      }
-      if constexpr (Act::dt == DT_F16) {
-        const uint32_t sel = 0x0C000C00u | ((4u + pp) << 16) | (uint32_t)pp;
-        q.t0 = __builtin_amdgcn_perm(q.o, q.e, sel) | 0x64006400u;
-      } else {
-        q.t0 = __builtin_bit_cast(uint32_t, (float)((q.e >> (8 * pp)) & 0xffu));
-        q.t1 = __builtin_bit_cast(uint32_t, (float)((q.o >> (8 * pp)) & 0xffu));
-      }
+    const int dword = I >> 3, part = I & 7;
+    const int i = dword / 4, dw = dword % 4;
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    auto bf_pair = [&](float a, float b) {
+      const bf16x2_t r = {(__bf16)__builtin_fmaf(a, q.sf[i], q.nzs[i]), (__bf16)__builtin_fmaf(b, q.sf[i], q.nzs[i])};
+      return __builtin_bit_cast(uint32_t, r);
+    };
+    auto f16_pair = [&](int pp) {
+      const uint32_t sel = 0x0C000C00u | ((4u + pp) << 16) | (uint32_t)pp;
+      const uint32_t bits = __builtin_amdgcn_perm(q.o, q.e, sel) | 0x64006400u;
+      return __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, bits) - q.zv[i]) * q.sv[i]);
+    };
+    if (part == 0) {
+      const uint32_t w = st.b[i][dw];
+      q.e = w & 0x0F0F0F0Fu;
+      q.o = (w >> 4) & 0x0F0F0F0Fu;
+    } else if (part == 7) {
+      *reinterpret_cast<u32x4*>(blds[i] + buf * kBufBytes + dw * 16) = q.outv;
+    } else if constexpr (Act::dt == DT_F16) {
+      if (part <= 4) q.outv[part - 1] = f16_pair(part - 1);
     } else {
-      if constexpr (Act::dt == DT_F16) {
-        const _Float16 z1024 = (_Float16)(1024.0f + (float)st.z[i]);
-        const f16x2 zv = {z1024, z1024}, sv = {sc, sc};
-        q.outv[pp] = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, q.t0) - zv) * sv);
-      } else {
-        const float sf = (float)sc;
-        const float nzs = -(float)st.z[i] * sf;       // exact
-        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-        const bf16x2_t r = {(__bf16)__builtin_fmaf(__builtin_bit_cast(float, q.t0), sf, nzs),
-                            (__bf16)__builtin_fmaf(__builtin_bit_cast(float, q.t1), sf, nzs)};
-        q.outv[pp] = __builtin_bit_cast(uint32_t, r);
-      }
-      if (pp == 3) *reinterpret_cast<u32x4*>(blds[i] + buf * kBufBytes + dw * 16) = q.outv;
+      if (part == 1) {
+        q.fe = __builtin_amdgcn_cvt_pk_f32_fp8((int)q.e, false);
+        q.fo = __builtin_amdgcn_cvt_pk_f32_fp8((int)q.o, false);
+      } else if (part == 4) {
+        q.fe = __builtin_amdgcn_cvt_pk_f32_fp8((int)q.e, true);
+        q.fo = __builtin_amdgcn_cvt_pk_f32_fp8((int)q.o, true);
+      } else if (part == 2) q.outv[0] = bf_pair(q.fe[0], q.fo[0]);
+      else if (part == 3) q.outv[1] = bf_pair(q.fe[1], q.fo[1]);
+      else if (part == 5) q.outv[2] = bf_pair(q.fe[0], q.fo[0]);
+      else q.outv[3] = bf_pair(q.fe[1], q.fo[1]);
     }
   };
 
@@ -198,17 +238,23 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
   // step earlier) are dequantized into the other buffer and the weights two steps
   // ahead are fetched into `nxt`.
   constexpr int kMfmas = 2 * TN * TM;
-  constexpr int kEvery = kMfmas / kPieces > 0 ? kMfmas / kPieces : 1;   // MFMAs per dequant piece
+  // pieces are spread evenly over the MFMAs of the step: piece I goes behind the
+  // first MFMA slot with (slot + 1) * kPieces / kMfmas > I
+  uint64_t tacc[6] = {0, 0, 0, 0, 0, 0};
   auto step64 = [&](int kt, int buf, int slot0, StageB& cur, StageB& nxt) {
-    load_b(nxt, kt + 2);
-    __builtin_amdgcn_sched_barrier(0);
+    uint64_t tp = QLIN_EXP_TIME ? __builtin_amdgcn_s_memtime() : 0;
+    auto mark = [&](int i) { if (QLIN_EXP_TIME) { __builtin_amdgcn_sched_barrier(0); const uint64_t t = __builtin_amdgcn_s_memtime(); tacc[i] += t - tp; tp = t; __builtin_amdgcn_sched_barrier(0);} };
     const Elem* Bb = Bs + buf * BNP * kPitch;
     DqState q;
+    dq_begin(cur, q);
     auto rd_w = [&](int a, int s) {
       return *reinterpret_cast<const u32x4*>(Bb + (wn0 + a * 16 + j) * kPitch + s * 32 + g * 8);
     };
     // the weight operand of row a + 1 is fetched from LDS while row a is multiplied
     u32x4 wnext = rd_w(0, 0);
+    constexpr int kHalf = TN * TM;                    // MFMAs per 32-wide step
+    constexpr int kXEvery = kHalf / TM;               // one activation load per kXEvery MFMAs
+    constexpr int kBEvery = kHalf / (3 * B_CH) > 0 ? kHalf / (3 * B_CH) : 1;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
 #pragma unroll
@@ -219,24 +265,26 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
 #pragma unroll
         for (int b = 0; b < TM; ++b) {
           mfma_agpr<Act>(acc[a][b], wcur, xring[slot0 + s][b]);
-          const int slot = (s * TN + a) * TM + b;
-          if (slot % kEvery == 0 && slot / kEvery < kPieces) {
-            dq_piece(cur, buf ^ 1, slot / kEvery, q);
-            // keep MFMAs, vector-ALU pieces and memory accesses in this order
-            __builtin_amdgcn_sched_barrier(0);
-          }
+          const int m = a * TM + b;                   // MFMA index inside this 32-wide step
+          const int slot = s * kHalf + m;
+          const int p0 = slot * kPieces / kMfmas, p1 = (slot + 1) * kPieces / kMfmas;
+#pragma unroll
+          for (int I = p0; I < p1; ++I) { if (!QLIN_EXP_NODQ) dq_piece(cur, buf ^ 1, I, q); }
+          // global loads, one at a time: the ring slot multiplied in the previous
+          // 32-wide step is refilled 3 steps ahead, and in the first half the weight
+          // chunks two 64-wide steps ahead are fetched
+          if (m % kXEvery == kXEvery / 2 && m / kXEvery < TM && !QLIN_EXP_NOX)
+            load_x1((slot0 + s + 3) & 3, m / kXEvery, 2 * kt + s + 3);
+          if (s == 0 && m % kBEvery == 0 && m / kBEvery < 3 * B_CH) load_b1(nxt, kt + 2, m / kBEvery);
+          // keep MFMAs, vector-ALU pieces and memory accesses in this order
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
-      // refill the ring slot, 4 steps ahead; fenced so that the new loads do not
-      // overlap the registers they replace
-      __builtin_amdgcn_sched_barrier(0);
-      load_x(slot0 + s, 2 * kt + s + 4);
-      __builtin_amdgcn_sched_barrier(0);
+      mark(2 * s);
+      mark(2 * s + 1);
     }
-    // pieces that did not fit behind an MFMA (small tiles)
-#pragma unroll
-    for (int I = kMfmas / kEvery; I < kPieces; ++I) dq_piece(cur, buf ^ 1, I, q);
-    __syncthreads();
+    if (!QLIN_EXP_NOBAR) __syncthreads();
+    mark(4);
   };
 
   StageB s0, s1;
@@ -250,6 +298,7 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
   }
   {
     DqState q;
+    dq_begin(s0, q);
 #pragma unroll
     for (int I = 0; I < kPieces; ++I) dq_piece(s0, 0, I, q);
   }
@@ -259,6 +308,11 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
     step64(kt + 1, 1, 2, s0, s1);
   }
 
+  if (QLIN_EXP_TIME && blockIdx.x == QLIN_EXP_TIME - 1 && threadIdx.x == 0) {
+    uint64_t* dbg = (uint64_t*)p.out;
+    for (int i = 0; i < 5; ++i) dbg[i] = tacc[i];
+    return;
+  }
   // the last MFMAs are still in the matrix pipe: wait before reading their results
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   // D = W-tile (rows n) x X-tile^T: lane holds n = 4 g + v (v = 0..3), m = j
