@@ -28,18 +28,6 @@
 #include "qlinear_common.hpp"
 #include "../../include/mi355x_qlinear.h"
 
-#ifndef QLIN_EXP_NODQ
-#define QLIN_EXP_NODQ 0
-#endif
-#ifndef QLIN_EXP_NOX
-#define QLIN_EXP_NOX 0
-#endif
-#ifndef QLIN_EXP_TIME
-#define QLIN_EXP_TIME 0
-#endif
-#ifndef QLIN_EXP_NOBAR
-#define QLIN_EXP_NOBAR 0
-#endif
 namespace qlin {
 
 struct GemmArgs {
@@ -117,10 +105,15 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
   const uint32_t xtile0 = (uint32_t)((m0 + wm0) >> 4);
   const uint32_t xtiles = (uint32_t)(Mp >> 4);
   u32x4 xring[4][TM];
+  uint32_t xtoff[TM];                                 // scalar: byte offset of tile b's block row
+#pragma unroll
+  for (int b = 0; b < TM; ++b) {
+    const uint32_t t = xtile0 + b < xtiles ? xtile0 + b : xtiles - 1;     // tiles past M: any valid block
+    xtoff[b] = __builtin_amdgcn_readfirstlane(t * (uint32_t)Q * 1024u);
+  }
   auto load_x1 = [&](int slot, int b, int q) {        // a step beyond the last re-reads the last (never used)
     const uint32_t qc = (uint32_t)(q < Q ? q : Q - 1);
-    const uint32_t t = xtile0 + b < xtiles ? xtile0 + b : xtiles - 1;     // tiles past M: any valid block
-    xring[slot][b] = __builtin_amdgcn_raw_buffer_load_b128(xr, xlane, (t * (uint32_t)Q + qc) * 1024u, 0);
+    xring[slot][b] = __builtin_amdgcn_raw_buffer_load_b128(xr, xlane, xtoff[b] + qc * 1024u, 0);
   };
   auto load_x = [&](int slot, int q) {
 #pragma unroll
@@ -240,10 +233,7 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
   constexpr int kMfmas = 2 * TN * TM;
   // pieces are spread evenly over the MFMAs of the step: piece I goes behind the
   // first MFMA slot with (slot + 1) * kPieces / kMfmas > I
-  uint64_t tacc[6] = {0, 0, 0, 0, 0, 0};
   auto step64 = [&](int kt, int buf, int slot0, StageB& cur, StageB& nxt) {
-    uint64_t tp = QLIN_EXP_TIME ? __builtin_amdgcn_s_memtime() : 0;
-    auto mark = [&](int i) { if (QLIN_EXP_TIME) { __builtin_amdgcn_sched_barrier(0); const uint64_t t = __builtin_amdgcn_s_memtime(); tacc[i] += t - tp; tp = t; __builtin_amdgcn_sched_barrier(0);} };
     const Elem* Bb = Bs + buf * BNP * kPitch;
     DqState q;
     dq_begin(cur, q);
@@ -269,22 +259,19 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
           const int slot = s * kHalf + m;
           const int p0 = slot * kPieces / kMfmas, p1 = (slot + 1) * kPieces / kMfmas;
 #pragma unroll
-          for (int I = p0; I < p1; ++I) { if (!QLIN_EXP_NODQ) dq_piece(cur, buf ^ 1, I, q); }
+          for (int I = p0; I < p1; ++I) dq_piece(cur, buf ^ 1, I, q);
           // global loads, one at a time: the ring slot multiplied in the previous
           // 32-wide step is refilled 3 steps ahead, and in the first half the weight
           // chunks two 64-wide steps ahead are fetched
-          if (m % kXEvery == kXEvery / 2 && m / kXEvery < TM && !QLIN_EXP_NOX)
+          if (m % kXEvery == kXEvery / 2 && m / kXEvery < TM)
             load_x1((slot0 + s + 3) & 3, m / kXEvery, 2 * kt + s + 3);
           if (s == 0 && m % kBEvery == 0 && m / kBEvery < 3 * B_CH) load_b1(nxt, kt + 2, m / kBEvery);
           // keep MFMAs, vector-ALU pieces and memory accesses in this order
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      mark(2 * s);
-      mark(2 * s + 1);
     }
-    if (!QLIN_EXP_NOBAR) __syncthreads();
-    mark(4);
+    __syncthreads();
   };
 
   StageB s0, s1;
@@ -308,11 +295,6 @@ __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
     step64(kt + 1, 1, 2, s0, s1);
   }
 
-  if (QLIN_EXP_TIME && blockIdx.x == QLIN_EXP_TIME - 1 && threadIdx.x == 0) {
-    uint64_t* dbg = (uint64_t*)p.out;
-    for (int i = 0; i < 5; ++i) dbg[i] = tacc[i];
-    return;
-  }
   // the last MFMAs are still in the matrix pipe: wait before reading their results
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   // D = W-tile (rows n) x X-tile^T: lane holds n = 4 g + v (v = 0..3), m = j
