@@ -153,7 +153,13 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
  *   scattered_w[pos] = top_w[sorted_pairs[pos]]   (esimd_moe_scatter, moe_ops.h:522-569).
  * mi_moe_combine: out[t] = sum_j w * y[inv[t*topk + j]], weights indexed by sorted
  *   position (weights_by_position = 1, esimd_moe_gather, moe_ops.h:627-676) or by
- *   pair; y is in the activation dtype, or fp32 when y_f32 = 1. */
+ *   pair; y is in the activation dtype, or fp32 when y_f32 = 1.
+ * mi_moe_shared_gate: gate[t] = sigmoid(x[t, :] . gate_weight[:]) in fp32
+ *   (moe_down_gate_precompute_kernel, V/csrc/moe_batch/moe.sycl:978-1010).
+ * mi_moe_combine_shared: mi_moe_combine + gate[t] * shared[t, :] (shared expert's
+ *   output, activation dtype; gate may be null = 1), summed in fp32 and rounded once
+ *   (the finalize step of moe_down_finalize_fp8_block_batched_kernel,
+ *   V/csrc/moe_batch/moe.sycl:1570-1663). */
 int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K, int act_dtype,
                      void* stream);
 int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
@@ -162,6 +168,11 @@ int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_
                    void* scattered_w, int K, int topk, int total, void* stream);
 int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
                    int weights_by_position, int act_dtype, int y_f32, void* stream);
+int mi_moe_shared_gate(const void* x, const void* gate_weight, float* gate, int T, int H, int act_dtype,
+                       void* stream);
+int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void* out, const void* shared,
+                          const float* gate, int H, int topk, int T, int weights_by_position, int act_dtype,
+                          int y_f32, void* stream);
 
 /* ---- MoE grouped FP8 block-scaled GEMM ----------------------------------------
  * out[r, :] = a[src(r), :] @ dequant(w[e])^T for the rows r of expert e,

@@ -347,12 +347,15 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(const u32x4* __restri
 
 // final[t] = sum_j w_j * y[pos(t, j)]; weights either per sorted position
 // (by_pos = 1, the reference's scattered_weights) or per pair (top_w).
+// With a shared expert: + gate[t] * shared[t], added in fp32 before the one rounding.
 template <class Act, bool Y32>
 __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ yv,
                                                       const int32_t* __restrict__ inv,
                                                       const typename Act::elem* __restrict__ w,
                                                       typename Act::v8* __restrict__ out, int H8, int topk,
-                                                      int T, int by_pos) {
+                                                      int T, int by_pos,
+                                                      const typename Act::v8* __restrict__ shared,
+                                                      const float* __restrict__ gate) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= (size_t)T * H8) return;
   const int t = (int)(i / H8), c = (int)(i % H8);
@@ -371,10 +374,34 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
       for (int e = 0; e < 8; ++e) acc[e] += wj * Act::to_f32(v[e]);
     }
   }
+  if (shared) {
+    const typename Act::v8 sv = shared[i];
+    const float gt = gate ? gate[t] : 1.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += gt * Act::to_f32(sv[e]);
+  }
   typename Act::v8 o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = Act::from_f32(acc[e]);
   out[i] = o;
+}
+
+// gate[t] = sigmoid(x[t, :] . gw[:]) in fp32, one wavefront per token.
+template <class Act>
+__global__ __launch_bounds__(256) void shared_gate_kernel(const typename Act::v8* __restrict__ x,
+                                                          const typename Act::v8* __restrict__ gw,
+                                                          float* __restrict__ gate, int T, int H8) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  float acc = 0.f;
+  for (int c = lane; c < H8; c += 64) {
+    const typename Act::v8 a = x[(size_t)t * H8 + c], b = gw[c];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += Act::to_f32(a[e]) * Act::to_f32(b[e]);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) gate[t] = 1.0f / (1.0f + __expf(-acc));
 }
 
 static inline dim3 grid1d(size_t n, int bs = 256) { return dim3((unsigned)((n + bs - 1) / bs)); }
@@ -469,9 +496,11 @@ int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_
   return launch_status();
 }
 
-int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
-                   int weights_by_position, int act_dtype, int y_f32, void* stream) {
+int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void* out, const void* shared,
+                          const float* gate, int H, int topk, int T, int weights_by_position, int act_dtype,
+                          int y_f32, void* stream) {
   if (!y || !inv || !w || !out) return MI_ERR_ARG;
+  if (gate && !shared) return MI_ERR_ARG;
   if (H <= 0 || (H % 8) || topk < 1 || T < 0) return MI_ERR_SHAPE;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
   if (!T) return MI_OK;
@@ -479,13 +508,35 @@ int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, 
   const dim3 grid = grid1d((size_t)T * (H / 8));
 #define QLIN_COMBINE(ACT, Y32, WT, OT)                                                                   \
   hipLaunchKernelGGL((combine_kernel<ACT, Y32>), grid, dim3(256), 0, st, y, inv, (const WT*)w, (OT*)out, \
-                     H / 8, topk, T, weights_by_position)
+                     H / 8, topk, T, weights_by_position, (const OT*)shared, gate)
   if (act_dtype == DT_F16) {
     if (y_f32) QLIN_COMBINE(ActF16, true, _Float16, f16x8); else QLIN_COMBINE(ActF16, false, _Float16, f16x8);
   } else {
     if (y_f32) QLIN_COMBINE(ActBF16, true, __bf16, bf16x8); else QLIN_COMBINE(ActBF16, false, __bf16, bf16x8);
   }
 #undef QLIN_COMBINE
+  return launch_status();
+}
+
+int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
+                   int weights_by_position, int act_dtype, int y_f32, void* stream) {
+  return mi_moe_combine_shared(y, inv, w, out, nullptr, nullptr, H, topk, T, weights_by_position, act_dtype,
+                               y_f32, stream);
+}
+
+int mi_moe_shared_gate(const void* x, const void* gate_weight, float* gate, int T, int H, int act_dtype,
+                       void* stream) {
+  if (!x || !gate_weight || !gate) return MI_ERR_ARG;
+  if (H <= 0 || (H % 8) || T < 0) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (!T) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(shared_gate_kernel<ActF16>, dim3((T + 3) / 4), dim3(256), 0, st, (const f16x8*)x,
+                       (const f16x8*)gate_weight, gate, T, H / 8);
+  else
+    hipLaunchKernelGGL(shared_gate_kernel<ActBF16>, dim3((T + 3) / 4), dim3(256), 0, st, (const bf16x8*)x,
+                       (const bf16x8*)gate_weight, gate, T, H / 8);
   return launch_status();
 }
 

@@ -151,6 +151,19 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
                                       output, top_k, act_quant)
 
 
+def moe_forward_full_fp8_block(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight,
+                               shared_gate_up_scale, down_weight, down_scale, shared_down_weight,
+                               shared_down_scale, shared_expert_gate_weight, top_k, num_shared_experts,
+                               n_routed_experts):
+    """Allocates the output and runs torch.ops.moe_ops.moe_forward_full_fp8_block
+    (V/python/custom_esimd_kernels_vllm/ops.py:1092-1125)."""
+    output = torch.empty_like(x)
+    return torch.ops.moe_ops.moe_forward_full_fp8_block(
+        x, logits, output, gate_up_weight, gate_up_scale, shared_gate_up_weight, shared_gate_up_scale,
+        down_weight, down_scale, shared_down_weight, shared_down_scale, shared_expert_gate_weight,
+        top_k, num_shared_experts, n_routed_experts)
+
+
 def precompute_moe_route(topk_weights, topk_ids, num_experts):
     """Same contract as the reference helper: (sorted_rows, sorted_weights, rows_per_expert),
     stable by expert; computed on the device by the sort kernel."""

@@ -572,6 +572,81 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
     return output
 
 
+def moe_forward_full_fp8_block(x, logits, output, gate_up_weight, gate_up_scale, shared_gate_up_weight,
+                               shared_gate_up_scale, down_weight, down_scale, shared_down_weight,
+                               shared_down_scale, shared_expert_gate_weight, top_k, num_shared_experts,
+                               n_routed_experts):
+    """Small-batch fused MoE decode step for 128x128 block-FP8 weights, w8a16:
+    softmax top-k (renormalised) -> routed experts (gate_up, SiLU*mul, down) weighted sum
+    + sigmoid(x . shared_expert_gate_weight) * shared expert.  Same arguments and checks as
+    the reference op (V/csrc/moe_batch/moe.sycl:1707-1853); bf16 is accepted besides fp16
+    and the 12-token limit is lifted (more tokens simply run the grouped kernels)."""
+    who = "moe_forward_full_fp8_block"
+    _chk(x.dim() == 2 and x.shape[0] >= 1, f"{who}: x must be [T, H] with T >= 1")
+    _chk_act(x, output, who)
+    _chk(tuple(output.shape) == tuple(x.shape), f"{who}: output must have x's shape")
+    _chk(output.data_ptr() != x.data_ptr(), f"{who} output must not alias x")
+    _chk(int(num_shared_experts) == 1, f"{who} requires one shared expert")
+    E, k = int(n_routed_experts), int(top_k)
+    _chk(E > 0 and 0 < k <= E, f"{who} requires 0 < top_k <= n_routed_experts")
+    T, H = x.shape
+    _chk(logits.dim() == 2 and tuple(logits.shape) == (T, E) and logits.dtype == x.dtype, f"{who}: logits must be [T, E] in x's dtype")
+    for name, w in (("gate_up_weight", gate_up_weight), ("down_weight", down_weight),
+                    ("shared_gate_up_weight", shared_gate_up_weight), ("shared_down_weight", shared_down_weight)):
+        _chk(w.dtype in (torch.float8_e4m3fn, torch.uint8), f"{who} requires e4m3 weights ({name} is {w.dtype})")
+    for name, t in (("gate_up_scale", gate_up_scale), ("down_scale", down_scale),
+                    ("shared_gate_up_scale", shared_gate_up_scale), ("shared_down_scale", shared_down_scale)):
+        _chk(t.dtype == torch.float32, f"{who}: {name} must be fp32")
+    _chk(gate_up_weight.dim() == 3 and gate_up_weight.shape[0] == E and gate_up_weight.shape[2] == H and
+         gate_up_weight.shape[1] % 2 == 0, f"{who}: gate_up_weight must be [E, 2I, H]")
+    I = gate_up_weight.shape[1] // 2
+    _chk(H % 128 == 0 and I % 128 == 0, f"{who}: hidden and intermediate sizes must be multiples of 128")
+    _chk(tuple(down_weight.shape) == (E, H, I), f"{who}: down_weight must be [E, H, I]")
+    _chk(tuple(shared_gate_up_weight.shape) == (2 * I, H) and tuple(shared_down_weight.shape) == (H, I),
+         f"{who}: shared weights must be [2I, H] and [H, I]")
+    _chk(tuple(gate_up_scale.shape) == (E, 2 * I // 128, H // 128) and tuple(down_scale.shape) == (E, H // 128, I // 128),
+         f"{who}: routed scales must be [E, 2I/128, H/128] and [E, H/128, I/128]")
+    _chk(tuple(shared_gate_up_scale.shape) == (2 * I // 128, H // 128) and
+         tuple(shared_down_scale.shape) == (H // 128, I // 128), f"{who}: shared scales must be [2I/128, H/128] and [H/128, I/128]")
+    _chk(tuple(shared_expert_gate_weight.shape) == (1, H) and shared_expert_gate_weight.dtype == x.dtype,
+         f"{who}: shared_expert_gate_weight must be [1, H] in x's dtype")
+    for name, t in (("logits", logits), ("output", output), ("gate_up_weight", gate_up_weight),
+                    ("gate_up_scale", gate_up_scale), ("shared_gate_up_weight", shared_gate_up_weight),
+                    ("shared_gate_up_scale", shared_gate_up_scale), ("down_weight", down_weight),
+                    ("down_scale", down_scale), ("shared_down_weight", shared_down_weight),
+                    ("shared_down_scale", shared_down_scale), ("shared_expert_gate_weight", shared_expert_gate_weight)):
+        _chk(t.device == x.device, f"{who}: {name} must be on the same device as x")
+        _chk(t.is_contiguous(), f"{who}: {name} must be contiguous")
+    dev = x.device
+    P = T * k
+    # routing and routed experts (w8a16 grouped GEMMs on the expert-sorted pairs)
+    top_w = torch.empty(T, k, dtype=x.dtype, device=dev)
+    top_ids = torch.empty(T, k, dtype=torch.int32, device=dev)
+    esimd_moe_topk(logits, top_w, top_ids, T)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    start = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
+    moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
+    inter = torch.empty(P, I, dtype=x.dtype, device=dev)
+    y = torch.empty(P, H, dtype=torch.float32, device=dev)
+    moe_gemm_fp8_block(x, None, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
+    moe_gemm_fp8_block(inter, None, None, down_weight, down_scale, start, y, H, I, E, False)
+    # shared expert: dense block-scaled GEMMs on all tokens
+    sh_gu = torch.empty(T, 2 * I, dtype=x.dtype, device=dev)
+    esimd_gemm_fp8_blockscale(x, shared_gate_up_weight, shared_gate_up_scale, sh_gu, 128, 128)
+    sh_inter = torch.empty(T, I, dtype=x.dtype, device=dev)
+    esimd_moe_silu_mul(sh_gu, sh_inter, 2 * I, I, T)
+    sh_out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    esimd_gemm_fp8_blockscale(sh_inter, shared_down_weight, shared_down_scale, sh_out, 128, 128)
+    gate = torch.empty(T, dtype=torch.float32, device=dev)
+    capi.call("mi_moe_shared_gate", x, capi.ptr(x), capi.ptr(shared_expert_gate_weight), capi.ptr(gate), T, H,
+              capi.act_dtype(x))
+    capi.call("mi_moe_combine_shared", y, capi.ptr(y), capi.ptr(inv), capi.ptr(top_w), capi.ptr(output),
+              capi.ptr(sh_out), capi.ptr(gate), H, k, T, 0, capi.act_dtype(output), 1)
+    return output
+
+
 def moe_combine(y, inv, top_w, output, top_k):
     """output[t] = sum_j top_w[t, j] * y[inv[t * top_k + j]]; y fp32 or the activation dtype."""
     who = "moe_combine"
@@ -688,6 +763,11 @@ def register():
     _define("moe_ops", "moe_topk(Tensor logits, int top_k, bool norm) -> (Tensor, Tensor)", moe_topk,
             lambda logits, top_k, norm: (logits.new_empty(logits.shape[0], top_k),
                                          logits.new_empty(logits.shape[0], top_k, dtype=torch.int32)))
+    _define("moe_ops", "moe_forward_full_fp8_block(Tensor x, Tensor logits, Tensor(a!) output, Tensor gate_up_weight, "
+                       "Tensor gate_up_scale, Tensor shared_gate_up_weight, Tensor shared_gate_up_scale, "
+                       "Tensor down_weight, Tensor down_scale, Tensor shared_down_weight, Tensor shared_down_scale, "
+                       "Tensor shared_expert_gate_weight, int top_k, int num_shared_experts, "
+                       "int n_routed_experts) -> Tensor(a!)", moe_forward_full_fp8_block, _ret(2))
     _define("moe_fp8_prefill_ops", "moe_prefill_gather_forward_fp8(Tensor selected_experts, int num_experts) -> Tensor[]",
             moe_prefill_gather_forward_fp8)
     # siblings without a reference counterpart

@@ -546,3 +546,27 @@ def max_rel_err(out: torch.Tensor, ref: torch.Tensor) -> float:
     r = ref.to(torch.float32)
     floor = r.abs().mean().clamp(min=1e-12)
     return float(((o - r).abs() / r.abs().clamp(min=float(floor))).max())
+
+
+def moe_forward_full(x, logits, w13, s13, shared_w13, shared_s13, w2, s2, shared_w2, shared_s2, shared_gate, top_k):
+    """Small-batch fused MoE decode step with one shared expert, fp32 throughout.
+    Follows the per-token loop of V/tests/test_moe_forward_full_fp8_block.py:49-80:
+    softmax -> top-k (lowest index wins ties) -> renormalise -> routed experts ->
+    + sigmoid(x . gate) * shared expert.  Weights are uint8 E4M3 codes with 128x128
+    block scales."""
+    top_w, top_ids = moe_topk(logits, top_k, out_dtype=torch.float32)
+    x32 = x.float()
+    out = torch.zeros_like(x32)
+    dw13 = fp8_dequant_block(w13, s13)
+    dw2 = fp8_dequant_block(w2, s2)
+    for t in range(x.shape[0]):
+        for j in range(top_k):
+            e = int(top_ids[t, j])
+            gate, up = (x32[t] @ dw13[e].t()).chunk(2, dim=-1)
+            inter = torch.nn.functional.silu(gate) * up
+            out[t] += top_w[t, j].float() * (inter @ dw2[e].t())
+    g = torch.sigmoid(x32 @ shared_gate.float().t())
+    gate, up = (x32 @ fp8_dequant_block(shared_w13, shared_s13).t()).chunk(2, dim=-1)
+    sh = torch.nn.functional.silu(gate) * up
+    out += g * (sh @ fp8_dequant_block(shared_w2, shared_s2).t())
+    return out

@@ -279,3 +279,59 @@ def test_moe_forward_small(v, dev, T, E, K, H, I, aq):
 def test_cfg3_moe_forward(v, dev):
     out = _check_forward(v, dev, 512, 128, 8, 2048, 768, True, seed=1237)
     assert torch.isfinite(out.float()).all()
+
+
+# ----------------------------------------------------------------- fused decode op with shared expert
+def _full_case(T, seed, dtype, experts=16, hidden=256, inter=128):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, hidden, generator=g) * 0.2).to(dtype)
+    logits = (torch.randn(T, experts, generator=g) * 0.4).to(dtype)
+    w13, s13 = O.fp8_quantize_block(torch.randn(experts, 2 * inter, hidden, generator=g) * 0.15)
+    w2, s2 = O.fp8_quantize_block(torch.randn(experts, hidden, inter, generator=g) * 0.15)
+    sw13, ss13 = O.fp8_quantize_block(torch.randn(2 * inter, hidden, generator=g) * 0.15)
+    sw2, ss2 = O.fp8_quantize_block(torch.randn(hidden, inter, generator=g) * 0.15)
+    gate = (torch.randn(1, hidden, generator=g) * 0.1).to(dtype)
+    return x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 8, 10, 12, 40])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_moe_forward_full_fp8_block(v, dev, T, dtype):
+    # V/tests/test_moe_forward_full_fp8_block.py:83-150 (same sizes, same bars); T = 40 is beyond
+    # the reference's 12-token limit
+    top_k = 4
+    x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate = _full_case(T, 100 + T, dtype)
+    expected = O.moe_forward_full(x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate, top_k)
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    out = torch.empty(T, x.shape[1], dtype=dtype, device=dev)
+    r = torch.ops.moe_ops.moe_forward_full_fp8_block(
+        x.to(dev), logits.to(dev), out, f8(w13), s13.to(dev), f8(sw13), ss13.to(dev), f8(w2), s2.to(dev),
+        f8(sw2), ss2.to(dev), gate.to(dev), top_k, 1, 16)
+    assert r.data_ptr() == out.data_ptr()
+    actual = out.cpu().float()
+    mean_rel = ((actual - expected).abs().mean() / expected.abs().mean()).item()
+    cos = torch.nn.functional.cosine_similarity(actual.flatten(), expected.flatten(), dim=0).item()
+    bar = 3e-3 if dtype == torch.float16 else 1e-2     # the reference's bar is for fp16
+    assert mean_rel < bar and cos > (0.9999 if dtype == torch.float16 else 0.999)
+
+
+def test_moe_forward_full_fp8_block_errors(v, dev):
+    top_k = 4
+    x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate = _full_case(4, 7, torch.float16)
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    xd = x.to(dev)
+    args = [xd, logits.to(dev), torch.empty_like(xd), f8(w13), s13.to(dev), f8(sw13), ss13.to(dev), f8(w2),
+            s2.to(dev), f8(sw2), ss2.to(dev), gate.to(dev), top_k, 1, 16]
+    op = torch.ops.moe_ops.moe_forward_full_fp8_block
+    bad = list(args); bad[2] = xd                                  # output aliases x
+    with pytest.raises(RuntimeError, match="alias"):
+        op(*bad)
+    bad = list(args); bad[13] = 2                                  # two shared experts
+    with pytest.raises(RuntimeError, match="one shared expert"):
+        op(*bad)
+    bad = list(args); bad[12] = 17                                 # top_k > experts
+    with pytest.raises(RuntimeError, match="top_k"):
+        op(*bad)
+    bad = list(args); bad[4] = s13.to(dev).double()                # scale dtype
+    with pytest.raises(RuntimeError):
+        op(*bad)

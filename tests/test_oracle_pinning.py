@@ -338,3 +338,37 @@ def test_matmul_ref_orientation():
     x = torch.tensor([[1.0, 2.0, 3.0]])
     w = torch.tensor([[1.0, 0.0, 0.0], [0.0, 0.0, 1.0]])
     assert O.matmul_ref(x, w).tolist() == [[1.0, 3.0]]
+
+
+def test_moe_forward_full_oracle_against_dense_formulation():
+    """The per-token loop of moe_forward_full must equal a dense restatement: every expert's
+    output computed for every token, masked by the routing matrix (no loop shared with the
+    oracle), plus the gated shared expert.  A transposed weight, a missing renormalisation or
+    a gate applied to the wrong term fails this."""
+    g = torch.Generator().manual_seed(5)
+    T, E, H, I, k = 5, 8, 128, 128, 3
+    x = (torch.randn(T, H, generator=g) * 0.2).half()
+    logits = (torch.randn(T, E, generator=g) * 0.4).half()
+    w13, s13 = O.fp8_quantize_block(torch.randn(E, 2 * I, H, generator=g) * 0.15)
+    w2, s2 = O.fp8_quantize_block(torch.randn(E, H, I, generator=g) * 0.15)
+    sw13, ss13 = O.fp8_quantize_block(torch.randn(2 * I, H, generator=g) * 0.15)
+    sw2, ss2 = O.fp8_quantize_block(torch.randn(H, I, generator=g) * 0.15)
+    gate = (torch.randn(1, H, generator=g) * 0.1).half()
+    got = O.moe_forward_full(x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate, k)
+    # dense restatement with library routines
+    probs = torch.softmax(logits.float(), -1)
+    tw, ti = torch.topk(probs, k, dim=-1)                     # no ties in this random case
+    tw = tw / tw.sum(-1, keepdim=True)
+    route = torch.zeros(T, E).scatter_(1, ti, tw)             # [T, E] routing weights
+    d13 = w13.view(torch.float8_e4m3fn).float() * s13.repeat_interleave(128, -2).repeat_interleave(128, -1)
+    d2 = w2.view(torch.float8_e4m3fn).float() * s2.repeat_interleave(128, -2).repeat_interleave(128, -1)
+    gu = torch.einsum("th,enh->ten", x.float(), d13)          # [T, E, 2I]
+    inter = torch.nn.functional.silu(gu[..., :I]) * gu[..., I:]
+    ye = torch.einsum("tei,ehi->teh", inter, d2)              # [T, E, H]
+    want = (route.unsqueeze(-1) * ye).sum(1)
+    ds13 = sw13.view(torch.float8_e4m3fn).float() * ss13.repeat_interleave(128, -2).repeat_interleave(128, -1)
+    ds2 = sw2.view(torch.float8_e4m3fn).float() * ss2.repeat_interleave(128, -2).repeat_interleave(128, -1)
+    sgu = x.float() @ ds13.t()
+    sh = (torch.nn.functional.silu(sgu[:, :I]) * sgu[:, I:]) @ ds2.t()
+    want = want + torch.sigmoid(x.float() @ gate.float().t()) * sh
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
