@@ -154,6 +154,13 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
  * mi_moe_combine: out[t] = sum_j w * y[inv[t*topk + j]], weights indexed by sorted
  *   position (weights_by_position = 1, esimd_moe_gather, moe_ops.h:627-676) or by
  *   pair; y is in the activation dtype, or fp32 when y_f32 = 1.
+ *   inv may be null: y is then already in pair order (row t*topk + j), as
+ *   moe_prefill_accumulate_forward_fp8 takes it
+ *   (S/csrc/moe_prefill/moe_prefill_fp8.sycl:413-436).
+ * mi_permute_rows: dst[i] = src[map[i]] (scatter = 0) or dst[map[i]] = src[i]
+ *   (scatter = 1) on rows of row_bytes (multiple of 16) bytes; moves grouped-GEMM
+ *   rows between expert-sorted and pair order (the reference's up/down prefill
+ *   kernels scatter to pair order themselves, moe_prefill_fp8.sycl:280-300, :385-411).
  * mi_moe_shared_gate: gate[t] = sigmoid(x[t, :] . gate_weight[:]) in fp32
  *   (moe_down_gate_precompute_kernel, V/csrc/moe_batch/moe.sycl:978-1010).
  * mi_moe_combine_shared: mi_moe_combine + gate[t] * shared[t, :] (shared expert's
@@ -168,6 +175,8 @@ int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_
                    void* scattered_w, int K, int topk, int total, void* stream);
 int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
                    int weights_by_position, int act_dtype, int y_f32, void* stream);
+int mi_permute_rows(const void* src, const int32_t* map, void* dst, int rows, long long row_bytes, int scatter,
+                    void* stream);
 int mi_moe_shared_gate(const void* x, const void* gate_weight, float* gate, int T, int H, int act_dtype,
                        void* stream);
 int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void* out, const void* shared,

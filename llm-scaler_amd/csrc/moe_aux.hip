@@ -345,6 +345,20 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(const u32x4* __restri
   if (c == 0 && weights) weights[pos] = top_w[pair];
 }
 
+// Row permutation of 16-byte chunks: dst[i] = src[map[i]] (gather) or
+// dst[map[i]] = src[i] (scatter); map is a permutation of 0 .. rows-1.
+__global__ __launch_bounds__(256) void permute_rows_kernel(const u32x4* __restrict__ src,
+                                                           const int32_t* __restrict__ map,
+                                                           u32x4* __restrict__ dst, int C, int rows,
+                                                           int scatter) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)rows * C) return;
+  const int r = (int)(i / C), c = (int)(i % C);
+  const int m = map[r];
+  if (scatter) dst[(size_t)m * C + c] = src[i];
+  else dst[i] = src[(size_t)m * C + c];
+}
+
 // final[t] = sum_j w_j * y[pos(t, j)]; weights either per sorted position
 // (by_pos = 1, the reference's scattered_weights) or per pair (top_w).
 // With a shared expert: + gate[t] * shared[t], added in fp32 before the one rounding.
@@ -361,7 +375,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
   const int t = (int)(i / H8), c = (int)(i % H8);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < topk; ++j) {
-    const int pos = inv[(size_t)t * topk + j];
+    const int pos = inv ? inv[(size_t)t * topk + j] : t * topk + j;   // no map: y is in pair order
     const float wj = Act::to_f32(w[by_pos ? pos : t * topk + j]);
     if constexpr (Y32) {
       const f32x4* y = (const f32x4*)yv;
@@ -499,7 +513,7 @@ int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_
 int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void* out, const void* shared,
                           const float* gate, int H, int topk, int T, int weights_by_position, int act_dtype,
                           int y_f32, void* stream) {
-  if (!y || !inv || !w || !out) return MI_ERR_ARG;
+  if (!y || !w || !out) return MI_ERR_ARG;
   if (gate && !shared) return MI_ERR_ARG;
   if (H <= 0 || (H % 8) || topk < 1 || T < 0) return MI_ERR_SHAPE;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
@@ -522,6 +536,17 @@ int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, 
                    int weights_by_position, int act_dtype, int y_f32, void* stream) {
   return mi_moe_combine_shared(y, inv, w, out, nullptr, nullptr, H, topk, T, weights_by_position, act_dtype,
                                y_f32, stream);
+}
+
+int mi_permute_rows(const void* src, const int32_t* map, void* dst, int rows, long long row_bytes, int scatter,
+                    void* stream) {
+  if (!src || !map || !dst) return MI_ERR_ARG;
+  if (rows < 0 || row_bytes <= 0 || (row_bytes % 16) || row_bytes / 16 > 0x7fffffff) return MI_ERR_SHAPE;
+  if (!rows) return MI_OK;
+  const int C = (int)(row_bytes / 16);
+  hipLaunchKernelGGL(permute_rows_kernel, grid1d((size_t)rows * C), dim3(256), 0, (hipStream_t)stream,
+                     (const u32x4*)src, map, (u32x4*)dst, C, rows, scatter);
+  return launch_status();
 }
 
 int mi_moe_shared_gate(const void* x, const void* gate_weight, float* gate, int T, int H, int act_dtype,

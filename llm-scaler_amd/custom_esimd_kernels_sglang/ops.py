@@ -42,3 +42,13 @@ def esimd_gemm_fp8_pert(input, weight, weight_scale, output):
 
 def esimd_gemm_int4_pgrp(input, weight, weight_scale, output):
     return _ops_gemm.esimd_gemm_int4_pgrp(input, weight, weight_scale, output)
+
+
+# FP8 MoE prefill with per-expert scalar scales (torch.ops.moe_fp8_prefill_ops),
+# S/python/custom_esimd_kernels_sglang/ops.py:1656-1675
+_moe_fp8_prefill = torch.ops.moe_fp8_prefill_ops
+
+
+def moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, top_k, num_experts):
+    return _moe_fp8_prefill.moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale,
+                                                 top_k, num_experts)

@@ -676,6 +676,132 @@ def moe_prefill_gather_forward_fp8(selected_experts, num_experts):
     return [start[:E], tokens, perm, start[1:] - start[:E]]
 
 # --------------------------------------------------------------------------
+# sglang FP8 MoE prefill ops (per-expert scalar scales), moe_fp8_prefill_ops
+# --------------------------------------------------------------------------
+def _expert_block_scales(scale, E, parts, rows_per_part, K, who):
+    """[E, parts] per-expert scalars -> [E, parts * rows_per_part / 128, K / 128] block scales
+    (every block of part p of expert e carries scale[e, p])."""
+    _chk(rows_per_part % 128 == 0 and K % 128 == 0,
+         f"{who}: intermediate and hidden sizes must be multiples of 128")
+    s = scale.to(torch.float32).reshape(-1)[:E * parts].reshape(E, parts, 1, 1)
+    return s.expand(E, parts, rows_per_part // 128, K // 128).reshape(E, parts * rows_per_part // 128, K // 128).contiguous()
+
+
+def _prefill_starts(expert_offsets, total):
+    """[E] exclusive offsets -> [E + 1] with the total appended."""
+    tail = torch.full((1,), total, dtype=torch.int32, device=expert_offsets.device)
+    return torch.cat([expert_offsets.reshape(-1), tail]).contiguous()
+
+
+def _permute_rows(src, map_, dst, scatter):
+    rows = map_.numel()
+    capi.call("mi_permute_rows", src, capi.ptr(src), capi.ptr(map_), capi.ptr(dst), rows,
+              src.shape[1] * src.element_size(), 1 if scatter else 0)
+    return dst
+
+
+def moe_prefill_up_forward_fp8(x, gate_up_weight, gate_up_scale, expert_offsets, expert_tokens, top_k):
+    """intermediate[pair] = silu(x[t] @ (s_gate w_gate)^T) * (x[t] @ (s_up w_up)^T) for pair = t*top_k + j,
+    rows grouped per expert by (expert_offsets, expert_tokens) as moe_prefill_gather_forward_fp8 returns them
+    (S/csrc/moe_prefill/moe_prefill_fp8.sycl:480-530).  -> [T*top_k, I] in pair order."""
+    who = "moe_prefill_up_forward_fp8"
+    _chk(x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(), f"{who}: x must be contiguous fp16/bf16 [T, H]")
+    _chk(gate_up_weight.dim() == 3, f"{who}: gate_up_weight must be [E, 2*I, H]")
+    _chk_fp8(gate_up_weight, who)
+    _chk(gate_up_scale.dtype == torch.float32, f"{who}: gate_up_scale must be float32")
+    _chk(expert_offsets.dtype == torch.int32 and expert_tokens.dtype == torch.int32, f"{who}: offsets and tokens must be int32")
+    E, two_i, H = gate_up_weight.shape
+    I = two_i // 2
+    _chk(x.shape[1] == H, f"{who}: x hidden dim must equal w13 last dim")
+    _chk(gate_up_scale.numel() >= 2 * E, f"{who}: gate_up_scale must have >= 2*E entries ([E,2] gate/up)")
+    P = expert_tokens.numel()
+    k = int(top_k)
+    dev = x.device
+    bs = _expert_block_scales(gate_up_scale, E, 2, I, H, who)
+    start = _prefill_starts(expert_offsets, P)
+    tokens = expert_tokens.contiguous()
+    row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
+    inter_sorted = torch.empty(P, I, dtype=x.dtype, device=dev)
+    moe_gemm_fp8_block(x, None, row_map, gate_up_weight, bs, start, inter_sorted, two_i, H, E, True)
+    return _permute_rows(inter_sorted, tokens, torch.empty_like(inter_sorted), scatter=True)
+
+
+def moe_prefill_down_forward_fp8(intermediate, down_weight, down_scale, expert_offsets, expert_tokens):
+    """expert_output[pair] = intermediate[pair] @ (s[e] w2[e])^T, both in pair order
+    (S/csrc/moe_prefill/moe_prefill_fp8.sycl:532-582)."""
+    who = "moe_prefill_down_forward_fp8"
+    _chk(intermediate.dim() == 2 and intermediate.dtype in (torch.float16, torch.bfloat16) and intermediate.is_contiguous(),
+         f"{who}: intermediate must be contiguous fp16/bf16 [T*k, I]")
+    _chk(down_weight.dim() == 3, f"{who}: down_weight must be [E, H, I]")
+    _chk_fp8(down_weight, who)
+    _chk(down_scale.dtype == torch.float32, f"{who}: down_scale must be float32")
+    _chk(expert_offsets.dtype == torch.int32 and expert_tokens.dtype == torch.int32, f"{who}: offsets and tokens must be int32")
+    E, H, I = down_weight.shape
+    _chk(intermediate.shape[1] == I, f"{who}: intermediate dim must equal w2 last dim")
+    _chk(down_scale.numel() >= E, f"{who}: down_scale must have >= E entries")
+    P = expert_tokens.numel()
+    bs = _expert_block_scales(down_scale, E, 1, H, I, who)
+    start = _prefill_starts(expert_offsets, P)
+    tokens = expert_tokens.contiguous()
+    y_sorted = torch.empty(P, H, dtype=intermediate.dtype, device=intermediate.device)
+    moe_gemm_fp8_block(intermediate, None, tokens, down_weight, bs, start, y_sorted, H, I, E, False)
+    return _permute_rows(y_sorted, tokens, torch.empty_like(y_sorted), scatter=True)
+
+
+def moe_prefill_accumulate_forward_fp8(output, routing_weights):
+    """routing_output[t] = sum_j routing_weights[t, j] * output[t*k + j]
+    (S/csrc/moe_prefill/moe_prefill_fp8.sycl:413-436, :584-611)."""
+    who = "moe_prefill_accumulate_forward_fp8"
+    _chk(output.dim() == 2 and routing_weights.dim() == 2, f"{who}: output [T*k, H], routing_weights [T, k]")
+    _chk(output.dtype in (torch.float16, torch.bfloat16) and routing_weights.dtype == output.dtype, f"{who}: fp16/bf16 tensors of one dtype")
+    T, k = routing_weights.shape
+    H = output.shape[1]
+    _chk(output.shape[0] >= T * k and H % 8 == 0, f"{who}: output too small or H not a multiple of 8")
+    res = torch.empty(T, H, dtype=output.dtype, device=output.device)
+    capi.call("mi_moe_combine_shared", output, capi.ptr(output.contiguous()), None, capi.ptr(routing_weights.contiguous()),
+              capi.ptr(res), None, None, H, k, T, 0, capi.act_dtype(res), 0)
+    return res
+
+
+def moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, top_k, num_experts):
+    """Prefill MoE with per-expert scalar scales: stable expert sort -> grouped gate_up GEMM with
+    SiLU*mul -> grouped down GEMM -> weighted combine (S/csrc/moe_prefill/moe_prefill_fp8.sycl:616-649).
+    The intermediate stays in expert-sorted order and the down output in fp32, so the two
+    pair-order round trips of the separate ops are not made here."""
+    who = "moe_prefill_full_fp8"
+    _chk(hidden_states.dtype in (torch.float16, torch.bfloat16), f"{who}: hidden_states must be fp16 (bf16 accepted)")
+    _chk(topk_weights.dtype == hidden_states.dtype, f"{who}: topk_weights must be fp16 (the activation dtype)")
+    _chk(topk_ids.dtype == torch.int32, f"{who}: topk_ids must be int32")
+    k, E = int(top_k), int(num_experts)
+    _chk(topk_ids.dim() == 2 and topk_ids.shape[1] == k, f"{who}: topk_ids must be [M, top_k]")
+    _chk(w13.dim() == 3 and w2.dim() == 3 and w13.shape[0] == E and w2.shape[0] == E, f"{who}: w13 [E,2I,H], w2 [E,H,I]")
+    _chk_fp8(w13, who)
+    _chk_fp8(w2, who)
+    x = hidden_states.contiguous()
+    T, H = x.shape
+    I = w2.shape[2]
+    _chk(tuple(w13.shape) == (E, 2 * I, H) and tuple(w2.shape) == (E, H, I), f"{who}: w13 [E,2I,H], w2 [E,H,I]")
+    _chk(w13_scale.dtype == torch.float32 and w2_scale.dtype == torch.float32, f"{who}: scales must be float32")
+    _chk(w13_scale.numel() >= 2 * E and w2_scale.numel() >= E, f"{who}: w13_scale [E,2], w2_scale [E]")
+    dev = x.device
+    P = T * k
+    ids = topk_ids.contiguous()
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    start = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
+    moe_sort(ids, E, sorted_pairs, start, inv, sorted_token, None)
+    inter = torch.empty(P, I, dtype=x.dtype, device=dev)
+    y = torch.empty(P, H, dtype=torch.float32, device=dev)
+    moe_gemm_fp8_block(x, None, sorted_token, w13, _expert_block_scales(w13_scale, E, 2, I, H, who), start, inter,
+                       2 * I, H, E, True)
+    moe_gemm_fp8_block(inter, None, None, w2, _expert_block_scales(w2_scale, E, 1, H, I, who), start, y, H, I, E, False)
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    moe_combine(y, inv, topk_weights.contiguous(), out, k)
+    return out
+
+
+# --------------------------------------------------------------------------
 # registration
 # --------------------------------------------------------------------------
 def _ret(idx):
@@ -770,6 +896,17 @@ def register():
                        "int n_routed_experts) -> Tensor(a!)", moe_forward_full_fp8_block, _ret(2))
     _define("moe_fp8_prefill_ops", "moe_prefill_gather_forward_fp8(Tensor selected_experts, int num_experts) -> Tensor[]",
             moe_prefill_gather_forward_fp8)
+    _define("moe_fp8_prefill_ops", "moe_prefill_full_fp8(Tensor hidden_states, Tensor topk_weights, Tensor topk_ids, "
+            "Tensor w13, Tensor w13_scale, Tensor w2, Tensor w2_scale, int top_k, int num_experts) -> Tensor",
+            moe_prefill_full_fp8, lambda h, *a: torch.empty_like(h))
+    _define("moe_fp8_prefill_ops", "moe_prefill_up_forward_fp8(Tensor x, Tensor gate_up_weight, Tensor gate_up_scale, "
+            "Tensor expert_offsets, Tensor expert_tokens, int top_k) -> Tensor", moe_prefill_up_forward_fp8,
+            lambda x, w, s, eo, et, k: x.new_empty(et.numel(), w.shape[1] // 2))
+    _define("moe_fp8_prefill_ops", "moe_prefill_down_forward_fp8(Tensor intermediate, Tensor down_weight, "
+            "Tensor down_scale, Tensor expert_offsets, Tensor expert_tokens) -> Tensor", moe_prefill_down_forward_fp8,
+            lambda i, w, s, eo, et: i.new_empty(et.numel(), w.shape[1]))
+    _define("moe_fp8_prefill_ops", "moe_prefill_accumulate_forward_fp8(Tensor output, Tensor routing_weights) -> Tensor",
+            moe_prefill_accumulate_forward_fp8, lambda o, w: o.new_empty(w.shape[0], o.shape[1]))
     # siblings without a reference counterpart
     _define(_V, "moe_sort(Tensor top_ids, int num_experts, Tensor(a!) sorted_pairs, Tensor(b!) expert_start, "
                 "Tensor(c!) inv, Tensor(d!)? sorted_token, Tensor(e!)? max_count) -> Tensor(a!)", moe_sort, _ret(2))

@@ -570,3 +570,29 @@ def moe_forward_full(x, logits, w13, s13, shared_w13, shared_s13, w2, s2, shared
     sh = torch.nn.functional.silu(gate) * up
     out += g * (sh @ fp8_dequant_block(shared_w2, shared_s2).t())
     return out
+
+
+def moe_prefill_scalar(x, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, return_parts=False):
+    """FP8 MoE prefill with per-expert scalar scales, fp32 throughout
+    (S/csrc/moe_prefill/moe_prefill_fp8.sycl:616-649; gate/up scales separate, :196-199):
+      gate = s13[e,0] * (x @ w13[e,:I]^T), up = s13[e,1] * (x @ w13[e,I:]^T),
+      inter = silu(gate) * up, y = s2[e] * (inter @ w2[e]^T), out[t] = sum_j w[t,j] * y[t,j].
+    return_parts also gives the [T*k, I] intermediate and the [T*k, H] expert output in pair order."""
+    T, H = x.shape
+    k = topk_ids.shape[1]
+    E, two_i, _ = w13.shape
+    I = two_i // 2
+    d13 = e4m3_decode(w13.reshape(-1, H)).reshape(E, two_i, H)
+    d2 = e4m3_decode(w2.reshape(-1, I)).reshape(E, H, I)
+    x32 = x.float()
+    inter = torch.zeros(T * k, I)
+    y = torch.zeros(T * k, H)
+    for t in range(T):
+        for j in range(k):
+            e = int(topk_ids[t, j])
+            gate = (x32[t] @ d13[e, :I].t()) * w13_scale[e, 0]
+            up = (x32[t] @ d13[e, I:].t()) * w13_scale[e, 1]
+            inter[t * k + j] = torch.nn.functional.silu(gate) * up
+            y[t * k + j] = (inter[t * k + j] @ d2[e].t()) * w2_scale[e]
+    out = (topk_weights.float().reshape(T, k, 1) * y.reshape(T, k, H)).sum(1)
+    return (out, inter, y) if return_parts else out

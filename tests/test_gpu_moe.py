@@ -13,6 +13,12 @@ TOL = 1e-2
 
 
 @pytest.fixture(scope="module")
+def s(dev):
+    import custom_esimd_kernels_sglang as sg
+    return sg
+
+
+@pytest.fixture(scope="module")
 def v(dev):
     import custom_esimd_kernels_vllm as mod
     return mod
@@ -335,3 +341,65 @@ def test_moe_forward_full_fp8_block_errors(v, dev):
     bad = list(args); bad[4] = s13.to(dev).double()                # scale dtype
     with pytest.raises(RuntimeError):
         op(*bad)
+
+
+# ----------------------------------------------------------------- sglang prefill ops, per-expert scalar scales
+def _prefill_case(T, E, H, I, k, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=g) * 0.3).to(dtype)
+    logits = torch.randn(T, E, generator=g).to(dtype)
+    tw, ti = O.moe_topk(logits, k)
+    w13f = torch.randn(E, 2 * I, H, generator=g) * 0.05
+    w2f = torch.randn(E, H, I, generator=g) * 0.05
+    s13 = torch.stack([w13f[:, :I].abs().amax((1, 2)), w13f[:, I:].abs().amax((1, 2))], 1) / 448.0
+    s2 = w2f.abs().amax((1, 2)) / 448.0
+    w13 = torch.cat([O.e4m3_quantize(w13f[:, :I] / s13[:, 0].view(E, 1, 1)), O.e4m3_quantize(w13f[:, I:] / s13[:, 1].view(E, 1, 1))], 1)
+    w2 = O.e4m3_quantize(w2f / s2.view(E, 1, 1))
+    return x, tw, ti, w13, s13.float().contiguous(), w2, s2.float().contiguous()
+
+
+@pytest.mark.parametrize("T,E,H,I,k,dtype", [(64, 8, 256, 128, 2, torch.float16), (200, 16, 512, 256, 4, torch.bfloat16),
+                                             (1, 4, 128, 128, 1, torch.float16)])
+def test_moe_prefill_full_fp8(s, dev, T, E, H, I, k, dtype):
+    x, tw, ti, w13, s13, w2, s2 = _prefill_case(T, E, H, I, k, 300 + T, dtype)
+    want, inter_ref, y_ref = O.moe_prefill_scalar(x, tw, ti, w13, s13, w2, s2, return_parts=True)
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    op = torch.ops.moe_fp8_prefill_ops
+    got = op.moe_prefill_full_fp8(x.to(dev), tw.to(dev), ti.to(dev), f8(w13), s13.to(dev), f8(w2), s2.to(dev), k, E)
+    assert got.shape == (T, H) and got.dtype == dtype
+    # the intermediate is a 16-bit tensor by the op's contract (w8a16): the reference value of the
+    # output is the down projection of the oracle's intermediate rounded to that dtype
+    ids = ti.reshape(-1).long()
+    d2 = O.e4m3_decode(w2.reshape(-1, I)).reshape(E, H, I)
+    y_r = torch.einsum("pi,phi->ph", inter_ref.to(dtype).float(), d2[ids]) * s2[ids].view(-1, 1)
+    want_r = (tw.float().reshape(T, k, 1) * y_r.reshape(T, k, H)).sum(1)
+    assert O.max_rel_err(got.cpu().float(), want_r) < TOL
+    mean_rel = ((got.cpu().float() - want).abs().mean() / want.abs().mean()).item()
+    assert mean_rel < 5e-3                                      # against the all-fp32 oracle
+    # the staged ops, each against the oracle's pair-ordered intermediates (teacher forcing:
+    # the down op is fed the up op's own rounded output)
+    offs, toks, perm, rows = op.moe_prefill_gather_forward_fp8(ti.to(dev), E)
+    inter = op.moe_prefill_up_forward_fp8(x.to(dev), f8(w13), s13.to(dev), offs, toks, k)
+    assert inter.shape == (T * k, I)
+    assert O.max_rel_err(inter.cpu().float(), inter_ref) < TOL
+    y = op.moe_prefill_down_forward_fp8(inter, f8(w2), s2.to(dev), offs, toks)
+    y_forced = torch.einsum("pi,phi->ph", inter.cpu().float(), d2[ids]) * s2[ids].view(-1, 1)
+    assert O.max_rel_err(y.cpu().float(), y_forced) < TOL
+    acc = op.moe_prefill_accumulate_forward_fp8(y, tw.to(dev))
+    acc_ref = (tw.float().reshape(T, k, 1) * y.cpu().float().reshape(T, k, H)).sum(1)
+    assert O.max_rel_err(acc.cpu().float(), acc_ref) < TOL
+    assert O.max_rel_err(acc.cpu().float(), want) < 3 * TOL     # free-running chain: three 16-bit roundings
+
+
+def test_permute_rows_roundtrip(v, dev):
+    from mi355x_qlinear import capi
+    g = torch.Generator().manual_seed(9)
+    rows, cols = 777, 264
+    src = torch.randn(rows, cols, generator=g).half().to(dev)
+    perm = torch.randperm(rows, generator=g).to(torch.int32).to(dev)
+    a = torch.empty_like(src)
+    b = torch.empty_like(src)
+    capi.call("mi_permute_rows", src, capi.ptr(src), capi.ptr(perm), capi.ptr(a), rows, cols * 2, 0)
+    assert torch.equal(a.cpu(), src.cpu()[perm.cpu().long()])
+    capi.call("mi_permute_rows", a, capi.ptr(a), capi.ptr(perm), capi.ptr(b), rows, cols * 2, 1)
+    assert torch.equal(b.cpu(), src.cpu())

@@ -372,3 +372,30 @@ def test_moe_forward_full_oracle_against_dense_formulation():
     sh = (torch.nn.functional.silu(sgu[:, :I]) * sgu[:, I:]) @ ds2.t()
     want = want + torch.sigmoid(x.float() @ gate.float().t()) * sh
     assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_moe_prefill_scalar_is_the_block_scaled_forward_with_constant_blocks():
+    """Per-expert scalar scales are the special case of 128x128 block scales in which every block of
+    the gate half, of the up half and of the down weight carries one value: the scalar-scale oracle
+    must agree with the (independently pinned) block-scale dequantisation + dense routing algebra."""
+    g = torch.Generator().manual_seed(11)
+    T, E, H, I, k = 6, 4, 128, 128, 2
+    x = (torch.randn(T, H, generator=g) * 0.3).half()
+    tw, ti = O.moe_topk(torch.randn(T, E, generator=g).half(), k)
+    w13 = torch.randint(0, 120, (E, 2 * I, H), generator=g, dtype=torch.int32).to(torch.uint8)
+    w2 = torch.randint(0, 120, (E, H, I), generator=g, dtype=torch.int32).to(torch.uint8)
+    s13 = torch.rand(E, 2, generator=g) * 1e-3 + 1e-4
+    s2 = torch.rand(E, generator=g) * 1e-3 + 1e-4
+    got, inter, y = O.moe_prefill_scalar(x, tw, ti, w13, s13, w2, s2, return_parts=True)
+    b13 = s13.view(E, 2, 1).expand(E, 2, H // 128).reshape(E, 2 * I // 128, H // 128)
+    b2 = s2.view(E, 1, 1).expand(E, H // 128, I // 128)
+    d13, d2 = O.fp8_dequant_block(w13, b13), O.fp8_dequant_block(w2, b2)
+    route = torch.zeros(T, E).scatter_(1, ti.long(), tw.float())
+    gu = torch.einsum("th,enh->ten", x.float(), d13)
+    it = torch.nn.functional.silu(gu[..., :I]) * gu[..., I:]
+    want = (route.unsqueeze(-1) * torch.einsum("tei,ehi->teh", it, d2)).sum(1)
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-7)
+    assert inter.shape == (T * k, I) and y.shape == (T * k, H)
+    # pair order: row t*k + j belongs to token t
+    e = int(ti[3, 1])
+    assert torch.allclose(inter[3 * k + 1], it[3, e], rtol=1e-4, atol=1e-7)
