@@ -82,8 +82,11 @@ int mi_gemv_int4_multi(const void* x, int nmat, const void* const* w, const void
  * (V/csrc/xpu/esimd_kernel_gemm.sycl:55-91, V/csrc/xpu/esimd_kernels/int4_GEMM.h:291-320),
  * without its 64-row limit; the zero-point operand (cfg2's asymmetric weights) has
  * no counterpart in the reference's kernels.
- * mi_gemm_int4 takes its scratch for the re-tiled activations from the stream-
- * ordered allocator; mi_gemm_int4_ws uses a caller-provided workspace of at least
+ * mi_gemm_int4 keeps its scratch for the re-tiled activations in a grow-only
+ * buffer per (device, stream), the convention of the reference's launchers
+ * (V/csrc/xpu/esimd_kernel_moe.sycl:45-67): the first call of a size allocates
+ * (not possible while the stream is being captured), later calls reuse it;
+ * mi_gemm_int4_ws uses a caller-provided workspace of at least
  * mi_gemm_int4_workspace() bytes (0 when no workspace is needed), 16-byte aligned,
  * which must stay untouched until the stream has passed the call. */
 int mi_gemm_int4(const void* x, const void* w, const void* scale, const void* zp, void* out, int M, int N,

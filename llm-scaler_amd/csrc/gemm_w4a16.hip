@@ -26,6 +26,7 @@
 // per 64-wide K step.  The weights are the MFMA A operand, so a lane ends up with
 // 4 consecutive output columns of one row and stores them as 8 bytes.
 #include "qlinear_common.hpp"
+#include "scratch.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -419,14 +420,12 @@ int mi_gemm_int4(const void* x, const void* w, const void* scale, const void* zp
   const int rc = mi_gemm_int4_workspace(M, N, K, &bytes);
   if (rc != MI_OK) return rc;
   if (!bytes) return mi_gemm_int4_ws(x, w, scale, zp, out, nullptr, 0, M, N, K, act_dtype, stream);
-  // stream-ordered scratch for the re-tiled activations; callers that must not
-  // allocate (or that capture the stream) pass their own through mi_gemm_int4_ws
-  hipStream_t st = (hipStream_t)stream;
-  void* ws = nullptr;
-  if (hipMallocAsync(&ws, (size_t)bytes, st) != hipSuccess) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
-  const int rc2 = mi_gemm_int4_ws(x, w, scale, zp, out, ws, bytes, M, N, K, act_dtype, stream);
-  if (hipFreeAsync(ws, st) != hipSuccess) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
-  return rc2;
+  // scratch for the re-tiled activations: this stream's grow-only buffer (the first
+  // call of a size allocates; callers that must never allocate pass their own
+  // workspace through mi_gemm_int4_ws)
+  void* ws = scratch_get((hipStream_t)stream, (size_t)bytes);
+  if (!ws) return MI_ERR_LAUNCH;
+  return mi_gemm_int4_ws(x, w, scale, zp, out, ws, bytes, M, N, K, act_dtype, stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,34 @@
+#include "scratch.hpp"
+
+#include <map>
+#include <mutex>
+#include <utility>
+
+namespace qlin {
+
+namespace {
+struct Buf {
+  void* p = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_mu;
+std::map<std::pair<int, hipStream_t>, Buf> g_bufs;
+}  // namespace
+
+void* scratch_get(hipStream_t stream, size_t bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  std::lock_guard<std::mutex> lock(g_mu);
+  Buf& b = g_bufs[{dev, stream}];
+  if (b.bytes >= bytes && b.p) return b.p;
+  size_t want = 1u << 20;                             // at least 1 MiB, then powers of two
+  while (want < bytes) want <<= 1;
+  void* p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  // the old buffer stays allocated: kernels already queued may still use it
+  b.p = p;
+  b.bytes = want;
+  return p;
+}
+
+}  // namespace qlin
