@@ -10,6 +10,14 @@
 // operand (M padded to 16 inside the matrix core — free while HBM-bound).  The
 // NW partial accumulators are reduced through LDS.
 //
+// Global loads are row-coalesced: consecutive lanes read one row's contiguous
+// bytes of a granule (loading MFMA operand layout directly makes every lane touch
+// a different 16-byte piece, and the texture addresser, not HBM, becomes the
+// limit), and a wave-private LDS tile turns them into operand layout.  The
+// weights always take this path (non-temporal loads); the activations only when
+// there are many rows (M > 32) — for few rows their direct loads are cheaper than
+// the extra LDS traffic.
+//
 // Lane mapping inside one granule (128 k): lane = (j = lane % 16, g = lane / 16)
 // holds the 32 consecutive k  [128 gi + 32 g, +32)  of weight row n0 + j and of
 // activation row j.  MFMA i (0..3) consumes the i-th 8-k slice of both.
@@ -50,7 +58,15 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr bool kIsQ4K = (FMT == 2);
   constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
 
-  __shared__ f32x4 red[NW - 1][RT][MT][64];
+  // wave-private staging tiles for the weights (one 16-row tile = 16 rows of one
+  // granule, padded pitch); the cross-wave reduction buffer overlays them at the end
+  constexpr int kWRowB = kIsFp8 ? 128 : 64;           // weight bytes per row per granule
+  constexpr int kWP = kWRowB + 16;                    // LDS pitch: operand reads hit distinct banks
+  constexpr int kXP = 256 + 16;                       // activation tile pitch
+  constexpr bool kXLds = MT >= 4;                     // stage the activations through LDS too
+  constexpr int kWStage = NW * RT * 16 * kWP;         // activation tiles follow the weight tiles
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
 
   int tile = blockIdx.x;
   int mat = 0;
@@ -102,10 +118,26 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
       for (int t = 0; t < RT; ++t) {
         const int n = n0 + t * 16 + j;
         const int nc = n < N ? n : N - 1;
-        const uint32_t woff =
-            (ok && n < nend) ? (uint32_t)n * wrow + (kIsFp8 ? (uint32_t)kl : ((uint32_t)kl >> 1)) : kOOB;
-        wa[u][t] = buf_load16(wr, woff);
-        if constexpr (kIsFp8) wb[u][t] = buf_load16(wr, (ok && n < nend) ? woff + 16 : kOOB);
+        // weights: row-coalesced (consecutive lanes read one row's contiguous bytes);
+        // they are turned into operand layout through LDS before use
+        if constexpr (kIsFp8) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int r = (lane >> 3) + 8 * h, c = lane & 7;
+            const int nr = n0 + t * 16 + r;
+            const bool okw = gi < G && gi * 128 + c * 16 < K && nr < nend;
+            // non-temporal: the weights are used once and should not displace x in L2
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(
+                wr, okw ? (uint32_t)nr * wrow + (uint32_t)(gi * 128 + c * 16) : kOOB, 0, 2);
+            if (h == 0) wa[u][t] = v; else wb[u][t] = v;
+          }
+        } else {
+          const int r = lane >> 2, c = lane & 3;
+          const int nr = n0 + t * 16 + r;
+          const bool okw = gi < G && gi * 128 + c * 32 < K && nr < nend;
+          wa[u][t] = __builtin_amdgcn_raw_buffer_load_b128(
+              wr, okw ? (uint32_t)nr * wrow + (uint32_t)(gi * 64 + c * 16) : kOOB, 0, 2);
+        }
         if constexpr (kIsInt4) {
           sc[u][t] = (float)s16[(size_t)nc * Kg + gic];
           zz[u][t] = zp ? (float)zp[(size_t)nc * Kg + gic] : 8.0f;
@@ -120,16 +152,52 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
       }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
+        if constexpr (kXLds) {
+          // many rows: row-coalesced as well (16 lanes read one row's 256 contiguous
+          // bytes of the granule), transposed through LDS before use
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
+          for (int i = 0; i < 4; ++i) {
+            const int r = (lane >> 4) + 4 * i, c = lane & 15;
+            const int m = mt * 16 + r;
+            const bool okx = gi < G && gi * 128 + c * 8 < K && m < M;
+            xa[u][mt][i] = buf_load16(xr, okx ? ((uint32_t)m * (uint32_t)K + (uint32_t)(gi * 128 + c * 8)) * 2u : kOOB);
+          }
+        } else {
+          // few rows: straight into operand layout (lane (j, g): row j, 32 consecutive k)
+          const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
+        }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
+      // activations through this wavefront's staging tile into MFMA operand layout:
+      // lane (j, g) ends up with row j, k = 32 g + 8 i .. + 7 of the granule
+#pragma unroll
+      for (int mt = 0; mt < (kXLds ? MT : 0); ++mt) {
+        unsigned char* xl = smem + kWStage + (wave * MT + mt) * 16 * kXP;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          *reinterpret_cast<u32x4*>(xl + ((lane >> 4) + 4 * i) * kXP + (lane & 15) * 16) = xa[u][mt][i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          xa[u][mt][i] = *reinterpret_cast<const u32x4*>(xl + j * kXP + g * 64 + i * 16);
+      }
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
+        // through this wavefront's staging tile into MFMA operand layout
+        unsigned char* wl = smem + (wave * RT + t) * 16 * kWP;
+        if constexpr (kIsFp8) {
+          *reinterpret_cast<u32x4*>(wl + (lane >> 3) * kWP + (lane & 7) * 16) = wa[u][t];
+          *reinterpret_cast<u32x4*>(wl + ((lane >> 3) + 8) * kWP + (lane & 7) * 16) = wb[u][t];
+          wa[u][t] = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32);
+          wb[u][t] = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32 + 16);
+        } else {
+          *reinterpret_cast<u32x4*>(wl + (lane >> 2) * kWP + (lane & 3) * 16) = wa[u][t];
+          wa[u][t] = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 16);
+        }
         V8 b[4];
         if constexpr (kIsFp8) {
           b[0] = fp8x8_to_act<Act>(wa[u][t][0], wa[u][t][1]);
@@ -171,6 +239,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   }
 
   // ---- reduce the NW partial tiles through LDS ----
+  __syncthreads();                                    // the buffer overlays the staging tiles
   if (wave > 0) {
 #pragma unroll
     for (int t = 0; t < RT; ++t)
@@ -215,7 +284,18 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
     tiles += a.tiles[i];
   }
   if (tiles == 0) return;
-  hipLaunchKernelGGL((skinny_kernel<Act, FMT, SC, MT, RT, NW, UN>), dim3(tiles), dim3(NW * 64), 0, st, a);
+  constexpr int kStage = NW * RT * 16 * ((FMT == 0 ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
+  constexpr int kRed = (NW - 1) * RT * MT * 1024;
+  constexpr int lds = kStage > kRed ? kStage : kRed;
+  auto kern = skinny_kernel<Act, FMT, SC, MT, RT, NW, UN>;
+  if (lds > 64 * 1024) {
+    static bool raised = false;                       // opt in to > 64 KiB of dynamic LDS once
+    if (!raised) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(NW * 64), lds, st, a);
 }
 
 template <class Act, int FMT, int SC>
