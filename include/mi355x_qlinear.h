@@ -186,6 +186,18 @@ int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void
                           const float* gate, int H, int topk, int T, int weights_by_position, int act_dtype,
                           int y_f32, void* stream);
 
+/* ---- RMS norm in front of a GEMV -------------------------------------------------
+ * Per row of length L:  a = x (+ residual; residual is then overwritten with the
+ * rounded sum);  out = a * rsqrt(mean(a^2) + eps) * weight[i % weight_len]
+ * (* silu(gate[i]) when gate is given), fp32 arithmetic, one rounding.  residual and
+ * gate may be null.  This is the normalisation half of the reference's fused
+ * decode ops — esimd_resadd_norm_gemv_{int4,fp8}_pert
+ * (V/csrc/xpu/esimd_kernels/resadd_norm_gemv_int4.h:56-100), esimd_norm_gemv_*_pert
+ * (per-head gated norm, norm_gemv_int4.h), esimd_rms_norm (esimd_kernel.sycl:488-502);
+ * the ops run it and then the GEMV entry point on its output. */
+int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weight, void* out, int rows, int L,
+               int weight_len, float eps, int act_dtype, void* stream);
+
 /* ---- MoE grouped FP8 block-scaled GEMM ----------------------------------------
  * out[r, :] = a[src(r), :] @ dequant(w[e])^T for the rows r of expert e,
  * expert_start[e] <= r < expert_start[e+1]; src(r) = row_map[r] if row_map else r.

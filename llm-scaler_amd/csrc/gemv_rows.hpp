@@ -240,8 +240,14 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     load_batch(buf[i], g_next, sb_next);
     advance(g_next, sb_next);
   }
-  float pert_scale = 1.0f;
-  if constexpr (kFp8 && SC == RS_PERT) pert_scale = ((const float*)a.s[0])[0];
+  float pert_scale[kRowsMaxMat];                      // one per-tensor scale per fused matrix
+#pragma unroll
+  for (int i = 0; i < kRowsMaxMat; ++i) {
+    pert_scale[i] = 1.0f;
+    if constexpr (kFp8 && SC == RS_PERT) {
+      if (i < a.nmat) pert_scale[i] = ((const float*)a.s[i])[0];
+    }
+  }
 
   {
 #pragma unroll
@@ -382,7 +388,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       if constexpr (kFp8 && SC == RS_PERN)
         os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, b.os_lo[r])
                          : __builtin_bit_cast(float, (uint32_t)b.os_lo[r] | ((uint32_t)b.os_hi[r] << 16));
-      if constexpr (kFp8 && SC == RS_PERT) os = pert_scale;
+      if constexpr (kFp8 && SC == RS_PERT) os = mat == 0 ? pert_scale[0] : (mat == 1 ? pert_scale[1] : pert_scale[2]);
 #pragma unroll
       for (int m = 0; m < MR; ++m) {
         const float v = wave_sum(acc[r][m]);

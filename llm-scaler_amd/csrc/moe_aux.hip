@@ -418,6 +418,46 @@ __global__ __launch_bounds__(256) void shared_gate_kernel(const typename Act::v8
   if (lane == 0) gate[t] = 1.0f / (1.0f + __expf(-acc));
 }
 
+// ---------------------------------------------------------------- RMS norm (+ residual add, + SiLU gate)
+// One workgroup per row of length L:  a = x (+ residual, which is then updated in
+// place with the rounded sum);  out = a * rsqrt(mean(a^2) + eps) * weight[i % wlen]
+// (* silu(gate)), fp32 throughout, one rounding at the store.
+template <class Act>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const typename Act::elem* __restrict__ x,
+                                                      typename Act::elem* residual,
+                                                      const typename Act::elem* __restrict__ gate,
+                                                      const typename Act::elem* __restrict__ weight,
+                                                      typename Act::elem* __restrict__ out, int L, int wlen,
+                                                      float eps) {
+  __shared__ float wsum[4];
+  const size_t base = (size_t)blockIdx.x * L;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < L; i += 256) {
+    float a = Act::to_f32(x[base + i]);
+    if (residual) a += Act::to_f32(residual[base + i]);
+    ss += a * a;
+  }
+  ss = wave_sum(ss);
+  if (lane == 0) wsum[wave] = ss;
+  __syncthreads();
+  const float tot = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+  const float inv = rsqrtf(tot / (float)L + eps);
+  for (int i = threadIdx.x; i < L; i += 256) {
+    float a = Act::to_f32(x[base + i]);
+    if (residual) {
+      a += Act::to_f32(residual[base + i]);
+      residual[base + i] = Act::from_f32(a);
+    }
+    float v = a * inv * Act::to_f32(weight[i % wlen]);
+    if (gate) {
+      const float z = Act::to_f32(gate[base + i]);
+      v *= z / (1.0f + __expf(-z));
+    }
+    out[base + i] = Act::from_f32(v);
+  }
+}
+
 static inline dim3 grid1d(size_t n, int bs = 256) { return dim3((unsigned)((n + bs - 1) / bs)); }
 
 }  // namespace qlin
@@ -546,6 +586,22 @@ int mi_permute_rows(const void* src, const int32_t* map, void* dst, int rows, lo
   const int C = (int)(row_bytes / 16);
   hipLaunchKernelGGL(permute_rows_kernel, grid1d((size_t)rows * C), dim3(256), 0, (hipStream_t)stream,
                      (const u32x4*)src, map, (u32x4*)dst, C, rows, scatter);
+  return launch_status();
+}
+
+int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weight, void* out, int rows, int L,
+               int weight_len, float eps, int act_dtype, void* stream) {
+  if (!x || !weight || !out) return MI_ERR_ARG;
+  if (rows < 0 || L <= 0 || weight_len <= 0 || (L % weight_len)) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (!rows) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(rmsnorm_kernel<ActF16>, dim3(rows), dim3(256), 0, st, (const _Float16*)x, (_Float16*)residual,
+                       (const _Float16*)gate, (const _Float16*)weight, (_Float16*)out, L, weight_len, eps);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<ActBF16>, dim3(rows), dim3(256), 0, st, (const __bf16*)x, (__bf16*)residual,
+                       (const __bf16*)gate, (const __bf16*)weight, (__bf16*)out, L, weight_len, eps);
   return launch_status();
 }
 

@@ -176,3 +176,37 @@ def precompute_moe_route(topk_weights, topk_ids, num_experts):
     tok = torch.empty(T * k, dtype=torch.int32, device=dev)
     moe_sort(ids, num_experts, pairs, start, inv, tok, None)
     return tok.to(torch.int64), topk_weights.reshape(-1)[pairs.long()].contiguous(), (start[1:] - start[:-1]).contiguous()
+
+
+# decode fusions: RMS norm (+ residual add / SiLU gate) + GEMV
+# (V/python/custom_esimd_kernels_vllm/ops.py:340-560)
+def esimd_rms_norm(input, output, weight, eps):
+    return _ops.esimd_rms_norm(input, output, weight, eps)
+
+
+def esimd_resadd_norm_gemv_int4_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
+                                     normed_out, eps):
+    return _ops.esimd_resadd_norm_gemv_int4_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale,
+                                                 output, normed_out, eps)
+
+
+def esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
+                                    normed_out, eps):
+    return _ops.esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale,
+                                                output, normed_out, eps)
+
+
+def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps):
+    return _ops.esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps)
+
+
+def esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    return _ops.esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)
+
+
+def esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    return _ops.esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)
+
+
+def esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    return _ops.esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)

@@ -676,6 +676,91 @@ def moe_prefill_gather_forward_fp8(selected_experts, num_experts):
     return [start[:E], tokens, perm, start[1:] - start[:E]]
 
 # --------------------------------------------------------------------------
+# decode fusions: RMS norm (+ residual add / + SiLU gate) in front of a GEMV
+# (V/csrc/xpu/torch_extension.cc:103-140).  Two launches here: the norm kernel,
+# then the GEMV entry point on its 16-bit output.
+# --------------------------------------------------------------------------
+def _rmsnorm(x, residual, gate, weight, out, rows, L, eps, who):
+    _chk(x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(), f"{who}: activations must be contiguous fp16/bf16")
+    for name, t in (("residual", residual), ("gate", gate), ("norm_weight", weight), ("normed output", out)):
+        if t is not None:
+            _chk(t.dtype == x.dtype and t.is_contiguous() and t.device == x.device, f"{who}: {name} must match the input's dtype/device and be contiguous")
+    _chk(x.numel() == rows * L and out.numel() >= rows * L, f"{who}: size mismatch")
+    _chk(weight.numel() >= 1 and L % weight.numel() == 0, f"{who}: norm_weight length must divide the row length")
+    capi.call("mi_rmsnorm", x, capi.ptr(x), capi.ptr(residual), capi.ptr(gate), capi.ptr(weight), capi.ptr(out),
+              rows, L, weight.numel(), float(eps), capi.act_dtype(x))
+    return out
+
+
+def esimd_rms_norm(input, output, weight, eps):
+    """output = input * rsqrt(mean(input^2) + eps) * weight, per row (esimd_kernel.sycl:488-502)."""
+    K = input.shape[-1]
+    return _rmsnorm(input, None, None, weight, output, input.numel() // K, K, eps, "esimd_rms_norm")
+
+
+def esimd_resadd_norm_gemv_int4_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
+                                     normed_out, eps):
+    """residual += hidden_states (in place); normed_out = rmsnorm(residual) * norm_weight;
+    output = normed_out @ dequant(int4 weight)^T  (resadd_norm_gemv_int4.h:1-30)."""
+    who = "esimd_resadd_norm_gemv_int4_pert"
+    K = hidden_states.shape[-1]
+    rows = hidden_states.numel() // K
+    _rmsnorm(hidden_states, residual, None, norm_weight, normed_out, rows, K, eps, who)
+    esimd_gemv_int4(normed_out.view(rows, K), gemv_weight, gemv_scale, output)
+    return output
+
+
+def esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
+                                    normed_out, eps):
+    """Same with an FP8 weight and a per-tensor scale (resadd_norm_gemv_fused.h)."""
+    who = "esimd_resadd_norm_gemv_fp8_pert"
+    K = hidden_states.shape[-1]
+    rows = hidden_states.numel() // K
+    _rmsnorm(hidden_states, residual, None, norm_weight, normed_out, rows, K, eps, who)
+    esimd_gemv_fp8_pert(normed_out.view(rows, K), gemv_weight, gemv_scale, output)
+    return output
+
+
+def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps):
+    """Residual add + RMS norm feeding two per-tensor FP8 GEMVs in one launch (resadd_norm_gemv2_fused.h)."""
+    who = "esimd_resadd_norm_gemv2_fp8_pert"
+    K = hidden_states.shape[-1]
+    rows = hidden_states.numel() // K
+    normed = torch.empty_like(hidden_states)
+    _rmsnorm(hidden_states, residual, None, norm_weight, normed, rows, K, eps, who)
+    esimd_gemv_fp8_pert_fused2(normed.view(rows, K), w0, s0, o0, w1, s1, o1)
+    return o0
+
+
+def _gated_norm(x, z, norm_weight, HV, V, eps, who):
+    HV, V = int(HV), int(V)
+    _chk(x.numel() % (HV * V) == 0 and z.numel() == x.numel(), f"{who}: x and z must hold HV*V elements per row")
+    _chk(norm_weight.numel() == V, f"{who}: norm_weight must have V entries")
+    normed = torch.empty_like(x)
+    _rmsnorm(x, None, z, norm_weight, normed, x.numel() // V, V, eps, who)
+    return normed.view(-1, HV * V)
+
+
+def esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    """Per-head RMS norm gated by silu(z), then INT4 GEMV over the HV*V vector (norm_gemv_int4.h)."""
+    esimd_gemv_int4(_gated_norm(x, z, norm_weight, HV, V, eps, "esimd_norm_gemv_int4_pert"), gemv_weight, gemv_scale, output)
+    return output
+
+
+def esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    """Per-head gated RMS norm, then per-tensor FP8 GEMV (norm_gemv_fused.h)."""
+    esimd_gemv_fp8_pert(_gated_norm(x, z, norm_weight, HV, V, eps, "esimd_norm_gemv_fp8_pert"), gemv_weight, gemv_scale, output)
+    return output
+
+
+def esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    """Per-head gated RMS norm, then 128x128 block-scaled FP8 GEMV (torch_extension_gemm.cc:42-45)."""
+    esimd_gemm_fp8_blockscale(_gated_norm(x, z, norm_weight, HV, V, eps, "esimd_norm_gemv_fp8_blockscale"),
+                              gemv_weight, gemv_scale, output, 128, 128)
+    return output
+
+
+# --------------------------------------------------------------------------
 # sglang FP8 MoE prefill ops (per-expert scalar scales), moe_fp8_prefill_ops
 # --------------------------------------------------------------------------
 def _expert_block_scales(scale, E, parts, rows_per_part, K, who):
@@ -855,6 +940,24 @@ def register():
         _define(ns, "esimd_gemv_fp8_blockscale_fused2(Tensor input, Tensor w0, Tensor s0, Tensor(a!) o0, "
                     "Tensor w1, Tensor s1, Tensor(b!) o1, int block_n, int block_k) -> Tensor(a!)",
                 esimd_gemv_fp8_blockscale_fused2, _ret(3))
+    for ns in (_V, _S):
+        _define(ns, "esimd_rms_norm(Tensor input, Tensor output, Tensor weight, float eps) -> Tensor", esimd_rms_norm, _ret(1))
+        _define(ns, "esimd_resadd_norm_gemv_int4_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
+                    "Tensor gemv_weight, Tensor gemv_scale, Tensor output, Tensor normed_out, float eps) -> Tensor",
+                esimd_resadd_norm_gemv_int4_pert, _ret(5))
+        _define(ns, "esimd_resadd_norm_gemv_fp8_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
+                    "Tensor gemv_weight, Tensor gemv_scale, Tensor output, Tensor normed_out, float eps) -> Tensor",
+                esimd_resadd_norm_gemv_fp8_pert, _ret(5))
+        _define(ns, "esimd_resadd_norm_gemv2_fp8_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
+                    "Tensor w0, Tensor s0, Tensor o0, Tensor w1, Tensor s1, Tensor o1, float eps) -> Tensor",
+                esimd_resadd_norm_gemv2_fp8_pert, _ret(5))
+        _define(ns, "esimd_norm_gemv_int4_pert(Tensor x, Tensor z, Tensor norm_weight, Tensor gemv_weight, "
+                    "Tensor gemv_scale, Tensor output, int HV, int V, float eps) -> Tensor", esimd_norm_gemv_int4_pert, _ret(5))
+        _define(ns, "esimd_norm_gemv_fp8_pert(Tensor x, Tensor z, Tensor norm_weight, Tensor gemv_weight, "
+                    "Tensor gemv_scale, Tensor output, int HV, int V, float eps) -> Tensor", esimd_norm_gemv_fp8_pert, _ret(5))
+    _define(_V, "esimd_norm_gemv_fp8_blockscale(Tensor x, Tensor z, Tensor norm_weight, Tensor gemv_weight, "
+                "Tensor gemv_scale, Tensor(a!) output, int HV, int V, float eps) -> Tensor(a!)",
+            esimd_norm_gemv_fp8_blockscale, _ret(5))
     _define(_S, "esimd_gemv_q4_k(Tensor input, Tensor weight, Tensor weight_scale, "
                 "Tensor weight_min, Tensor output) -> Tensor", esimd_gemv_q4_k, _ret(4))
     # siblings without a reference counterpart

@@ -596,3 +596,26 @@ def moe_prefill_scalar(x, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, 
             y[t * k + j] = (inter[t * k + j] @ d2[e].t()) * w2_scale[e]
     out = (topk_weights.float().reshape(T, k, 1) * y.reshape(T, k, H)).sum(1)
     return (out, inter, y) if return_parts else out
+
+
+def rmsnorm(x, weight, eps, residual=None, gate=None, heads=None):
+    """RMS norm as the reference's fused decode ops define it, fp32:
+    a = x (+ residual);  normed = a * rsqrt(mean(a^2) + eps) * weight (* silu(gate)),
+    per row, or per head of len(weight) elements when `heads` is given
+    (V/tests/test_resadd_norm_gemv_int4.py:41-58, V/tests/test_norm_gemv_int4.py:36-68).
+    Returns (normed fp32, updated residual rounded to x's dtype or None)."""
+    a = x.float()
+    new_res = None
+    if residual is not None:
+        a = a + residual.float()
+        new_res = a.to(x.dtype)
+    shape = a.shape
+    if heads is not None:
+        a = a.reshape(-1, weight.numel())
+    var = a.pow(2).mean(dim=-1, keepdim=True)
+    normed = a * torch.rsqrt(var + eps) * weight.float()
+    normed = normed.reshape(shape)
+    if gate is not None:
+        z = gate.float()
+        normed = normed * (z * torch.sigmoid(z))
+    return normed, new_res

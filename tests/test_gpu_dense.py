@@ -379,3 +379,125 @@ def test_cfg2_w4a16_prefill_gemm(ops, dev):
     out2 = torch.empty_like(out)
     v.esimd_gemm_int4_pgrp_zp((x * 2).to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out2)
     assert torch.equal(out2.cpu().float(), 2 * o.float())
+
+
+# ----------------------------------------------------------------- decode fusions: RMS norm + GEMV
+def _ulp_close(a, b, dtype, ulps=2):
+    """|a - b| within `ulps` units in the last place of the 16-bit dtype"""
+    eps = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    return bool(((a - b).abs() <= ulps * eps * b.abs().clamp_min(1e-30) + 1e-7).all())
+
+
+@pytest.mark.parametrize("N,K", [(16, 128), (256, 512), (128, 2048), (128, 4096)])
+@pytest.mark.parametrize("kind", ["int4", "fp8"])
+def test_resadd_norm_gemv(ops, dev, N, K, kind):
+    # V/tests/test_resadd_norm_gemv_int4.py:60-105 (same shapes)
+    v, _ = ops
+    g = torch.Generator().manual_seed(42)
+    eps = 1e-6
+    hidden = torch.randn(1, K, generator=g).half()
+    residual = torch.randn(1, K, generator=g).half()
+    nw = (torch.randn(K, generator=g) * 0.1 + 1.0).half()
+    out = torch.empty(1, N, dtype=torch.float16, device=dev)
+    normed_out = torch.empty(1, K, dtype=torch.float16, device=dev)
+    res_d = residual.to(dev).clone()
+    if kind == "int4":
+        _, packed, scale, _ = O.make_int4_case(1, K, N, seed=5)
+        v.esimd_resadd_norm_gemv_int4_pert(hidden.to(dev), res_d, nw.to(dev), packed.view(torch.int32).to(dev),
+                                           scale.to(dev), out, normed_out, eps)
+        wd = O.int4_dequant(packed, scale, out_dtype=torch.float16)
+    else:
+        w8 = O.e4m3_quantize((torch.randn(N, K, generator=g) * 100).clamp(-448, 448))
+        sc = torch.tensor([3.0e-3])
+        v.esimd_resadd_norm_gemv_fp8_pert(hidden.to(dev), res_d, nw.to(dev), w8.view(torch.float8_e4m3fn).to(dev),
+                                          sc.to(dev), out, normed_out, eps)
+        wd = O.fp8_dequant_per_tensor(w8, sc)
+    normed_ref, res_ref = O.rmsnorm(hidden, nw, eps, residual=residual)
+    assert torch.equal(res_d.cpu().view(torch.int16), res_ref.view(torch.int16))        # one exact rounding
+    assert _ulp_close(normed_out.cpu().float(), normed_ref, torch.float16)
+    ref = O.matmul_ref(normed_out.cpu(), wd)                                              # GEMV on the op's own normed vector
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+    # free-running against the all-fp32 chain: the reference's own (mean) bar
+    full = normed_ref @ wd.float().t()
+    assert ((out.cpu().float() - full).abs().mean() / full.abs().mean()).item() < 5e-3
+
+
+def test_resadd_norm_gemv2_and_rms_norm(ops, dev):
+    v, _ = ops
+    g = torch.Generator().manual_seed(3)
+    K, N0, N1, eps = 2048, 96, 640, 1e-5
+    hidden = torch.randn(1, K, generator=g).to(torch.bfloat16)
+    residual = torch.randn(1, K, generator=g).to(torch.bfloat16)
+    nw = (torch.randn(K, generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+    w0 = O.e4m3_quantize(torch.randn(N0, K, generator=g) * 50)
+    w1 = O.e4m3_quantize(torch.randn(N1, K, generator=g) * 50)
+    s0, s1 = torch.tensor([2.0e-3]), torch.tensor([5.0e-3])
+    o0 = torch.empty(1, N0, dtype=torch.bfloat16, device=dev)
+    o1 = torch.empty(1, N1, dtype=torch.bfloat16, device=dev)
+    res_d = residual.to(dev).clone()
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    r = v.esimd_resadd_norm_gemv2_fp8_pert(hidden.to(dev), res_d, nw.to(dev), f8(w0), s0.to(dev), o0, f8(w1), s1.to(dev), o1, eps)
+    assert r.data_ptr() == o0.data_ptr()
+    normed_ref, res_ref = O.rmsnorm(hidden, nw, eps, residual=residual)
+    assert torch.equal(res_d.cpu().view(torch.int16), res_ref.view(torch.int16))
+    nr = normed_ref.to(torch.bfloat16)
+    for o, w, s in ((o0, w0, s0), (o1, w1, s1)):
+        ref = O.matmul_ref(nr, O.fp8_dequant_per_tensor(w, s))
+        assert O.max_rel_err(o.cpu(), ref) < 2 * TOL       # normed vector may differ by an ulp from the oracle's
+    # plain RMS norm, several rows
+    x = torch.randn(5, 384, generator=g).half()
+    w = torch.rand(384, generator=g).half()
+    y = torch.empty_like(x, device=dev)
+    v.esimd_rms_norm(x.to(dev), y, w.to(dev), 1e-6)
+    assert _ulp_close(y.cpu().float(), O.rmsnorm(x, w, 1e-6)[0], torch.float16)
+
+
+@pytest.mark.parametrize("HV,V,N", [(1, 128, 16), (4, 128, 32), (8, 128, 256), (16, 128, 2048)])
+@pytest.mark.parametrize("kind", ["int4", "fp8", "block"])
+def test_norm_gemv_gated(ops, dev, HV, V, N, kind):
+    # V/tests/test_norm_gemv_int4.py:36-110: per-head RMS norm gated by silu(z), then the GEMV
+    v, _ = ops
+    g = torch.Generator().manual_seed(HV * 7 + N)
+    K, eps = HV * V, 1e-6
+    if kind == "block":
+        N = -(-N // 128) * 128          # the block quantiser of the oracle wants whole 128x128 blocks
+    x = torch.randn(1, K, generator=g).half()
+    z = torch.randn(1, K, generator=g).half()
+    nw = (torch.randn(V, generator=g) * 0.1 + 1.0).half()
+    out = torch.empty(1, N, dtype=torch.float16, device=dev)
+    normed_ref, _ = O.rmsnorm(x, nw, eps, gate=z, heads=HV)
+    nr = normed_ref.half()
+    if kind == "int4":
+        _, packed, scale, _ = O.make_int4_case(1, K, N, seed=6)
+        v.esimd_norm_gemv_int4_pert(x.to(dev), z.to(dev), nw.to(dev), packed.to(dev), scale.to(dev), out, HV, V, eps)
+        wd = O.int4_dequant(packed, scale, out_dtype=torch.float16)
+    elif kind == "fp8":
+        w8 = O.e4m3_quantize((torch.randn(N, K, generator=g) * 100).clamp(-448, 448))
+        sc = torch.tensor([1.0e-3])
+        v.esimd_norm_gemv_fp8_pert(x.to(dev), z.to(dev), nw.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev), out, HV, V, eps)
+        wd = O.fp8_dequant_per_tensor(w8, sc)
+    else:
+        w8, sc = O.fp8_quantize_block(torch.randn(N, K, generator=g) * 0.1)
+        v.esimd_norm_gemv_fp8_blockscale(x.to(dev), z.to(dev), nw.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev), out, HV, V, eps)
+        wd = O.fp8_dequant_block(w8, sc)
+    ref = O.matmul_ref(nr, wd)
+    assert O.max_rel_err(out.cpu(), ref) < 2 * TOL
+
+
+def test_fp8_pert_fused_distinct_scales(ops, dev):
+    """Every fused matrix carries its own per-tensor scale."""
+    v, _ = ops
+    g = torch.Generator().manual_seed(8)
+    K = 1024
+    x = torch.randn(1, K, generator=g).half()
+    ws = [O.e4m3_quantize(torch.randn(n, K, generator=g) * 40) for n in (48, 200, 136)]
+    ss = [torch.tensor([1.0e-3]), torch.tensor([7.0e-3]), torch.tensor([2.5e-4])]
+    outs = [torch.empty(1, w.shape[0], dtype=torch.float16, device=dev) for w in ws]
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    v.esimd_gemv_fp8_pert_fused3(x.to(dev), f8(ws[0]), ss[0].to(dev), outs[0], f8(ws[1]), ss[1].to(dev), outs[1],
+                                 f8(ws[2]), ss[2].to(dev), outs[2])
+    for o, w, s in zip(outs, ws, ss):
+        assert O.max_rel_err(o.cpu(), O.matmul_ref(x, O.fp8_dequant_per_tensor(w, s))) < TOL
+    o2 = [torch.empty_like(outs[0]), torch.empty_like(outs[1])]
+    v.esimd_gemv_fp8_pert_fused2(x.to(dev), f8(ws[0]), ss[0].to(dev), o2[0], f8(ws[1]), ss[1].to(dev), o2[1])
+    assert torch.equal(o2[0], outs[0]) and torch.equal(o2[1], outs[1])

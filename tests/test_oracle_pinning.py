@@ -399,3 +399,26 @@ def test_moe_prefill_scalar_is_the_block_scaled_forward_with_constant_blocks():
     # pair order: row t*k + j belongs to token t
     e = int(ti[3, 1])
     assert torch.allclose(inter[3 * k + 1], it[3, e], rtol=1e-4, atol=1e-7)
+
+
+def test_rmsnorm_oracle_against_library_and_hand_values():
+    """rms_norm of the library for the plain case; hand values for the residual and gated forms."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 64, generator=g).half()
+    w = torch.rand(64, generator=g).half()
+    got, none = O.rmsnorm(x, w, 1e-6)
+    assert none is None
+    want = torch.nn.functional.rms_norm(x.float(), (64,), w.float(), 1e-6)
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-7)
+    # residual: a = x + r = [3, 4] -> rms = sqrt(12.5); gate z = 0 -> silu(0) = 0 kills the output
+    xs, rs = torch.tensor([[1.0, 1.0]]).half(), torch.tensor([[2.0, 3.0]]).half()
+    ws = torch.tensor([1.0, 2.0]).half()
+    n, nr = O.rmsnorm(xs, ws, 0.0, residual=rs)
+    assert torch.equal(nr, torch.tensor([[3.0, 4.0]]).half())
+    assert torch.allclose(n, torch.tensor([[3.0 / 12.5 ** 0.5, 8.0 / 12.5 ** 0.5]]), rtol=1e-6)
+    n0, _ = O.rmsnorm(xs, ws, 0.0, gate=torch.zeros(1, 2).half())
+    assert torch.equal(n0, torch.zeros(1, 2))
+    # heads: each head of len(weight) elements is normalised on its own
+    xh = torch.tensor([[3.0, 4.0, 6.0, 8.0]]).half()
+    nh, _ = O.rmsnorm(xh, torch.ones(2).half(), 0.0, heads=2)
+    assert torch.allclose(nh, torch.tensor([[3 / 12.5 ** 0.5, 4 / 12.5 ** 0.5, 6 / 50 ** 0.5, 8 / 50 ** 0.5]]), rtol=1e-6)
