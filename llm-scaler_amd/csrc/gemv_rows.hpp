@@ -7,7 +7,9 @@
 // once per workgroup in LDS, already laid out in the order the lanes consume
 // them, so the inner loop touches global memory for weights only.  The K
 // reduction finishes inside the wavefront with cross-lane adds; no LDS
-// reduction, no barrier after the staging one.
+// reduction, no barrier after the staging one.  When a whole activation row fits
+// in one batch (K <= SPU spans) and M <= 2, every wavefront keeps its share of
+// the activations in registers instead (XREG): no LDS, no barrier at all.
 //
 // Per-format arithmetic (x = activation, all sums in fp32):
 //   fp8   : sum x * e4m3(w), exact conversion to 16 bit, scale applied per row
@@ -80,7 +82,7 @@ __device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_
 // weight loads of the next batch are in flight while the current one is
 // consumed (two register buffers).  Weight loads carry the non-temporal hint:
 // every byte is used exactly once.
-template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI>
+template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI, bool XREG>
 __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   constexpr bool kFp8 = FMT == RF_FP8;
   constexpr bool kNib = !kFp8;
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     u32x4 w[RW][SPU];
     float s[RW][SPU];          // per-lane scale of the chunk (int4 group / q4k sub-block / fp8 block)
     float z[RW][SPU];          // int4 zero-point / q4k min
-    uint16_t os_lo[RW], os_hi[RW];   // fp8 per-channel scale of the row, raw halves (fp32 or fp16)
+    uint32_t os_lo[RW], os_hi[RW];   // fp8 per-channel scale of the row, raw halves (fp32 or fp16)
   };
 
   // Kernel arguments are selected with uniform compares, never indexed
@@ -205,7 +207,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     const uint32_t dead = (uint32_t)(!(p < total && m < M && k < K)) << 31;
     return (((uint32_t)m * K + k) * 2u) | dead;
   };
-  auto x_store = [&](int p, u32x4 v) {
+  auto x_arrange = [&](u32x4 v) -> u32x4 {
     if constexpr (kNib) {
       // natural pairs (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x4)(x1 x5)(x2 x6)(x3 x7)
       const uint32_t d0 = v[0], d1 = v[1], d2 = v[2], d3 = v[3];
@@ -221,11 +223,60 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       }
       v = u32x4{e0, e1, e2, e3};
     }
-    if (p < total) xs[p] = v;
+    return v;
   };
-  u32x4 xpre[XPRE];
+  auto x_store = [&](int p, u32x4 v) {
+    if (p < total) xs[p] = x_arrange(v);
+  };
+  // what the planted constants contribute (c1) and sum x (c2) over one 32-k
+  // chunk = four arranged pieces, summed in a fixed order
+  auto chunk_sums = [&](const u32x4 (&pc)[4], float& k1, float& k2) {
+    float lo = 0.f, hi = 0.f;
+    auto pair_sum = [](uint32_t bits) -> float {
+      if constexpr (Act::dt == DT_F16) {
+        const f16x2 h = __builtin_bit_cast(f16x2, bits);
+        return (float)h[0] + (float)h[1];
+      } else {
+        const bf16x2 h = __builtin_bit_cast(bf16x2, bits);
+        return (float)h[0] + (float)h[1];
+      }
+    };
 #pragma unroll
-  for (int t = 0; t < XPRE; ++t) xpre[t] = buf_load16(xr, x_offset(threadIdx.x + t * NWV * 64));
+    for (int i = 0; i < 4; ++i) {
+      lo += pair_sum(pc[i][0]);
+      hi += pair_sum(pc[i][1]);
+      lo += pair_sum(pc[i][2]);
+      hi += pair_sum(pc[i][3]);
+    }
+    if constexpr (Act::dt == DT_F16) {
+      k1 = 1024.0f * (lo + hi);                      // hi already holds x / 16
+      k2 = lo + 16.0f * hi;
+    } else {
+      k1 = 128.0f * (lo + hi);
+      k2 = lo + hi;
+    }
+  };
+  // XREG: the lane's own pieces of every span, loaded straight into registers
+  constexpr int XM = XREG ? MR : 1, XS = XREG ? SPU : 1;
+  u32x4 xreg[XM][XS][PPL];
+  float c1r[XM][XS], c2r[XM][XS];
+  if constexpr (XREG) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int sp = 0; sp < SPU; ++sp)
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) {
+          const int k = sp * SPAN_K + (lane * PPL + i) * 8;
+          const uint32_t dead = (uint32_t)(!(m < M && k < K)) << 31;
+          xreg[m][sp][i] = buf_load16(xr, (((uint32_t)m * K + k) * 2u) | dead);
+        }
+  }
+  u32x4 xpre[XPRE];
+  if constexpr (!XREG) {
+#pragma unroll
+    for (int t = 0; t < XPRE; ++t) xpre[t] = buf_load16(xr, x_offset(threadIdx.x + t * NWV * 64));
+  }
 
   auto advance = [&](int& g, int& sb) {
     if (++sb == nbatch) { sb = 0; g += stride; }
@@ -240,58 +291,46 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     load_batch(buf[i], g_next, sb_next);
     advance(g_next, sb_next);
   }
-  float pert_scale[kRowsMaxMat];                      // one per-tensor scale per fused matrix
-#pragma unroll
-  for (int i = 0; i < kRowsMaxMat; ++i) {
-    pert_scale[i] = 1.0f;
-    if constexpr (kFp8 && SC == RS_PERT) {
-      if (i < a.nmat) pert_scale[i] = ((const float*)a.s[i])[0];
+  // one per-tensor scale per fused matrix (scalars, so they stay in registers)
+  float pert0 = 1.0f, pert1 = 1.0f, pert2 = 1.0f;
+  if constexpr (kFp8 && SC == RS_PERT) {
+    pert0 = ((const float*)a.s[0])[0];
+    if constexpr (MULTI) {
+      if (a.nmat > 1) pert1 = ((const float*)a.s[1])[0];
+      if (a.nmat > 2) pert2 = ((const float*)a.s[2])[0];
     }
   }
 
-  {
+  if constexpr (XREG) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int sp = 0; sp < SPU; ++sp) {
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) xreg[m][sp][i] = x_arrange(xreg[m][sp][i]);
+        if constexpr (kNib) chunk_sums(xreg[m][sp], c1r[m][sp], c2r[m][sp]);
+      }
+  } else {
 #pragma unroll
     for (int t = 0; t < XPRE; ++t) x_store(threadIdx.x + t * NWV * 64, xpre[t]);
     for (int p = threadIdx.x + XPRE * NWV * 64; p < total; p += NWV * 64)
       x_store(p, buf_load16(xr, x_offset(p)));
     if constexpr (kNib) {
-      // per 32-k chunk: what the planted constants contribute (c1) and sum x (c2),
-      // summed in a fixed order from the staged image
+      // per 32-k chunk sums, from the staged image
       __syncthreads();
       const int chunks = MR * nspan * 64;
       for (int c = threadIdx.x; c < chunks; c += NWV * 64) {
         const int m = c / (nspan * 64);
         const int sl = c - m * (nspan * 64);
         const int s = sl >> 6, l = sl & 63;
-        float lo = 0.f, hi = 0.f;
-        auto pair_sum = [](uint32_t bits) -> float {
-          if constexpr (Act::dt == DT_F16) {
-            const f16x2 h = __builtin_bit_cast(f16x2, bits);
-            return (float)h[0] + (float)h[1];
-          } else {
-            const bf16x2 h = __builtin_bit_cast(bf16x2, bits);
-            return (float)h[0] + (float)h[1];
-          }
-        };
+        u32x4 pc[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const u32x4 v = xs[m * pieces_per_row + (s * 4 + i) * 64 + l];
-          lo += pair_sum(v[0]);
-          hi += pair_sum(v[1]);
-          lo += pair_sum(v[2]);
-          hi += pair_sum(v[3]);
-        }
-        if constexpr (Act::dt == DT_F16) {
-          c1[c] = 1024.0f * (lo + hi);               // hi already holds x / 16
-          c2[c] = lo + 16.0f * hi;
-        } else {
-          c1[c] = 128.0f * (lo + hi);
-          c2[c] = lo + hi;
-        }
+        for (int i = 0; i < 4; ++i) pc[i] = xs[m * pieces_per_row + (s * 4 + i) * 64 + l];
+        chunk_sums(pc, c1[c], c2[c]);
       }
     }
+    __syncthreads();
   }
-  __syncthreads();
 
   float acc[RW][MR];
 #pragma unroll
@@ -308,7 +347,10 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 #pragma unroll
         for (int m = 0; m < MR; ++m)
 #pragma unroll
-          for (int i = 0; i < PPL; ++i) xp[m][i] = xs[m * pieces_per_row + (s * PPL + i) * 64 + lane];
+          for (int i = 0; i < PPL; ++i) {
+            if constexpr (XREG) xp[m][i] = xreg[m][sp][i];
+            else xp[m][i] = xs[m * pieces_per_row + (s * PPL + i) * 64 + lane];
+          }
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
           const u32x4 w = b.w[r][sp];
@@ -361,8 +403,13 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
             const float zz = b.z[r][sp];
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
-              const float k1 = c1[(m * nspan + s) * 64 + lane];
-              const float k2 = c2[(m * nspan + s) * 64 + lane];
+              float k1, k2;
+              if constexpr (XREG) {
+                k1 = c1r[m][sp]; k2 = c2r[m][sp];
+              } else {
+                k1 = c1[(m * nspan + s) * 64 + lane];
+                k2 = c2[(m * nspan + s) * 64 + lane];
+              }
               if constexpr (FMT == RF_INT4)
                 acc[r][m] += sc * (part[m] - k1 - zz * k2);
               else
@@ -386,9 +433,9 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       const int n = row0 + r;
       float os = 1.0f;
       if constexpr (kFp8 && SC == RS_PERN)
-        os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, b.os_lo[r])
-                         : __builtin_bit_cast(float, (uint32_t)b.os_lo[r] | ((uint32_t)b.os_hi[r] << 16));
-      if constexpr (kFp8 && SC == RS_PERT) os = mat == 0 ? pert_scale[0] : (mat == 1 ? pert_scale[1] : pert_scale[2]);
+        os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)b.os_lo[r])
+                         : __builtin_bit_cast(float, b.os_lo[r] | (b.os_hi[r] << 16));
+      if constexpr (kFp8 && SC == RS_PERT) os = mat == 0 ? pert0 : (mat == 1 ? pert1 : pert2);
 #pragma unroll
       for (int m = 0; m < MR; ++m) {
         const float v = wave_sum(acc[r][m]);
@@ -438,11 +485,10 @@ static inline int device_cu_count() {
   return cus;
 }
 
-template <class Act, int FMT, int SC, int MR, int RW>
+template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG>
 static void launch_rows_rw(RowsArgs a, hipStream_t st) {
   constexpr int NWV = 8;
   constexpr int NBUF = 2;
-  constexpr int SPU = FMT == RF_FP8 ? 4 : 2;
   int groups = 0;
   for (int i = 0; i < kRowsMaxMat; ++i) {
     a.groups[i] = i < a.nmat ? (a.N[i] + RW - 1) / RW : 0;
@@ -462,28 +508,40 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st) {
   const int needed = (groups + NWV - 1) / NWV;
   const int wgs = needed < best_wgs ? needed : best_wgs;
   a.total_waves = wgs * NWV;
-  const size_t lds = rows_lds_bytes(FMT, MR, a.K);
+  const size_t lds = XREG ? 0 : rows_lds_bytes(FMT, MR, a.K);
   if (a.nmat == 1)
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false>), dim3(wgs), dim3(NWV * 64),
-                       lds, st, a);
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false, XREG>), dim3(wgs),
+                       dim3(NWV * 64), lds, st, a);
   else
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true>), dim3(wgs), dim3(NWV * 64),
-                       lds, st, a);
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG>), dim3(wgs),
+                       dim3(NWV * 64), lds, st, a);
 }
 
+// Batch shape by row length.  Rows of up to one batch (fp8: 4 spans = 4096 k,
+// nibble formats: 2 or 3 spans = 4096 / 6144 k) with M <= 2 keep the
+// activations in registers; longer rows stage them in LDS.
 template <class Act, int FMT, int SC, int MR>
 static void launch_rows(RowsArgs a, hipStream_t st) {
   constexpr int ppl = FMT == RF_FP8 ? 2 : 4;
   constexpr int span_k = 64 * ppl * 8;
   constexpr int SPU = FMT == RF_FP8 ? 4 : 2;
+  constexpr bool kRegOk = MR <= 2;
   a.nspan = (a.K + span_k - 1) / span_k;
+  if constexpr (FMT != RF_FP8 && kRegOk) {
+    if (a.nspan == 3) return launch_rows_rw<Act, FMT, SC, MR, 2, 3, true>(a, st);
+  }
   const int per_batch = a.nspan < SPU ? a.nspan : SPU;     // loads per row per batch
-  if (per_batch >= 4)
-    launch_rows_rw<Act, FMT, SC, MR, 1>(a, st);
-  else if (per_batch >= 2)
-    launch_rows_rw<Act, FMT, SC, MR, 2>(a, st);
-  else
-    launch_rows_rw<Act, FMT, SC, MR, 4>(a, st);
+  const bool one_batch = kRegOk && a.nspan <= SPU;
+  if (per_batch >= 4) {
+    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 1, SPU, true>(a, st); }
+    launch_rows_rw<Act, FMT, SC, MR, 1, SPU, false>(a, st);
+  } else if (per_batch >= 2) {
+    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 2, SPU, true>(a, st); }
+    launch_rows_rw<Act, FMT, SC, MR, 2, SPU, false>(a, st);
+  } else {
+    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 4, SPU, true>(a, st); }
+    launch_rows_rw<Act, FMT, SC, MR, 4, SPU, false>(a, st);
+  }
 }
 
 template <class Act, int FMT, int SC>
