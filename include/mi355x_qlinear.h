@@ -126,6 +126,55 @@ int mi_dequant_q4k(const void* ql, const void* scale, const void* qmin, void* ou
                    void* stream);
 int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int K, void* stream);
 
+/* ---- other GGUF formats: weight preparation, dequant, decode GEMV (fp16) ------
+ * Resident representations (what the reference's ops read):
+ *   Q4_0: packed [N,K/2] u8 interleaved nibbles (byte j = elem 2j | elem 2j+1 << 4),
+ *         scale [N,K/32] fp16; w = (nib - 8) * scale.
+ *   Q8_0: qs [N,K] int8, scale [N,K/32] fp16; w = qs * scale.
+ *   Q5_K: ql [N,K/2] interleaved low nibbles, qh [N,K/8] (per 512-k tile, bit b of
+ *         byte t = fifth bit of element b*64+t), scale/qmin [N,K/32] fp16;
+ *         w = fp16(fp16(v5 * scale) - qmin).
+ *   Q6_K: ql [N,K/2], qh [N,K/4] (per 512-k tile, 2-bit field p of byte t = top
+ *         bits of element p*128+t), scale [N,K/16] fp16; w = (v6 - 32) * scale.
+ * mi_q4_0_repack / mi_q8_0_repack / mi_q5k_repack / mi_q6k_repack: raw GGML rows
+ *   ([N, K/32*18], [N, K/32*34], [N, K/256*176], [N, K/256*210] bytes) -> resident
+ *   (_xpu_repack_q4_0, _xpu_repack_q8_0, _xpu_repack_q5_k, _xpu_repack_q6_k,
+ *   sglang/patches/sglang_for_multi_arc.patch:2173-2193, 3031-3044, 2725-2740,
+ *   2996-3008).  K % 32 == 0; K % 512 == 0 for the K-quants (whole shuffle tiles).
+ * mi_dequant_*: resident -> dense fp16 [N,K] with the fp16 roundings of
+ *   _xpu_dequant_q4_0_packed / _q8_0 / _q5_k / _q6_k (same patch :2196-2213,
+ *   3047-3054, 2952-2970, 3011-3026), the reference's route for M > 1.
+ * mi_gemv_*: out [M,N] fp16 = x [M,K] fp16 @ w^T, fp32 accumulation.  Replace
+ *   esimd_gemv_q4_0, esimd_gemm_q4_0, esimd_gemv_q8_0(_m), esimd_gemv_q5_k,
+ *   esimd_gemv_q6_k(_m) (S/csrc/xpu/torch_extension.cc:48-106), for any M (rows
+ *   are processed four at a time, each pass streaming the weight once).
+ * mi_q4_0_quantize: x [rows,K] fp16/bf16 -> qweight [rows,K/8] int32 (nibble i of
+ *   word w = element 8w+i, value + 8) + scale [rows,K/128] fp16 = max/-8, the
+ *   layout mi_gemv_int4 reads.  GGML's quantize_row_q4_0 rule on 128-wide blocks;
+ *   replaces q4_0_quantize (V/csrc/xpu/torch_extension_q4_0.cc:27-75,
+ *   V/csrc/xpu/q4_0_quant.sycl:30-120).  K % 128 == 0. */
+int mi_q4_0_repack(const void* raw, void* packed, void* scale, int N, int K, void* stream);
+int mi_q8_0_repack(const void* raw, void* qs, void* scale, int N, int K, void* stream);
+int mi_q5k_repack(const void* raw, void* ql, void* qh, void* scale, void* qmin, int N, int K,
+                  void* stream);
+int mi_q6k_repack(const void* raw, void* ql, void* qh, void* scale, int N, int K, void* stream);
+int mi_dequant_q4_0(const void* packed, const void* scale, void* out, int N, int K, void* stream);
+int mi_dequant_q8_0(const void* qs, const void* scale, void* out, int N, int K, void* stream);
+int mi_dequant_q5k(const void* ql, const void* qh, const void* scale, const void* qmin, void* out,
+                   int N, int K, void* stream);
+int mi_dequant_q6k(const void* ql, const void* qh, const void* scale, void* out, int N, int K,
+                   void* stream);
+int mi_gemv_q4_0(const void* x, const void* packed, const void* scale, void* out, int M, int N, int K,
+                 void* stream);
+int mi_gemv_q8_0(const void* x, const void* qs, const void* scale, void* out, int M, int N, int K,
+                 void* stream);
+int mi_gemv_q5k(const void* x, const void* ql, const void* qh, const void* scale, const void* qmin,
+                void* out, int M, int N, int K, void* stream);
+int mi_gemv_q6k(const void* x, const void* ql, const void* qh, const void* scale, void* out, int M,
+                int N, int K, void* stream);
+int mi_q4_0_quantize(const void* x, void* qweight, void* scale, int rows, int K, int in_dtype,
+                     void* stream);
+
 /* ---- MoE routing and permutation --------------------------------------------
  * mi_moe_topk: fp32 softmax over E experts -> top-K (lowest index wins ties,
  *   descending probability) -> optional renormalisation; top_w in the activation

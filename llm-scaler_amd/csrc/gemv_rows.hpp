@@ -21,7 +21,14 @@
 //           zero-point's  z * C2, C2 = sum x_k  are precomputed per 32-k chunk
 //           at staging time, and the group scale multiplies the corrected
 //           partial:  acc += s * (dot - C1 - z C2);
-//   Q4_K  : same planting; acc += s * (dot - C1) - min * C2.
+//   Q4_K  : same planting; acc += s * (dot - C1) - min * C2;
+//   Q4_0  : the Q4_K path with min = 8 s (32-wide groups, w = (nib - 8) s);
+//   Q5_K  : Q4_K plus the fifth bit, OR-ed into the planted constant (bit 4 for
+//           even, bit 8 for odd nibbles) from the tile-shuffled qh bytes;
+//   Q6_K  : two high bits OR-ed in the same way, the constant and the zero point
+//           32 removed exactly in 16 bit before the dot product, one scale per 16;
+//   Q8_0  : bytes planted as 0x6400 | (q ^ 0x80) = 1152 + q, 1152 removed exactly
+//           in 16 bit, one scale per 32.
 // The dequantized weight is therefore never rounded to 16 bit here; against a
 // reference that rounds it the difference is below 2^-9 relative per weight.
 #pragma once
@@ -36,6 +43,7 @@ struct RowsArgs {
   const void* w[kRowsMaxMat];
   const void* s[kRowsMaxMat];
   const void* z[kRowsMaxMat];
+  const void* h[kRowsMaxMat];     // Q5_K / Q6_K high bits (tile-shuffled)
   void* out[kRowsMaxMat];
   int N[kRowsMaxMat];
   int groups[kRowsMaxMat];     // row groups (RW rows each) per matrix
@@ -46,7 +54,8 @@ struct RowsArgs {
   int scale_f16;
 };
 
-enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2 };
+enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2, RF_Q40 = 3, RF_Q80 = 4, RF_Q5K = 5, RF_Q6K = 6 };
+constexpr bool rows_byte_fmt(int fmt) { return fmt == RF_FP8 || fmt == RF_Q80; }   // one byte per weight
 enum : int { RS_PERN = 0, RS_PERT = 1, RS_BLOCK = 2 };
 
 template <class Act> struct Dot2;
@@ -85,10 +94,13 @@ __device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_
 template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI, bool XREG>
 __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   constexpr bool kFp8 = FMT == RF_FP8;
-  constexpr bool kNib = !kFp8;
-  constexpr int PPL = kFp8 ? 2 : 4;
+  constexpr bool kByte = rows_byte_fmt(FMT);
+  constexpr bool kNib = !kByte;
+  constexpr bool kHigh = FMT == RF_Q5K || FMT == RF_Q6K;
+  constexpr bool kSums = kNib && FMT != RF_Q6K;       // formats that use the per-chunk sums
+  constexpr int PPL = kByte ? 2 : 4;
   constexpr int SPAN_K = 64 * PPL * 8;               // k covered by one wave load: 1024 / 2048
-  constexpr int SPAN_B = kFp8 ? SPAN_K : SPAN_K / 2; // bytes of one weight row per span
+  constexpr int SPAN_B = kByte ? SPAN_K : SPAN_K / 2; // bytes of one weight row per span
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int K = a.K, M = a.M;
@@ -100,13 +112,14 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   float* c1 = reinterpret_cast<float*>(smem + (size_t)MR * pieces_per_row * 16);   // [MR][nspan*64]
   float* c2 = c1 + MR * nspan * 64;
 
-  const uint32_t wrow = kFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
+  const uint32_t wrow = kByte ? (uint32_t)K : ((uint32_t)K >> 1);
   const int nbatch = (nspan + SPU - 1) / SPU;        // batches per row group
   const int stride = a.total_waves;
   const int ngroups = a.groups[0] + a.groups[1] + a.groups[2];
 
   struct Batch {                                     // one batch = RW rows x SPU spans
     u32x4 w[RW][SPU];
+    u32x4 h[RW][SPU][kHigh ? 2 : 1];   // the lane's 32 high-bit bytes (Q5_K / Q6_K)
     float s[RW][SPU];          // per-lane scale of the chunk (int4 group / q4k sub-block / fp8 block)
     float z[RW][SPU];          // int4 zero-point / q4k min
     uint32_t os_lo[RW], os_hi[RW];   // fp8 per-channel scale of the row, raw halves (fp32 or fp16)
@@ -134,6 +147,8 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     locate(live ? g : 0, mat, row0);
     const int N = QLIN_PICK(N, mat);
     const __amdgpu_buffer_rsrc_t wr = make_rsrc(QLIN_PICK(w, mat), (uint32_t)N * wrow);
+    const __amdgpu_buffer_rsrc_t hr =
+        make_rsrc(QLIN_PICK(h, mat), kHigh ? (uint32_t)N * (FMT == RF_Q5K ? ((uint32_t)K >> 3) : ((uint32_t)K >> 2)) : 0u);
     const _Float16* s16 = (const _Float16*)QLIN_PICK(s, mat);
     const float* s32 = (const float*)QLIN_PICK(s, mat);
     const uint8_t* zp = (const uint8_t*)QLIN_PICK(z, mat);
@@ -164,11 +179,24 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
           gi = gi < Kg ? gi : Kg - 1;
           b.s[r][sp] = (float)s16[(size_t)nc * Kg + gi];
           b.z[r][sp] = zp ? (float)zp[(size_t)nc * Kg + gi] : 8.0f;
-        } else if constexpr (FMT == RF_Q4K) {
+        } else if constexpr (FMT == RF_Q4K || FMT == RF_Q5K) {
           const int Kc = K >> 5;
           const int ci = chunk < Kc ? chunk : Kc - 1;
           b.s[r][sp] = (float)s16[(size_t)nc * Kc + ci];
           b.z[r][sp] = (float)qmin[(size_t)nc * Kc + ci];
+        } else if constexpr (FMT == RF_Q40) {
+          const int Kc = K >> 5;
+          const int ci = chunk < Kc ? chunk : Kc - 1;
+          b.s[r][sp] = (float)s16[(size_t)nc * Kc + ci];
+        } else if constexpr (FMT == RF_Q6K) {
+          // the lane's 32 k span two 16-wide groups: both fp16 scales in one 32-bit load
+          const int Kc = K >> 5;
+          const int ci = chunk < Kc ? chunk : Kc - 1;
+          b.s[r][sp] = reinterpret_cast<const float*>(s16)[(size_t)nc * Kc + ci];
+        } else if constexpr (FMT == RF_Q80) {
+          const int Kc = K >> 5;
+          const int c8 = (s * SPAN_K + lane * 16) >> 5;
+          b.s[r][sp] = (float)s16[(size_t)nc * Kc + (c8 < Kc ? c8 : Kc - 1)];
         } else if constexpr (SC == RS_BLOCK) {
           const int Kb = (K + 127) >> 7;
           const int kblk = (s * SPAN_K + lane * 16) >> 7;
@@ -186,6 +214,18 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
         const uint32_t dead = (uint32_t)(!(live && (row0 + r < N) && (kb < wrow))) << 31;
         b.w[r][sp] = __builtin_amdgcn_raw_buffer_load_b128(
             wr, ((uint32_t)(row0 + r) * wrow + kb) | dead, 0, 2 /* nt */);
+        if constexpr (kHigh) {
+          // per 512-k tile the high bits of element b*64 + t (Q5_K, 1 bit) or
+          // p*128 + t (Q6_K, 2 bits) sit in byte t: the lane's 32 consecutive k
+          // are 32 consecutive bytes, one bit field
+          constexpr uint32_t tile_b = FMT == RF_Q5K ? 64u : 128u;
+          const uint32_t hrow = FMT == RF_Q5K ? ((uint32_t)K >> 3) : ((uint32_t)K >> 2);
+          const uint32_t tile = (uint32_t)(sb * SPU + sp) * 4u + ((uint32_t)lane >> 4);
+          const uint32_t within = FMT == RF_Q5K ? ((uint32_t)lane & 1u) * 32u : ((uint32_t)lane & 3u) * 32u;
+          const uint32_t ho = ((uint32_t)(row0 + r) * hrow + tile * tile_b + within) | dead;
+          b.h[r][sp][0] = __builtin_amdgcn_raw_buffer_load_b128(hr, ho, 0, 2);
+          b.h[r][sp][1] = __builtin_amdgcn_raw_buffer_load_b128(hr, ho + 16u, 0, 2);
+        }
       }
   };
 
@@ -308,14 +348,14 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       for (int sp = 0; sp < SPU; ++sp) {
 #pragma unroll
         for (int i = 0; i < PPL; ++i) xreg[m][sp][i] = x_arrange(xreg[m][sp][i]);
-        if constexpr (kNib) chunk_sums(xreg[m][sp], c1r[m][sp], c2r[m][sp]);
+        if constexpr (kSums) chunk_sums(xreg[m][sp], c1r[m][sp], c2r[m][sp]);
       }
   } else {
 #pragma unroll
     for (int t = 0; t < XPRE; ++t) x_store(threadIdx.x + t * NWV * 64, xpre[t]);
     for (int p = threadIdx.x + XPRE * NWV * 64; p < total; p += NWV * 64)
       x_store(p, buf_load16(xr, x_offset(p)));
-    if constexpr (kNib) {
+    if constexpr (kSums) {
       // per 32-k chunk sums, from the staged image
       __syncthreads();
       const int chunks = MR * nspan * 64;
@@ -375,7 +415,32 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 #pragma unroll
               for (int m = 0; m < MR; ++m) acc[r][m] += part[m];
             }
+          } else if constexpr (FMT == RF_Q80) {
+            // int8 -> fp16 exactly: 0x6400 | (q ^ 0x80) = 1152 + q, minus 1152
+            const f16x2 k1152 = {(_Float16)1152.0f, (_Float16)1152.0f};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t u = w[d] ^ 0x80808080u;
+              const uint32_t p0 = __builtin_bit_cast(
+                  uint32_t, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - k1152);
+              const uint32_t p1 = __builtin_bit_cast(
+                  uint32_t, __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - k1152);
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                part[m] = Dot2<Act>::run(p0, xp[m][d >> 1][(d & 1) * 2], part[m]);
+                part[m] = Dot2<Act>::run(p1, xp[m][d >> 1][(d & 1) * 2 + 1], part[m]);
+              }
+            }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * b.s[r][sp];
           } else {
+            float part_hi[MR];                       // Q6_K: second 16-wide group of the lane
+#pragma unroll
+            for (int m = 0; m < MR; ++m) part_hi[m] = 0.f;
+            // bit field of the lane inside its high-bit bytes (the same for every span:
+            // a span covers whole 512-k tiles)
+            const uint32_t hshift = FMT == RF_Q5K ? (((uint32_t)lane & 15u) >> 1) : ((((uint32_t)lane & 15u) >> 2) * 2u);
+            constexpr uint32_t hmask = FMT == RF_Q5K ? 0x01010101u : 0x03030303u;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
               uint32_t t0, t1, t2, t3;
@@ -391,18 +456,45 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
                 t2 = ((w[d] >> 8) & 0x000F000Fu) | 0x43004300u;
                 t3 = ((w[d] >> 12) & 0x000F000Fu) | 0x43004300u;
               }
+              if constexpr (kHigh && Act::dt == DT_F16) {
+                // elements 8d .. 8d+3 have their high bits in bytes of hA, 8d+4 .. 8d+7 in hB;
+                // pair (i, i+4) takes byte i of each, moved to bit 4 (even) / bit 8 (odd nibbles)
+                const uint32_t hA = (b.h[r][sp][d >> 1][(d & 1) * 2] >> hshift) & hmask;
+                const uint32_t hB = (b.h[r][sp][d >> 1][(d & 1) * 2 + 1] >> hshift) & hmask;
+                t0 |= __builtin_amdgcn_perm(hB, hA, 0x0C040C00u) << 4;
+                t1 |= __builtin_amdgcn_perm(hB, hA, 0x0C050C01u) << 8;
+                t2 |= __builtin_amdgcn_perm(hB, hA, 0x0C060C02u) << 4;
+                t3 |= __builtin_amdgcn_perm(hB, hA, 0x0C070C03u) << 8;
+              }
+              if constexpr (FMT == RF_Q6K && Act::dt == DT_F16) {
+                // exact in fp16: (1024 + v6) - 1056 = v6 - 32, (1024 + 16 v6) - 1536 = 16 (v6 - 32)
+                const f16x2 ke = {(_Float16)1056.0f, (_Float16)1056.0f};
+                const f16x2 ko = {(_Float16)1536.0f, (_Float16)1536.0f};
+                t0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, t0) - ke);
+                t1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, t1) - ko);
+                t2 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, t2) - ke);
+                t3 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, t3) - ko);
+              }
 #pragma unroll
               for (int m = 0; m < MR; ++m) {
-                part[m] = Dot2<Act>::run(t0, xp[m][d][0], part[m]);
-                part[m] = Dot2<Act>::run(t1, xp[m][d][1], part[m]);
-                part[m] = Dot2<Act>::run(t2, xp[m][d][2], part[m]);
-                part[m] = Dot2<Act>::run(t3, xp[m][d][3], part[m]);
+                float& pt = (FMT == RF_Q6K && d >= 2) ? part_hi[m] : part[m];
+                pt = Dot2<Act>::run(t0, xp[m][d][0], pt);
+                pt = Dot2<Act>::run(t1, xp[m][d][1], pt);
+                pt = Dot2<Act>::run(t2, xp[m][d][2], pt);
+                pt = Dot2<Act>::run(t3, xp[m][d][3], pt);
               }
             }
-            const float sc = b.s[r][sp];
-            const float zz = b.z[r][sp];
+            if constexpr (FMT == RF_Q6K) {
+              const uint32_t two = __builtin_bit_cast(uint32_t, b.s[r][sp]);
+              const float s_lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(two & 0xFFFFu));
+              const float s_hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(two >> 16));
 #pragma unroll
-            for (int m = 0; m < MR; ++m) {
+              for (int m = 0; m < MR; ++m) acc[r][m] += s_lo * part[m] + s_hi * part_hi[m];
+            }
+            const float sc = b.s[r][sp];
+            const float zz = FMT == RF_Q40 ? 8.0f * sc : b.z[r][sp];
+#pragma unroll
+            for (int m = 0; m < (FMT == RF_Q6K ? 0 : MR); ++m) {
               float k1, k2;
               if constexpr (XREG) {
                 k1 = c1r[m][sp]; k2 = c2r[m][sp];
@@ -465,11 +557,11 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 
 // LDS bytes the kernel needs for a given shape.
 static inline size_t rows_lds_bytes(int fmt, int MR, int K) {
-  const int ppl = fmt == RF_FP8 ? 2 : 4;
+  const int ppl = rows_byte_fmt(fmt) ? 2 : 4;
   const int span_k = 64 * ppl * 8;
   const int nspan = (K + span_k - 1) / span_k;
   size_t b = (size_t)MR * nspan * ppl * 64 * 16;
-  if (fmt != RF_FP8) b += (size_t)2 * MR * nspan * 64 * 4;
+  if (!rows_byte_fmt(fmt)) b += (size_t)2 * MR * nspan * 64 * 4;
   return b;
 }
 
@@ -522,12 +614,15 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st) {
 // activations in registers; longer rows stage them in LDS.
 template <class Act, int FMT, int SC, int MR>
 static void launch_rows(RowsArgs a, hipStream_t st) {
-  constexpr int ppl = FMT == RF_FP8 ? 2 : 4;
+  constexpr bool kByte = rows_byte_fmt(FMT);
+  constexpr bool kHigh = FMT == RF_Q5K || FMT == RF_Q6K;   // three loads per row and span: fewer rows in flight
+  constexpr int ppl = kByte ? 2 : 4;
   constexpr int span_k = 64 * ppl * 8;
-  constexpr int SPU = FMT == RF_FP8 ? 4 : 2;
+  constexpr int SPU = kByte ? 4 : 2;
   constexpr bool kRegOk = MR <= 2;
+  constexpr int RW2 = kHigh ? 1 : 2, RW4 = kHigh ? 2 : 4;
   a.nspan = (a.K + span_k - 1) / span_k;
-  if constexpr (FMT != RF_FP8 && kRegOk) {
+  if constexpr (!kByte && !kHigh && kRegOk) {
     if (a.nspan == 3) return launch_rows_rw<Act, FMT, SC, MR, 2, 3, true>(a, st);
   }
   const int per_batch = a.nspan < SPU ? a.nspan : SPU;     // loads per row per batch
@@ -536,11 +631,11 @@ static void launch_rows(RowsArgs a, hipStream_t st) {
     if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 1, SPU, true>(a, st); }
     launch_rows_rw<Act, FMT, SC, MR, 1, SPU, false>(a, st);
   } else if (per_batch >= 2) {
-    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 2, SPU, true>(a, st); }
-    launch_rows_rw<Act, FMT, SC, MR, 2, SPU, false>(a, st);
+    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, RW2, SPU, true>(a, st); }
+    launch_rows_rw<Act, FMT, SC, MR, RW2, SPU, false>(a, st);
   } else {
-    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 4, SPU, true>(a, st); }
-    launch_rows_rw<Act, FMT, SC, MR, 4, SPU, false>(a, st);
+    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, RW4, SPU, true>(a, st); }
+    launch_rows_rw<Act, FMT, SC, MR, RW4, SPU, false>(a, st);
   }
 }
 

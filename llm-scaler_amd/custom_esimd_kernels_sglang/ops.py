@@ -20,6 +20,70 @@ def q4_k_dequant(weight, weight_scale, weight_min, output):
     return _ops.q4_k_dequant(weight, weight_scale, weight_min, output)
 
 
+# other GGUF formats, S/python/custom_esimd_kernels_sglang/ops.py (esimd_gemv_q4_0 ... esimd_gemv_q6_k_m)
+def esimd_gemv_q4_0(input, weight, weight_scale, output):
+    """weight [N, K/2] uint8 interleaved nibbles, weight_scale [N, K/32] fp16; w = (nib - 8) * scale."""
+    return _ops.esimd_gemv_q4_0(input, weight, weight_scale, output)
+
+
+def esimd_gemm_q4_0(input, weight, weight_scale, output):
+    return _ops.esimd_gemm_q4_0(input, weight, weight_scale, output)
+
+
+def esimd_gemv_q8_0(input, weight, weight_scale, output):
+    """weight [N, K] int8, weight_scale [N, K/32] fp16; w = qs * scale."""
+    return _ops.esimd_gemv_q8_0(input, weight, weight_scale, output)
+
+
+def esimd_gemv_q8_0_m(input, weight, weight_scale, output):
+    return _ops.esimd_gemv_q8_0_m(input, weight, weight_scale, output)
+
+
+def esimd_gemv_q5_k(input, ql, qh, weight_scale, weight_min, output):
+    return _ops.esimd_gemv_q5_k(input, ql, qh, weight_scale, weight_min, output)
+
+
+def esimd_gemv_q6_k(input, ql, qh, weight_scale, output):
+    return _ops.esimd_gemv_q6_k(input, ql, qh, weight_scale, output)
+
+
+def esimd_gemv_q6_k_m(input, ql, qh, weight_scale, output):
+    return _ops.esimd_gemv_q6_k_m(input, ql, qh, weight_scale, output)
+
+
+# weight preparation on the device (the reference does these in torch at load time)
+def q4_0_repack(qweight, weight, weight_scale):
+    return _ops.q4_0_repack(qweight, weight, weight_scale)
+
+
+def q8_0_repack(qweight, weight, weight_scale):
+    return _ops.q8_0_repack(qweight, weight, weight_scale)
+
+
+def q5_k_repack(qweight, ql, qh, weight_scale, weight_min):
+    return _ops.q5_k_repack(qweight, ql, qh, weight_scale, weight_min)
+
+
+def q6_k_repack(qweight, ql, qh, weight_scale):
+    return _ops.q6_k_repack(qweight, ql, qh, weight_scale)
+
+
+def q4_0_dequant(weight, weight_scale, output):
+    return _ops.q4_0_dequant(weight, weight_scale, output)
+
+
+def q8_0_dequant(weight, weight_scale, output):
+    return _ops.q8_0_dequant(weight, weight_scale, output)
+
+
+def q5_k_dequant(ql, qh, weight_scale, weight_min, output):
+    return _ops.q5_k_dequant(ql, qh, weight_scale, weight_min, output)
+
+
+def q6_k_dequant(ql, qh, weight_scale, output):
+    return _ops.q6_k_dequant(ql, qh, weight_scale, output)
+
+
 def esimd_gemv_fp8_pern(input, weight, weight_scale, output, N, K):
     return _ops.esimd_gemv_fp8_pern(input, weight, weight_scale, output, N, K)
 

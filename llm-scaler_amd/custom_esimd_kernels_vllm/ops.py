@@ -210,3 +210,9 @@ def esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output,
 
 def esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
     return _ops.esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)
+
+
+def q4_0_quantize(input, out_qweight, out_scale):
+    """torch.ops.custom_esimd_kernels_vllm.q4_0_quantize (the reference registers it from its
+    q4_0_quant_ops module): [M, K] fp16/bf16 -> int32 [M, K/8] + fp16 scale [M, K/128]."""
+    return _ops.q4_0_quantize(input, out_qweight, out_scale)

@@ -297,6 +297,233 @@ def q4_k_dequant(weight, weight_scale, weight_min, output):
 
 
 # --------------------------------------------------------------------------
+# Other GGUF formats: Q4_0, Q8_0, Q5_K, Q6_K (S/csrc/xpu/torch_extension.cc:48-106)
+# and the group-128 Q4_0 quantizer (V/csrc/xpu/torch_extension_q4_0.cc:27-75)
+# --------------------------------------------------------------------------
+def _chk_gguf_io(x, o, N, K, who):
+    _chk(x.dtype == torch.float16 and o.dtype == torch.float16, f"{who}: input and output must be fp16")
+    _chk(x.is_contiguous() and o.is_contiguous(), f"{who}: input and output must be contiguous")
+    _chk(x.numel() % K == 0, f"{who}: input numel {x.numel()} is not a multiple of K={K}")
+    M = x.numel() // K
+    _chk(o.numel() == M * N, f"{who}: output has {o.numel()} elements, expected M*N={M * N}")
+    return M
+
+
+def _chk_u8(t, shape, nm, who, dtypes=(torch.uint8,)):
+    _chk(t.dtype in dtypes and t.is_contiguous() and tuple(t.shape) == tuple(shape),
+         f"{who}: {nm} must be contiguous {'/'.join(str(d) for d in dtypes)} {list(shape)}, got {t.dtype} {list(t.shape)}")
+
+
+def _chk_f16(t, numel, nm, who):
+    _chk(t.dtype == torch.float16 and t.is_contiguous() and t.numel() == numel,
+         f"{who}: {nm} must be contiguous fp16 with {numel} elements")
+
+
+def _gemv_q4_0(input, weight, weight_scale, output, who):
+    _chk(weight.dtype == torch.uint8 and weight.dim() == 2 and weight.is_contiguous(),
+         f"{who}: weight must be contiguous uint8 [N, K/2]")
+    N, K = weight.shape[0], weight.shape[1] * 2
+    _chk(K % 32 == 0, f"{who}: K={K} must be a multiple of 32")
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale [N, K/32]", who)
+    M = _chk_gguf_io(input, output, N, K, who)
+    capi.call("mi_gemv_q4_0", input, capi.ptr(input), capi.ptr(weight), capi.ptr(weight_scale), capi.ptr(output), M, N, K)
+    return output
+
+
+def esimd_gemv_q4_0(input, weight, weight_scale, output):
+    """weight [N, K/2] uint8 interleaved nibbles, scale [N, K/32] fp16; w = (nib - 8) * scale."""
+    return _gemv_q4_0(input, weight, weight_scale, output, "esimd_gemv_q4_0")
+
+
+def esimd_gemm_q4_0(input, weight, weight_scale, output):
+    """The reference's M >= 2 op on the same layout; one kernel family serves both here."""
+    return _gemv_q4_0(input, weight, weight_scale, output, "esimd_gemm_q4_0")
+
+
+def _gemv_q8_0(input, weight, weight_scale, output, who):
+    _chk(weight.dtype in (torch.int8, torch.uint8) and weight.dim() == 2 and weight.is_contiguous(),
+         f"{who}: weight must be contiguous int8 [N, K]")
+    N, K = weight.shape
+    _chk(K % 32 == 0, f"{who}: K={K} must be a multiple of 32")
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale [N, K/32]", who)
+    M = _chk_gguf_io(input, output, N, K, who)
+    capi.call("mi_gemv_q8_0", input, capi.ptr(input), capi.ptr(weight), capi.ptr(weight_scale), capi.ptr(output), M, N, K)
+    return output
+
+
+def esimd_gemv_q8_0(input, weight, weight_scale, output):
+    """weight [N, K] int8, scale [N, K/32] fp16; w = qs * scale."""
+    return _gemv_q8_0(input, weight, weight_scale, output, "esimd_gemv_q8_0")
+
+
+def esimd_gemv_q8_0_m(input, weight, weight_scale, output):
+    return _gemv_q8_0(input, weight, weight_scale, output, "esimd_gemv_q8_0_m")
+
+
+def esimd_gemv_q5_k(input, ql, qh, weight_scale, weight_min, output):
+    """ql [N, K/2], qh [N, K/8] (tile-shuffled fifth bits), scale / min [N, K/32] fp16."""
+    who = "esimd_gemv_q5_k"
+    _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be contiguous uint8 [N, K/2]")
+    N, K = ql.shape[0], ql.shape[1] * 2
+    _chk(K % 512 == 0, f"{who}: K={K} must be a multiple of 512")
+    _chk_u8(qh, (N, K // 8), "qh", who)
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale [N, K/32]", who)
+    _chk_f16(weight_min, N * (K // 32), "weight_min [N, K/32]", who)
+    M = _chk_gguf_io(input, output, N, K, who)
+    capi.call("mi_gemv_q5k", input, capi.ptr(input), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale),
+              capi.ptr(weight_min), capi.ptr(output), M, N, K)
+    return output
+
+
+def _gemv_q6_k(input, ql, qh, weight_scale, output, who):
+    _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be contiguous uint8 [N, K/2]")
+    N, K = ql.shape[0], ql.shape[1] * 2
+    _chk(K % 512 == 0, f"{who}: K={K} must be a multiple of 512")
+    _chk_u8(qh, (N, K // 4), "qh", who)
+    _chk_f16(weight_scale, N * (K // 16), "weight_scale [N, K/16]", who)
+    M = _chk_gguf_io(input, output, N, K, who)
+    capi.call("mi_gemv_q6k", input, capi.ptr(input), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale),
+              capi.ptr(output), M, N, K)
+    return output
+
+
+def esimd_gemv_q6_k(input, ql, qh, weight_scale, output):
+    """ql [N, K/2], qh [N, K/4] (tile-shuffled top two bits), scale [N, K/16] fp16; w = (v6 - 32) * scale."""
+    return _gemv_q6_k(input, ql, qh, weight_scale, output, "esimd_gemv_q6_k")
+
+
+def esimd_gemv_q6_k_m(input, ql, qh, weight_scale, output):
+    return _gemv_q6_k(input, ql, qh, weight_scale, output, "esimd_gemv_q6_k_m")
+
+
+def _raw_rows(qweight, block_bytes, block_elems, who):
+    _chk(qweight.dtype == torch.uint8 and qweight.dim() == 2 and qweight.is_contiguous(),
+         f"{who}: qweight must be contiguous uint8 [N, blocks*{block_bytes}]")
+    _chk(qweight.shape[1] % block_bytes == 0, f"{who}: row length {qweight.shape[1]} is not a multiple of {block_bytes}")
+    return qweight.shape[0], qweight.shape[1] // block_bytes * block_elems
+
+
+def q4_0_repack(qweight, weight, weight_scale):
+    """Raw GGML q4_0 rows [N, K/32*18] -> (weight [N, K/2] interleaved nibbles, scale [N, K/32])."""
+    who = "q4_0_repack"
+    N, K = _raw_rows(qweight, 18, 32, who)
+    _chk_u8(weight, (N, K // 2), "weight", who)
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    capi.call("mi_q4_0_repack", qweight, capi.ptr(qweight), capi.ptr(weight), capi.ptr(weight_scale), N, K)
+    return weight
+
+
+def q8_0_repack(qweight, weight, weight_scale):
+    """Raw GGML q8_0 rows [N, K/32*34] -> (weight [N, K] int8, scale [N, K/32])."""
+    who = "q8_0_repack"
+    N, K = _raw_rows(qweight, 34, 32, who)
+    _chk_u8(weight, (N, K), "weight", who, (torch.int8, torch.uint8))
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    capi.call("mi_q8_0_repack", qweight, capi.ptr(qweight), capi.ptr(weight), capi.ptr(weight_scale), N, K)
+    return weight
+
+
+def q5_k_repack(qweight, ql, qh, weight_scale, weight_min):
+    """Raw GGML q5_K rows [N, K/256*176] -> (ql, tile-shuffled qh, scale, min)."""
+    who = "q5_k_repack"
+    N, K = _raw_rows(qweight, 176, 256, who)
+    _chk(K % 512 == 0, f"{who}: K={K} must be a multiple of 512")
+    _chk_u8(ql, (N, K // 2), "ql", who)
+    _chk_u8(qh, (N, K // 8), "qh", who)
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    _chk_f16(weight_min, N * (K // 32), "weight_min", who)
+    capi.call("mi_q5k_repack", qweight, capi.ptr(qweight), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale),
+              capi.ptr(weight_min), N, K)
+    return ql
+
+
+def q6_k_repack(qweight, ql, qh, weight_scale):
+    """Raw GGML q6_K rows [N, K/256*210] -> (ql, tile-shuffled qh, scale [N, K/16])."""
+    who = "q6_k_repack"
+    N, K = _raw_rows(qweight, 210, 256, who)
+    _chk(K % 512 == 0, f"{who}: K={K} must be a multiple of 512")
+    _chk_u8(ql, (N, K // 2), "ql", who)
+    _chk_u8(qh, (N, K // 4), "qh", who)
+    _chk_f16(weight_scale, N * (K // 16), "weight_scale", who)
+    capi.call("mi_q6k_repack", qweight, capi.ptr(qweight), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale), N, K)
+    return ql
+
+
+def _chk_dense_out(output, N, K, who):
+    _chk(output.dtype == torch.float16 and output.is_contiguous() and output.numel() == N * K,
+         f"{who}: output must be contiguous fp16 [N, K]")
+
+
+def q4_0_dequant(weight, weight_scale, output):
+    who = "q4_0_dequant"
+    _chk(weight.dtype == torch.uint8 and weight.dim() == 2 and weight.is_contiguous(), f"{who}: weight must be uint8 [N, K/2]")
+    N, K = weight.shape[0], weight.shape[1] * 2
+    _chk(K % 32 == 0, f"{who}: K must be a multiple of 32")
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    _chk_dense_out(output, N, K, who)
+    capi.call("mi_dequant_q4_0", weight, capi.ptr(weight), capi.ptr(weight_scale), capi.ptr(output), N, K)
+    return output
+
+
+def q8_0_dequant(weight, weight_scale, output):
+    who = "q8_0_dequant"
+    _chk(weight.dtype in (torch.int8, torch.uint8) and weight.dim() == 2 and weight.is_contiguous(),
+         f"{who}: weight must be int8 [N, K]")
+    N, K = weight.shape
+    _chk(K % 32 == 0, f"{who}: K must be a multiple of 32")
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    _chk_dense_out(output, N, K, who)
+    capi.call("mi_dequant_q8_0", weight, capi.ptr(weight), capi.ptr(weight_scale), capi.ptr(output), N, K)
+    return output
+
+
+def q5_k_dequant(ql, qh, weight_scale, weight_min, output):
+    who = "q5_k_dequant"
+    _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be uint8 [N, K/2]")
+    N, K = ql.shape[0], ql.shape[1] * 2
+    _chk(K % 512 == 0, f"{who}: K must be a multiple of 512")
+    _chk_u8(qh, (N, K // 8), "qh", who)
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    _chk_f16(weight_min, N * (K // 32), "weight_min", who)
+    _chk_dense_out(output, N, K, who)
+    capi.call("mi_dequant_q5k", ql, capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale), capi.ptr(weight_min),
+              capi.ptr(output), N, K)
+    return output
+
+
+def q6_k_dequant(ql, qh, weight_scale, output):
+    who = "q6_k_dequant"
+    _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be uint8 [N, K/2]")
+    N, K = ql.shape[0], ql.shape[1] * 2
+    _chk(K % 512 == 0, f"{who}: K must be a multiple of 512")
+    _chk_u8(qh, (N, K // 4), "qh", who)
+    _chk_f16(weight_scale, N * (K // 16), "weight_scale", who)
+    _chk_dense_out(output, N, K, who)
+    capi.call("mi_dequant_q6k", ql, capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale), capi.ptr(output), N, K)
+    return output
+
+
+def q4_0_quantize(input, out_qweight, out_scale):
+    """V/csrc/xpu/torch_extension_q4_0.cc:27-75: [M, K] fp16/bf16 -> int32 [M, K/8] + fp16 scale [M, K/128]."""
+    who = "q4_0_quantize"
+    _chk(input.dim() == 2, f"{who}: input must be 2D")
+    _chk(input.is_contiguous(), f"{who}: input must be contiguous")
+    _chk(out_qweight.is_contiguous(), f"{who}: out_qweight must be contiguous")
+    _chk(out_scale.is_contiguous(), f"{who}: out_scale must be contiguous")
+    _chk(out_qweight.dtype == torch.int32, f"{who}: out_qweight must be int32")
+    _chk(out_scale.dtype == torch.float16, f"{who}: out_scale must be float16")
+    M, K = input.shape
+    _chk(K % 128 == 0, f"{who}: K must be divisible by 128 (got {K})")
+    _chk(out_qweight.shape[0] == M, f"{who}: out_qweight row count mismatch")
+    _chk(out_qweight.shape[1] == K // 8, f"{who}: out_qweight col count must be K/8")
+    _chk(out_scale.shape[0] == M, f"{who}: out_scale row count mismatch")
+    _chk(out_scale.shape[1] == K // 128, f"{who}: out_scale col count must be K/128")
+    _chk(input.dtype in (torch.float16, torch.bfloat16), f"{who}: input dtype must be bfloat16 or float16 (got {input.dtype})")
+    capi.call("mi_q4_0_quantize", input, capi.ptr(input), capi.ptr(out_qweight), capi.ptr(out_scale), M, K,
+              capi.act_dtype(input))
+
+
+# --------------------------------------------------------------------------
 # dequant-only siblings
 # --------------------------------------------------------------------------
 def int4_dequant(weight, weight_scale, weight_zp, output):
@@ -965,6 +1192,34 @@ def register():
                 "Tensor(c!) weight_min) -> Tensor(a!)", q4_k_repack, _ret(1))
     _define(_S, "q4_k_dequant(Tensor weight, Tensor weight_scale, Tensor weight_min, "
                 "Tensor(a!) output) -> Tensor(a!)", q4_k_dequant, _ret(3))
+    # other GGUF formats (S/csrc/xpu/torch_extension.cc:48-106) and their weight preparation
+    _define(_S, "esimd_gemv_q4_0(Tensor input, Tensor weight, Tensor weight_scale, Tensor output) -> Tensor",
+            esimd_gemv_q4_0, _ret(3))
+    _define(_S, "esimd_gemm_q4_0(Tensor input, Tensor weight, Tensor weight_scale, Tensor output) -> Tensor",
+            esimd_gemm_q4_0, _ret(3))
+    _define(_S, "esimd_gemv_q8_0(Tensor input, Tensor weight, Tensor weight_scale, Tensor output) -> Tensor",
+            esimd_gemv_q8_0, _ret(3))
+    _define(_S, "esimd_gemv_q8_0_m(Tensor input, Tensor weight, Tensor weight_scale, Tensor output) -> Tensor",
+            esimd_gemv_q8_0_m, _ret(3))
+    _define(_S, "esimd_gemv_q5_k(Tensor input, Tensor ql, Tensor qh, Tensor weight_scale, Tensor weight_min, "
+                "Tensor output) -> Tensor", esimd_gemv_q5_k, _ret(5))
+    _define(_S, "esimd_gemv_q6_k(Tensor input, Tensor ql, Tensor qh, Tensor weight_scale, Tensor output) -> Tensor",
+            esimd_gemv_q6_k, _ret(4))
+    _define(_S, "esimd_gemv_q6_k_m(Tensor input, Tensor ql, Tensor qh, Tensor weight_scale, Tensor output) -> Tensor",
+            esimd_gemv_q6_k_m, _ret(4))
+    _define(_S, "q4_0_repack(Tensor qweight, Tensor(a!) weight, Tensor(b!) weight_scale) -> Tensor(a!)", q4_0_repack, _ret(1))
+    _define(_S, "q8_0_repack(Tensor qweight, Tensor(a!) weight, Tensor(b!) weight_scale) -> Tensor(a!)", q8_0_repack, _ret(1))
+    _define(_S, "q5_k_repack(Tensor qweight, Tensor(a!) ql, Tensor(b!) qh, Tensor(c!) weight_scale, "
+                "Tensor(d!) weight_min) -> Tensor(a!)", q5_k_repack, _ret(1))
+    _define(_S, "q6_k_repack(Tensor qweight, Tensor(a!) ql, Tensor(b!) qh, Tensor(c!) weight_scale) -> Tensor(a!)",
+            q6_k_repack, _ret(1))
+    _define(_S, "q4_0_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output) -> Tensor(a!)", q4_0_dequant, _ret(2))
+    _define(_S, "q8_0_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output) -> Tensor(a!)", q8_0_dequant, _ret(2))
+    _define(_S, "q5_k_dequant(Tensor ql, Tensor qh, Tensor weight_scale, Tensor weight_min, Tensor(a!) output) -> Tensor(a!)",
+            q5_k_dequant, _ret(4))
+    _define(_S, "q6_k_dequant(Tensor ql, Tensor qh, Tensor weight_scale, Tensor(a!) output) -> Tensor(a!)",
+            q6_k_dequant, _ret(3))
+    _define(_V, "q4_0_quantize(Tensor input, Tensor(a!) out_qweight, Tensor(b!) out_scale) -> ()", q4_0_quantize, None)
     _define(_V, "int4_dequant(Tensor weight, Tensor weight_scale, Tensor? weight_zp, "
                 "Tensor(a!) output) -> Tensor(a!)", int4_dequant, _ret(3))
     _define(_V, "fp8_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output, str mode) -> Tensor(a!)",

@@ -1,0 +1,234 @@
+"""GPU parity for the weight-preparation side: GGUF Q4_0 / Q8_0 / Q5_K / Q6_K repack,
+dequant and decode GEMV, and the group-128 Q4_0 quantizer, through torch.ops ->
+ctypes -> the C ABI, against the CPU oracle.
+
+Bars: repack outputs, dequantized weights and quantizer outputs bit-exact; GEMV
+outputs within max relative error 1e-2 of the fp32-accumulated reference on the
+oracle's dequantized weights.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as G
+from oracle import qlinear_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops(dev):
+    import custom_esimd_kernels_vllm as v
+    import custom_esimd_kernels_sglang as s
+    return v, s
+
+
+def _t(a):
+    return torch.from_numpy(np.ascontiguousarray(a))
+
+
+def _f16u(rng, shape, lo, hi):
+    return rng.uniform(lo, hi, size=shape).astype(np.float16)
+
+
+def _raw_case(kind, N, K, seed):
+    rng = np.random.default_rng(seed)
+    if kind == "q4_0":
+        d = _f16u(rng, (N, K // 32), -0.02, 0.02)
+        return G.q4_0_build_raw(rng.integers(0, 16, size=(N, K), dtype=np.uint8), d)
+    if kind == "q8_0":
+        d = _f16u(rng, (N, K // 32), -0.002, 0.002)
+        return G.q8_0_build_raw(rng.integers(-128, 128, size=(N, K)).astype(np.int8), d)
+    nsb = K // 256
+    if kind == "q5_k":
+        sc12 = O.q4k_pack_scales(rng.integers(0, 64, size=(N, nsb, 8)), rng.integers(0, 64, size=(N, nsb, 8)))
+        return G.q5k_build_raw(rng.integers(0, 32, size=(N, K)), sc12, _f16u(rng, (N, nsb), 0.0005, 0.005),
+                               _f16u(rng, (N, nsb), 0.0, 0.003))
+    sc = rng.integers(-128, 128, size=(N, nsb, 16)).astype(np.int8)
+    return G.q6k_build_raw(rng.integers(0, 64, size=(N, K)), sc, _f16u(rng, (N, nsb), 0.00002, 0.0002))
+
+
+def _repack_oracle(kind, raw):
+    return {"q4_0": G.q4_0_repack, "q8_0": G.q8_0_repack, "q5_k": G.q5k_repack, "q6_k": G.q6k_repack}[kind](raw)
+
+
+def _dequant_oracle(kind, rep):
+    return {"q4_0": G.q4_0_dequant, "q8_0": G.q8_0_dequant, "q5_k": G.q5k_dequant, "q6_k": G.q6k_dequant}[kind](*rep)
+
+
+def _repack_gpu(s, kind, raw, dev):
+    N = raw.shape[0]
+    r = _t(raw).to(dev)
+    if kind == "q4_0":
+        K = raw.shape[1] // 18 * 32
+        out = (torch.empty(N, K // 2, dtype=torch.uint8, device=dev), torch.empty(N, K // 32, dtype=torch.float16, device=dev))
+        s.q4_0_repack(r, *out)
+    elif kind == "q8_0":
+        K = raw.shape[1] // 34 * 32
+        out = (torch.empty(N, K, dtype=torch.int8, device=dev), torch.empty(N, K // 32, dtype=torch.float16, device=dev))
+        s.q8_0_repack(r, *out)
+    elif kind == "q5_k":
+        K = raw.shape[1] // 176 * 256
+        out = (torch.empty(N, K // 2, dtype=torch.uint8, device=dev), torch.empty(N, K // 8, dtype=torch.uint8, device=dev),
+               torch.empty(N, K // 32, dtype=torch.float16, device=dev), torch.empty(N, K // 32, dtype=torch.float16, device=dev))
+        s.q5_k_repack(r, *out)
+    else:
+        K = raw.shape[1] // 210 * 256
+        out = (torch.empty(N, K // 2, dtype=torch.uint8, device=dev), torch.empty(N, K // 4, dtype=torch.uint8, device=dev),
+               torch.empty(N, K // 16, dtype=torch.float16, device=dev))
+        s.q6_k_repack(r, *out)
+    return out, K
+
+
+def _same(a_gpu, b_np):
+    a = a_gpu.cpu().numpy()
+    if a.dtype == np.float16:
+        return np.array_equal(a.view(np.uint16), np.asarray(b_np).view(np.uint16))
+    return np.array_equal(a.view(np.uint8), np.asarray(b_np).view(np.uint8))
+
+
+KINDS = ["q4_0", "q8_0", "q5_k", "q6_k"]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("N,K", [(3, 512), (64, 2048), (17, 5120)])
+def test_repack_and_dequant_bit_exact(ops, dev, kind, N, K):
+    _, s = ops
+    raw = _raw_case(kind, N, K, seed=N + K)
+    ref = _repack_oracle(kind, raw)
+    got, K2 = _repack_gpu(s, kind, raw, dev)
+    assert K2 == K
+    for g, r in zip(got, ref):
+        assert _same(g, r)
+    dense = torch.empty(N, K, dtype=torch.float16, device=dev)
+    getattr(s, f"{kind}_dequant")(*got, dense)
+    assert _same(dense, _dequant_oracle(kind, ref))
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_dequant_extreme_scales(ops, dev, kind):
+    # negative, subnormal-product and large scales / mins: roundings must still match bit for bit
+    _, s = ops
+    N, K = 8, 1024
+    raw = _raw_case(kind, N, K, seed=99)
+    rep = [np.array(a) for a in _repack_oracle(kind, raw)]
+    sc = rep[-2] if kind == "q5_k" else rep[-1]
+    sc[0, :4] = np.array([-0.875, 6.0e-5, 1.0e-7, 300.0], dtype=np.float16)
+    if kind == "q5_k":
+        rep[-1][0, :4] = np.array([0.3333, -2.5, 6.0e-8, 1000.0], dtype=np.float16)
+    dense = torch.empty(N, K, dtype=torch.float16, device=dev)
+    getattr(s, f"{kind}_dequant")(*[_t(a).to(dev) for a in rep], dense)
+    assert _same(dense, _dequant_oracle(kind, rep))
+
+
+def _gemv(s, kind, x, rep, out, name=None):
+    name = name or f"esimd_gemv_{kind}"
+    return getattr(s, name)(x, *rep, out)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("M,N,K", [(1, 64, 512), (1, 1000, 4096), (1, 520, 5120), (2, 96, 2048), (3, 33, 1024),
+                                   (4, 256, 8192), (1, 40, 14336), (7, 48, 1536), (16, 130, 2048)])
+def test_gemv(ops, dev, kind, M, N, K):
+    _, s = ops
+    raw = _raw_case(kind, N, K, seed=7 * M + N + K)
+    rep = _repack_oracle(kind, raw)
+    wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32))
+    g = torch.Generator().manual_seed(K + M)
+    x = torch.randn(M, K, generator=g).half()
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    ret = _gemv(s, kind, x.to(dev), [_t(a).to(dev) for a in rep], out)
+    assert ret.data_ptr() == out.data_ptr()
+    ref = O.matmul_ref(x, wd)
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
+@pytest.mark.parametrize("name,kind", [("esimd_gemm_q4_0", "q4_0"), ("esimd_gemv_q8_0_m", "q8_0"), ("esimd_gemv_q6_k_m", "q6_k")])
+def test_small_m_variants(ops, dev, name, kind):
+    _, s = ops
+    M, N, K = 6, 200, 2048
+    raw = _raw_case(kind, N, K, seed=5)
+    rep = _repack_oracle(kind, raw)
+    wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32))
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(3)).half()
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    _gemv(s, kind, x.to(dev), [_t(a).to(dev) for a in rep], out, name)
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, wd)) < TOL
+
+
+@pytest.mark.parametrize("kind", ["q5_k", "q6_k"])
+def test_gemv_every_high_bit_field(ops, dev, kind):
+    # weights whose low nibbles are zero: the output depends on the high bits alone,
+    # one 64- (Q5_K) or 128-element (Q6_K) field of one 512-tile at a time
+    _, s = ops
+    N, K = 16, 1024
+    span = 64 if kind == "q5_k" else 128
+    for f in range(K // span):
+        v = np.zeros((N, K), dtype=np.int64)
+        v[:, f * span:(f + 1) * span] = 16 if kind == "q5_k" else 48
+        if kind == "q5_k":
+            sc12 = O.q4k_pack_scales(np.full((N, K // 256, 8), 1), np.zeros((N, K // 256, 8), dtype=np.int64))
+            raw = G.q5k_build_raw(v, sc12, np.full((N, K // 256), 0.5, np.float16), np.zeros((N, K // 256), np.float16))
+        else:
+            raw = G.q6k_build_raw(v, np.ones((N, K // 256, 16), np.int8), np.full((N, K // 256), 0.5, np.float16))
+        rep = _repack_oracle(kind, raw)
+        wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32))
+        x = torch.randn(1, K, generator=torch.Generator().manual_seed(f)).half()
+        out = torch.empty(1, N, dtype=torch.float16, device=dev)
+        _gemv(s, kind, x.to(dev), [_t(a).to(dev) for a in rep], out)
+        assert O.max_rel_err(out.cpu(), O.matmul_ref(x, wd)) < TOL, f"field {f}"
+
+
+def test_gguf_shape_errors(ops, dev):
+    _, s = ops
+    x = torch.zeros(1, 256, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError):          # Q5_K needs whole 512-tiles
+        s.esimd_gemv_q5_k(x, torch.zeros(4, 128, dtype=torch.uint8, device=dev), torch.zeros(4, 32, dtype=torch.uint8, device=dev),
+                          torch.zeros(4, 8, dtype=torch.float16, device=dev), torch.zeros(4, 8, dtype=torch.float16, device=dev),
+                          torch.zeros(1, 4, dtype=torch.float16, device=dev))
+    with pytest.raises(RuntimeError):          # bf16 activations are not part of the GGUF path
+        s.esimd_gemv_q8_0(x.bfloat16(), torch.zeros(4, 256, dtype=torch.int8, device=dev),
+                          torch.zeros(4, 8, dtype=torch.float16, device=dev), torch.zeros(1, 4, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(RuntimeError):
+        s.q4_0_repack(torch.zeros(4, 19, dtype=torch.uint8, device=dev), torch.zeros(4, 16, dtype=torch.uint8, device=dev),
+                      torch.zeros(4, 1, dtype=torch.float16, device=dev))
+
+
+# ------------------------------------------------------------- quantizer ----
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", [(1, 128), (4, 256), (16, 128), (256, 512), (1024, 2048), (512, 5120)])
+def test_q4_0_quantize_bit_exact(ops, dev, dt, M, K):
+    # shapes of V/tests/test_q4_0_quant_xpu.py:52-61
+    v, _ = ops
+    g = torch.Generator().manual_seed(M * 7 + K)
+    x = (torch.randn(M, K, generator=g) * 0.5).to(dt)
+    x[0, :4] = torch.tensor([7.0, -7.0, 3.0, -3.0]).to(dt)          # known-answer block when K == 128 ... and ties
+    if M > 1:
+        x[1, :] = 0                                                  # all-zero blocks
+    q = torch.empty(M, K // 8, dtype=torch.int32, device=dev)
+    sc = torch.empty(M, K // 128, dtype=torch.float16, device=dev)
+    assert v.q4_0_quantize(x.to(dev), q, sc) is None
+    rq, rs = G.q4_0_quantize(x.float().numpy())
+    assert np.array_equal(sc.cpu().numpy().view(np.uint16), rs.view(np.uint16))
+    assert np.array_equal(q.cpu().numpy(), rq)
+
+
+def test_q4_0_quantize_feeds_int4_gemv(ops, dev):
+    # quantize on the device, run the int4 GEMV on the result, compare with the dense product
+    v, _ = ops
+    N, K = 512, 4096
+    g = torch.Generator().manual_seed(11)
+    w = (torch.randn(N, K, generator=g) * 0.05).half()
+    x = torch.randn(1, K, generator=g).half()
+    q = torch.empty(N, K // 8, dtype=torch.int32, device=dev)
+    sc = torch.empty(N, K // 128, dtype=torch.float16, device=dev)
+    v.q4_0_quantize(w.to(dev), q, sc)
+    out = torch.empty(1, N, dtype=torch.float16, device=dev)
+    v.esimd_gemv_int4(x.to(dev), q.view(torch.uint8), sc, out)
+    wd = O.int4_dequant(q.cpu().view(torch.uint8), sc.cpu(), out_dtype=torch.float16)
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, wd)) < TOL
+    # and the quantization itself stays inside the Q4_0 envelope: |w - deq| <= |d|
+    err = (wd.float() - w.float()).abs()
+    assert bool((err <= sc.cpu().float().abs().repeat_interleave(128, dim=1) + 1e-4).all())
