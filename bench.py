@@ -125,6 +125,106 @@ def wl_q4k(M: int, dev):
                 kernel="gemv_rows_kernel" if M <= 4 else "skinny_kernel", cpu=cpu)
 
 
+def wl_gguf(kind: str, M: int, dev):
+    """Decode GEMV on the other GGUF formats at the cfg4 shape (next-row workloads)."""
+    import custom_esimd_kernels_sglang as s
+    import numpy as np
+    from oracle import gguf_oracle as G
+    from oracle import qlinear_oracle as O
+    K = N = 5120
+    rng = np.random.default_rng(1240)
+    f16u = lambda shape, lo, hi: rng.uniform(lo, hi, size=shape).astype(np.float16)
+    nsb = K // 256
+    if kind == "q4_0":
+        raw = G.q4_0_build_raw(rng.integers(0, 16, size=(N, K), dtype=np.uint8), f16u((N, K // 32), -0.02, 0.02))
+        rep, deq, op = G.q4_0_repack(raw), G.q4_0_dequant, s.esimd_gemv_q4_0
+    elif kind == "q8_0":
+        raw = G.q8_0_build_raw(rng.integers(-128, 128, size=(N, K)).astype(np.int8), f16u((N, K // 32), -0.002, 0.002))
+        rep, deq, op = G.q8_0_repack(raw), G.q8_0_dequant, s.esimd_gemv_q8_0
+    elif kind == "q5_k":
+        sc12 = O.q4k_pack_scales(rng.integers(0, 64, size=(N, nsb, 8)), rng.integers(0, 64, size=(N, nsb, 8)))
+        raw = G.q5k_build_raw(rng.integers(0, 32, size=(N, K)), sc12, f16u((N, nsb), 0.0005, 0.005), f16u((N, nsb), 0.0, 0.003))
+        rep, deq, op = G.q5k_repack(raw), G.q5k_dequant, s.esimd_gemv_q5_k
+    else:
+        raw = G.q6k_build_raw(rng.integers(0, 64, size=(N, K)), rng.integers(-128, 128, size=(N, nsb, 16)).astype(np.int8),
+                              f16u((N, nsb), 0.00002, 0.0002))
+        rep, deq, op = G.q6k_repack(raw), G.q6k_dequant, s.esimd_gemv_q6_k
+    rep_t = [torch.from_numpy(np.ascontiguousarray(a)) for a in rep]
+    per = sum(t.numel() * t.element_size() for t in rep_t)
+    R = _copies(per)
+    g = torch.Generator().manual_seed(96)
+    W = [[t.to(dev) for t in rep_t]]
+    for _ in range(R - 1):
+        p = torch.randperm(N, generator=g)
+        W.append([t[p].to(dev) for t in rep_t])
+    x = torch.randn(M, K, generator=g).half()
+    xd = x.to(dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        op(xd, *W[i % R], out)
+
+    def cpu():
+        return O.matmul_ref(x, torch.from_numpy(deq(*rep).astype(np.float32))).to(torch.float16)
+
+    return dict(launch=launch, R=R, bytes=per + 2 * M * K + 2 * M * N, flops=2 * M * N * K, bound="hbm", dtype="f16",
+                name=f"next: GGUF {kind} (repacked) decode GEMV M={M} K={K} N={N} fp16", kernel="gemv_rows_kernel", cpu=cpu)
+
+
+def wl_q4_0_quantize(dev):
+    """On-device group-128 Q4_0 quantization of a [14336, 4096] bf16 weight (next-row workload)."""
+    import custom_esimd_kernels_vllm as v
+    from oracle import gguf_oracle as G
+    rows, K = 14336, 4096
+    g = torch.Generator().manual_seed(95)
+    w = (torch.randn(rows, K, generator=g) * 0.02).bfloat16()
+    R = _copies(rows * K * 2)
+    ws = [w.to(dev)] + [w[torch.randperm(rows, generator=g)].to(dev) for _ in range(R - 1)]
+    q = torch.empty(rows, K // 8, dtype=torch.int32, device=dev)
+    sc = torch.empty(rows, K // 128, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        v.q4_0_quantize(ws[i % R], q, sc)
+
+    def cpu():
+        return G.q4_0_quantize(w.float().numpy())
+
+    return dict(launch=launch, R=R, bytes=rows * K * 2 + rows * K // 2 + rows * (K // 128) * 2, flops=0, bound="hbm",
+                dtype="f32", name=f"next: q4_0_quantize (group 128) [{rows}, {K}] bf16 -> int4 + fp16 scales",
+                kernel="q4_0_quantize_kernel", cpu=cpu)
+
+
+def wl_resadd_norm_gemv(dev):
+    """Residual add + RMS norm fused into the FP8 per-tensor GEMV, K=4096 N=14336 fp16 (next-row workload)."""
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    K, N = 4096, 14336
+    g = torch.Generator().manual_seed(94)
+    w8 = O.e4m3_quantize((torch.randn(N, K, generator=g) * 100).clamp(-448, 448))
+    R = _copies(N * K)
+    ws = [w8.to(dev).view(torch.float8_e4m3fn)] + [w8[torch.randperm(N, generator=g)].to(dev).view(torch.float8_e4m3fn)
+                                                    for _ in range(R - 1)]
+    h = torch.zeros(1, K).half()       # the op adds it into `residual` in place on every launch: keep that stationary
+    res = torch.randn(1, K, generator=g).half()
+    nw = (torch.randn(K, generator=g) * 0.1 + 1.0).half()
+    sc = torch.tensor([2.0e-4])
+    hd, nwd, scd = h.to(dev), nw.to(dev), sc.to(dev)
+    resd = res.to(dev)
+    out = torch.empty(1, N, dtype=torch.float16, device=dev)
+    normed = torch.empty(1, K, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        v.esimd_resadd_norm_gemv_fp8_pert(hd, resd, nwd, ws[i % R], scd, out, normed, 1e-6)
+
+    def cpu():
+        nr, _ = O.rmsnorm(h, nw, 1e-6, residual=res)
+        return O.matmul_ref(nr.half(), O.fp8_dequant_per_tensor(w8, sc)).half()
+
+    return dict(launch=launch, R=R, bytes=N * K + 4 + 2 * N + 5 * 2 * K, flops=2 * N * K, bound="hbm", dtype="f16",
+                name=f"next: resadd + RMS norm + FP8 per-tensor GEMV M=1 K={K} N={N} fp16 (one fused launch)",
+                kernel="gemv_rows_kernel", cpu=cpu)
+
+
 def wl_gemm_w4a16(dev):
     import custom_esimd_kernels_vllm as v
     from oracle import qlinear_oracle as O
@@ -202,6 +302,12 @@ WORKLOADS = {
     "cfg3": wl_moe,
     "cfg4_m1": lambda dev: wl_q4k(1, dev),
     "cfg4_m64": lambda dev: wl_q4k(64, dev),
+    "next_q4_0_m1": lambda dev: wl_gguf("q4_0", 1, dev),
+    "next_q8_0_m1": lambda dev: wl_gguf("q8_0", 1, dev),
+    "next_q5_k_m1": lambda dev: wl_gguf("q5_k", 1, dev),
+    "next_q6_k_m1": lambda dev: wl_gguf("q6_k", 1, dev),
+    "next_q4_0_quantize": wl_q4_0_quantize,
+    "next_resadd_norm_gemv": wl_resadd_norm_gemv,
 }
 HEADLINE = "cfg1_m1"
 

@@ -247,6 +247,24 @@ int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void
 int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weight, void* out, int rows, int L,
                int weight_len, float eps, int act_dtype, void* stream);
 
+/* The same normalisation fused into the decode GEMV (one launch, M == 1):
+ *   x' = rmsnorm(x (+ residual)) (* silu(gate)) per head of norm_len elements
+ *   (norm_len == K: the whole row), out[i] = x' @ dequant(w[i])^T for nmat <= 3
+ *   matrices.  fmt 0 = FP8 per-tensor scale (scale[i] -> fp32 [1]), 1 = FP8 128x128
+ *   block scale, 2 = INT4 group 128 (scale[i] fp16 [N, K/128]).  residual (in place),
+ *   gate and normed_out may be null.  Every workgroup normalises its own copy of the
+ *   row; the in-place residual and normed_out are written by the workgroup that
+ *   arrives last at a per-stream device counter, after all others have read their
+ *   inputs.  Rows longer than 16384 fall back to mi_rmsnorm + the GEMV (normed_out
+ *   is then required).  Replaces the launch of esimd_resadd_norm_gemv_{int4,fp8}_pert,
+ *   esimd_resadd_norm_gemv2_fp8_pert, esimd_norm_gemv_{int4,fp8}_pert and
+ *   esimd_norm_gemv_fp8_blockscale (V/csrc/xpu/torch_extension.cc:103-133,
+ *   V/csrc/xpu/esimd_kernels/resadd_norm_gemv_fused.h:1-24, norm_gemv_fused.h). */
+int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* norm_weight,
+                 void* normed_out, int norm_len, float eps, int fmt, int nmat, const void* const* w,
+                 const void* const* scale, void* const* out, const int* N, int K, int act_dtype,
+                 void* stream);
+
 /* ---- MoE grouped FP8 block-scaled GEMM ----------------------------------------
  * out[r, :] = a[src(r), :] @ dequant(w[e])^T for the rows r of expert e,
  * expert_start[e] <= r < expert_start[e+1]; src(r) = row_map[r] if row_map else r.

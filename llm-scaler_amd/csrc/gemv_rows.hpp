@@ -52,6 +52,17 @@ struct RowsArgs {
   int nspan;                   // ceil(K / span_k)
   int total_waves;             // persistent grid size in wavefronts
   int scale_f16;
+  // Fused RMS norm of the activation row (NORM kernels, M == 1):
+  //   a = x (+ residual);  x' = a * rsqrt(mean_head(a^2) + eps) * weight[k % n_len] (* silu(gate))
+  // per head of n_len elements (n_len == K: the whole row).  The workgroup that
+  // arrives last writes `residual` (the rounded sum, in place) and `n_out`.
+  const void* n_res;
+  const void* n_gate;
+  const void* n_weight;
+  void* n_out;
+  unsigned int* n_arrive;      // zeroed counter; the kernel leaves it at zero again
+  int n_len;
+  float n_eps;
 };
 
 enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2, RF_Q40 = 3, RF_Q80 = 4, RF_Q5K = 5, RF_Q6K = 6 };
@@ -91,8 +102,10 @@ __device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_
 // weight loads of the next batch are in flight while the current one is
 // consumed (two register buffers).  Weight loads carry the non-temporal hint:
 // every byte is used exactly once.
-template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI, bool XREG>
+template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI, bool XREG,
+          bool NORM = false>
 __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
+  static_assert(!NORM || (MR == 1 && !XREG), "the fused norm stages one activation row through LDS");
   constexpr bool kFp8 = FMT == RF_FP8;
   constexpr bool kByte = rows_byte_fmt(FMT);
   constexpr bool kNib = !kByte;
@@ -111,6 +124,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   u32x4* xs = reinterpret_cast<u32x4*>(smem);        // [MR][pieces_per_row]
   float* c1 = reinterpret_cast<float*>(smem + (size_t)MR * pieces_per_row * 16);   // [MR][nspan*64]
   float* c2 = c1 + MR * nspan * 64;
+  float* nrm = reinterpret_cast<float*>(smem + (size_t)MR * pieces_per_row * 16 + (kByte ? 0 : (size_t)2 * MR * nspan * 64 * 4));   // NORM: [K/8] piece sums, [NWV] wave sums, flag
 
   const uint32_t wrow = kByte ? (uint32_t)K : ((uint32_t)K >> 1);
   const int nbatch = (nspan + SPU - 1) / SPU;        // batches per row group
@@ -317,6 +331,26 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 #pragma unroll
     for (int t = 0; t < XPRE; ++t) xpre[t] = buf_load16(xr, x_offset(threadIdx.x + t * NWV * 64));
   }
+  // NORM: residual, gate and norm weight of the same pieces (a null operand reads zeros)
+  u32x4 nres[NORM ? XPRE : 1], ngate[NORM ? XPRE : 1], nwgt[NORM ? XPRE : 1];
+  if constexpr (NORM) {
+    const __amdgpu_buffer_rsrc_t rr = make_rsrc(a.n_res, a.n_res ? (uint32_t)K * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t gr = make_rsrc(a.n_gate, a.n_gate ? (uint32_t)K * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t wr_n = make_rsrc(a.n_weight, (uint32_t)a.n_len * 2u);
+#pragma unroll
+    for (int t = 0; t < XPRE; ++t) {
+      nres[t] = ngate[t] = nwgt[t] = u32x4{0u, 0u, 0u, 0u};
+      if (t * NWV * 64 < total) {                     // uniform: this group of pieces exists
+        const uint32_t off = x_offset(threadIdx.x + t * NWV * 64);
+        const uint32_t k0 = (off & 0x7FFFFFFFu) >> 1;
+        const uint32_t kw = a.n_len == K ? k0 : k0 % (uint32_t)a.n_len;
+        nres[t] = buf_load16(rr, off);
+        ngate[t] = buf_load16(gr, off);
+        nwgt[t] = buf_load16(wr_n, (kw * 2u) | (off & 0x80000000u));
+      }
+    }
+  }
+  unsigned int n_prev = 0;                            // NORM: workgroups that arrived before this one
 
   auto advance = [&](int& g, int& sb) {
     if (++sb == nbatch) { sb = 0; g += stride; }
@@ -341,6 +375,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     }
   }
 
+  u32x4 res_new[NORM ? XPRE : 1], normed[NORM ? XPRE : 1];   // NORM: what the last workgroup writes back
   if constexpr (XREG) {
 #pragma unroll
     for (int m = 0; m < MR; ++m)
@@ -350,6 +385,108 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
         for (int i = 0; i < PPL; ++i) xreg[m][sp][i] = x_arrange(xreg[m][sp][i]);
         if constexpr (kSums) chunk_sums(xreg[m][sp], c1r[m][sp], c2r[m][sp]);
       }
+  } else if constexpr (NORM) {
+    using E = typename Act::elem;
+    const int V = a.n_len;
+    float av[XPRE][8];
+    float ssp[XPRE];
+#pragma unroll
+    for (int t = 0; t < XPRE; ++t) {
+      ssp[t] = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) av[t][e] = 0.f;
+      if (t * NWV * 64 >= total) continue;            // uniform
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const E h = __builtin_bit_cast(E, (uint16_t)(xpre[t][e >> 1] >> (16 * (e & 1))));
+        const E r = __builtin_bit_cast(E, (uint16_t)(nres[t][e >> 1] >> (16 * (e & 1))));
+        av[t][e] = Act::to_f32(h) + Act::to_f32(r);
+        ssp[t] += av[t][e] * av[t][e];
+      }
+    }
+    const bool whole = V == K;
+    if (whole) {
+      const float ws = wave_sum((ssp[0] + ssp[1]) + (ssp[2] + ssp[3]));
+      if (lane == 0) nrm[(K >> 3) + wave] = ws;
+    } else {
+#pragma unroll
+      for (int t = 0; t < XPRE; ++t) {
+        const int pidx = threadIdx.x + t * NWV * 64;
+        const uint32_t off = x_offset(pidx);
+        if (!(off >> 31)) nrm[(off >> 4)] = ssp[t];   // natural piece index k0 / 8
+      }
+    }
+    __syncthreads();                                  // every thread has consumed its loads
+    // Arrival count: whoever comes last knows that all workgroups hold their copy of the
+    // row in registers, and may overwrite the residual.  The final count is looked at only
+    // at the end of the kernel.
+    // Relaxed is enough: the barrier above already orders every thread's (completed) loads
+    // before the increment, the last workgroup reads nothing the others wrote, and its
+    // stores depend on the value it gets back.  A release / acquire pair would add cache
+    // write-backs and a wait for every load in flight.
+    // Two levels keep the chain of same-address read-modify-writes short (each takes tens of
+    // nanoseconds at the memory side): 16 counters by workgroup index, then one on top.
+    if (threadIdx.x == 0) {
+      const unsigned int sub = blockIdx.x & 15u;
+      const unsigned int members = (gridDim.x - sub + 15u) >> 4;
+      unsigned int* c1p = a.n_arrive + sub * 16u;       // 64 bytes apart
+      const unsigned int p1 = __hip_atomic_fetch_add(c1p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      n_prev = 0xFFFFFFFFu;
+      if (p1 == members - 1) {                          // last of its group: report to the top counter
+        __hip_atomic_store(c1p, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        n_prev = __hip_atomic_fetch_add(a.n_arrive + 256, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    float wtot = 0.f;
+    if (whole) {
+#pragma unroll
+      for (int w = 0; w < NWV; ++w) wtot += nrm[(K >> 3) + w];
+    }
+#pragma unroll
+    for (int t = 0; t < XPRE; ++t) {
+      if (t * NWV * 64 >= total) continue;
+      const uint32_t off = x_offset(threadIdx.x + t * NWV * 64);
+      float tot = wtot;
+      if (!whole) {
+        tot = 0.f;
+        const int k0 = (int)((off & 0x7FFFFFFFu) >> 1);
+        const int hp = (k0 / V) * (V >> 3);
+        if (!(off >> 31))
+          for (int jj = 0; jj < (V >> 3); ++jj) tot += nrm[hp + jj];
+      }
+      const float inv = rsqrtf(tot / (float)V + a.n_eps);
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        uint32_t rw = 0, nw = 0;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const int e = e2 * 2 + h2;
+          const E wv = __builtin_bit_cast(E, (uint16_t)(nwgt[t][e2] >> (16 * h2)));
+          float v = av[t][e] * inv * Act::to_f32(wv);
+          if (a.n_gate) {
+            const float z = Act::to_f32(__builtin_bit_cast(E, (uint16_t)(ngate[t][e2] >> (16 * h2))));
+            v *= z / (1.0f + __expf(-z));
+          }
+          rw |= (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(av[t][e])) << (16 * h2);
+          nw |= (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(v)) << (16 * h2);
+        }
+        res_new[t][e2] = rw;
+        normed[t][e2] = nw;
+      }
+      x_store(threadIdx.x + t * NWV * 64, normed[t]);
+    }
+    if constexpr (kSums) {
+      __syncthreads();
+      const int chunks = nspan * 64;
+      for (int c = threadIdx.x; c < chunks; c += NWV * 64) {
+        const int s = c >> 6, l = c & 63;
+        u32x4 pc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pc[i] = xs[(s * 4 + i) * 64 + l];
+        chunk_sums(pc, c1[c], c2[c]);
+      }
+    }
+    __syncthreads();
   } else {
 #pragma unroll
     for (int t = 0; t < XPRE; ++t) x_store(threadIdx.x + t * NWV * 64, xpre[t]);
@@ -552,6 +689,27 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       if (sq[i] == nbatch - 1) finish(buf[i], gq[i]);
     }
   }
+  if constexpr (NORM) {
+    float* flag = nrm + (K >> 3) + NWV;
+    if (threadIdx.x == 0) {
+      const unsigned int groups = gridDim.x < 16u ? gridDim.x : 16u;
+      const bool last = n_prev == groups - 1;
+      if (last) __hip_atomic_store(a.n_arrive + 256, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *flag = last ? 1.0f : 0.0f;
+    }
+    __syncthreads();
+    if (*flag != 0.0f) {
+#pragma unroll
+      for (int t = 0; t < XPRE; ++t) {
+        if (t * NWV * 64 >= total) continue;
+        const uint32_t off = x_offset(threadIdx.x + t * NWV * 64);
+        if (!(off >> 31)) {
+          if (a.n_res) *reinterpret_cast<u32x4*>((char*)const_cast<void*>(a.n_res) + off) = res_new[t];
+          if (a.n_out) *reinterpret_cast<u32x4*>((char*)a.n_out + off) = normed[t];
+        }
+      }
+    }
+  }
 #undef QLIN_PICK
 }
 
@@ -565,6 +723,12 @@ static inline size_t rows_lds_bytes(int fmt, int MR, int K) {
   return b;
 }
 
+// extra LDS of the fused norm: one partial sum per 8-k piece, one per wavefront, one flag
+static inline size_t rows_norm_lds_bytes(int K) { return ((size_t)(K >> 3) + 16) * 4; }
+
+// rows the fused norm can stage: XPRE (4) pieces of 8 k per thread, 512 threads
+constexpr int kRowsNormMaxK = 4 * 512 * 8;
+
 static inline int device_cu_count() {
   static int cus = 0;
   if (!cus) {
@@ -577,7 +741,7 @@ static inline int device_cu_count() {
   return cus;
 }
 
-template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG>
+template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG, bool NORM = false>
 static void launch_rows_rw(RowsArgs a, hipStream_t st) {
   constexpr int NWV = 8;
   constexpr int NBUF = 2;
@@ -600,12 +764,12 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st) {
   const int needed = (groups + NWV - 1) / NWV;
   const int wgs = needed < best_wgs ? needed : best_wgs;
   a.total_waves = wgs * NWV;
-  const size_t lds = XREG ? 0 : rows_lds_bytes(FMT, MR, a.K);
+  const size_t lds = XREG ? 0 : rows_lds_bytes(FMT, MR, a.K) + (NORM ? rows_norm_lds_bytes(a.K) : 0);
   if (a.nmat == 1)
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false, XREG>), dim3(wgs),
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false, XREG, NORM>), dim3(wgs),
                        dim3(NWV * 64), lds, st, a);
   else
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG>), dim3(wgs),
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG, NORM>), dim3(wgs),
                        dim3(NWV * 64), lds, st, a);
 }
 
@@ -637,6 +801,23 @@ static void launch_rows(RowsArgs a, hipStream_t st) {
     if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, RW4, SPU, true>(a, st); }
     launch_rows_rw<Act, FMT, SC, MR, RW4, SPU, false>(a, st);
   }
+}
+
+// M == 1 with the RMS norm fused into the activation staging (LDS path).
+template <class Act, int FMT, int SC>
+static void launch_rows_norm(RowsArgs a, hipStream_t st) {
+  constexpr bool kByte = rows_byte_fmt(FMT);
+  constexpr int ppl = kByte ? 2 : 4;
+  constexpr int span_k = 64 * ppl * 8;
+  constexpr int SPU = kByte ? 4 : 2;
+  a.nspan = (a.K + span_k - 1) / span_k;
+  const int per_batch = a.nspan < SPU ? a.nspan : SPU;
+  if (per_batch >= 4)
+    launch_rows_rw<Act, FMT, SC, 1, 1, SPU, false, true>(a, st);
+  else if (per_batch >= 2)
+    launch_rows_rw<Act, FMT, SC, 1, 2, SPU, false, true>(a, st);
+  else
+    launch_rows_rw<Act, FMT, SC, 1, 4, SPU, false, true>(a, st);
 }
 
 template <class Act, int FMT, int SC>

@@ -1,0 +1,63 @@
+// RMS norm (+ residual add, + SiLU gate) fused into the decode GEMV.
+//
+// One launch: every workgroup of the one-wavefront-per-row GEMV normalises the
+// activation row itself while it stages it in LDS (the row is a few KiB and sits
+// in L2), so the GEMV does not wait for a separate norm kernel.  The in-place
+// residual update and the normalised row are written by the workgroup that
+// arrives last at a device-wide counter: by then every workgroup holds its copy
+// of the inputs in registers, so no workgroup can read a half-updated residual.
+// Rows too long for the staging registers take the two-kernel route.
+#include "gemv_rows.hpp"
+#include "scratch.hpp"
+#include "../../include/mi355x_qlinear.h"
+
+using namespace qlin;
+
+extern "C" {
+
+int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
+                 int norm_len, float eps, int fmt, int nmat, const void* const* w, const void* const* scale,
+                 void* const* out, const int* N, int K, int act_dtype, void* stream) {
+  if (!x || !norm_weight || !w || !scale || !out || !N) return MI_ERR_ARG;
+  if (nmat < 1 || nmat > kRowsMaxMat) return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (fmt < 0 || fmt > 2) return MI_ERR_ARG;
+  if (K <= 0 || norm_len <= 0 || (norm_len % 8) || (K % norm_len)) return MI_ERR_SHAPE;
+  if (fmt == 0 ? (K % 16) : (K % 128)) return MI_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  RowsArgs r{};
+  r.x = x; r.nmat = nmat; r.M = 1; r.K = K; r.scale_f16 = 0;
+  for (int i = 0; i < nmat; ++i) {
+    if (!w[i] || !scale[i] || !out[i] || N[i] < 0) return MI_ERR_ARG;
+    if ((uint64_t)N[i] * (uint64_t)K >= (1ull << 31)) return MI_ERR_SHAPE;
+    r.w[i] = w[i]; r.s[i] = scale[i]; r.out[i] = out[i]; r.N[i] = N[i];
+  }
+  const int rfmt = fmt == 2 ? RF_INT4 : RF_FP8;
+  const bool fused = K <= kRowsNormMaxK && rows_lds_bytes(rfmt, 1, K) + rows_norm_lds_bytes(K) <= 64 * 1024;
+  if (!fused) {
+    // two kernels: the norm writes the row (into normed_out, or over x's scratch copy), then the GEMV
+    if (!normed_out) return MI_ERR_ARG;
+    const int rc = mi_rmsnorm(x, residual, gate, norm_weight, normed_out, K / norm_len, norm_len, norm_len, eps,
+                              act_dtype, stream);
+    if (rc != MI_OK) return rc;
+    const float* const* fs = reinterpret_cast<const float* const*>(scale);
+    if (fmt == 0) return mi_gemm_fp8_pert_multi(normed_out, nmat, w, fs, out, N, 1, K, act_dtype, stream);
+    if (fmt == 1) return mi_gemm_fp8_blockscale_multi(normed_out, nmat, w, fs, out, N, 1, K, act_dtype, stream);
+    return mi_gemv_int4_multi(normed_out, nmat, w, scale, nullptr, out, N, 1, K, act_dtype, stream);
+  }
+  r.n_res = residual; r.n_gate = gate; r.n_weight = norm_weight; r.n_out = normed_out;
+  r.n_len = norm_len; r.n_eps = eps;
+  r.n_arrive = arrival_counter_get(st);
+  if (!r.n_arrive) return MI_ERR_LAUNCH;
+  const bool f16 = act_dtype == DT_F16;
+  if (fmt == 0) {
+    if (f16) launch_rows_norm<ActF16, RF_FP8, RS_PERT>(r, st); else launch_rows_norm<ActBF16, RF_FP8, RS_PERT>(r, st);
+  } else if (fmt == 1) {
+    if (f16) launch_rows_norm<ActF16, RF_FP8, RS_BLOCK>(r, st); else launch_rows_norm<ActBF16, RF_FP8, RS_BLOCK>(r, st);
+  } else {
+    if (f16) launch_rows_norm<ActF16, RF_INT4, RS_PERN>(r, st); else launch_rows_norm<ActBF16, RF_INT4, RS_PERN>(r, st);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -13,6 +13,7 @@ struct Buf {
 };
 std::mutex g_mu;
 std::map<std::pair<int, hipStream_t>, Buf> g_bufs;
+std::map<std::pair<int, hipStream_t>, unsigned int*> g_counters;
 }  // namespace
 
 void* scratch_get(hipStream_t stream, size_t bytes) {
@@ -29,6 +30,19 @@ void* scratch_get(hipStream_t stream, size_t bytes) {
   b.p = p;
   b.bytes = want;
   return p;
+}
+
+unsigned int* arrival_counter_get(hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  std::lock_guard<std::mutex> lock(g_mu);
+  unsigned int*& c = g_counters[{dev, stream}];
+  if (c) return c;
+  void* p = nullptr;
+  if (hipMalloc(&p, 2048) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  if (hipMemset(p, 0, 2048) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(p); return nullptr; }
+  c = static_cast<unsigned int*>(p);
+  return c;
 }
 
 }  // namespace qlin

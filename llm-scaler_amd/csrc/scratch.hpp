@@ -20,4 +20,9 @@ namespace qlin {
 // nullptr when the allocation fails (e.g. under stream capture)
 void* scratch_get(hipStream_t stream, size_t bytes);
 
+// A zero-initialised block of 512 32-bit counters per (device, stream) for kernels that
+// count arriving workgroups and leave the counters at zero again when they finish.
+// Allocated and cleared on first use (not under stream capture); nullptr on failure.
+unsigned int* arrival_counter_get(hipStream_t stream);
+
 }  // namespace qlin

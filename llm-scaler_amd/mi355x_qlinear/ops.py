@@ -925,66 +925,112 @@ def esimd_rms_norm(input, output, weight, eps):
     return _rmsnorm(input, None, None, weight, output, input.numel() // K, K, eps, "esimd_rms_norm")
 
 
+_NORM_FP8_PERT, _NORM_FP8_BLOCK, _NORM_INT4 = 0, 1, 2
+
+
+def _norm_gemv(x, residual, gate, norm_weight, normed_out, norm_len, eps, fmt, ws, ss, outs, who):
+    """One launch: RMS norm (+ residual add / SiLU gate) of the single activation row, fused
+    into the decode GEMV over `ws`.  More than one row takes the norm kernel + GEMV route."""
+    _chk(x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(), f"{who}: activations must be contiguous fp16/bf16")
+    for name, t in (("residual", residual), ("gate", gate), ("norm_weight", norm_weight), ("normed output", normed_out)):
+        if t is not None:
+            _chk(t.dtype == x.dtype and t.is_contiguous() and t.device == x.device,
+                 f"{who}: {name} must match the input's dtype/device and be contiguous")
+    if fmt == _NORM_INT4:
+        K = ws[0].shape[1] * (2 if ws[0].dtype == torch.uint8 else 8)
+    else:
+        K = ws[0].shape[1]
+    _chk(x.numel() % K == 0, f"{who}: input numel {x.numel()} is not a multiple of K={K}")
+    rows = x.numel() // K
+    norm_len = int(norm_len)
+    _chk(norm_weight.numel() == norm_len and K % norm_len == 0, f"{who}: norm_weight must have {norm_len} entries dividing K={K}")
+    for t in (residual, gate):
+        if t is not None:
+            _chk(t.numel() == x.numel(), f"{who}: residual / gate must have the input's size")
+    if normed_out is not None:
+        _chk(normed_out.numel() >= x.numel(), f"{who}: normed output is too small")
+    if rows != 1:
+        normed = normed_out if normed_out is not None else torch.empty_like(x)
+        _rmsnorm(x, residual, gate, norm_weight, normed, x.numel() // norm_len, norm_len, eps, who)
+        xin = normed.view(rows, K)
+        if fmt == _NORM_INT4:
+            return _int4_multi(xin, ws, ss, [None] * len(ws), outs, who)
+        if fmt == _NORM_FP8_PERT:
+            return _fp8_pert_multi(xin, ws, ss, outs, who)
+        return esimd_gemm_fp8_blockscale(xin, ws[0], ss[0], outs[0], 128, 128)
+    Ns = []
+    for w, sc, o in zip(ws, ss, outs):
+        _chk(w.dim() == 2 and w.is_contiguous(), f"{who}: weights must be contiguous 2-D tensors")
+        _chk_act(x, o, who)
+        if fmt == _NORM_INT4:
+            _chk(w.dtype in (torch.uint8, torch.int32), f"{who}: int4 weight must be uint8 [N, K/2] or int32 [N, K/8]")
+            _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+            _chk(sc.dtype == torch.float16 and sc.is_contiguous() and sc.numel() == w.shape[0] * (K // 128),
+                 f"{who}: gemv_scale must be contiguous fp16 [N, K/128]")
+        else:
+            _chk_fp8(w, who)
+            _chk(w.shape[1] == K, f"{who}: all weights must be [N, K={K}]")
+            if fmt == _NORM_FP8_PERT:
+                _chk(sc.dtype == torch.float32 and sc.numel() >= 1, f"{who}: gemv_scale must be an fp32 scalar tensor")
+            else:
+                _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+                _chk(sc.dtype == torch.float32 and sc.is_contiguous() and sc.numel() == -(-w.shape[0] // 128) * (K // 128),
+                     f"{who}: gemv_scale must be contiguous fp32 [ceil(N/128), K/128]")
+        _chk(o.numel() == w.shape[0], f"{who}: output has {o.numel()} elements, expected N={w.shape[0]}")
+        Ns.append(w.shape[0])
+    capi.call("mi_norm_gemv", x, capi.ptr(x), capi.ptr(residual), capi.ptr(gate), capi.ptr(norm_weight),
+              capi.ptr(normed_out), norm_len, float(eps), fmt, len(ws), capi.ptr_array(ws), capi.ptr_array(ss),
+              capi.ptr_array(outs), capi.int_array(Ns), K, capi.act_dtype(x))
+    return outs[0]
+
+
 def esimd_resadd_norm_gemv_int4_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
                                      normed_out, eps):
     """residual += hidden_states (in place); normed_out = rmsnorm(residual) * norm_weight;
     output = normed_out @ dequant(int4 weight)^T  (resadd_norm_gemv_int4.h:1-30)."""
-    who = "esimd_resadd_norm_gemv_int4_pert"
     K = hidden_states.shape[-1]
-    rows = hidden_states.numel() // K
-    _rmsnorm(hidden_states, residual, None, norm_weight, normed_out, rows, K, eps, who)
-    esimd_gemv_int4(normed_out.view(rows, K), gemv_weight, gemv_scale, output)
-    return output
+    return _norm_gemv(hidden_states, residual, None, norm_weight, normed_out, K, eps, _NORM_INT4,
+                      [gemv_weight], [gemv_scale], [output], "esimd_resadd_norm_gemv_int4_pert")
 
 
 def esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
                                     normed_out, eps):
     """Same with an FP8 weight and a per-tensor scale (resadd_norm_gemv_fused.h)."""
-    who = "esimd_resadd_norm_gemv_fp8_pert"
     K = hidden_states.shape[-1]
-    rows = hidden_states.numel() // K
-    _rmsnorm(hidden_states, residual, None, norm_weight, normed_out, rows, K, eps, who)
-    esimd_gemv_fp8_pert(normed_out.view(rows, K), gemv_weight, gemv_scale, output)
-    return output
+    return _norm_gemv(hidden_states, residual, None, norm_weight, normed_out, K, eps, _NORM_FP8_PERT,
+                      [gemv_weight], [gemv_scale], [output], "esimd_resadd_norm_gemv_fp8_pert")
 
 
 def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps):
     """Residual add + RMS norm feeding two per-tensor FP8 GEMVs in one launch (resadd_norm_gemv2_fused.h)."""
-    who = "esimd_resadd_norm_gemv2_fp8_pert"
     K = hidden_states.shape[-1]
-    rows = hidden_states.numel() // K
-    normed = torch.empty_like(hidden_states)
-    _rmsnorm(hidden_states, residual, None, norm_weight, normed, rows, K, eps, who)
-    esimd_gemv_fp8_pert_fused2(normed.view(rows, K), w0, s0, o0, w1, s1, o1)
-    return o0
+    return _norm_gemv(hidden_states, residual, None, norm_weight, None, K, eps, _NORM_FP8_PERT,
+                      [w0, w1], [s0, s1], [o0, o1], "esimd_resadd_norm_gemv2_fp8_pert")
 
 
-def _gated_norm(x, z, norm_weight, HV, V, eps, who):
+def _gated_norm_gemv(x, z, norm_weight, HV, V, eps, fmt, weight, scale, output, who):
     HV, V = int(HV), int(V)
     _chk(x.numel() % (HV * V) == 0 and z.numel() == x.numel(), f"{who}: x and z must hold HV*V elements per row")
     _chk(norm_weight.numel() == V, f"{who}: norm_weight must have V entries")
-    normed = torch.empty_like(x)
-    _rmsnorm(x, None, z, norm_weight, normed, x.numel() // V, V, eps, who)
-    return normed.view(-1, HV * V)
+    return _norm_gemv(x, None, z, norm_weight, None, V, eps, fmt, [weight], [scale], [output], who)
 
 
 def esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
     """Per-head RMS norm gated by silu(z), then INT4 GEMV over the HV*V vector (norm_gemv_int4.h)."""
-    esimd_gemv_int4(_gated_norm(x, z, norm_weight, HV, V, eps, "esimd_norm_gemv_int4_pert"), gemv_weight, gemv_scale, output)
-    return output
+    return _gated_norm_gemv(x, z, norm_weight, HV, V, eps, _NORM_INT4, gemv_weight, gemv_scale, output,
+                            "esimd_norm_gemv_int4_pert")
 
 
 def esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
     """Per-head gated RMS norm, then per-tensor FP8 GEMV (norm_gemv_fused.h)."""
-    esimd_gemv_fp8_pert(_gated_norm(x, z, norm_weight, HV, V, eps, "esimd_norm_gemv_fp8_pert"), gemv_weight, gemv_scale, output)
-    return output
+    return _gated_norm_gemv(x, z, norm_weight, HV, V, eps, _NORM_FP8_PERT, gemv_weight, gemv_scale, output,
+                            "esimd_norm_gemv_fp8_pert")
 
 
 def esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
     """Per-head gated RMS norm, then 128x128 block-scaled FP8 GEMV (torch_extension_gemm.cc:42-45)."""
-    esimd_gemm_fp8_blockscale(_gated_norm(x, z, norm_weight, HV, V, eps, "esimd_norm_gemv_fp8_blockscale"),
-                              gemv_weight, gemv_scale, output, 128, 128)
-    return output
+    return _gated_norm_gemv(x, z, norm_weight, HV, V, eps, _NORM_FP8_BLOCK, gemv_weight, gemv_scale, output,
+                            "esimd_norm_gemv_fp8_blockscale")
 
 
 # --------------------------------------------------------------------------

@@ -501,3 +501,51 @@ def test_fp8_pert_fused_distinct_scales(ops, dev):
     o2 = [torch.empty_like(outs[0]), torch.empty_like(outs[1])]
     v.esimd_gemv_fp8_pert_fused2(x.to(dev), f8(ws[0]), ss[0].to(dev), o2[0], f8(ws[1]), ss[1].to(dev), o2[1])
     assert torch.equal(o2[0], outs[0]) and torch.equal(o2[1], outs[1])
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,K", [(14336, 4096), (5000, 16384), (520, 20480), (3000, 1024)])
+def test_resadd_norm_gemv_many_workgroups_and_repeats(ops, dev, dt, N, K):
+    """Fused launch on a full grid, three calls in a row on the same buffers: the arrival
+    counter must come back to zero each time and the residual must be updated exactly once
+    per call.  K = 20480 exceeds the fused staging and takes the norm kernel + GEMV route."""
+    v, _ = ops
+    g = torch.Generator().manual_seed(N + K)
+    eps = 1e-6
+    hidden = (torch.randn(1, K, generator=g) * 0.5).to(dt)
+    residual = torch.randn(1, K, generator=g).to(dt)
+    nw = (torch.randn(K, generator=g) * 0.1 + 1.0).to(dt)
+    w8 = O.e4m3_quantize((torch.randn(N, K, generator=g) * 100).clamp(-448, 448))
+    sc = torch.tensor([1.0e-3])
+    wd = O.fp8_dequant_per_tensor(w8, sc)
+    out = torch.empty(1, N, dtype=dt, device=dev)
+    normed_out = torch.empty(1, K, dtype=dt, device=dev)
+    res_d = residual.to(dev).clone()
+    hd, nwd, wdv, scd = hidden.to(dev), nw.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev)
+    res_ref = residual
+    for _ in range(3):
+        v.esimd_resadd_norm_gemv_fp8_pert(hd, res_d, nwd, wdv, scd, out, normed_out, eps)
+        normed_ref, res_ref = O.rmsnorm(hidden, nw, eps, residual=res_ref)
+        assert torch.equal(res_d.cpu().view(torch.int16), res_ref.view(torch.int16))
+        assert _ulp_close(normed_out.cpu().float(), normed_ref, dt)
+        assert O.max_rel_err(out.cpu(), O.matmul_ref(normed_out.cpu(), wd)) < TOL
+
+
+def test_norm_gemv_several_rows(ops, dev):
+    # more than one activation row: the norm kernel + GEMV route, same results
+    v, _ = ops
+    g = torch.Generator().manual_seed(77)
+    rows, K, N, eps = 3, 1024, 200, 1e-6
+    hidden = torch.randn(rows, K, generator=g).half()
+    residual = torch.randn(rows, K, generator=g).half()
+    nw = (torch.randn(K, generator=g) * 0.1 + 1.0).half()
+    _, packed, scale, _ = O.make_int4_case(1, K, N, seed=9)
+    out = torch.empty(rows, N, dtype=torch.float16, device=dev)
+    normed_out = torch.empty(rows, K, dtype=torch.float16, device=dev)
+    res_d = residual.to(dev).clone()
+    v.esimd_resadd_norm_gemv_int4_pert(hidden.to(dev), res_d, nw.to(dev), packed.to(dev), scale.to(dev), out, normed_out, eps)
+    normed_ref, res_ref = O.rmsnorm(hidden, nw, eps, residual=residual)
+    assert torch.equal(res_d.cpu().view(torch.int16), res_ref.view(torch.int16))
+    assert _ulp_close(normed_out.cpu().float(), normed_ref, torch.float16)
+    wd = O.int4_dequant(packed, scale, out_dtype=torch.float16)
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(normed_out.cpu(), wd)) < TOL
