@@ -69,6 +69,10 @@ enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2, RF_Q40 = 3, RF_Q80 = 4, RF_Q5K
 constexpr bool rows_byte_fmt(int fmt) { return fmt == RF_FP8 || fmt == RF_Q80; }   // one byte per weight
 enum : int { RS_PERN = 0, RS_PERT = 1, RS_BLOCK = 2 };
 
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+
 template <class Act> struct Dot2;
 template <> struct Dot2<ActF16> {
   static __device__ __forceinline__ float run(uint32_t a, uint32_t b, float c) {
@@ -134,8 +138,11 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   struct Batch {                                     // one batch = RW rows x SPU spans
     u32x4 w[RW][SPU];
     u32x4 h[RW][SPU][kHigh ? 2 : 1];   // the lane's 32 high-bit bytes (Q5_K / Q6_K)
-    float s[RW][SPU];          // per-lane scale of the chunk (int4 group / q4k sub-block / fp8 block)
-    float z[RW][SPU];          // int4 zero-point / q4k min
+    // per-lane side data of the chunk, kept as the raw loaded bits: converting here would
+    // make the load's first use sit right behind it, and a wait for one load is a wait for
+    // every older load in flight (the previous batch's weights)
+    uint32_t s[RW][SPU];       // scale: fp16 bits (int4 group, GGUF sub-block; Q6_K: two), fp32 bits (fp8 block)
+    uint32_t z[RW][SPU];       // int4 zero-point byte / Q4_K, Q5_K min fp16 bits
     uint32_t os_lo[RW], os_hi[RW];   // fp8 per-channel scale of the row, raw halves (fp32 or fp16)
   };
 
@@ -166,7 +173,9 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     const _Float16* s16 = (const _Float16*)QLIN_PICK(s, mat);
     const float* s32 = (const float*)QLIN_PICK(s, mat);
     const uint8_t* zp = (const uint8_t*)QLIN_PICK(z, mat);
-    const _Float16* qmin = (const _Float16*)QLIN_PICK(z, mat);
+    const uint16_t* qminu = (const uint16_t*)QLIN_PICK(z, mat);
+    const uint16_t* s16u = reinterpret_cast<const uint16_t*>(s16);
+    const uint8_t* zsrc = zp ? zp : reinterpret_cast<const uint8_t*>(s16);   // always a readable address
     if constexpr (kFp8 && SC == RS_PERN) {
 #pragma unroll
       for (int r = 0; r < RW; ++r) {
@@ -191,30 +200,30 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
           const int Kg = K >> 7;
           int gi = chunk >> 2;
           gi = gi < Kg ? gi : Kg - 1;
-          b.s[r][sp] = (float)s16[(size_t)nc * Kg + gi];
-          b.z[r][sp] = zp ? (float)zp[(size_t)nc * Kg + gi] : 8.0f;
+          b.s[r][sp] = s16u[(size_t)nc * Kg + gi];
+          b.z[r][sp] = zsrc[(size_t)nc * Kg + gi];      // no zero-points: a dummy byte, replaced by 8 at use
         } else if constexpr (FMT == RF_Q4K || FMT == RF_Q5K) {
           const int Kc = K >> 5;
           const int ci = chunk < Kc ? chunk : Kc - 1;
-          b.s[r][sp] = (float)s16[(size_t)nc * Kc + ci];
-          b.z[r][sp] = (float)qmin[(size_t)nc * Kc + ci];
+          b.s[r][sp] = s16u[(size_t)nc * Kc + ci];
+          b.z[r][sp] = qminu[(size_t)nc * Kc + ci];
         } else if constexpr (FMT == RF_Q40) {
           const int Kc = K >> 5;
           const int ci = chunk < Kc ? chunk : Kc - 1;
-          b.s[r][sp] = (float)s16[(size_t)nc * Kc + ci];
+          b.s[r][sp] = s16u[(size_t)nc * Kc + ci];
         } else if constexpr (FMT == RF_Q6K) {
           // the lane's 32 k span two 16-wide groups: both fp16 scales in one 32-bit load
           const int Kc = K >> 5;
           const int ci = chunk < Kc ? chunk : Kc - 1;
-          b.s[r][sp] = reinterpret_cast<const float*>(s16)[(size_t)nc * Kc + ci];
+          b.s[r][sp] = reinterpret_cast<const uint32_t*>(s16)[(size_t)nc * Kc + ci];
         } else if constexpr (FMT == RF_Q80) {
           const int Kc = K >> 5;
           const int c8 = (s * SPAN_K + lane * 16) >> 5;
-          b.s[r][sp] = (float)s16[(size_t)nc * Kc + (c8 < Kc ? c8 : Kc - 1)];
+          b.s[r][sp] = s16u[(size_t)nc * Kc + (c8 < Kc ? c8 : Kc - 1)];
         } else if constexpr (SC == RS_BLOCK) {
           const int Kb = (K + 127) >> 7;
           const int kblk = (s * SPAN_K + lane * 16) >> 7;
-          b.s[r][sp] = s32[(size_t)(nc >> 7) * Kb + (kblk < Kb ? kblk : Kb - 1)];
+          b.s[r][sp] = reinterpret_cast<const uint32_t*>(s32)[(size_t)(nc >> 7) * Kb + (kblk < Kb ? kblk : Kb - 1)];
         }
       }
     }
@@ -365,6 +374,8 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     load_batch(buf[i], g_next, sb_next);
     advance(g_next, sb_next);
   }
+  // nothing below may be scheduled above the prefetch: the weight loads go out first
+  __builtin_amdgcn_sched_barrier(0);
   // one per-tensor scale per fused matrix (scalars, so they stay in registers)
   float pert0 = 1.0f, pert1 = 1.0f, pert2 = 1.0f;
   if constexpr (kFp8 && SC == RS_PERT) {
@@ -515,11 +526,15 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
 
+  const bool has_zp = FMT == RF_INT4 && a.z[0] != nullptr;   // zero-points come for all matrices or for none
   auto compute = [&](const Batch& b, int sb) {
 #pragma unroll
     for (int sp = 0; sp < SPU; ++sp) {
       const int s = sb * SPU + sp;
-      if (s < nspan) {                                // wave-uniform
+      // wave-uniform.  With the activations in registers a span past the row's end holds
+      // zero weights and zero activations and is simply computed: the loop body then has
+      // no branches, which keeps the wait counts of the loads in flight exact.
+      if (XREG || s < nspan) {
         u32x4 xp[MR][PPL];
 #pragma unroll
         for (int m = 0; m < MR; ++m)
@@ -547,7 +562,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
             }
             if constexpr (SC == RS_BLOCK) {
 #pragma unroll
-              for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * b.s[r][sp];
+              for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * __builtin_bit_cast(float, b.s[r][sp]);
             } else {
 #pragma unroll
               for (int m = 0; m < MR; ++m) acc[r][m] += part[m];
@@ -569,7 +584,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
               }
             }
 #pragma unroll
-            for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * b.s[r][sp];
+            for (int m = 0; m < MR; ++m) acc[r][m] += part[m] * f16_bits_to_f32(b.s[r][sp]);
           } else {
             float part_hi[MR];                       // Q6_K: second 16-wide group of the lane
 #pragma unroll
@@ -622,14 +637,16 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
               }
             }
             if constexpr (FMT == RF_Q6K) {
-              const uint32_t two = __builtin_bit_cast(uint32_t, b.s[r][sp]);
-              const float s_lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(two & 0xFFFFu));
-              const float s_hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(two >> 16));
+              const uint32_t two = b.s[r][sp];
+              const float s_lo = f16_bits_to_f32(two & 0xFFFFu);
+              const float s_hi = f16_bits_to_f32(two >> 16);
 #pragma unroll
               for (int m = 0; m < MR; ++m) acc[r][m] += s_lo * part[m] + s_hi * part_hi[m];
             }
-            const float sc = b.s[r][sp];
-            const float zz = FMT == RF_Q40 ? 8.0f * sc : b.z[r][sp];
+            const float sc = f16_bits_to_f32(b.s[r][sp]);
+            const float zz = FMT == RF_Q40    ? 8.0f * sc
+                             : FMT == RF_INT4 ? (has_zp ? (float)b.z[r][sp] : 8.0f)
+                                              : f16_bits_to_f32(b.z[r][sp]);
 #pragma unroll
             for (int m = 0; m < (FMT == RF_Q6K ? 0 : MR); ++m) {
               float k1, k2;
@@ -650,8 +667,16 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     }
   };
 
-  // finish the K reduction inside the wavefront, lane 0 stores, accumulators reset
+  // finish the K reduction inside the wavefront, lane 0 stores, accumulators reset.
+  // The stored values keep their registers until the next batch's loads have been issued
+  // (see the loop): stores and loads retire through one in-order counter, so reusing a
+  // store's data register any earlier would make the compiler wait for every load in flight.
   using Elem = typename Act::elem;
+  uint32_t stored[RW][MR];
+#pragma unroll
+  for (int r = 0; r < RW; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) stored[r][m] = 0u;
   auto finish = [&](const Batch& b, int g) {
     int mat, row0;
     locate(g, mat, row0);
@@ -669,24 +694,37 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       for (int m = 0; m < MR; ++m) {
         const float v = wave_sum(acc[r][m]);
         acc[r][m] = 0.f;
-        if (lane == 0 && n < N && m < M) out[(size_t)m * N + n] = Act::from_f32(v * os);
+        stored[r][m] = (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(v * os));
+        asm volatile("" : "+v"(stored[r][m]));        // the store below reads exactly this register
+        if (lane == 0 && n < N && m < M)
+          out[(size_t)m * N + n] = __builtin_bit_cast(Elem, (uint16_t)stored[r][m]);
       }
     }
   };
 
   // ---- walk the wave's batches; buffer indices are static after unrolling ----
-  bool more = true;
-  while (more) {
+  // Both halves of a ring turn always issue their loads (a batch past the end loads
+  // nothing) and the only way out is at the bottom: an exit in the middle would reach the
+  // loop header with the other slot's loads still in flight, and the compiler would then
+  // have to drain every load there on every turn.
+  while (gq[0] < ngroups) {
 #pragma unroll
     for (int i = 0; i < NBUF; ++i) {
-      constexpr int dummy = 0; (void)dummy;
       const int j = (i + NBUF - 1) % NBUF;
       gq[j] = g_next; sq[j] = sb_next;
       load_batch(buf[j], g_next, sb_next);
+      // the next batch's loads are issued before the current batch is consumed: without
+      // the fence the compiler rotates the loop (compute first), which halves the prefetch
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) asm volatile("" ::"v"(stored[r][m]));
       advance(g_next, sb_next);
-      if (gq[i] >= ngroups) { more = false; break; }
-      compute(buf[i], sq[i]);
-      if (sq[i] == nbatch - 1) finish(buf[i], gq[i]);
+      if (gq[i] < ngroups) {                          // uniform; rejoins before the next loads
+        compute(buf[i], sq[i]);
+        if (sq[i] == nbatch - 1) finish(buf[i], gq[i]);
+      }
     }
   }
   if constexpr (NORM) {

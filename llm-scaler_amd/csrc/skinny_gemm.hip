@@ -344,6 +344,7 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
   if (FMT == 2 && (a.K % 32)) return MI_ERR_SHAPE;
   for (int i = 0; i < a.nmat; ++i) {
     if (a.N[i] < 0 || !a.w[i] || !a.out[i]) return MI_ERR_ARG;
+    if (FMT == 1 && (a.z[i] != nullptr) != (a.z[0] != nullptr)) return MI_ERR_ARG;   // zero-points for all or none
     if ((uint64_t)a.N[i] * (uint64_t)a.K >= (1ull << 31)) return MI_ERR_SHAPE;
     a.tiles[i] = (a.N[i] + 15) / 16;
   }
