@@ -103,13 +103,26 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 
   // Out-of-range granules / lanes / rows load zeros for both operands, so the
   // loop body needs no branches: a zero weight times a zero activation adds 0.
-  for (int gbase = wave; gbase < G; gbase += NW * UN) {
-    u32x4 wa[UN][RT], wb[UN][RT];
-    u32x4 xa[UN][MT][4];
-    float sc[UN][RT];                                // int4 / q4k scale, block scale
-    float zz[UN][RT];
+  //
+  // A stage = U granules of this wavefront (gbase, gbase + NW, ...): their loads, and
+  // later their conversion + MFMAs.  With UN >= 2 the granules of a turn are split into
+  // two stages in a ring, so that the loads of the next stage are in flight while the
+  // current one is consumed (continuous streaming instead of load bursts).
+  constexpr int US = UN >= 2 ? UN / 2 : UN;           // granules per stage
+  struct Stage {
+    u32x4 wa[US][RT], wb[US][RT];
+    u32x4 xa[US][MT][4];
+    uint32_t sc[US][RT];                              // raw bits: int4 / q4k scale (fp16), block scale (fp32)
+    uint32_t zz[US][RT];                              // raw: int4 zero-point byte / q4k min (fp16)
+  };
+  const uint16_t* s16u = reinterpret_cast<const uint16_t*>(s16);
+  const uint16_t* qminu = reinterpret_cast<const uint16_t*>(qmin);
+  const uint8_t* zsrc = zp ? zp : reinterpret_cast<const uint8_t*>(s16);   // always a readable address
+  const bool has_zp = zp != nullptr;
+
+  auto load_stage = [&](Stage& st, int gbase) {
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
+    for (int u = 0; u < US; ++u) {
       const int gi = gbase + u * NW;
       const int kl = gi * 128 + g * 32;
       const bool ok = (gi < G) && (kl < K);
@@ -129,25 +142,27 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
             // non-temporal: the weights are used once and should not displace x in L2
             const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(
                 wr, okw ? (uint32_t)nr * wrow + (uint32_t)(gi * 128 + c * 16) : kOOB, 0, 2);
-            if (h == 0) wa[u][t] = v; else wb[u][t] = v;
+            if (h == 0) st.wa[u][t] = v; else st.wb[u][t] = v;
           }
         } else {
           const int r = lane >> 2, c = lane & 3;
           const int nr = n0 + t * 16 + r;
           const bool okw = gi < G && gi * 128 + c * 32 < K && nr < nend;
-          wa[u][t] = __builtin_amdgcn_raw_buffer_load_b128(
+          st.wa[u][t] = __builtin_amdgcn_raw_buffer_load_b128(
               wr, okw ? (uint32_t)nr * wrow + (uint32_t)(gi * 64 + c * 16) : kOOB, 0, 2);
         }
+        // side data stays raw until it is used: a conversion here would wait for the load,
+        // and with it for every older load in flight
         if constexpr (kIsInt4) {
-          sc[u][t] = (float)s16[(size_t)nc * Kg + gic];
-          zz[u][t] = zp ? (float)zp[(size_t)nc * Kg + gic] : 8.0f;
+          st.sc[u][t] = s16u[(size_t)nc * Kg + gic];
+          st.zz[u][t] = zsrc[(size_t)nc * Kg + gic];
         } else if constexpr (kIsQ4K) {
           const int sb = gic * 4 + g;
           const int sbc = sb < Kb32 ? sb : Kb32 - 1;
-          sc[u][t] = (float)s16[(size_t)nc * Kb32 + sbc];
-          zz[u][t] = (float)qmin[(size_t)nc * Kb32 + sbc];
+          st.sc[u][t] = s16u[(size_t)nc * Kb32 + sbc];
+          st.zz[u][t] = qminu[(size_t)nc * Kb32 + sbc];
         } else if constexpr (kBlock) {
-          sc[u][t] = s32[(size_t)(min(n0 + t * 16, N - 1) >> 7) * Kb + gic];
+          st.sc[u][t] = reinterpret_cast<const uint32_t*>(s32)[(size_t)(min(n0 + t * 16, N - 1) >> 7) * Kb + gic];
         }
       }
 #pragma unroll
@@ -160,19 +175,21 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
             const int r = (lane >> 4) + 4 * i, c = lane & 15;
             const int m = mt * 16 + r;
             const bool okx = gi < G && gi * 128 + c * 8 < K && m < M;
-            xa[u][mt][i] = buf_load16(xr, okx ? ((uint32_t)m * (uint32_t)K + (uint32_t)(gi * 128 + c * 8)) * 2u : kOOB);
+            st.xa[u][mt][i] = buf_load16(xr, okx ? ((uint32_t)m * (uint32_t)K + (uint32_t)(gi * 128 + c * 8)) * 2u : kOOB);
           }
         } else {
           // few rows: straight into operand layout (lane (j, g): row j, 32 consecutive k)
           const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
+          for (int i = 0; i < 4; ++i) st.xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
         }
       }
     }
-    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  auto compute_stage = [&](Stage& st) {
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
+    for (int u = 0; u < US; ++u) {
       // activations through this wavefront's staging tile into MFMA operand layout:
       // lane (j, g) ends up with row j, k = 32 g + 8 i .. + 7 of the granule
 #pragma unroll
@@ -180,45 +197,51 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
         unsigned char* xl = smem + kWStage + (wave * MT + mt) * 16 * kXP;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          *reinterpret_cast<u32x4*>(xl + ((lane >> 4) + 4 * i) * kXP + (lane & 15) * 16) = xa[u][mt][i];
+          *reinterpret_cast<u32x4*>(xl + ((lane >> 4) + 4 * i) * kXP + (lane & 15) * 16) = st.xa[u][mt][i];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          xa[u][mt][i] = *reinterpret_cast<const u32x4*>(xl + j * kXP + g * 64 + i * 16);
+          st.xa[u][mt][i] = *reinterpret_cast<const u32x4*>(xl + j * kXP + g * 64 + i * 16);
       }
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
         // through this wavefront's staging tile into MFMA operand layout
         unsigned char* wl = smem + (wave * RT + t) * 16 * kWP;
+        u32x4 wa = st.wa[u][t], wb = st.wb[u][t];
         if constexpr (kIsFp8) {
-          *reinterpret_cast<u32x4*>(wl + (lane >> 3) * kWP + (lane & 7) * 16) = wa[u][t];
-          *reinterpret_cast<u32x4*>(wl + ((lane >> 3) + 8) * kWP + (lane & 7) * 16) = wb[u][t];
-          wa[u][t] = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32);
-          wb[u][t] = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32 + 16);
+          *reinterpret_cast<u32x4*>(wl + (lane >> 3) * kWP + (lane & 7) * 16) = wa;
+          *reinterpret_cast<u32x4*>(wl + ((lane >> 3) + 8) * kWP + (lane & 7) * 16) = wb;
+          wa = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32);
+          wb = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32 + 16);
         } else {
-          *reinterpret_cast<u32x4*>(wl + (lane >> 2) * kWP + (lane & 3) * 16) = wa[u][t];
-          wa[u][t] = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 16);
+          *reinterpret_cast<u32x4*>(wl + (lane >> 2) * kWP + (lane & 3) * 16) = wa;
+          wa = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 16);
         }
         V8 b[4];
+        float scf = 0.f;
         if constexpr (kIsFp8) {
-          b[0] = fp8x8_to_act<Act>(wa[u][t][0], wa[u][t][1]);
-          b[1] = fp8x8_to_act<Act>(wa[u][t][2], wa[u][t][3]);
-          b[2] = fp8x8_to_act<Act>(wb[u][t][0], wb[u][t][1]);
-          b[3] = fp8x8_to_act<Act>(wb[u][t][2], wb[u][t][3]);
+          b[0] = fp8x8_to_act<Act>(wa[0], wa[1]);
+          b[1] = fp8x8_to_act<Act>(wa[2], wa[3]);
+          b[2] = fp8x8_to_act<Act>(wb[0], wb[1]);
+          b[3] = fp8x8_to_act<Act>(wb[2], wb[3]);
+          if constexpr (kBlock) scf = __builtin_bit_cast(float, st.sc[u][t]);
         } else if constexpr (kIsInt4) {
+          const float sf = (float)__builtin_bit_cast(_Float16, (uint16_t)st.sc[u][t]);
+          const float zf = has_zp ? (float)st.zz[u][t] : 8.0f;
           if constexpr (Act::dt == DT_F16) {
-            const _Float16 s = (_Float16)sc[u][t];
-            const _Float16 z = (_Float16)(1024.0f + zz[u][t]);
+            const _Float16 s = (_Float16)sf;
+            const _Float16 z = (_Float16)(1024.0f + zf);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[u][t][i], s, z);
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[i], s, z);
           } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[u][t][i], sc[u][t], zz[u][t]);
+            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[i], sf, zf);
           }
         } else {
           if constexpr (Act::dt == DT_F16) {
+            const _Float16 s = __builtin_bit_cast(_Float16, (uint16_t)st.sc[u][t]);
+            const _Float16 mn = __builtin_bit_cast(_Float16, (uint16_t)st.zz[u][t]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              b[i] = q4kx8_to_f16(wa[u][t][i], (_Float16)sc[u][t], (_Float16)zz[u][t]);
+            for (int i = 0; i < 4; ++i) b[i] = q4kx8_to_f16(wa[i], s, mn);
           }
         }
 #pragma unroll
@@ -226,15 +249,36 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
           if constexpr (kBlock) {
             f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < 4; ++i) tt = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], tt);
-            acc[t][mt] += tt * sc[u][t];
+            for (int i = 0; i < 4; ++i) tt = Act::mfma(as_v8<V8>(st.xa[u][mt][i]), b[i], tt);
+            acc[t][mt] += tt * scf;
           } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              acc[t][mt] = Act::mfma(as_v8<V8>(xa[u][mt][i]), b[i], acc[t][mt]);
+              acc[t][mt] = Act::mfma(as_v8<V8>(st.xa[u][mt][i]), b[i], acc[t][mt]);
           }
         }
       }
+    }
+  };
+
+  if constexpr (UN >= 2) {
+    // two-stage ring; the only exit is at the bottom (stages past the end load zeros)
+    Stage s0, s1;
+    load_stage(s0, wave);
+    for (int gbase = wave; gbase < G; gbase += NW * UN) {
+      load_stage(s1, gbase + NW * US);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_stage(s0);
+      load_stage(s0, gbase + NW * UN);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_stage(s1);
+    }
+  } else {
+    Stage s0;
+    for (int gbase = wave; gbase < G; gbase += NW * UN) {
+      load_stage(s0, gbase);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_stage(s0);
     }
   }
 
