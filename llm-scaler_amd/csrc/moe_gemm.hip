@@ -205,11 +205,17 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
           for (int i = 0; i < WL; ++i) *reinterpret_cast<u32x4*>(wlds[i] + par * kWBuf) = r[s].w[i];
 #pragma unroll
           for (int i = 0; i < NAI; ++i) *reinterpret_cast<u32x4*>(alds[i]) = r[s].a[i];
+          // The activation scale is taken out of the ring slot before the slot is reloaded
+          // below.  Left to the scheduler, the multiply sinks under the reload, old and new
+          // value overlap, and the loop latch gets a register copy of the NEW value, i.e. a
+          // wait for every load in flight on each turn.
+          float xs_now = A8 ? r[s].xs : 1.0f;
+          asm volatile("" : "+v"(xs_now));
           float sc[RT];
 #pragma unroll
           for (int t = 0; t < RT; ++t) {
             const float ws = wsc[(size_t)nb[t] * Kb + gi];
-            sc[t] = A8 ? r[s].xs * ws : ws;
+            sc[t] = A8 ? xs_now * ws : ws;
           }
           // prefetch D granules ahead, across the tile-group boundary
           {
