@@ -201,6 +201,8 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
  *   V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:5-7).
  * mi_moe_silu_mul: out[r, c] = silu(in[r, c]) * in[r, n_half + c]
  *   (esimd_moe_silu_mul, V/csrc/xpu/esimd_kernels/moe_ops.h:576-621).
+ * mi_moe_gelu_tanh_mul: the same with the tanh form of GELU on the gate half
+ *   (esimd_moe_gelu_tanh_mul, moe_ops.h:680-728; exp argument held in [-30, 30]).
  * mi_moe_scatter: scattered[pos] = hidden[sorted_pairs[pos] / topk], optional
  *   scattered_w[pos] = top_w[sorted_pairs[pos]]   (esimd_moe_scatter, moe_ops.h:522-569).
  * mi_moe_combine: out[t] = sum_j w * y[inv[t*topk + j]], weights indexed by sorted
@@ -223,6 +225,8 @@ int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K
                      void* stream);
 int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
                     void* stream);
+int mi_moe_gelu_tanh_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
+                         void* stream);
 int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_pairs, void* scattered,
                    void* scattered_w, int K, int topk, int total, void* stream);
 int mi_moe_combine(const void* y, const int32_t* inv, const void* w, void* out, int H, int topk, int T,
@@ -243,9 +247,13 @@ int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void
  * decode ops — esimd_resadd_norm_gemv_{int4,fp8}_pert
  * (V/csrc/xpu/esimd_kernels/resadd_norm_gemv_int4.h:56-100), esimd_norm_gemv_*_pert
  * (per-head gated norm, norm_gemv_int4.h), esimd_rms_norm (esimd_kernel.sycl:488-502);
- * the ops run it and then the GEMV entry point on its output. */
+ * the ops run it and then the GEMV entry point on its output.  With a residual the sum is
+ * multiplied by residual_scale before it is stored and normalised (1 for the plain add;
+ * esimd_fused_scaled_add_rms_norm, V/csrc/xpu/torch_extension.cc:145-148).  x and out may be
+ * the same buffer (esimd_fused_add_rms_norm writes the normalised row over hidden_states). */
 int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weight, void* out, int rows, int L,
-               int weight_len, float eps, int act_dtype, void* stream);
+               int weight_len, float eps, int act_dtype,
+               float residual_scale, void* stream);
 
 /* The same normalisation fused into the decode GEMV (one launch, M == 1):
  *   x' = rmsnorm(x (+ residual)) (* silu(gate)) per head of norm_len elements

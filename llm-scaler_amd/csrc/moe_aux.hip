@@ -318,7 +318,10 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* 
 }
 
 // ---------------------------------------------------------------- elementwise
-template <class Act>
+// out[r, c] = act(gate) * up with act = SiLU, or (GELU) the tanh form of GELU:
+// 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), tanh through exp(2z) with 2z held in
+// [-30, 30] so that large gates saturate instead of producing inf / inf.
+template <class Act, bool GELU>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const typename Act::elem* __restrict__ in,
                                                        typename Act::elem* __restrict__ out, int n_gate_up,
                                                        int n_half, int rows) {
@@ -327,7 +330,14 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const typename Act::elem*
   const int r = (int)(i / n_half), c = (int)(i % n_half);
   const float g = Act::to_f32(in[(size_t)r * n_gate_up + c]);
   const float u = Act::to_f32(in[(size_t)r * n_gate_up + n_half + c]);
-  out[i] = Act::from_f32(g / (1.0f + expf(-g)) * u);
+  if constexpr (GELU) {
+    float two_z = 2.0f * (0.7978845608f * (g + 0.044715f * (g * g * g)));
+    two_z = two_z > 30.0f ? 30.0f : (two_z < -30.0f ? -30.0f : two_z);
+    const float e = expf(two_z);
+    out[i] = Act::from_f32(0.5f * g * (1.0f + (e - 1.0f) / (e + 1.0f)) * u);
+  } else {
+    out[i] = Act::from_f32(g / (1.0f + expf(-g)) * u);
+  }
 }
 
 // scattered[pos] = hidden[pair / topk], weights[pos] = top_w[pair]   (pos -> pair = sorted_pairs[pos])
@@ -421,21 +431,23 @@ __global__ __launch_bounds__(256) void shared_gate_kernel(const typename Act::v8
 // ---------------------------------------------------------------- RMS norm (+ residual add, + SiLU gate)
 // One workgroup per row of length L:  a = x (+ residual, which is then updated in
 // place with the rounded sum);  out = a * rsqrt(mean(a^2) + eps) * weight[i % wlen]
-// (* silu(gate)), fp32 throughout, one rounding at the store.
+// (* silu(gate)), fp32 throughout, one rounding at the store; x and out may be one buffer
+// (every element is read and written by the same thread).  With a residual the sum is
+// multiplied by res_scale first (1 for the plain residual add).
 template <class Act>
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const typename Act::elem* __restrict__ x,
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const typename Act::elem* x,
                                                       typename Act::elem* residual,
                                                       const typename Act::elem* __restrict__ gate,
                                                       const typename Act::elem* __restrict__ weight,
-                                                      typename Act::elem* __restrict__ out, int L, int wlen,
-                                                      float eps) {
+                                                      typename Act::elem* out, int L, int wlen,
+                                                      float eps, float res_scale) {
   __shared__ float wsum[4];
   const size_t base = (size_t)blockIdx.x * L;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float ss = 0.f;
   for (int i = threadIdx.x; i < L; i += 256) {
     float a = Act::to_f32(x[base + i]);
-    if (residual) a += Act::to_f32(residual[base + i]);
+    if (residual) a = (a + Act::to_f32(residual[base + i])) * res_scale;
     ss += a * a;
   }
   ss = wave_sum(ss);
@@ -446,7 +458,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const typename Act::elem* 
   for (int i = threadIdx.x; i < L; i += 256) {
     float a = Act::to_f32(x[base + i]);
     if (residual) {
-      a += Act::to_f32(residual[base + i]);
+      a = (a + Act::to_f32(residual[base + i])) * res_scale;
       residual[base + i] = Act::from_f32(a);
     }
     float v = a * inv * Act::to_f32(weight[i % wlen]);
@@ -520,22 +532,30 @@ int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K
   return launch_status();
 }
 
-int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
-                    void* stream) {
+static int act_mul_launch(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
+                          bool gelu, void* stream) {
   if (!in || !out) return MI_ERR_ARG;
   if (rows < 0 || n_half <= 0 || n_gate_up != 2 * n_half) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
   if (!rows) return MI_OK;
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid = grid1d((size_t)rows * n_half);
-  if (act_dtype == DT_F16)
-    hipLaunchKernelGGL(silu_mul_kernel<ActF16>, grid, dim3(256), 0, st, (const _Float16*)in, (_Float16*)out,
-                       n_gate_up, n_half, rows);
-  else if (act_dtype == DT_BF16)
-    hipLaunchKernelGGL(silu_mul_kernel<ActBF16>, grid, dim3(256), 0, st, (const __bf16*)in, (__bf16*)out,
-                       n_gate_up, n_half, rows);
-  else
-    return MI_ERR_ARG;
+#define QLIN_ACT_MUL(ACT, ELEM, G) \
+  hipLaunchKernelGGL((silu_mul_kernel<ACT, G>), grid, dim3(256), 0, st, (const ELEM*)in, (ELEM*)out, n_gate_up, n_half, rows)
+  if (act_dtype == DT_F16) { if (gelu) QLIN_ACT_MUL(ActF16, _Float16, true); else QLIN_ACT_MUL(ActF16, _Float16, false); }
+  else { if (gelu) QLIN_ACT_MUL(ActBF16, __bf16, true); else QLIN_ACT_MUL(ActBF16, __bf16, false); }
+#undef QLIN_ACT_MUL
   return launch_status();
+}
+
+int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
+                    void* stream) {
+  return act_mul_launch(in, out, n_gate_up, n_half, rows, act_dtype, false, stream);
+}
+
+int mi_moe_gelu_tanh_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,
+                         void* stream) {
+  return act_mul_launch(in, out, n_gate_up, n_half, rows, act_dtype, true, stream);
 }
 
 int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_pairs, void* scattered,
@@ -590,7 +610,8 @@ int mi_permute_rows(const void* src, const int32_t* map, void* dst, int rows, lo
 }
 
 int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weight, void* out, int rows, int L,
-               int weight_len, float eps, int act_dtype, void* stream) {
+               int weight_len, float eps, int act_dtype, float residual_scale,
+               void* stream) {
   if (!x || !weight || !out) return MI_ERR_ARG;
   if (rows < 0 || L <= 0 || weight_len <= 0 || (L % weight_len)) return MI_ERR_SHAPE;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
@@ -598,10 +619,10 @@ int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weig
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == DT_F16)
     hipLaunchKernelGGL(rmsnorm_kernel<ActF16>, dim3(rows), dim3(256), 0, st, (const _Float16*)x, (_Float16*)residual,
-                       (const _Float16*)gate, (const _Float16*)weight, (_Float16*)out, L, weight_len, eps);
+                       (const _Float16*)gate, (const _Float16*)weight, (_Float16*)out, L, weight_len, eps, residual_scale);
   else
     hipLaunchKernelGGL(rmsnorm_kernel<ActBF16>, dim3(rows), dim3(256), 0, st, (const __bf16*)x, (__bf16*)residual,
-                       (const __bf16*)gate, (const __bf16*)weight, (__bf16*)out, L, weight_len, eps);
+                       (const __bf16*)gate, (const __bf16*)weight, (__bf16*)out, L, weight_len, eps, residual_scale);
   return launch_status();
 }
 

@@ -38,7 +38,7 @@ int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* no
     // two kernels: the norm writes the row (into normed_out, or over x's scratch copy), then the GEMV
     if (!normed_out) return MI_ERR_ARG;
     const int rc = mi_rmsnorm(x, residual, gate, norm_weight, normed_out, K / norm_len, norm_len, norm_len, eps,
-                              act_dtype, stream);
+                              act_dtype, 1.0f, stream);
     if (rc != MI_OK) return rc;
     const float* const* fs = reinterpret_cast<const float* const*>(scale);
     if (fmt == 0) return mi_gemm_fp8_pert_multi(normed_out, nmat, w, fs, out, N, 1, K, act_dtype, stream);

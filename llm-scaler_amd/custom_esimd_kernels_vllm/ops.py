@@ -109,6 +109,11 @@ def esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows):
     return _ops.esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows)
 
 
+def esimd_moe_gelu_tanh_mul(input, output, N_gate_up, N_half, total_rows):
+    """GELU_tanh(gate) * up activation."""
+    return _ops.esimd_moe_gelu_tanh_mul(input, output, N_gate_up, N_half, total_rows)
+
+
 def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T):
     return _ops.esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T)
 
@@ -180,6 +185,25 @@ def precompute_moe_route(topk_weights, topk_ids, num_experts):
 
 # decode fusions: RMS norm (+ residual add / SiLU gate) + GEMV
 # (V/python/custom_esimd_kernels_vllm/ops.py:340-560)
+def esimd_fused_add_rms_norm(hidden_states, residual, weight, eps):
+    """residual = hidden_states + residual (in place); hidden_states = rmsnorm(residual) * weight."""
+    return _ops.esimd_fused_add_rms_norm(hidden_states, residual, weight, eps)
+
+
+def esimd_fused_scaled_add_rms_norm(hidden_states, residual, weight, eps, scalar):
+    """residual = (hidden_states + residual) * scalar (in place); hidden_states = rmsnorm(residual) * weight."""
+    return _ops.esimd_fused_scaled_add_rms_norm(hidden_states, residual, weight, eps, scalar)
+
+
+def esimd_fused_add_rms_norm_batched(hidden_states, residual, weight, eps):
+    return _ops.esimd_fused_add_rms_norm_batched(hidden_states, residual, weight, eps)
+
+
+def esimd_rms_norm_gated(x, z, weight, output, eps):
+    """output = rmsnorm(x) * weight * silu(z); x, z [rows, V], weight [V]."""
+    return _ops.esimd_rms_norm_gated(x, z, weight, output, eps)
+
+
 def esimd_rms_norm(input, output, weight, eps):
     return _ops.esimd_rms_norm(input, output, weight, eps)
 

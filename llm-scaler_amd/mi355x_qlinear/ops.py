@@ -638,15 +638,23 @@ def act_quant_fp8(x, q, scale):
     return q
 
 
-def esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows):
-    who = "esimd_moe_silu_mul"
+def _act_mul(input, output, N_gate_up, N_half, total_rows, entry, who):
     _chk_act(input, output, who)
     _chk(int(N_gate_up) == 2 * int(N_half), f"{who}: N_gate_up must be 2 * N_half")
     _chk(input.numel() >= int(total_rows) * int(N_gate_up) and output.numel() >= int(total_rows) * int(N_half),
          f"{who}: tensors too small for total_rows")
-    capi.call("mi_moe_silu_mul", input, capi.ptr(input), capi.ptr(output), int(N_gate_up), int(N_half),
+    capi.call(entry, input, capi.ptr(input), capi.ptr(output), int(N_gate_up), int(N_half),
               int(total_rows), capi.act_dtype(input))
     return output
+
+
+def esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows):
+    return _act_mul(input, output, N_gate_up, N_half, total_rows, "mi_moe_silu_mul", "esimd_moe_silu_mul")
+
+
+def esimd_moe_gelu_tanh_mul(input, output, N_gate_up, N_half, total_rows):
+    """GELU_tanh(gate) * up (V/csrc/xpu/esimd_kernels/moe_ops.h:680-728)."""
+    return _act_mul(input, output, N_gate_up, N_half, total_rows, "mi_moe_gelu_tanh_mul", "esimd_moe_gelu_tanh_mul")
 
 
 def esimd_moe_scatter(hidden_states, router_top_value, sorted_token_ids, scattered_hidden, scattered_weights,
@@ -907,7 +915,7 @@ def moe_prefill_gather_forward_fp8(selected_experts, num_experts):
 # (V/csrc/xpu/torch_extension.cc:103-140).  Two launches here: the norm kernel,
 # then the GEMV entry point on its 16-bit output.
 # --------------------------------------------------------------------------
-def _rmsnorm(x, residual, gate, weight, out, rows, L, eps, who):
+def _rmsnorm(x, residual, gate, weight, out, rows, L, eps, who, residual_scale=1.0):
     _chk(x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(), f"{who}: activations must be contiguous fp16/bf16")
     for name, t in (("residual", residual), ("gate", gate), ("norm_weight", weight), ("normed output", out)):
         if t is not None:
@@ -915,8 +923,39 @@ def _rmsnorm(x, residual, gate, weight, out, rows, L, eps, who):
     _chk(x.numel() == rows * L and out.numel() >= rows * L, f"{who}: size mismatch")
     _chk(weight.numel() >= 1 and L % weight.numel() == 0, f"{who}: norm_weight length must divide the row length")
     capi.call("mi_rmsnorm", x, capi.ptr(x), capi.ptr(residual), capi.ptr(gate), capi.ptr(weight), capi.ptr(out),
-              rows, L, weight.numel(), float(eps), capi.act_dtype(x))
+              rows, L, weight.numel(), float(eps), capi.act_dtype(x), float(residual_scale))
     return out
+
+
+def esimd_fused_add_rms_norm(hidden_states, residual, weight, eps):
+    """residual = hidden_states + residual (in place); hidden_states = rmsnorm(residual) * weight (in place)
+    (V/csrc/xpu/torch_extension.cc:141-143; one row in the reference, any number here)."""
+    K = hidden_states.shape[-1]
+    return _rmsnorm(hidden_states, residual, None, weight, hidden_states, hidden_states.numel() // K, K, eps,
+                    "esimd_fused_add_rms_norm")
+
+
+def esimd_fused_add_rms_norm_batched(hidden_states, residual, weight, eps):
+    """The same for any number of rows (torch_extension.cc:154-156)."""
+    K = hidden_states.shape[-1]
+    return _rmsnorm(hidden_states, residual, None, weight, hidden_states, hidden_states.numel() // K, K, eps,
+                    "esimd_fused_add_rms_norm_batched")
+
+
+def esimd_fused_scaled_add_rms_norm(hidden_states, residual, weight, eps, scalar):
+    """residual = (hidden_states + residual) * scalar (in place); hidden_states = rmsnorm(residual) * weight
+    (torch_extension.cc:145-148)."""
+    K = hidden_states.shape[-1]
+    return _rmsnorm(hidden_states, residual, None, weight, hidden_states, hidden_states.numel() // K, K, eps,
+                    "esimd_fused_scaled_add_rms_norm", residual_scale=float(scalar))
+
+
+def esimd_rms_norm_gated(x, z, weight, output, eps):
+    """output = rmsnorm(x) * weight * silu(z) per row of V = len(weight) elements
+    (torch_extension.cc:150-152)."""
+    V = weight.numel()
+    _chk(x.numel() % V == 0 and z.numel() == x.numel(), "esimd_rms_norm_gated: x and z must be [rows, V]")
+    return _rmsnorm(x, None, z, weight, output, x.numel() // V, V, eps, "esimd_rms_norm_gated")
 
 
 def esimd_rms_norm(input, output, weight, eps):
@@ -1215,6 +1254,14 @@ def register():
                 esimd_gemv_fp8_blockscale_fused2, _ret(3))
     for ns in (_V, _S):
         _define(ns, "esimd_rms_norm(Tensor input, Tensor output, Tensor weight, float eps) -> Tensor", esimd_rms_norm, _ret(1))
+        _define(ns, "esimd_fused_add_rms_norm(Tensor hidden_states, Tensor residual, Tensor weight, float eps) -> Tensor",
+                esimd_fused_add_rms_norm, _ret(0))
+        _define(ns, "esimd_fused_scaled_add_rms_norm(Tensor hidden_states, Tensor residual, Tensor weight, float eps, "
+                    "float scalar) -> Tensor", esimd_fused_scaled_add_rms_norm, _ret(0))
+        _define(ns, "esimd_rms_norm_gated(Tensor x, Tensor z, Tensor weight, Tensor output, float eps) -> Tensor",
+                esimd_rms_norm_gated, _ret(3))
+        _define(ns, "esimd_fused_add_rms_norm_batched(Tensor hidden_states, Tensor residual, Tensor weight, float eps) -> Tensor",
+                esimd_fused_add_rms_norm_batched, _ret(0))
         _define(ns, "esimd_resadd_norm_gemv_int4_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
                     "Tensor gemv_weight, Tensor gemv_scale, Tensor output, Tensor normed_out, float eps) -> Tensor",
                 esimd_resadd_norm_gemv_int4_pert, _ret(5))
@@ -1285,6 +1332,8 @@ def register():
                 esimd_moe_scatter_fused, _ret(3))
         _define(ns, "esimd_moe_silu_mul(Tensor input, Tensor output, int N_gate_up, int N_half, int total_rows) -> Tensor",
                 esimd_moe_silu_mul, _ret(1))
+        _define(ns, "esimd_moe_gelu_tanh_mul(Tensor input, Tensor output, int N_gate_up, int N_half, int total_rows) -> Tensor",
+                esimd_moe_gelu_tanh_mul, _ret(1))
         _define(ns, "esimd_moe_gather(Tensor moe_output, Tensor topk_ids, Tensor scattered_weights, "
                     "Tensor final_hidden, int K, int topk, int T) -> Tensor", esimd_moe_gather, _ret(3))
     _define(_V, "esimd_moe_gemm_fp8_blockscale(Tensor input, Tensor weight, Tensor weight_scale, Tensor(a!) output, "

@@ -380,6 +380,15 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return g * torch.sigmoid(g) * u
 
 
+def gelu_tanh_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """[rows, 2I] -> [rows, I] fp32: GELU_tanh(gate) * up, gate = first half
+    (V/csrc/xpu/esimd_kernels/moe_ops.h:696-723; the textbook tanh form, which
+    torch.nn.functional.gelu(approximate="tanh") implements)."""
+    half = gate_up.shape[-1] // 2
+    g, u = gate_up[..., :half].float(), gate_up[..., half:].float()
+    return torch.nn.functional.gelu(g, approximate="tanh") * u
+
+
 def moe_forward(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, *, act_quant: bool,
                 act_dtype=torch.bfloat16):
     """Routed-experts MoE forward (no shared expert), per-token / per-route loop.

@@ -549,3 +549,32 @@ def test_norm_gemv_several_rows(ops, dev):
     assert _ulp_close(normed_out.cpu().float(), normed_ref, torch.float16)
     wd = O.int4_dequant(packed, scale, out_dtype=torch.float16)
     assert O.max_rel_err(out.cpu(), O.matmul_ref(normed_out.cpu(), wd)) < TOL
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_norm_only_ops(ops, dev, dt):
+    # esimd_fused_add_rms_norm (+ _batched, scaled) work in place; esimd_rms_norm_gated is per row of V
+    v, _ = ops
+    g = torch.Generator().manual_seed(31)
+    rows, K, eps = 5, 2048, 1e-6
+    h = torch.randn(rows, K, generator=g).to(dt)
+    r = torch.randn(rows, K, generator=g).to(dt)
+    w = (torch.randn(K, generator=g) * 0.1 + 1.0).to(dt)
+    for name, scalar in (("esimd_fused_add_rms_norm", None), ("esimd_fused_add_rms_norm_batched", None),
+                         ("esimd_fused_scaled_add_rms_norm", 0.70703125)):
+        hd, rd = h.to(dev).clone(), r.to(dev).clone()
+        args = (hd, rd, w.to(dev), eps) + (() if scalar is None else (scalar,))
+        ret = getattr(v, name)(*args)
+        assert ret.data_ptr() == hd.data_ptr()
+        a = (h.float() + r.float()) * (1.0 if scalar is None else scalar)
+        assert torch.equal(rd.cpu().view(torch.int16), a.to(dt).view(torch.int16))
+        ref = a * torch.rsqrt(a.pow(2).mean(dim=-1, keepdim=True) + eps) * w.float()
+        assert _ulp_close(hd.cpu().float(), ref, dt)
+    V = 128
+    x = torch.randn(24, V, generator=g).to(dt)
+    z = torch.randn(24, V, generator=g).to(dt)
+    wv = (torch.randn(V, generator=g) * 0.1 + 1.0).to(dt)
+    out = torch.empty(24, V, dtype=dt, device=dev)
+    v.esimd_rms_norm_gated(x.to(dev), z.to(dev), wv.to(dev), out, eps)
+    ref, _ = O.rmsnorm(x, wv, eps, gate=z, heads=24)
+    assert _ulp_close(out.cpu().float(), ref, dt)

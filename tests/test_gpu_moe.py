@@ -135,6 +135,19 @@ def test_silu_mul(v, dev):
     assert O.max_rel_err(out.cpu(), ref) < 8e-3     # bf16 output rounding is 2^-9
 
 
+def test_gelu_tanh_mul(v, dev):
+    g = torch.Generator().manual_seed(15)
+    x = (torch.randn(29, 384, generator=g) * 3).half()
+    x[0, :8] = torch.tensor([40.0, -40.0, 11.5, -11.5, 0.0, 1e-4, 60000.0, -60000.0]).half()   # saturating gates
+    x[0, 192:200] = 1.0
+    out = torch.empty(29, 192, dtype=torch.float16, device=dev)
+    v.esimd_moe_gelu_tanh_mul(x.to(dev), out, 384, 192, 29)
+    ref = O.gelu_tanh_mul(x)
+    assert torch.isfinite(out.cpu().float()).all()
+    assert out[0, 1].item() == 0.0 and out[0, 7].item() == 0.0          # gelu(-large) = -0
+    assert O.max_rel_err(out.cpu(), ref) < 2e-3
+
+
 # ------------------------------------------------------------------ grouped GEMM
 def _grouped_ref(x, dw, counts):
     ref = torch.empty(x.shape[0], dw.shape[1], dtype=torch.float32)

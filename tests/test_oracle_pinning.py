@@ -422,3 +422,15 @@ def test_rmsnorm_oracle_against_library_and_hand_values():
     xh = torch.tensor([[3.0, 4.0, 6.0, 8.0]]).half()
     nh, _ = O.rmsnorm(xh, torch.ones(2).half(), 0.0, heads=2)
     assert torch.allclose(nh, torch.tensor([[3 / 12.5 ** 0.5, 4 / 12.5 ** 0.5, 6 / 50 ** 0.5, 8 / 50 ** 0.5]]), rtol=1e-6)
+
+
+def test_gelu_tanh_mul_closed_form():
+    # the tanh form written out (exp-based tanh as the reference's kernel computes it), gate = first half
+    gu = torch.tensor([[0.0, 1.0, -2.0, 3.0, 2.0, 2.0, 2.0, 0.5]])
+    out = O.gelu_tanh_mul(gu)
+    g = gu[0, :4].double()
+    z = 0.7978845608 * (g + 0.044715 * g ** 3)
+    e = torch.exp(2 * z)
+    exp = 0.5 * g * (1 + (e - 1) / (e + 1)) * gu[0, 4:].double()
+    assert torch.allclose(out[0].double(), exp, rtol=1e-6, atol=1e-7)
+    assert out[0, 0] == 0 and abs(out[0, 1].item() - 0.8411920 * 2.0) < 1e-5    # gelu_tanh(1) = 0.841192
