@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
 
 A step is one launch of the hot-path op on one batch of seeded synthetic input.
-The headline workload (default) is BASELINE.json configs[1]: FP8 per-channel
+The headline workload (default) is the second benchmark configuration: FP8 per-channel
 weight-only GEMV, M=1, K=4096, N=14336, bf16 activations.  Each step uses the
 next of R distinct weight copies (R x weight bytes >> the 256 MB Infinity Cache)
 so the figure is HBM bandwidth, not cache bandwidth.  The K timed steps are

@@ -131,29 +131,6 @@ __device__ __forceinline__ bf16x8 int4x8_to_bf16(uint32_t w, float s, float z) {
   return out;
 }
 
-// bf16 on the packed-fp16 pipe: d = nib - z is formed exactly as an fp16 pair
-// ((0x6400 | nib) - (1024 + z)), each half is multiplied by the fp16 scale in
-// fp32 (exact: 5 x 11 significant bits, one mixed-precision fma) and the pair is
-// rounded once to bf16 — bit-identical to int4x8_to_bf16 at two thirds of the
-// VALU work.  z1024 = 1024 + z.
-__device__ __forceinline__ bf16x8 int4x8_to_bf16_mix(uint32_t w, _Float16 s, _Float16 z1024) {
-  const uint32_t e = w & 0x0F0F0F0Fu;
-  const uint32_t o = (w >> 4) & 0x0F0F0F0Fu;
-  f16x2 zv = {z1024, z1024};
-  const float sf = (float)s;
-  bf16x8 out;
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const uint32_t sel = 0x0C000C00u | ((4u + p) << 16) | (uint32_t)p;
-    const uint32_t bits = __builtin_amdgcn_perm(o, e, sel) | 0x64006400u;
-    f16x2 v = __builtin_bit_cast(f16x2, bits);
-    v = v - zv;
-    out[2 * p] = (__bf16)((float)v[0] * sf);
-    out[2 * p + 1] = (__bf16)((float)v[1] * sf);
-  }
-  return out;
-}
-
 // ---- Q4_K repacked sub-block -> fp16, two roundings ---------------------------
 // w = fp16(fp16(nib * scale) - min): the product is rounded before the
 // subtraction, exactly as two separate fp16 ops do; contraction into an fma
