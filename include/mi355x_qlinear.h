@@ -221,6 +221,12 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
  *   output, activation dtype; gate may be null = 1), summed in fp32 and rounded once
  *   (the finalize step of moe_down_finalize_fp8_block_batched_kernel,
  *   V/csrc/moe_batch/moe.sycl:1570-1663). */
+/* mi_moe_sort and mi_act_quant_fp8 of the token activations x [rows, H] in one launch
+ * (the two are independent; the sort is a single latency-bound workgroup).  No counterpart
+ * in the reference: its MoE path keeps 16-bit activations. */
+int mi_moe_sort_quant(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
+                      int32_t* sorted_token, int32_t* max_count, int T, int K, int E, const void* x,
+                      void* q, float* scale, long long rows, int H, int act_dtype, void* stream);
 int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K, int act_dtype,
                      void* stream);
 int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,

@@ -138,7 +138,7 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* wave_t
   return v + (wave ? wave_tot[wave - 1] : 0u);
 }
 
-__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
+__device__ __forceinline__ void moe_sort_body(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
     int32_t* __restrict__ max_count, int T, int K, int E) {
@@ -276,6 +276,13 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
   }
 }
 
+__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
+    const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
+    int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
+    int32_t* __restrict__ max_count, int T, int K, int E) {
+  moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+}
+
 // ---------------------------------------------------------------- activation quant
 // Per row, per 128-wide group: s = max|x| / 448 (clamped at 1e-12), q = e4m3(x / s).
 // 16 lanes own one group (8 elements each); the group maximum is a DPP butterfly
@@ -287,10 +294,9 @@ __device__ __forceinline__ float dpp_max(float v) {
 }
 
 template <class Act>
-__global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* __restrict__ x,
-                                                        u32x2* __restrict__ q, float* __restrict__ s,
-                                                        size_t groups16) {   // 16-lane groups in total
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;     // one lane = 8 elements
+__device__ __forceinline__ void act_quant_body(const typename Act::v8* __restrict__ x, u32x2* __restrict__ q,
+                                               float* __restrict__ s, size_t groups16, size_t i) {
+  // one lane = 8 elements, lane index i
   const bool live = (i >> 4) < groups16;
   typename Act::v8 v;
   if (live) v = x[i];
@@ -315,6 +321,28 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* 
     q[i] = u32x2{(uint32_t)lo, (uint32_t)hi};
     if ((threadIdx.x & 15) == 0) s[i >> 4] = scale;
   }
+}
+
+template <class Act>
+__global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* __restrict__ x,
+                                                        u32x2* __restrict__ q, float* __restrict__ s,
+                                                        size_t groups16) {   // 16-lane groups in total
+  act_quant_body<Act>(x, q, s, groups16, (size_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+// The expert sort (one workgroup, latency-bound) and the quantisation of the token
+// activations (independent of the routing) in one launch: workgroup 0 sorts, the others
+// quantise 1024 lanes' worth each.
+template <class Act>
+__global__ __launch_bounds__(kSortThreads) void moe_sort_quant_kernel(
+    const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
+    int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
+    int32_t* __restrict__ max_count, int T, int K, int E, const typename Act::v8* __restrict__ x,
+    u32x2* __restrict__ q, float* __restrict__ s, size_t groups16) {
+  if (blockIdx.x == 0)
+    moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+  else
+    act_quant_body<Act>(x, q, s, groups16, (size_t)(blockIdx.x - 1) * kSortThreads + threadIdx.x);
 }
 
 // ---------------------------------------------------------------- elementwise
@@ -510,6 +538,28 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
   if (T > 0 && (!top_ids || !sorted_pairs || !inv)) return MI_ERR_ARG;   // T == 0 only fills expert_start
   hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(kSortThreads), 0, (hipStream_t)stream, top_ids,
                      sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+  return launch_status();
+}
+
+int mi_moe_sort_quant(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
+                      int32_t* sorted_token, int32_t* max_count, int T, int K, int E, const void* x, void* q,
+                      float* scale, long long rows, int H, int act_dtype, void* stream) {
+  if (!expert_start || !x || !q || !scale) return MI_ERR_ARG;
+  if (T < 0 || K < 1 || E < 1 || E > 1024) return MI_ERR_SHAPE;
+  if (T > 0 && (!top_ids || !sorted_pairs || !inv)) return MI_ERR_ARG;
+  if (rows < 0 || H <= 0 || (H % 128)) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  const size_t groups16 = (size_t)rows * (H / 128);
+  const unsigned grid = 1u + (unsigned)((groups16 * 16 + kSortThreads - 1) / kSortThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(moe_sort_quant_kernel<ActF16>, dim3(grid), dim3(kSortThreads), 0, st, top_ids, sorted_pairs,
+                       expert_start, inv, sorted_token, max_count, T, K, E, (const f16x8*)x, (u32x2*)q, scale,
+                       groups16);
+  else
+    hipLaunchKernelGGL(moe_sort_quant_kernel<ActBF16>, dim3(grid), dim3(kSortThreads), 0, st, top_ids, sorted_pairs,
+                       expert_start, inv, sorted_token, max_count, T, K, E, (const bf16x8*)x, (u32x2*)q, scale,
+                       groups16);
   return launch_status();
 }
 

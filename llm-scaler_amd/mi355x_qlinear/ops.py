@@ -788,13 +788,18 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
     start = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(P, dtype=torch.int32, device=dev)
     sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
-    moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
     inter = torch.empty(P, I, dtype=x.dtype, device=dev)
     y = torch.empty(P, H, dtype=torch.float32, device=dev)      # fp32: the combine adds K rounded terms otherwise
     if act_quant:
         xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
         xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)
-        act_quant_fp8(x, xq, xs)
+        # the expert sort and the quantisation of x do not depend on each other: one launch
+        capi.call("mi_moe_sort_quant", top_ids, capi.ptr(top_ids), capi.ptr(sorted_pairs), capi.ptr(start),
+                  capi.ptr(inv), capi.ptr(sorted_token), None, T, k, E, capi.ptr(x), capi.ptr(xq), capi.ptr(xs),
+                  T, H, capi.act_dtype(x))
+    else:
+        moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
+    if act_quant:
         moe_gemm_fp8_block(xq, xs, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
         iq = torch.empty(P, I, dtype=torch.uint8, device=dev)
         isc = torch.empty(P, I // 128, dtype=torch.float32, device=dev)
