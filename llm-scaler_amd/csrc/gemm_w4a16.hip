@@ -60,7 +60,6 @@ constexpr int kPitch = kBK + 8;                      // elements per LDS row (14
 
 template <class Act, int BM, int BN>
 __global__ __launch_bounds__(256) void gemm_w4a16_kernel(const GemmArgs p) {
-  using V8 = typename Act::v8;
   using Elem = typename Act::elem;
   constexpr int WM = BM / 2, WN = BN / 2;             // wave sub-tile
   constexpr int TM = WM / 16, TN = WN / 16;

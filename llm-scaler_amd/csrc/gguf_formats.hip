@@ -8,6 +8,7 @@
 // Dequant: resident representation -> dense fp16 with the reference's fp16
 // roundings.  GEMV: the one-wavefront-per-row decode kernel, fp16 only.
 #include "gemv_rows.hpp"
+#include "gguf_skinny.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -335,6 +336,9 @@ static int run_gguf_gemv(RowsArgs r, int M, hipStream_t st) {
   if (M < 0 || r.N[0] < 0 || r.K <= 0) return MI_ERR_SHAPE;
   if ((uint64_t)r.N[0] * (uint64_t)r.K >= (1ull << 31)) return MI_ERR_SHAPE;
   if (M == 0 || r.N[0] == 0) return MI_OK;
+  // more than four rows: the MFMA kernel (64 rows per pass)
+  if (M > 4)
+    return gguf_skinny(FMT, r.x, r.w[0], r.h[0], r.s[0], r.z[0], r.out[0], M, r.N[0], r.K, st);
   // rows per launch: as many (4, 2, 1) as the staged activations allow in 64 KiB of LDS
   int step = 4;
   while (step > 1 && rows_lds_bytes(FMT, step, r.K) > 64 * 1024) step >>= 1;

@@ -159,6 +159,61 @@ __device__ __forceinline__ f16x8 q4kx8_to_f16(uint32_t w, _Float16 s, _Float16 m
   return out;
 }
 
+// Q8_0: eight signed bytes -> fp16(q) * s, one rounding.  0x6400 | (q ^ 0x80) = 1152 + q
+// exactly; the subtraction is exact, the product rounds once.
+__device__ __forceinline__ f16x8 i8x8_to_f16(uint32_t w0, uint32_t w1, _Float16 s) {
+#pragma clang fp contract(off)
+  const f16x2 k1152 = {(_Float16)1152.0f, (_Float16)1152.0f};
+  const f16x2 sv = {s, s};
+  f16x8 out;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const uint32_t u = (p < 2 ? w0 : w1) ^ 0x80808080u;
+    const uint32_t sel = (p & 1) ? 0x04030402u : 0x04010400u;
+    f16x2 v = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, u, sel));
+    v = (v - k1152) * sv;
+    out[2 * p] = v[0];
+    out[2 * p + 1] = v[1];
+  }
+  return out;
+}
+
+// Q5_K (BITS = 1) / Q6_K (BITS = 2): eight nibbles in w plus their high bits — bytes of hA
+// (elements 0..3) and hB (elements 4..7), the field starting at bit `shift` of each byte.
+//   Q5_K: fp16(fp16(v * s) - m) with v = nib + 16 h (two roundings, like Q4_K);
+//   Q6_K: (v - 32) * s with v = nib + 16 h (exact difference, one rounding; m unused).
+template <int BITS>
+__device__ __forceinline__ f16x8 kqx8_to_f16(uint32_t w, uint32_t hA, uint32_t hB, uint32_t shift, _Float16 s,
+                                             _Float16 m) {
+#pragma clang fp contract(off)
+  constexpr uint32_t mask = BITS == 1 ? 0x01010101u : 0x03030303u;
+  const uint32_t e = w & 0x0F0F0F0Fu;
+  const uint32_t o = (w >> 4) & 0x0F0F0F0Fu;
+  const uint32_t a = (hA >> shift) & mask, bq = (hB >> shift) & mask;
+  const f16x2 sv = {s, s};
+  const f16x2 mv = {m, m};
+  const f16x2 base = BITS == 1 ? f16x2{(_Float16)1024.0f, (_Float16)1024.0f} : f16x2{(_Float16)1056.0f, (_Float16)1056.0f};
+  f16x8 out;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const uint32_t sel = 0x0C000C00u | ((4u + p) << 16) | (uint32_t)p;
+    // elements 2p, 2p+1: their high-bit bytes are bytes (2p % 4), (2p % 4) + 1 of hA (p < 2) or hB
+    const uint32_t hsrc = p < 2 ? a : bq;
+    const uint32_t hsel = (p & 1) ? 0x0C030C02u : 0x0C010C00u;
+    const uint32_t hi = __builtin_amdgcn_perm(hsrc, hsrc, hsel) << 4;
+    const uint32_t bits = __builtin_amdgcn_perm(o, e, sel) | 0x64006400u | hi;
+    f16x2 v = __builtin_bit_cast(f16x2, bits) - base;
+    f16x2 prod = v * sv;
+    if constexpr (BITS == 1) {
+      asm volatile("" : "+v"(prod));                  // keep the product as its own rounded value
+      prod = prod - mv;
+    }
+    out[2 * p] = prod[0];
+    out[2 * p + 1] = prod[1];
+  }
+  return out;
+}
+
 // Sum over the 64 lanes with DPP (cross-lane operands inside the VALU, no LDS
 // round trips): butterfly inside each row of 16 lanes, then the four row totals
 // are read out with v_readlane.  Every lane returns the same total.

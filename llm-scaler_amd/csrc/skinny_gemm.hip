@@ -1,380 +1,10 @@
-// Weight-streaming ("skinny") quantized GEMV / small-M GEMM for gfx950.
-//
-// Regime: M <= 64 rows of activations against an [N, K] quantized weight.  The
-// weight is read exactly once at full HBM rate; everything else (activations,
-// scales) comes out of L2.  One workgroup owns up to 64 output columns (weight
-// rows, in 16-row tiles) and all of K; its NW wavefronts interleave 128-wide K granules so that the
-// workgroup as a whole walks each weight row front to back, and every lane
-// issues 128-bit loads.  Weights are dequantized in registers to the activation
-// type and fed to v_mfma_f32_16x16x32_{f16,bf16} with the activations as the A
-// operand (M padded to 16 inside the matrix core — free while HBM-bound).  The
-// NW partial accumulators are reduced through LDS.
-//
-// Global loads are row-coalesced: consecutive lanes read one row's contiguous
-// bytes of a granule (loading MFMA operand layout directly makes every lane touch
-// a different 16-byte piece, and the texture addresser, not HBM, becomes the
-// limit), and a wave-private LDS tile turns them into operand layout.  The
-// weights always take this path (non-temporal loads); the activations only when
-// there are many rows (M > 32) — for few rows their direct loads are cheaper than
-// the extra LDS traffic.
-//
-// Lane mapping inside one granule (128 k): lane = (j = lane % 16, g = lane / 16)
-// holds the 32 consecutive k  [128 gi + 32 g, +32)  of weight row n0 + j and of
-// activation row j.  MFMA i (0..3) consumes the i-th 8-k slice of both.
-#include "qlinear_common.hpp"
-#include "gemv_rows.hpp"
+// Entry points of the weight-streaming GEMV / small-M GEMM for FP8 (per-channel, per-tensor,
+// 128x128 block), INT4 group 128 and GGUF Q4_K: M <= 4 takes the one-wavefront-per-row
+// kernel (gemv_rows.hpp), larger M the MFMA kernel (skinny_kernel.hpp).
+#include "skinny_kernel.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
-
-constexpr int kMaxMat = 3;
-
-struct SkinnyArgs {
-  const void* x;
-  const void* w[kMaxMat];
-  const void* s[kMaxMat];     // scales (format specific)
-  const void* z[kMaxMat];     // int4: zero-points (may be null); q4k: mins
-  void* out[kMaxMat];
-  int N[kMaxMat];
-  int tiles[kMaxMat];         // 16-row tiles per matrix
-  int nmat;
-  int M, K;
-  int rpw;                    // weight rows owned by one workgroup (<= 16 RT)
-  int scale_f16;              // fp8 per-channel: scale is fp16 instead of fp32
-};
-
-enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
-
-// ---------------------------------------------------------------- kernel
-// FMT: 0 = fp8 (SC selects the scale mode), 1 = int4 g128, 2 = Q4_K repacked.
-// MT = 16-row activation tiles (M <= 16 MT), RT = 16-row weight tiles per
-// workgroup, NW = wavefronts splitting K, UN = granules in flight per wave.
-template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
-__global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
-  using V8 = typename Act::v8;
-  using Elem = typename Act::elem;
-  constexpr bool kIsFp8 = (FMT == 0);
-  constexpr bool kIsInt4 = (FMT == 1);
-  constexpr bool kIsQ4K = (FMT == 2);
-  constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
-
-  // wave-private staging tiles for the weights (one 16-row tile = 16 rows of one
-  // granule, padded pitch); the cross-wave reduction buffer overlays them at the end
-  constexpr int kWRowB = kIsFp8 ? 128 : 64;           // weight bytes per row per granule
-  constexpr int kWP = kWRowB + 16;                    // LDS pitch: operand reads hit distinct banks
-  constexpr int kXP = 256 + 16;                       // activation tile pitch
-  constexpr bool kXLds = MT >= 4;                     // stage the activations through LDS too
-  constexpr int kWStage = NW * RT * 16 * kWP;         // activation tiles follow the weight tiles
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
-
-  int tile = blockIdx.x;
-  int mat = 0;
-#pragma unroll
-  for (int i = 0; i + 1 < kMaxMat; ++i) {
-    if (mat == i && i + 1 < a.nmat && tile >= a.tiles[i]) { tile -= a.tiles[i]; mat = i + 1; }
-  }
-  const int N = a.N[mat];
-  const int K = a.K, M = a.M;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int j = lane & 15, g = lane >> 4;
-  const int n0 = tile * a.rpw;
-  const int nend = min(N, n0 + a.rpw);                // rows past it belong to the next workgroup
-  const int G = (K + 127) >> 7;
-
-  const uint32_t wrow = kIsFp8 ? (uint32_t)K : ((uint32_t)K >> 1);
-  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
-  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
-
-  const _Float16* s16 = (const _Float16*)a.s[mat];
-  const float* s32 = (const float*)a.s[mat];
-  const uint8_t* zp = (const uint8_t*)a.z[mat];
-  const _Float16* qmin = (const _Float16*)a.z[mat];
-  const int Kg = K >> 7;                             // int4 groups per row
-  const int Kb32 = K >> 5;                           // q4k sub-blocks per row
-  const int Kb = G;                                  // fp8 block columns
-
-  f32x4 acc[RT][MT];
-#pragma unroll
-  for (int t = 0; t < RT; ++t)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // Out-of-range granules / lanes / rows load zeros for both operands, so the
-  // loop body needs no branches: a zero weight times a zero activation adds 0.
-  //
-  // A stage = U granules of this wavefront (gbase, gbase + NW, ...): their loads, and
-  // later their conversion + MFMAs.  With UN >= 2 the granules of a turn are split into
-  // two stages in a ring, so that the loads of the next stage are in flight while the
-  // current one is consumed (continuous streaming instead of load bursts).
-  constexpr int US = UN >= 2 ? UN / 2 : UN;           // granules per stage
-  struct Stage {
-    u32x4 wa[US][RT], wb[US][RT];
-    u32x4 xa[US][MT][4];
-    uint32_t sc[US][RT];                              // raw bits: int4 / q4k scale (fp16), block scale (fp32)
-    uint32_t zz[US][RT];                              // raw: int4 zero-point byte / q4k min (fp16)
-  };
-  const uint16_t* s16u = reinterpret_cast<const uint16_t*>(s16);
-  const uint16_t* qminu = reinterpret_cast<const uint16_t*>(qmin);
-  const uint8_t* zsrc = zp ? zp : reinterpret_cast<const uint8_t*>(s16);   // always a readable address
-  const bool has_zp = zp != nullptr;
-
-  auto load_stage = [&](Stage& st, int gbase) {
-#pragma unroll
-    for (int u = 0; u < US; ++u) {
-      const int gi = gbase + u * NW;
-      const int kl = gi * 128 + g * 32;
-      const bool ok = (gi < G) && (kl < K);
-      const int gic = gi < G ? gi : G - 1;
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const int n = n0 + t * 16 + j;
-        const int nc = n < N ? n : N - 1;
-        // weights: row-coalesced (consecutive lanes read one row's contiguous bytes);
-        // they are turned into operand layout through LDS before use
-        if constexpr (kIsFp8) {
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const int r = (lane >> 3) + 8 * h, c = lane & 7;
-            const int nr = n0 + t * 16 + r;
-            const bool okw = gi < G && gi * 128 + c * 16 < K && nr < nend;
-            // non-temporal: the weights are used once and should not displace x in L2
-            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(
-                wr, okw ? (uint32_t)nr * wrow + (uint32_t)(gi * 128 + c * 16) : kOOB, 0, 2);
-            if (h == 0) st.wa[u][t] = v; else st.wb[u][t] = v;
-          }
-        } else {
-          const int r = lane >> 2, c = lane & 3;
-          const int nr = n0 + t * 16 + r;
-          const bool okw = gi < G && gi * 128 + c * 32 < K && nr < nend;
-          st.wa[u][t] = __builtin_amdgcn_raw_buffer_load_b128(
-              wr, okw ? (uint32_t)nr * wrow + (uint32_t)(gi * 64 + c * 16) : kOOB, 0, 2);
-        }
-        // side data stays raw until it is used: a conversion here would wait for the load,
-        // and with it for every older load in flight
-        if constexpr (kIsInt4) {
-          st.sc[u][t] = s16u[(size_t)nc * Kg + gic];
-          st.zz[u][t] = zsrc[(size_t)nc * Kg + gic];
-        } else if constexpr (kIsQ4K) {
-          const int sb = gic * 4 + g;
-          const int sbc = sb < Kb32 ? sb : Kb32 - 1;
-          st.sc[u][t] = s16u[(size_t)nc * Kb32 + sbc];
-          st.zz[u][t] = qminu[(size_t)nc * Kb32 + sbc];
-        } else if constexpr (kBlock) {
-          st.sc[u][t] = reinterpret_cast<const uint32_t*>(s32)[(size_t)(min(n0 + t * 16, N - 1) >> 7) * Kb + gic];
-        }
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if constexpr (kXLds) {
-          // many rows: row-coalesced as well (16 lanes read one row's 256 contiguous
-          // bytes of the granule), transposed through LDS before use
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int r = (lane >> 4) + 4 * i, c = lane & 15;
-            const int m = mt * 16 + r;
-            const bool okx = gi < G && gi * 128 + c * 8 < K && m < M;
-            st.xa[u][mt][i] = buf_load16(xr, okx ? ((uint32_t)m * (uint32_t)K + (uint32_t)(gi * 128 + c * 8)) * 2u : kOOB);
-          }
-        } else {
-          // few rows: straight into operand layout (lane (j, g): row j, 32 consecutive k)
-          const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) st.xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
-        }
-      }
-    }
-  };
-
-  auto compute_stage = [&](Stage& st) {
-#pragma unroll
-    for (int u = 0; u < US; ++u) {
-      // activations through this wavefront's staging tile into MFMA operand layout:
-      // lane (j, g) ends up with row j, k = 32 g + 8 i .. + 7 of the granule
-#pragma unroll
-      for (int mt = 0; mt < (kXLds ? MT : 0); ++mt) {
-        unsigned char* xl = smem + kWStage + (wave * MT + mt) * 16 * kXP;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          *reinterpret_cast<u32x4*>(xl + ((lane >> 4) + 4 * i) * kXP + (lane & 15) * 16) = st.xa[u][mt][i];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          st.xa[u][mt][i] = *reinterpret_cast<const u32x4*>(xl + j * kXP + g * 64 + i * 16);
-      }
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        // through this wavefront's staging tile into MFMA operand layout
-        unsigned char* wl = smem + (wave * RT + t) * 16 * kWP;
-        u32x4 wa = st.wa[u][t], wb = st.wb[u][t];
-        if constexpr (kIsFp8) {
-          *reinterpret_cast<u32x4*>(wl + (lane >> 3) * kWP + (lane & 7) * 16) = wa;
-          *reinterpret_cast<u32x4*>(wl + ((lane >> 3) + 8) * kWP + (lane & 7) * 16) = wb;
-          wa = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32);
-          wb = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 32 + 16);
-        } else {
-          *reinterpret_cast<u32x4*>(wl + (lane >> 2) * kWP + (lane & 3) * 16) = wa;
-          wa = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 16);
-        }
-        V8 b[4];
-        float scf = 0.f;
-        if constexpr (kIsFp8) {
-          b[0] = fp8x8_to_act<Act>(wa[0], wa[1]);
-          b[1] = fp8x8_to_act<Act>(wa[2], wa[3]);
-          b[2] = fp8x8_to_act<Act>(wb[0], wb[1]);
-          b[3] = fp8x8_to_act<Act>(wb[2], wb[3]);
-          if constexpr (kBlock) scf = __builtin_bit_cast(float, st.sc[u][t]);
-        } else if constexpr (kIsInt4) {
-          const float sf = (float)__builtin_bit_cast(_Float16, (uint16_t)st.sc[u][t]);
-          const float zf = has_zp ? (float)st.zz[u][t] : 8.0f;
-          if constexpr (Act::dt == DT_F16) {
-            const _Float16 s = (_Float16)sf;
-            const _Float16 z = (_Float16)(1024.0f + zf);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_f16(wa[i], s, z);
-          } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = int4x8_to_bf16(wa[i], sf, zf);
-          }
-        } else {
-          if constexpr (Act::dt == DT_F16) {
-            const _Float16 s = __builtin_bit_cast(_Float16, (uint16_t)st.sc[u][t]);
-            const _Float16 mn = __builtin_bit_cast(_Float16, (uint16_t)st.zz[u][t]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = q4kx8_to_f16(wa[i], s, mn);
-          }
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          if constexpr (kBlock) {
-            f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) tt = Act::mfma(as_v8<V8>(st.xa[u][mt][i]), b[i], tt);
-            acc[t][mt] += tt * scf;
-          } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              acc[t][mt] = Act::mfma(as_v8<V8>(st.xa[u][mt][i]), b[i], acc[t][mt]);
-          }
-        }
-      }
-    }
-  };
-
-  if constexpr (UN >= 2) {
-    // two-stage ring; the only exit is at the bottom (stages past the end load zeros)
-    Stage s0, s1;
-    load_stage(s0, wave);
-    for (int gbase = wave; gbase < G; gbase += NW * UN) {
-      load_stage(s1, gbase + NW * US);
-      __builtin_amdgcn_sched_barrier(0);
-      compute_stage(s0);
-      load_stage(s0, gbase + NW * UN);
-      __builtin_amdgcn_sched_barrier(0);
-      compute_stage(s1);
-    }
-  } else {
-    Stage s0;
-    for (int gbase = wave; gbase < G; gbase += NW * UN) {
-      load_stage(s0, gbase);
-      __builtin_amdgcn_sched_barrier(0);
-      compute_stage(s0);
-    }
-  }
-
-  // ---- reduce the NW partial tiles through LDS ----
-  __syncthreads();                                    // the buffer overlays the staging tiles
-  if (wave > 0) {
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) red[wave - 1][t][mt][lane] = acc[t][mt];
-  }
-  __syncthreads();
-  if (wave != 0) return;
-#pragma unroll
-  for (int w = 0; w < NW - 1; ++w)
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[t][mt] += red[w][t][mt][lane];
-
-  // D layout: lane holds output column n0 + 16 t + j, rows mt*16 + 4 g + v.
-  Elem* out = (Elem*)a.out[mat];
-#pragma unroll
-  for (int t = 0; t < RT; ++t) {
-    const int n = n0 + t * 16 + j;
-    if (n < nend) {
-      float os = 1.0f;
-      if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[n] : s32[n];
-      if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int m = mt * 16 + g * 4 + v;
-          if (m < M) out[(size_t)m * N + n] = Act::from_f32(acc[t][mt][v] * os);
-        }
-    }
-  }
-}
-
-template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
-static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
-  int tiles = 0;
-  a.rpw = rpw;
-  for (int i = 0; i < a.nmat; ++i) {
-    a.tiles[i] = (a.N[i] + rpw - 1) / rpw;
-    tiles += a.tiles[i];
-  }
-  if (tiles == 0) return;
-  constexpr int kStage = NW * RT * 16 * ((FMT == 0 ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
-  constexpr int kRed = (NW - 1) * RT * MT * 1024;
-  constexpr int lds = kStage > kRed ? kStage : kRed;
-  auto kern = skinny_kernel<Act, FMT, SC, MT, RT, NW, UN>;
-  if (lds > 64 * 1024) {
-    static bool raised = false;                       // opt in to > 64 KiB of dynamic LDS once
-    if (!raised) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      raised = true;
-    }
-  }
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(NW * 64), lds, st, a);
-}
-
-template <class Act, int FMT, int SC>
-static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
-  if (a.M == 0) return MI_OK;
-  {
-    // One workgroup per CU and round, R weight rows each (a multiple of 8, at most
-    // 64): wide workgroups re-read the activations from L2 least often, and an
-    // exact multiple of the CU count leaves no partial last round.  Rows of a
-    // workgroup's last 16-row tile beyond R are dead lanes that load nothing.
-    long ntot = 0;
-    for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
-    const int cus = device_cu_count();
-    int rounds = (int)((ntot + (long)cus * 64 - 1) / ((long)cus * 64));
-    if (rounds < 1) rounds = 1;
-    int rpw = (int)((ntot + (long)cus * rounds - 1) / ((long)cus * rounds));
-    // block scales: tiles must not straddle a 128-row scale block
-    rpw = (FMT == 0 && SC == SC_BLOCK) ? ((rpw + 15) & ~15) : ((rpw + 7) & ~7);
-    if (rpw > 64) rpw = 64;
-    if (rpw <= 16) {
-      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 1, 8, 4>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 1, 8, 2>(a, rpw, st);
-      else launch_one<Act, FMT, SC, 4, 1, 8, 1>(a, rpw, st);
-    } else if (rpw <= 32) {
-      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
-      else launch_one<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
-    } else {
-      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 4, 4, 1>(a, rpw, st);
-      else launch_one<Act, FMT, SC, 4, 4, 4, 1>(a, rpw, st);
-    }
-  }
-  return launch_status();
-}
 
 // Runs M in chunks of 64 rows (the skinny kernel's limit); each chunk streams
 // the weight once, so this is meant for decode-sized M.

@@ -130,7 +130,8 @@ def _gemv(s, kind, x, rep, out, name=None):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 512), (1, 1000, 4096), (1, 520, 5120), (2, 96, 2048), (3, 33, 1024),
-                                   (4, 256, 8192), (1, 40, 14336), (7, 48, 1536), (16, 130, 2048)])
+                                   (4, 256, 8192), (1, 40, 14336), (7, 48, 1536), (16, 130, 2048), (33, 72, 1024),
+                                   (64, 520, 5120), (100, 40, 512)])
 def test_gemv(ops, dev, kind, M, N, K):
     _, s = ops
     raw = _raw_case(kind, N, K, seed=7 * M + N + K)
@@ -158,10 +159,12 @@ def test_small_m_variants(ops, dev, name, kind):
     assert O.max_rel_err(out.cpu(), O.matmul_ref(x, wd)) < TOL
 
 
+@pytest.mark.parametrize("M", [1, 8])
 @pytest.mark.parametrize("kind", ["q5_k", "q6_k"])
-def test_gemv_every_high_bit_field(ops, dev, kind):
+def test_gemv_every_high_bit_field(ops, dev, kind, M):
     # weights whose low nibbles are zero: the output depends on the high bits alone,
-    # one 64- (Q5_K) or 128-element (Q6_K) field of one 512-tile at a time
+    # one 64- (Q5_K) or 128-element (Q6_K) field of one 512-tile at a time (M = 1: the row
+    # kernel, M = 8: the MFMA kernel)
     _, s = ops
     N, K = 16, 1024
     span = 64 if kind == "q5_k" else 128
@@ -175,8 +178,8 @@ def test_gemv_every_high_bit_field(ops, dev, kind):
             raw = G.q6k_build_raw(v, np.ones((N, K // 256, 16), np.int8), np.full((N, K // 256), 0.5, np.float16))
         rep = _repack_oracle(kind, raw)
         wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32))
-        x = torch.randn(1, K, generator=torch.Generator().manual_seed(f)).half()
-        out = torch.empty(1, N, dtype=torch.float16, device=dev)
+        x = torch.randn(M, K, generator=torch.Generator().manual_seed(f)).half()
+        out = torch.empty(M, N, dtype=torch.float16, device=dev)
         _gemv(s, kind, x.to(dev), [_t(a).to(dev) for a in rep], out)
         assert O.max_rel_err(out.cpu(), O.matmul_ref(x, wd)) < TOL, f"field {f}"
 
