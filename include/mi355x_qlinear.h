@@ -295,6 +295,28 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
                           int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,
                           int out_f32, void* stream);
 
+/* The same GEMM with the per-expert-scalar scale of the reference's per-tensor MoE
+ * kernels and their epilogues:
+ *   scale_per_expert = 1: w_scale is [E] fp32 (one factor per expert); K may then be
+ *     any multiple of 16 (the chunks of the last 128-granule past K read as zeros).
+ *     scale_per_expert = 0: block scales [E, ceil(N/128), ceil(K/128)] as above.
+ *   fuse_act: 0 none, 1 silu(gate) * up, 2 gelu_tanh(gate) * up (exp argument held in
+ *     [-30, 30]); gate = weight rows [0, N/2), up = rows [N/2, N); N/2 need not be a
+ *     multiple of 128.
+ *   out_map (optional, [total_rows] int32): the row of expert-sorted position r is
+ *     written to out[out_map[r]] (the reference's kernels write pair order themselves);
+ *   row_weight (optional, activation dtype, indexed by destination row): the row is
+ *     multiplied by it before rounding (routing weight of the down projection).
+ * Replaces moe_up_fp8_grouped_gelu_tanh_kernel / moe_down_fp8_grouped_kernel
+ * (V/csrc/moe_batch/moe_fp8_grouped.h:98-245, :247-341), moe_up_routed_e4m3_gelu_tanh_kernel
+ * / moe_down_routed_e4m3_vllm_layout_kernel (V/csrc/moe_batch/moe.sycl:458-558, :870-924)
+ * and the scatter at the end of the sglang prefill kernels
+ * (S/csrc/moe_prefill/moe_prefill_fp8.sycl:280-300, :385-411). */
+int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
+                            const float* w_scale, int scale_per_expert, const int32_t* expert_start, void* out,
+                            const int32_t* out_map, const void* row_weight, int a_rows, int total_rows, int E,
+                            int N, int K, int fuse_act, int act_dtype, int out_f32, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

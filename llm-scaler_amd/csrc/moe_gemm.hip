@@ -16,8 +16,13 @@
 //             acc += (A8 . W8)_granule * xs[row, g] * ws[n / 128, g]
 //   A16 : fp16 / bf16 activations (w8a16, the reference's mode): weights are
 //         converted exactly to 16 bit and ws is applied to the granule partial.
-// Optional fused epilogue: SiLU(gate) * up, where a workgroup pairs weight row n
-// (gate) with row n + N/2 (up) and writes N/2 columns.
+// The weight scale is one value per 128 x 128 block or one per expert.  K may end
+// in a partial granule (any multiple of 16): the chunks past K are loaded as zeros
+// on both operands.
+// Optional fused epilogue: act(gate) * up with act = SiLU or tanh-GELU, where a
+// workgroup pairs weight row n (gate) with row n + N/2 (up) and writes N/2 columns.
+// Output rows may be scattered through a map (sorted position -> destination row)
+// and scaled by a per-destination-row weight.
 #include "qlinear_common.hpp"
 #include "../../include/mi355x_qlinear.h"
 
@@ -28,10 +33,14 @@ struct MoeGemmArgs {
   const float* a_scale;       // A8: [rows, K/128]
   const int32_t* row_map;     // optional: sorted position -> source row of `a` / `a_scale`
   const void* w;              // [E, N, K] e4m3
-  const float* w_scale;       // [E, ceil(N/128), K/128]
+  const float* w_scale;       // [E, ceil(N/128), ceil(K/128)], or [E]
   const int32_t* start;       // [E+1]
   void* out;                  // [total_rows, N_out], activation dtype or fp32 (out_f32)
+  const int32_t* out_map;     // optional: sorted position -> row of `out`
+  const void* row_weight;     // optional, activation dtype: factor per row of `out`
   int out_f32;
+  int gelu;                   // fused epilogue: tanh-GELU instead of SiLU
+  int s_e, s_nb, s_g;         // w_scale strides: expert, 128-row block, granule (0, 0 = per expert)
   int E, N, K;                // N = weight rows per expert
   int n_out;                  // output columns (N, or N/2 with the fused SiLU*mul)
   int tiles_per_expert;       // workgroups per expert
@@ -89,7 +98,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 15, g = lane >> 4;
   const int K = p.K, N = p.N;
-  const int G = K >> 7, Kb = G;
+  const int G = (K + 127) >> 7, Kb = G;
+  const int ktail = K - ((G - 1) << 7);               // k extent of the last granule (128 = whole)
   const int half = N >> 1;
   const int limit = SILU ? half : N;                  // columns
   const int groups = (limit + kCols - 1) / kCols;     // tile groups per expert
@@ -103,13 +113,14 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
 
   // cooperative weight staging slots of this thread
   uint32_t wvoff[WL];
-  int wcol[WL];
+  int wcol[WL], wch[WL];
   unsigned char* wlds[WL];
 #pragma unroll
   for (int i = 0; i < WL; ++i) {
     const int c = tid + 256 * i;
     const int row = c >> 3, t = row >> 4, r = row & 15, ch = c & 7;
     wcol[i] = col0 + tile_col(t) + r;
+    wch[i] = ch * 16;
     wvoff[i] = (uint32_t)(tile_hi(t) + wcol[i]) * (uint32_t)K + (uint32_t)ch * 16u;
     wlds[i] = smem + row * kWPitch + ch * 16;
   }
@@ -123,7 +134,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   const int Nb = (N + 127) >> 7;
   // read through a restrict kernel argument so the (uniform) scale loads stay on the
   // scalar unit and do not queue behind the vector prefetch
-  const float* __restrict__ wsc = w_scale + (size_t)e * Nb * Kb;
+  const float* __restrict__ wsc = w_scale + (size_t)e * p.s_e;
+  const int s_nb = p.s_nb, s_g = p.s_g;
   const uint32_t tg_stride = (uint32_t)kCols * (uint32_t)K;   // weight bytes between tile groups
 
   struct Regs {                                       // one granule in flight
@@ -145,6 +157,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       xsoff = (src * (uint32_t)Kb * 4u) | ((uint32_t)(!ok) << 31);
     }
     uint32_t aoff[NAI];
+    int ach[NAI];
     unsigned char* alds[NAI];
 #pragma unroll
     for (int i = 0; i < NAI; ++i) {
@@ -156,20 +169,23 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
       aoff[i] = (src * (uint32_t)K * a_esz + (uint32_t)ch * 16u) | ((uint32_t)(!ok) << 31);
       alds[i] = al + row * APitch + ch * 16;
+      ach[i] = A8 ? ch * 16 : ch * 8;                 // first k of the chunk inside the granule
     }
 
     // issue the loads of granule gi of tile group tg (dead beyond the last one)
     auto load_granule = [&](Regs& r, int tg, int gi) {
       const uint32_t dead = tg < ntg ? 0u : 0x80000000u;
       const uint32_t wso = (uint32_t)tg * tg_stride + (uint32_t)gi * 128u;
+      const int kext = gi == G - 1 ? ktail : 128;     // uniform
 #pragma unroll
       for (int i = 0; i < WL; ++i) {
-        const bool ok = wcol[i] + tg * kCols < limit;
+        const bool ok = wcol[i] + tg * kCols < limit && wch[i] < kext;
         r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i] | dead | ((uint32_t)(!ok) << 31), wso, 2);
       }
 #pragma unroll
       for (int i = 0; i < NAI; ++i)
-        r.a[i] = __builtin_amdgcn_raw_buffer_load_b128(ar, aoff[i] | dead, (uint32_t)gi * AGran, 0);
+        r.a[i] = __builtin_amdgcn_raw_buffer_load_b128(ar, aoff[i] | dead | ((uint32_t)(ach[i] >= kext) << 31),
+                                                       (uint32_t)gi * AGran, 0);
       if constexpr (A8)
         r.xs = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xsr, xsoff | dead, (uint32_t)gi * 4u, 0));
     };
@@ -214,7 +230,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
           float sc[RT];
 #pragma unroll
           for (int t = 0; t < RT; ++t) {
-            const float ws = wsc[(size_t)nb[t] * Kb + gi];
+            const float ws = wsc[nb[t] * s_nb + gi * s_g];
             sc[t] = A8 ? xs_now * ws : ws;
           }
           // prefetch D granules ahead, across the tile-group boundary
@@ -275,7 +291,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       if (active && m < cnt) {
         Elem* out = (Elem*)p.out;
         float* out32 = (float*)p.out;
-        const size_t orow = (size_t)(r0 + m) * p.n_out;
+        const int dst = p.out_map ? p.out_map[r0 + m] : r0 + m;
+        const size_t orow = (size_t)dst * p.n_out;
+        const float rw = p.row_weight ? Act::to_f32(((const Elem*)p.row_weight)[dst]) : 1.0f;
         constexpr int NO = SILU ? RT / 2 : RT;
 #pragma unroll
         for (int o = 0; o < NO; ++o) {
@@ -286,9 +304,17 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
           for (int v = 0; v < 4; ++v) {
             if constexpr (SILU) {
               const float gate = acc[t][v], up = acc[t + 1][v];
-              v4[v] = gate / (1.0f + __expf(-gate)) * up;
+              if (p.gelu) {
+                // 0.5 g (1 + tanh z), tanh through exp(2z) with 2z held in [-30, 30]
+                float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
+                two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
+                const float ex = __expf(two_z);
+                v4[v] = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up * rw;
+              } else {
+                v4[v] = gate / (1.0f + __expf(-gate)) * up * rw;
+              }
             } else {
-              v4[v] = acc[t][v];
+              v4[v] = acc[t][v] * rw;
             }
           }
           if (n + 3 < limit && (p.n_out & 3) == 0) {
@@ -329,7 +355,7 @@ static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
 
 template <class Act, bool A8, bool SILU>
 static int dispatch_moe2(const MoeGemmArgs& p, hipStream_t st) {
-  const int G = p.K / 128;
+  const int G = (p.K + 127) / 128;
   const int cols = SILU ? p.N / 2 : p.N;
   // Wide workgroups (8 weight tiles) re-read the expert's activation rows least
   // often; narrower ones keep the device filled when there are few tiles.
@@ -354,14 +380,16 @@ using namespace qlin;
 
 extern "C" {
 
-int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
-                          const float* w_scale, const int32_t* expert_start, void* out, int a_rows,
-                          int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,
-                          int out_f32, void* stream) {
+int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
+                            const float* w_scale, int scale_per_expert, const int32_t* expert_start, void* out,
+                            const int32_t* out_map, const void* row_weight, int a_rows, int total_rows, int E,
+                            int N, int K, int fuse_act, int act_dtype, int out_f32, void* stream) {
   if (!a || !w || !w_scale || !expert_start || !out) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (E < 0 || N <= 0 || K <= 0 || (K % 128) || a_rows < 0 || total_rows < 0) return MI_ERR_SHAPE;
-  if (fuse_silu_mul && (N % 2)) return MI_ERR_SHAPE;
+  if (fuse_act < 0 || fuse_act > 2) return MI_ERR_ARG;
+  if (E < 0 || N <= 0 || K <= 0 || (K % 16) || a_rows < 0 || total_rows < 0) return MI_ERR_SHAPE;
+  if (a_scale && (K % 128)) return MI_ERR_SHAPE;      // quantised activations carry whole 128-groups
+  if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || (uint64_t)a_rows * (uint64_t)K * 2 >= (1ull << 31))
     return MI_ERR_SHAPE;
   if (!E || !total_rows) return MI_OK;
@@ -369,14 +397,27 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
   p.a = a; p.a_scale = a_scale; p.row_map = row_map; p.w = w; p.w_scale = w_scale;
   p.start = expert_start; p.out = out; p.E = E; p.N = N; p.K = K; p.a_rows = a_rows;
   p.total_rows = total_rows;
+  p.out_map = out_map; p.row_weight = row_weight;
   p.out_f32 = out_f32;
+  p.gelu = fuse_act == 2;
+  const int Kb = (K + 127) / 128, Nb = (N + 127) / 128;
+  if (scale_per_expert) { p.s_e = 1; p.s_nb = 0; p.s_g = 0; }
+  else { p.s_e = Nb * Kb; p.s_nb = Kb; p.s_g = 1; }
   hipStream_t st = (hipStream_t)stream;
   if (a_scale) {
-    return act_dtype == DT_F16 ? dispatch_moe<ActF16, true>(p, fuse_silu_mul, st)
-                               : dispatch_moe<ActBF16, true>(p, fuse_silu_mul, st);
+    return act_dtype == DT_F16 ? dispatch_moe<ActF16, true>(p, fuse_act, st)
+                               : dispatch_moe<ActBF16, true>(p, fuse_act, st);
   }
-  return act_dtype == DT_F16 ? dispatch_moe<ActF16, false>(p, fuse_silu_mul, st)
-                             : dispatch_moe<ActBF16, false>(p, fuse_silu_mul, st);
+  return act_dtype == DT_F16 ? dispatch_moe<ActF16, false>(p, fuse_act, st)
+                             : dispatch_moe<ActBF16, false>(p, fuse_act, st);
+}
+
+int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
+                          const float* w_scale, const int32_t* expert_start, void* out, int a_rows,
+                          int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,
+                          int out_f32, void* stream) {
+  return mi_moe_gemm_fp8_grouped(a, a_scale, row_map, w, w_scale, 0, expert_start, out, nullptr, nullptr, a_rows,
+                                 total_rows, E, N, K, fuse_silu_mul ? 1 : 0, act_dtype, out_f32, stream);
 }
 
 }  // extern "C"

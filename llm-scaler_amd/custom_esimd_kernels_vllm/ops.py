@@ -169,6 +169,39 @@ def moe_forward_full_fp8_block(x, logits, gate_up_weight, gate_up_scale, shared_
         top_k, num_shared_experts, n_routed_experts)
 
 
+# ---- per-expert-scale FP8 MoE with the tanh-GELU gate (V/python/custom_esimd_kernels_vllm/ops.py:1693-1800)
+def moe_forward_full_gelu_tanh(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
+                               n_routed_experts):
+    return _moe.moe_forward_full_gelu_tanh(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                                           top_k, n_routed_experts)
+
+
+def moe_forward_full_fp8_grouped(x, gate_up_weight, gate_up_scale, down_weight, down_scale, routing_weights,
+                                 expert_offsets, expert_tokens, top_k, n_routed_experts):
+    return _moe.moe_forward_full_fp8_grouped(x, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                                             routing_weights, expert_offsets, expert_tokens, top_k,
+                                             n_routed_experts)
+
+
+def moe_forward_full_gelu_tanh_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight,
+                                      down_scale, top_k, n_routed_experts):
+    return _moe.moe_forward_full_gelu_tanh_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale,
+                                                  down_weight, down_scale, top_k, n_routed_experts)
+
+
+def moe_forward_full_gelu_tanh_routed_decode(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale,
+                                             down_weight, down_scale, top_k, n_routed_experts):
+    return _moe.moe_forward_full_gelu_tanh_routed_decode(x, topk_weights, topk_indices, gate_up_weight,
+                                                         gate_up_scale, down_weight, down_scale, top_k,
+                                                         n_routed_experts)
+
+
+def moe_forward_full_gelu_tanh_decode(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                                      per_expert_scale, top_k, n_routed_experts):
+    return _moe.moe_forward_full_gelu_tanh_decode(x, logits, gate_up_weight, gate_up_scale, down_weight,
+                                                  down_scale, per_expert_scale, top_k, n_routed_experts)
+
+
 def precompute_moe_route(topk_weights, topk_ids, num_experts):
     """Same contract as the reference helper: (sorted_rows, sorted_weights, rows_per_expert),
     stable by expert; computed on the device by the sort kernel."""

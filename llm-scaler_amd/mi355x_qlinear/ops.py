@@ -701,13 +701,27 @@ def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, t
     return final_hidden
 
 
-def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse, who):
+_ACT_NONE, _ACT_SILU, _ACT_GELU_TANH = 0, 1, 2
+
+
+def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse, who, *, per_expert=False,
+              out_map=None, row_weight=None):
+    """Grouped GEMM over expert-sorted rows.  fuse: False / True (SiLU) or one of _ACT_*.
+    per_expert: w_scale holds one fp32 per expert instead of 128x128 block scales.
+    out_map (int32): sorted position -> row of `out`; row_weight (activation dtype): factor
+    per row of `out`."""
     _chk_fp8(w, who)
     _chk(w.numel() == E * N * K, f"{who}: weight must be [num_experts, N, K]")
-    _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
-    _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and
-         w_scale.numel() == E * ((N + 127) // 128) * (K // 128),
-         f"{who}: weight_scale must be contiguous fp32 [E, ceil(N/128), K/128]")
+    fuse = int(fuse)
+    if per_expert:
+        _chk(K % 16 == 0, f"{who}: K={K} must be a multiple of 16")
+        _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() >= E,
+             f"{who}: weight_scale must be contiguous fp32 [E]")
+    else:
+        _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+        _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and
+             w_scale.numel() == E * ((N + 127) // 128) * (K // 128),
+             f"{who}: weight_scale must be contiguous fp32 [E, ceil(N/128), K/128]")
     _chk(expert_start.dtype in (torch.int32, torch.uint32) and expert_start.numel() >= E + 1,
          f"{who}: expert_idx must be int32/uint32 [num_experts+1]")
     _chk(out.dtype in (torch.float16, torch.bfloat16, torch.float32) and out.is_contiguous(),
@@ -720,9 +734,14 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
         _chk(out.dtype in (a.dtype, torch.float32), f"{who}: output must be fp32 or share the activation dtype")
     else:
         adt = capi.act_dtype(out) if out.dtype != torch.float32 else capi.DT_BF16
-    capi.call("mi_moe_gemm_fp8_block", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), capi.ptr(w),
-              capi.ptr(w_scale), capi.ptr(expert_start), capi.ptr(out), a_rows, total, E, N, K,
-              1 if fuse else 0, adt, 1 if out.dtype == torch.float32 else 0)
+    if out_map is not None:
+        _chk(out_map.dtype == torch.int32 and out_map.is_contiguous(), f"{who}: the output row map must be int32")
+    if row_weight is not None:
+        _chk(out.dtype != torch.float32 and row_weight.dtype == out.dtype and row_weight.is_contiguous() and
+             row_weight.numel() >= total, f"{who}: row weights must share the output dtype, one per output row")
+    capi.call("mi_moe_gemm_fp8_grouped", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), capi.ptr(w),
+              capi.ptr(w_scale), 1 if per_expert else 0, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map),
+              capi.ptr(row_weight), a_rows, total, E, N, K, fuse, adt, 1 if out.dtype == torch.float32 else 0)
     return out
 
 
@@ -1123,9 +1142,8 @@ def moe_prefill_up_forward_fp8(x, gate_up_weight, gate_up_scale, expert_offsets,
     start = _prefill_starts(expert_offsets, P)
     tokens = expert_tokens.contiguous()
     row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
-    inter_sorted = torch.empty(P, I, dtype=x.dtype, device=dev)
-    moe_gemm_fp8_block(x, None, row_map, gate_up_weight, bs, start, inter_sorted, two_i, H, E, True)
-    return _permute_rows(inter_sorted, tokens, torch.empty_like(inter_sorted), scatter=True)
+    out = torch.empty(P, I, dtype=x.dtype, device=dev)
+    return _moe_gemm(x, None, row_map, gate_up_weight, bs, start, out, E, two_i, H, _ACT_SILU, who, out_map=tokens)
 
 
 def moe_prefill_down_forward_fp8(intermediate, down_weight, down_scale, expert_offsets, expert_tokens):
@@ -1145,9 +1163,8 @@ def moe_prefill_down_forward_fp8(intermediate, down_weight, down_scale, expert_o
     bs = _expert_block_scales(down_scale, E, 1, H, I, who)
     start = _prefill_starts(expert_offsets, P)
     tokens = expert_tokens.contiguous()
-    y_sorted = torch.empty(P, H, dtype=intermediate.dtype, device=intermediate.device)
-    moe_gemm_fp8_block(intermediate, None, tokens, down_weight, bs, start, y_sorted, H, I, E, False)
-    return _permute_rows(y_sorted, tokens, torch.empty_like(y_sorted), scatter=True)
+    out = torch.empty(P, H, dtype=intermediate.dtype, device=intermediate.device)
+    return _moe_gemm(intermediate, None, tokens, down_weight, bs, start, out, E, H, I, _ACT_NONE, who, out_map=tokens)
 
 
 def moe_prefill_accumulate_forward_fp8(output, routing_weights):
@@ -1201,6 +1218,182 @@ def moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, 
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     moe_combine(y, inv, topk_weights.contiguous(), out, k)
     return out
+
+
+# --------------------------------------------------------------------------
+# per-expert-scale FP8 MoE with the tanh-GELU gate (moe_ops: the gemma-style family)
+# weights in the FusedMoE layout: gate_up [E, 2I, H], down [E, H, I] e4m3, scales [E] fp32
+# --------------------------------------------------------------------------
+def _chk_pert_moe(x, gate_up_weight, gate_up_scale, down_weight, down_scale, who):
+    _chk(x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(),
+         f"{who}: x must be contiguous fp16 (bf16 accepted) [T, H]")
+    if gate_up_weight is not None:
+        _chk(gate_up_weight.dim() == 3 and gate_up_weight.shape[1] % 2 == 0, f"{who}: gate_up_weight must be [E, 2*I, H]")
+        _chk_fp8(gate_up_weight, who)
+        _chk(gate_up_scale.dtype == torch.float32 and gate_up_scale.numel() >= gate_up_weight.shape[0],
+             f"{who}: gate_up_scale must be float32 [E]")
+    if down_weight is not None:
+        _chk(down_weight.dim() == 3, f"{who}: down_weight must be [E, H, I]")
+        _chk_fp8(down_weight, who)
+        _chk(down_scale.dtype == torch.float32 and down_scale.numel() >= down_weight.shape[0],
+             f"{who}: down_scale must be float32 [E]")
+
+
+def moe_up_fp8_grouped(x, gate_up_weight, gate_up_scale, expert_offsets, expert_tokens, top_k, n_routed_experts):
+    """intermediate[pair] = gelu_tanh(x[t] @ (s[e] w_gate[e])^T) * (x[t] @ (s[e] w_up[e])^T), pair = t*top_k + j,
+    for the pairs grouped per expert by (expert_offsets [E] exclusive, expert_tokens [T*top_k])
+    (V/csrc/moe_batch/moe_fp8_grouped.h:348-408).  -> [T*top_k, I] in pair order."""
+    who = "moe_up_fp8_grouped"
+    _chk_pert_moe(x, gate_up_weight, gate_up_scale, None, None, who)
+    _chk(expert_offsets.dtype == torch.int32 and expert_tokens.dtype == torch.int32, f"{who}: offsets and tokens must be int32")
+    E, two_i, H = gate_up_weight.shape
+    _chk(E == int(n_routed_experts) and x.shape[1] == H, f"{who}: x [T, H] against gate_up_weight [E, 2*I, H]")
+    k = int(top_k)
+    P = x.shape[0] * k
+    _chk(expert_tokens.numel() == P and expert_offsets.numel() >= E, f"{who}: expert_tokens must hold T*top_k pairs")
+    tokens = expert_tokens.contiguous()
+    row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
+    out = torch.empty(P, two_i // 2, dtype=x.dtype, device=x.device)
+    return _moe_gemm(x, None, row_map, gate_up_weight, gate_up_scale.contiguous(), _prefill_starts(expert_offsets[:E], P),
+                     out, E, two_i, H, _ACT_GELU_TANH, who, per_expert=True, out_map=tokens)
+
+
+def moe_down_fp8_grouped(intermediate, down_weight, down_scale, routing_weights, expert_offsets, expert_tokens,
+                         top_k, n_routed_experts):
+    """out[pair] = routing_weights[pair] * (intermediate[pair] @ (s[e] w2[e])^T), pair order in and out
+    (V/csrc/moe_batch/moe_fp8_grouped.h:410-433)."""
+    who = "moe_down_fp8_grouped"
+    _chk_pert_moe(intermediate, None, None, down_weight, down_scale, who)
+    _chk(expert_offsets.dtype == torch.int32 and expert_tokens.dtype == torch.int32, f"{who}: offsets and tokens must be int32")
+    E, H, I = down_weight.shape
+    P = intermediate.shape[0]
+    _chk(E == int(n_routed_experts) and intermediate.shape[1] == I, f"{who}: intermediate [T*top_k, I] against down_weight [E, H, I]")
+    _chk(routing_weights.dtype == intermediate.dtype and routing_weights.numel() == P and expert_tokens.numel() == P,
+         f"{who}: routing_weights and expert_tokens must hold one entry per pair, weights in the activation dtype")
+    tokens = expert_tokens.contiguous()
+    out = torch.empty(P, H, dtype=intermediate.dtype, device=intermediate.device)
+    return _moe_gemm(intermediate, None, tokens, down_weight, down_scale.contiguous(), _prefill_starts(expert_offsets[:E], P),
+                     out, E, H, I, _ACT_NONE, who, per_expert=True, out_map=tokens,
+                     row_weight=routing_weights.contiguous().reshape(-1))
+
+
+def moe_forward_full_fp8_grouped(x, gate_up_weight, gate_up_scale, down_weight, down_scale, routing_weights,
+                                 expert_offsets, expert_tokens, top_k, n_routed_experts):
+    """Up (tanh-GELU), down and the sum over each token's top_k routes in one call
+    (V/csrc/moe_batch/moe_fp8_grouped.h:471-500).  The intermediate stays in expert-sorted order and
+    the down output in fp32 until the weighted sum, which rounds once."""
+    who = "moe_forward_full_fp8_grouped"
+    _chk_pert_moe(x, gate_up_weight, gate_up_scale, down_weight, down_scale, who)
+    _chk(expert_offsets.dtype == torch.int32 and expert_tokens.dtype == torch.int32, f"{who}: offsets and tokens must be int32")
+    E, two_i, H = gate_up_weight.shape
+    I = two_i // 2
+    _chk(tuple(down_weight.shape) == (E, H, I) and x.shape[1] == H and E == int(n_routed_experts),
+         f"{who}: gate_up_weight [E, 2*I, H], down_weight [E, H, I], x [T, H]")
+    k = int(top_k)
+    T = x.shape[0]
+    P = T * k
+    _chk(routing_weights.dtype == x.dtype and routing_weights.numel() == P and expert_tokens.numel() == P,
+         f"{who}: routing_weights and expert_tokens must hold one entry per pair, weights in the activation dtype")
+    tokens = expert_tokens.contiguous()
+    start = _prefill_starts(expert_offsets[:E], P)
+    row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
+    inter = torch.empty(P, I, dtype=x.dtype, device=x.device)
+    _moe_gemm(x, None, row_map, gate_up_weight, gate_up_scale.contiguous(), start, inter, E, two_i, H, _ACT_GELU_TANH, who,
+              per_expert=True)
+    y = torch.empty(P, H, dtype=torch.float32, device=x.device)
+    _moe_gemm(inter, None, None, down_weight, down_scale.contiguous(), start, y, E, H, I, _ACT_NONE, who, per_expert=True,
+              out_map=tokens)
+    out = torch.empty(T, H, dtype=x.dtype, device=x.device)
+    capi.call("mi_moe_combine", y, capi.ptr(y), None, capi.ptr(routing_weights.contiguous()), capi.ptr(out), H, k, T, 0,
+              capi.act_dtype(out), 1)
+    return out
+
+
+def _moe_pert_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
+                     act, accumulate, who):
+    _chk_pert_moe(x, gate_up_weight, gate_up_scale, down_weight, down_scale, who)
+    _chk(topk_weights.dtype == x.dtype, f"{who}: topk_weights must be fp16 (the activation dtype) [T, top_k]")
+    _chk(topk_indices.dtype == torch.int32, f"{who}: topk_indices must be int32 [T, top_k]")
+    E, two_i, H = gate_up_weight.shape
+    I = two_i // 2
+    T = x.shape[0]
+    k = int(top_k)
+    P = T * k
+    _chk(tuple(down_weight.shape) == (E, H, I) and x.shape[1] == H, f"{who}: gate_up_weight [E, 2*I, H], down_weight [E, H, I], x [T, H]")
+    _chk(topk_weights.numel() == P and topk_indices.numel() == P, f"{who}: routing tensors must be [T, top_k]")
+    dev = x.device
+    ids = topk_indices.contiguous().reshape(T, k)
+    top_w = topk_weights.contiguous().reshape(T, k)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    start = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
+    moe_sort(ids, E, sorted_pairs, start, inv, sorted_token, None)
+    inter = torch.empty(P, I, dtype=x.dtype, device=dev)
+    _moe_gemm(x, None, sorted_token, gate_up_weight, gate_up_scale.contiguous(), start, inter, E, two_i, H, act, who,
+              per_expert=True)
+    if not accumulate:
+        out = torch.empty(P, H, dtype=x.dtype, device=dev)
+        return _moe_gemm(inter, None, None, down_weight, down_scale.contiguous(), start, out, E, H, I, _ACT_NONE, who,
+                         per_expert=True, out_map=sorted_pairs, row_weight=top_w.reshape(-1))
+    y = torch.empty(P, H, dtype=torch.float32, device=dev)
+    _moe_gemm(inter, None, None, down_weight, down_scale.contiguous(), start, y, E, H, I, _ACT_NONE, who, per_expert=True)
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    return moe_combine(y, inv, top_w, out, k)
+
+
+def moe_forward_full_gelu_tanh_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight,
+                                      down_scale, top_k, n_routed_experts):
+    """out[t] = sum_j w[t, j] * down_e(gelu_tanh(gate_e(x[t])) * up_e(x[t])), e = topk_indices[t, j], with the
+    caller's routing (V/csrc/moe_batch/moe.sycl:2249-2293)."""
+    return _moe_pert_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                            top_k, _ACT_GELU_TANH, True, "moe_forward_full_gelu_tanh_routed")
+
+
+def moe_forward_full_gelu_tanh_routed_decode(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale,
+                                             down_weight, down_scale, top_k, n_routed_experts):
+    """The one-token form of moe_forward_full_gelu_tanh_routed (V/csrc/moe_batch/moe.sycl:2096-2170)."""
+    who = "moe_forward_full_gelu_tanh_routed_decode"
+    _chk(x.dim() == 2 and x.shape[0] == 1, f"{who}: the decode op takes one token")
+    return _moe_pert_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                            top_k, _ACT_GELU_TANH, True, who)
+
+
+def moe_forward_full_gelu_tanh_routed_no_accum(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale,
+                                               down_weight, down_scale, top_k, n_routed_experts):
+    """The routing-weighted per-route rows [T*top_k, H] without the sum over routes
+    (V/csrc/moe_batch/moe.sycl:2297-2335)."""
+    return _moe_pert_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                            top_k, _ACT_GELU_TANH, False, "moe_forward_full_gelu_tanh_routed_no_accum")
+
+
+def moe_forward_full_gelu_tanh(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
+                               n_routed_experts):
+    """Softmax top-k with renormalisation, then moe_forward_full_gelu_tanh_routed
+    (V/csrc/moe_batch/moe.sycl:2044-2094)."""
+    who = "moe_forward_full_gelu_tanh"
+    _chk(logits.dim() == 2 and logits.shape[1] == int(n_routed_experts) and logits.dtype == x.dtype,
+         f"{who}: logits must be [T, n_routed_experts] in the activation dtype")
+    top_w, top_ids = moe_topk(logits, int(top_k), True)
+    return _moe_pert_routed(x, top_w, top_ids, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
+                            _ACT_GELU_TANH, True, who)
+
+
+def moe_forward_full_gelu_tanh_decode(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                                      per_expert_scale, top_k, n_routed_experts):
+    """One token: softmax top-k, routing weights multiplied by per_expert_scale[e] and rounded to the
+    activation dtype (MoeFoldExpertScale, V/csrc/moe_batch/moe_decode_gemv.h:146-158), then the routed
+    forward (V/csrc/moe_batch/moe.sycl:2172-2241)."""
+    who = "moe_forward_full_gelu_tanh_decode"
+    _chk(x.dim() == 2 and x.shape[0] == 1, f"{who}: the decode op takes one token")
+    _chk(logits.dim() == 2 and logits.shape[1] == int(n_routed_experts) and logits.dtype == x.dtype,
+         f"{who}: logits must be [1, n_routed_experts] in the activation dtype")
+    _chk(per_expert_scale.dtype == torch.float32 and per_expert_scale.numel() >= int(n_routed_experts),
+         f"{who}: per_expert_scale must be float32 [n_routed_experts]")
+    top_w, top_ids = moe_topk(logits, int(top_k), True)
+    top_w = (top_w.float() * per_expert_scale.reshape(-1)[top_ids.long()]).to(x.dtype)
+    return _moe_pert_routed(x, top_w, top_ids, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
+                            _ACT_GELU_TANH, True, who)
 
 
 # --------------------------------------------------------------------------
@@ -1352,6 +1545,29 @@ def register():
                        "Tensor down_weight, Tensor down_scale, Tensor shared_down_weight, Tensor shared_down_scale, "
                        "Tensor shared_expert_gate_weight, int top_k, int num_shared_experts, "
                        "int n_routed_experts) -> Tensor(a!)", moe_forward_full_fp8_block, _ret(2))
+    _pert = ("Tensor gate_up_weight, Tensor gate_up_scale, Tensor down_weight, Tensor down_scale, "
+             "int top_k, int n_routed_experts) -> Tensor")
+    _define("moe_ops", "moe_forward_full_gelu_tanh(Tensor x, Tensor logits, " + _pert, moe_forward_full_gelu_tanh,
+            lambda x, *a: torch.empty_like(x))
+    for name, fn in (("moe_forward_full_gelu_tanh_routed", moe_forward_full_gelu_tanh_routed),
+                     ("moe_forward_full_gelu_tanh_routed_decode", moe_forward_full_gelu_tanh_routed_decode)):
+        _define("moe_ops", name + "(Tensor x, Tensor topk_weights, Tensor topk_indices, " + _pert, fn,
+                lambda x, *a: torch.empty_like(x))
+    _define("moe_ops", "moe_forward_full_gelu_tanh_routed_no_accum(Tensor x, Tensor topk_weights, Tensor topk_indices, "
+            + _pert, moe_forward_full_gelu_tanh_routed_no_accum,
+            lambda x, tw, *a: x.new_empty(tw.numel(), x.shape[1]))
+    _define("moe_ops", "moe_forward_full_gelu_tanh_decode(Tensor x, Tensor logits, Tensor gate_up_weight, "
+            "Tensor gate_up_scale, Tensor down_weight, Tensor down_scale, Tensor per_expert_scale, int top_k, "
+            "int n_routed_experts) -> Tensor", moe_forward_full_gelu_tanh_decode, lambda x, *a: torch.empty_like(x))
+    _define("moe_ops", "moe_up_fp8_grouped(Tensor x, Tensor gate_up_weight, Tensor gate_up_scale, Tensor expert_offsets, "
+            "Tensor expert_tokens, int top_k, int n_routed_experts) -> Tensor", moe_up_fp8_grouped,
+            lambda x, w, s, eo, et, k, e: x.new_empty(et.numel(), w.shape[1] // 2))
+    _define("moe_ops", "moe_down_fp8_grouped(Tensor intermediate, Tensor down_weight, Tensor down_scale, "
+            "Tensor routing_weights, Tensor expert_offsets, Tensor expert_tokens, int top_k, int n_routed_experts) -> Tensor",
+            moe_down_fp8_grouped, lambda i, w, *a: i.new_empty(i.shape[0], w.shape[1]))
+    _define("moe_ops", "moe_forward_full_fp8_grouped(Tensor x, Tensor gate_up_weight, Tensor gate_up_scale, "
+            "Tensor down_weight, Tensor down_scale, Tensor routing_weights, Tensor expert_offsets, Tensor expert_tokens, "
+            "int top_k, int n_routed_experts) -> Tensor", moe_forward_full_fp8_grouped, lambda x, *a: torch.empty_like(x))
     _define("moe_fp8_prefill_ops", "moe_prefill_gather_forward_fp8(Tensor selected_experts, int num_experts) -> Tensor[]",
             moe_prefill_gather_forward_fp8)
     _define("moe_fp8_prefill_ops", "moe_prefill_full_fp8(Tensor hidden_states, Tensor topk_weights, Tensor topk_ids, "

@@ -581,12 +581,18 @@ def moe_forward_full(x, logits, w13, s13, shared_w13, shared_s13, w2, s2, shared
     return out
 
 
-def moe_prefill_scalar(x, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, return_parts=False):
+def moe_prefill_scalar(x, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, return_parts=False, act="silu"):
     """FP8 MoE prefill with per-expert scalar scales, fp32 throughout
     (S/csrc/moe_prefill/moe_prefill_fp8.sycl:616-649; gate/up scales separate, :196-199):
       gate = s13[e,0] * (x @ w13[e,:I]^T), up = s13[e,1] * (x @ w13[e,I:]^T),
       inter = silu(gate) * up, y = s2[e] * (inter @ w2[e]^T), out[t] = sum_j w[t,j] * y[t,j].
+    w13_scale of shape [E] is one scale for both halves, and act="gelu_tanh" the tanh form of
+    GELU on the gate: the per-route loop of V/tests/test_moe_full_gelu_tanh.py:14-29 and
+    V/tests/test_moe_fp8_grouped.py:6-15 (kept in fp32 here).
     return_parts also gives the [T*k, I] intermediate and the [T*k, H] expert output in pair order."""
+    if w13_scale.dim() == 1:
+        w13_scale = torch.stack([w13_scale, w13_scale], 1)
+    fn = torch.nn.functional.silu if act == "silu" else (lambda g: torch.nn.functional.gelu(g, approximate="tanh"))
     T, H = x.shape
     k = topk_ids.shape[1]
     E, two_i, _ = w13.shape
@@ -601,7 +607,7 @@ def moe_prefill_scalar(x, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, 
             e = int(topk_ids[t, j])
             gate = (x32[t] @ d13[e, :I].t()) * w13_scale[e, 0]
             up = (x32[t] @ d13[e, I:].t()) * w13_scale[e, 1]
-            inter[t * k + j] = torch.nn.functional.silu(gate) * up
+            inter[t * k + j] = fn(gate) * up
             y[t * k + j] = (inter[t * k + j] @ d2[e].t()) * w2_scale[e]
     out = (topk_weights.float().reshape(T, k, 1) * y.reshape(T, k, H)).sum(1)
     return (out, inter, y) if return_parts else out

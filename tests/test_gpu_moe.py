@@ -416,3 +416,116 @@ def test_permute_rows_roundtrip(v, dev):
     assert torch.equal(a.cpu(), src.cpu()[perm.cpu().long()])
     capi.call("mi_permute_rows", a, capi.ptr(a), capi.ptr(perm), capi.ptr(b), rows, cols * 2, 1)
     assert torch.equal(b.cpu(), src.cpu())
+
+
+# ----------------------------------------------------------------- per-expert-scale ops with the tanh-GELU gate (moe_ops)
+def _pert_case(T, E, H, I, k, seed, dtype):
+    """Weights as V/tests/test_moe_full_gelu_tanh.py:39-44 draws them (clamped normal / 0.3 -> e4m3, with
+    per-expert scales varied here so that a wrong scale index shows)."""
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=g) * 0.05).to(dtype)
+    logits = torch.randn(T, E, generator=g).to(dtype)
+    tw, ti = O.moe_topk(logits, k)
+    w13 = O.e4m3_quantize((torch.randn(E, 2 * I, H, generator=g) * 0.05).clamp(-0.3, 0.3) / 0.3)
+    w2 = O.e4m3_quantize((torch.randn(E, H, I, generator=g) * 0.05).clamp(-0.3, 0.3) / 0.3)
+    s13 = (0.3 * (0.5 + torch.rand(E, generator=g))).float()
+    s2 = (0.3 * (0.5 + torch.rand(E, generator=g))).float()
+    return x, logits, tw.to(dtype), ti, w13, s13, w2, s2
+
+
+@pytest.mark.parametrize("T,E,H,I,k,dtype", [(2, 16, 2816, 704, 8, torch.float16), (40, 8, 256, 144, 2, torch.float16),
+                                             (1, 16, 512, 256, 4, torch.float16), (70, 4, 384, 80, 2, torch.bfloat16)])
+def test_moe_gelu_tanh_family(v, dev, T, E, H, I, k, dtype):
+    """K = 704, 144, 80 end in a partial 128-granule; I = 704, 144, 80 put the gate / up boundary inside a
+    128-row block."""
+    x, logits, tw, ti, w13, s13, w2, s2 = _pert_case(T, E, H, I, k, 500 + T, dtype)
+    want, inter_ref, y_ref = O.moe_prefill_scalar(x, tw, ti, w13, s13, w2, s2, return_parts=True, act="gelu_tanh")
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    op = torch.ops.moe_ops
+    d = lambda t: t.to(dev)
+    # down projection of the rounded intermediate: the value a w8a16 chain should produce
+    ids = ti.reshape(-1).long()
+    d2 = O.e4m3_decode(w2.reshape(-1, I)).reshape(E, H, I)
+    y_r = torch.einsum("pi,phi->ph", inter_ref.to(dtype).float(), d2[ids]) * s2[ids].view(-1, 1)
+    want_r = (tw.float().reshape(T, k, 1) * y_r.reshape(T, k, H)).sum(1)
+
+    got = op.moe_forward_full_gelu_tanh_routed(d(x), d(tw), d(ti), f8(w13), d(s13), f8(w2), d(s2), k, E)
+    assert got.shape == (T, H) and got.dtype == dtype
+    assert O.max_rel_err(got.cpu().float(), want_r) < TOL
+    assert ((got.cpu().float() - want).abs().mean() / want.abs().mean()).item() < 5e-3
+    # internal softmax top-k
+    got2 = op.moe_forward_full_gelu_tanh(d(x), d(logits), f8(w13), d(s13), f8(w2), d(s2), k, E)
+    assert O.max_rel_err(got2.cpu().float(), want_r) < TOL
+    # per-route rows, weighted, in pair order
+    rows = op.moe_forward_full_gelu_tanh_routed_no_accum(d(x), d(tw), d(ti), f8(w13), d(s13), f8(w2), d(s2), k, E)
+    assert rows.shape == (T * k, H)
+    assert O.max_rel_err(rows.cpu().float(), y_r * tw.float().reshape(-1, 1)) < TOL
+    if T == 1:
+        got3 = op.moe_forward_full_gelu_tanh_routed_decode(d(x), d(tw), d(ti), f8(w13), d(s13), f8(w2), d(s2), k, E)
+        assert torch.equal(got3.cpu(), got.cpu())
+        pes = (0.5 + torch.rand(E, generator=torch.Generator().manual_seed(3))).float()
+        got4 = op.moe_forward_full_gelu_tanh_decode(d(x), d(logits), f8(w13), d(s13), f8(w2), d(s2), d(pes), k, E)
+        tw_f = (tw.float() * pes[ti.long()]).to(dtype)
+        want4 = (tw_f.float().reshape(T, k, 1) * y_r.reshape(T, k, H)).sum(1)
+        assert O.max_rel_err(got4.cpu().float(), want4) < TOL
+    # the grouped ops on the sglang gather's expert grouping
+    offs, toks, _, _ = torch.ops.moe_fp8_prefill_ops.moe_prefill_gather_forward_fp8(d(ti), E)
+    inter = op.moe_up_fp8_grouped(d(x), f8(w13), d(s13), offs, toks, k, E)
+    assert inter.shape == (T * k, I)
+    assert O.max_rel_err(inter.cpu().float(), inter_ref) < TOL
+    rw = d(tw.reshape(-1).contiguous())
+    part = op.moe_down_fp8_grouped(inter, f8(w2), d(s2), rw, offs, toks, k, E)
+    forced = torch.einsum("pi,phi->ph", inter.cpu().float(), d2[ids]) * s2[ids].view(-1, 1) * tw.float().reshape(-1, 1)
+    assert O.max_rel_err(part.cpu().float(), forced) < TOL
+    full = op.moe_forward_full_fp8_grouped(d(x), f8(w13), d(s13), f8(w2), d(s2), rw, offs, toks, k, E)
+    assert O.max_rel_err(full.cpu().float(), want_r) < TOL
+
+
+def test_moe_fp8_grouped_reference_shape(v, dev):
+    """E=128, top_k=8, H=2816, I=704, T=256 (V/tests/test_moe_fp8_grouped.py:16-37): the three routes through
+    the kernels agree, and a sample of tokens matches the fp32 per-route loop."""
+    T, E, H, I, k = 256, 128, 2816, 704, 8
+    g = torch.Generator(device=dev).manual_seed(42)
+    x = (torch.randn(T, H, generator=g, device=dev) * 0.05).half()
+    logits = torch.randn(T, E, generator=g, device=dev).half()
+    w13 = ((torch.randn(E, 2 * I, H, generator=g, device=dev) * 0.05).clamp(-0.3, 0.3) / 0.3).to(torch.float8_e4m3fn)
+    w2 = ((torch.randn(E, H, I, generator=g, device=dev) * 0.05).clamp(-0.3, 0.3) / 0.3).to(torch.float8_e4m3fn)
+    s13 = torch.full((E,), 0.3, device=dev)
+    s2 = torch.full((E,), 0.3, device=dev)
+    op = torch.ops.moe_ops
+    tw, ti = op.moe_topk(logits, k, True)
+    offs, toks, _, _ = torch.ops.moe_fp8_prefill_ops.moe_prefill_gather_forward_fp8(ti, E)
+    rw = tw.reshape(-1).contiguous()
+    inter = op.moe_up_fp8_grouped(x, w13, s13, offs, toks, k, E)
+    part = op.moe_down_fp8_grouped(inter, w2, s2, rw, offs, toks, k, E)
+    staged = part.view(T, k, H).float().sum(1)
+    full = op.moe_forward_full_fp8_grouped(x, w13, s13, w2, s2, rw, offs, toks, k, E)
+    routed = op.moe_forward_full_gelu_tanh_routed(x, tw, ti, w13, s13, w2, s2, k, E)
+    assert O.max_rel_err(full.cpu().float(), staged.cpu()) < TOL
+    assert O.max_rel_err(routed.cpu().float(), full.cpu().float()) < 2e-3
+    sample = [0, 101, 255]
+    tic = ti.cpu()
+    used = sorted(set(tic[sample].reshape(-1).tolist()))
+    remap = {e: i for i, e in enumerate(used)}
+    ti_s = torch.tensor([[remap[int(e)] for e in tic[t]] for t in sample], dtype=torch.int32)
+    w13_s = w13.view(torch.uint8)[used].cpu()
+    w2_s = w2.view(torch.uint8)[used].cpu()
+    want = O.moe_prefill_scalar(x.cpu()[sample], tw.cpu()[sample], ti_s, w13_s, torch.full((len(used),), 0.3), w2_s,
+                                torch.full((len(used),), 0.3), act="gelu_tanh")
+    assert O.max_rel_err(full.cpu().float()[sample], want) < 2 * TOL      # intermediate rounded to fp16 on the device
+
+
+def test_moe_gemm_grouped_argument_errors(v, dev):
+    from mi355x_qlinear import capi
+    E, N, K, R = 2, 64, 72, 4          # K not a multiple of 16
+    a = torch.zeros(R, K, dtype=torch.float16, device=dev)
+    w = torch.zeros(E, N, K, dtype=torch.uint8, device=dev)
+    sc = torch.ones(E, device=dev)
+    start = torch.tensor([0, 2, 4], dtype=torch.int32, device=dev)
+    out = torch.zeros(R, N, dtype=torch.float16, device=dev)
+    args = lambda k, act: (capi.ptr(a), None, None, capi.ptr(w), capi.ptr(sc), 1, capi.ptr(start), capi.ptr(out), None, None,
+                           R, R, E, N, k, act, capi.DT_F16, 0)
+    with pytest.raises(RuntimeError):
+        capi.call("mi_moe_gemm_fp8_grouped", a, *args(K, 0))
+    with pytest.raises(RuntimeError):
+        capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 3))
