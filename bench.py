@@ -292,6 +292,52 @@ def wl_moe(dev):
                 kernel="moe_gemm_kernel", cpu=cpu)
 
 
+def wl_moe_gelu(dev):
+    """Per-expert-scale FP8 MoE with the tanh-GELU gate at the shape of the reference's own test
+    (vllm/custom-esimd-kernels-vllm/tests/test_moe_fp8_grouped.py:16): routing given, sort + grouped
+    gate_up GEMM with the fused GELU * up + grouped down GEMM + weighted sum."""
+    import custom_esimd_kernels_vllm  # noqa: F401  (registers torch.ops.moe_ops)
+    from oracle import qlinear_oracle as O
+    T, E, K, H, I = 256, 128, 8, 2816, 704
+    g = torch.Generator(device=dev).manual_seed(97)
+    x = (torch.randn(T, H, generator=g, device=dev) * 0.05).half()
+    logits = torch.randn(T, E, generator=g, device=dev).half()
+    tw, ti = torch.ops.moe_ops.moe_topk(logits, K, True)
+    wbytes = E * 3 * H * I
+    R = _copies(wbytes)
+    W = []
+    for _ in range(R):
+        w13 = ((torch.randn(E, 2 * I, H, generator=g, device=dev) * 0.05).clamp(-0.3, 0.3) / 0.3).to(torch.float8_e4m3fn)
+        w2 = ((torch.randn(E, H, I, generator=g, device=dev) * 0.05).clamp(-0.3, 0.3) / 0.3).to(torch.float8_e4m3fn)
+        W.append((w13, w2))
+    s13 = torch.full((E,), 0.3, device=dev)
+    s2 = torch.full((E,), 0.3, device=dev)
+
+    def launch(i):
+        a, b = W[i % R]
+        torch.ops.moe_ops.moe_forward_full_gelu_tanh_routed(x, tw, ti, a, s13, b, s2, K, E)
+
+    n_cpu = 2                                    # tokens of the CPU sample
+
+    def cpu():
+        tic = ti.cpu()[:n_cpu]
+        used = sorted(set(tic.reshape(-1).tolist()))
+        remap = {e: i for i, e in enumerate(used)}
+        ti_s = torch.tensor([[remap[int(e)] for e in row] for row in tic], dtype=torch.int32)
+        a, b = W[0]
+        sc = torch.full((len(used),), 0.3)
+        return O.moe_prefill_scalar(x.cpu()[:n_cpu], tw.cpu()[:n_cpu], ti_s, a.view(torch.uint8)[used].cpu(), sc,
+                                    b.view(torch.uint8)[used].cpu(), sc, act="gelu_tanh")
+
+    P = T * K
+    alg_bytes = wbytes + 8 * E + 2 * T * H + 6 * P + 2 * T * H
+    flops = 2 * P * 3 * H * I
+    return dict(launch=launch, R=R, bytes=alg_bytes, flops=flops, bound="hbm", dtype="fp16",
+                name=f"next: per-expert-scale FP8 MoE, tanh-GELU gate (sort+gate_up/GELU+down+combine) "
+                     f"T={T} E={E} top{K} H={H} I={I} fp16 (w8a16)",
+                kernel="moe_gemm_kernel", cpu=cpu, cpu_scale=n_cpu / T)
+
+
 WORKLOADS = {
     "cfg1_m1": lambda dev: wl_fp8_pern(1, dev),
     "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
@@ -308,6 +354,7 @@ WORKLOADS = {
     "next_q6_k_m1": lambda dev: wl_gguf("q6_k", 1, dev),
     "next_q4_0_quantize": wl_q4_0_quantize,
     "next_resadd_norm_gemv": wl_resadd_norm_gemv,
+    "next_moe_gelu_grouped": wl_moe_gelu,
 }
 HEADLINE = "cfg1_m1"
 
