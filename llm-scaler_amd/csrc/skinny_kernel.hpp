@@ -389,6 +389,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
   constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
   constexpr int kRed = (NW - 1) * RT * MT * 1024;
   constexpr int lds = kStage > kRed ? kStage : kRed;
+  static_assert(lds <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
   auto kern = skinny_kernel<Act, FMT, SC, MT, RT, NW, UN>;
   if (lds > 64 * 1024) {
     static bool raised = false;                       // opt in to > 64 KiB of dynamic LDS once
@@ -427,7 +428,7 @@ static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
       else launch_one<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
     } else {
       if (a.M <= 16) launch_one<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 4, 4, 1>(a, rpw, st);
+      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 4, 8, 1>(a, rpw, st);
       else launch_one<Act, FMT, SC, 4, 4, 4, 1>(a, rpw, st);
     }
   }

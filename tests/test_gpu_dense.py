@@ -578,3 +578,27 @@ def test_norm_only_ops(ops, dev, dt):
     v.esimd_rms_norm_gated(x.to(dev), z.to(dev), wv.to(dev), out, eps)
     ref, _ = O.rmsnorm(x, wv, eps, gate=z, heads=24)
     assert _ulp_close(out.cpu().float(), ref, dt)
+
+
+# ----------------------------------------------------------------- few weight rows, many activation rows
+@pytest.mark.parametrize("M,K,N,dt", [(64, 4096, 1024, torch.bfloat16), (17, 8192, 512, torch.float16),
+                                      (40, 4096, 2000, torch.float16), (64, 2176, 72, torch.bfloat16)])
+def test_fp8_pern_small_n_repeatable(ops, dev, M, K, N, dt):
+    """Shapes with fewer 64-row blocks than compute units; repeated calls agree bit for bit."""
+    v, _ = ops
+    x, w8, s = O.make_fp8_pern_case(M, K, N, seed=M + N, act_dtype=dt)
+    xd, wd, sd = x.to(dev), w8.to(dev), s.to(dev)
+    outs = []
+    for _ in range(3):
+        out = torch.full((M, N), float("nan"), dtype=dt, device=dev)
+        v.esimd_gemv_fp8_pern(xd, wd, sd, out, N, K)
+        outs.append(out.cpu())
+    ref = O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))
+    assert O.max_rel_err(outs[0], ref) < TOL
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+def test_int4_small_n_many_rows(ops, dev):
+    v, _ = ops
+    assert _run_int4(v, dev, 48, 4096, 1536, torch.bfloat16, seed=77) < TOL
+    assert _run_int4(v, dev, 64, 2048, 4096, torch.float16, seed=78) < TOL
