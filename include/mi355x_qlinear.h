@@ -317,6 +317,32 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
                             const int32_t* out_map, const void* row_weight, int a_rows, int total_rows, int E,
                             int N, int K, int fuse_act, int act_dtype, int out_f32, void* stream);
 
+/* ---- Decode MoE on K-major per-tensor FP8 expert weights --------------------------
+ * The routed experts of the reference's per-tensor FP8 MoE decode op keep the reduction
+ * index outermost: gate_up [E, H, 2I], down [E, I, H] e4m3, one fp32 scale per expert
+ * (moe_forward_full, V/csrc/moe_batch/moe.sycl:1855-1940; kernels moe_up_routed_e4m3_kernel
+ * :371-456, moe_down_routed_e4m3_kernel :815-868, moe_down_finalize_e4m3_kernel :1386-1421).
+ * route r = t * top_k + j uses expert route_expert[r] and token t.
+ * mi_moe_kmajor_up:   partial[r][s][:] = sum over split s's rows k of x[t][k] * W13[e][k][:]
+ *                     (fp32 [routes, splits, 2I], unscaled); 2I % 32 == 0.
+ * mi_moe_kmajor_down: inter[i] = act(s13[e] gate[i]) * (s13[e] up[i]) with gate / up summed over
+ *                     the up partials in split order and the product rounded to the activation
+ *                     type; partial[r][s][:] = sum over split s's rows i of inter[i] * W2[e][i][:]
+ *                     (fp32 [routes, splits, H], unscaled); gelu = 0: SiLU, 1: tanh-GELU; H % 16 == 0.
+ * mi_moe_kmajor_finalize: out[t][:] = sum_j top_w[t][j] * s2[e] * sum_s partial[r][s][:]
+ *                     + gate[t] * shared[t][:] (shared / gate optional), rounded once.
+ * `splits` (K split over workgroups, rows per split = ceil(K / splits) rounded up to 8, at most
+ * 1024) is the caller's choice: about two workgroups per compute unit over
+ * routes * ceil(N / 1024) column blocks fills the device. */
+int mi_moe_kmajor_up(const void* x, const void* w, const int32_t* route_expert, float* partial, int routes,
+                     int top_k, int H, int two_i, int splits, int act_dtype, void* stream);
+int mi_moe_kmajor_down(const float* up_partial, int up_splits, const float* up_scale, const void* w2,
+                       const int32_t* route_expert, float* partial, int routes, int I, int H, int splits,
+                       int gelu, int act_dtype, void* stream);
+int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_scale, const int32_t* route_expert,
+                           const void* top_w, const void* shared, const float* gate, void* out, int T, int top_k,
+                           int H, int act_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,3 +4,4 @@ importing it registers the torch.ops and re-exports the thin wrappers."""
 import mi355x_qlinear  # noqa: F401  (registers torch.ops.* for ROCm tensors)
 
 from .ops import *  # noqa: F401,F403
+from . import moe_ops  # noqa: F401,E402

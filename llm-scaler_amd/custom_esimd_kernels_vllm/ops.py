@@ -202,6 +202,16 @@ def moe_forward_full_gelu_tanh_decode(x, logits, gate_up_weight, gate_up_scale, 
                                                   down_scale, per_expert_scale, top_k, n_routed_experts)
 
 
+def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight, shared_gate_up_scale,
+                     down_weight, down_scale, shared_down_weight, shared_down_scale, shared_expert_gate_weight,
+                     top_k, num_shared_experts, n_routed_experts):
+    """V/python/custom_esimd_kernels_vllm/ops.py:1063-1090."""
+    return _moe.moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight,
+                                 shared_gate_up_scale, down_weight, down_scale, shared_down_weight,
+                                 shared_down_scale, shared_expert_gate_weight, top_k, num_shared_experts,
+                                 n_routed_experts)
+
+
 def precompute_moe_route(topk_weights, topk_ids, num_experts):
     """Same contract as the reference helper: (sorted_rows, sorted_weights, rows_per_expert),
     stable by expert; computed on the device by the sort kernel."""

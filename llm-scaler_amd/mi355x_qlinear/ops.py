@@ -1397,6 +1397,83 @@ def moe_forward_full_gelu_tanh_decode(x, logits, gate_up_weight, gate_up_scale, 
 
 
 # --------------------------------------------------------------------------
+# per-tensor FP8 MoE decode on K-major routed weights (moe_ops.moe_forward_full / _v2)
+# --------------------------------------------------------------------------
+def _km_splits(routes, K, N, dev):
+    """Workgroups over K per (route, 1024-column block): about two per compute unit in total,
+    at least 32 rows each, at most 1024 rows (the kernels' staging vector)."""
+    cblocks = (N + 1023) // 1024
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    want = -(-2 * cus // max(1, routes * cblocks))
+    return max(min(want, max(1, K // 32)), -(-K // 1024))
+
+
+def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight, shared_gate_up_scale,
+                     down_weight, down_scale, shared_down_weight, shared_down_scale, shared_expert_gate_weight,
+                     top_k, num_shared_experts, n_routed_experts):
+    """Per-tensor FP8 MoE decode step (V/csrc/moe_batch/moe.sycl:1855-1940): softmax top-k (renormalised),
+    routed experts on K-major weights gate_up [E, H, 2I] / down [E, I, H] with one fp32 scale per expert,
+    SiLU(gate) * up, + sigmoid(x . shared_expert_gate_weight[s]) * shared expert s (N-major
+    [S, 2I, H] / [S, H, I], scales [S]).  -> [T, H].  E4M3 only; bf16 accepted besides fp16."""
+    who = "moe_forward_full"
+    _chk(x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(), f"{who}: x must be contiguous fp16 [T, H]")
+    E, k, S = int(n_routed_experts), int(top_k), int(num_shared_experts)
+    T, H = x.shape
+    _chk(E > 0 and 0 < k <= E and S >= 0, f"{who}: requires 0 < top_k <= n_routed_experts")
+    _chk(logits.dim() == 2 and tuple(logits.shape) == (T, E) and logits.dtype == x.dtype, f"{who}: logits must be [T, E] in x's dtype")
+    _chk(gate_up_weight.dim() == 3 and gate_up_weight.shape[0] == E and gate_up_weight.shape[1] == H and
+         gate_up_weight.shape[2] % 32 == 0, f"{who}: gate_up_weight must be [E, H, 2*I] with I a multiple of 16")
+    I = gate_up_weight.shape[2] // 2
+    _chk(tuple(down_weight.shape) == (E, I, H) and H % 16 == 0, f"{who}: down_weight must be [E, I, H], H a multiple of 16")
+    _chk_fp8(gate_up_weight, who)
+    _chk_fp8(down_weight, who)
+    _chk(gate_up_scale.dtype == torch.float32 and gate_up_scale.numel() >= E and down_scale.dtype == torch.float32 and
+         down_scale.numel() >= E, f"{who}: routed scales must be float32 [E]")
+    dev = x.device
+    P = T * k
+    top_w, top_ids = moe_topk(logits, k, True)
+    route_expert = top_ids.reshape(-1)
+    adt = capi.act_dtype(x)
+    s_up = _km_splits(P, H, 2 * I, dev)
+    up_part = torch.empty(P, s_up, 2 * I, dtype=torch.float32, device=dev)
+    capi.call("mi_moe_kmajor_up", x, capi.ptr(x), capi.ptr(gate_up_weight), capi.ptr(route_expert), capi.ptr(up_part), P, k,
+              H, 2 * I, s_up, adt)
+    s_dn = _km_splits(P, I, H, dev)
+    dn_part = torch.empty(P, s_dn, H, dtype=torch.float32, device=dev)
+    capi.call("mi_moe_kmajor_down", x, capi.ptr(up_part), s_up, capi.ptr(gate_up_scale.contiguous()), capi.ptr(down_weight),
+              capi.ptr(route_expert), capi.ptr(dn_part), P, I, H, s_dn, 0, adt)
+    shared = gate = None
+    if S > 0:
+        _chk(S == 1, f"{who}: one shared expert is supported")
+        _chk_fp8(shared_gate_up_weight, who)
+        _chk_fp8(shared_down_weight, who)
+        _chk(shared_gate_up_weight.numel() == 2 * I * H and shared_down_weight.numel() == H * I,
+             f"{who}: shared weights must be [1, 2*I, H] and [1, H, I]")
+        _chk(shared_gate_up_scale.dtype == torch.float32 and shared_down_scale.dtype == torch.float32,
+             f"{who}: shared scales must be float32")
+        _chk(shared_expert_gate_weight.dtype == x.dtype and shared_expert_gate_weight.numel() == H,
+             f"{who}: shared_expert_gate_weight must be [1, H] in x's dtype")
+        sh_gu = torch.empty(T, 2 * I, dtype=x.dtype, device=dev)
+        esimd_gemm_fp8_pert(x, shared_gate_up_weight.reshape(2 * I, H), shared_gate_up_scale.reshape(-1)[:1], sh_gu)
+        sh_inter = torch.empty(T, I, dtype=x.dtype, device=dev)
+        esimd_moe_silu_mul(sh_gu, sh_inter, 2 * I, I, T)
+        shared = torch.empty(T, H, dtype=x.dtype, device=dev)
+        esimd_gemm_fp8_pert(sh_inter, shared_down_weight.reshape(H, I), shared_down_scale.reshape(-1)[:1], shared)
+        gate = torch.empty(T, dtype=torch.float32, device=dev)
+        capi.call("mi_moe_shared_gate", x, capi.ptr(x), capi.ptr(shared_expert_gate_weight.contiguous()), capi.ptr(gate), T, H, adt)
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    capi.call("mi_moe_kmajor_finalize", x, capi.ptr(dn_part), s_dn, capi.ptr(down_scale.contiguous()), capi.ptr(route_expert),
+              capi.ptr(top_w), capi.ptr(shared), capi.ptr(gate), capi.ptr(out), T, k, H, adt)
+    return out
+
+
+def moe_forward_full_v2(*args):
+    """The reference's variant for more than one token (V/csrc/moe_batch/moe.sycl:2337-2430): same
+    arguments and result as moe_forward_full; one implementation serves both here."""
+    return moe_forward_full(*args)
+
+
+# --------------------------------------------------------------------------
 # registration
 # --------------------------------------------------------------------------
 def _ret(idx):
@@ -1559,6 +1636,12 @@ def register():
     _define("moe_ops", "moe_forward_full_gelu_tanh_decode(Tensor x, Tensor logits, Tensor gate_up_weight, "
             "Tensor gate_up_scale, Tensor down_weight, Tensor down_scale, Tensor per_expert_scale, int top_k, "
             "int n_routed_experts) -> Tensor", moe_forward_full_gelu_tanh_decode, lambda x, *a: torch.empty_like(x))
+    _full = ("(Tensor x, Tensor logits, Tensor gate_up_weight, Tensor gate_up_scale, Tensor shared_gate_up_weight, "
+             "Tensor shared_gate_up_scale, Tensor down_weight, Tensor down_scale, Tensor shared_down_weight, "
+             "Tensor shared_down_scale, Tensor shared_expert_gate_weight, int top_k, int num_shared_experts, "
+             "int n_routed_experts) -> Tensor")
+    _define("moe_ops", "moe_forward_full" + _full, moe_forward_full, lambda x, *a: torch.empty_like(x))
+    _define("moe_ops", "moe_forward_full_v2" + _full, moe_forward_full_v2, lambda x, *a: torch.empty_like(x))
     _define("moe_ops", "moe_up_fp8_grouped(Tensor x, Tensor gate_up_weight, Tensor gate_up_scale, Tensor expert_offsets, "
             "Tensor expert_tokens, int top_k, int n_routed_experts) -> Tensor", moe_up_fp8_grouped,
             lambda x, w, s, eo, et, k, e: x.new_empty(et.numel(), w.shape[1] // 2))

@@ -581,6 +581,36 @@ def moe_forward_full(x, logits, w13, s13, shared_w13, shared_s13, w2, s2, shared
     return out
 
 
+def moe_forward_full_kmajor(x, logits, w13, s13, shared_w13, shared_s13, w2, s2, shared_w2, shared_s2, shared_gate,
+                            top_k):
+    """Per-tensor FP8 MoE decode step on K-major routed weights, fp32 throughout: what the kernels of
+    V/csrc/moe_batch/moe.sycl compute for moe_forward_full (:1855-1940) — routed up :371-456
+    (gate_up [E, H, 2I]: element [e, k, n]; scale gate_up_scale[e]; SiLU(gate) * up), routed down :815-868
+    (down [E, I, H]: element [e, i, h]; times routing weight and down_scale[e]), shared up :647-692
+    (shared_gate_up [2I, H], N-major), finalize :1386-1421 (sigmoid(x . gate) * shared down [H, I]).
+    Weights are uint8 E4M3 codes; shared_w13 / shared_w2 may be None (no shared expert)."""
+    top_w, top_ids = moe_topk(logits, top_k, out_dtype=torch.float32)
+    x32 = x.float()
+    T, H = x.shape
+    E, _, two_i = w13.shape
+    I = two_i // 2
+    d13 = e4m3_decode(w13.reshape(-1, two_i)).reshape(E, H, two_i)
+    d2 = e4m3_decode(w2.reshape(-1, H)).reshape(E, I, H)
+    out = torch.zeros_like(x32)
+    for t in range(T):
+        for j in range(top_k):
+            e = int(top_ids[t, j])
+            gu = (x32[t] @ d13[e]) * s13[e]
+            inter = torch.nn.functional.silu(gu[:I]) * gu[I:]
+            out[t] += top_w[t, j].float() * s2[e] * (inter @ d2[e])
+    if shared_w13 is not None:
+        gu = (x32 @ e4m3_decode(shared_w13.reshape(two_i, H)).t()) * shared_s13.reshape(-1)[0]
+        sh = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+        y = (sh @ e4m3_decode(shared_w2.reshape(H, I)).t()) * shared_s2.reshape(-1)[0]
+        out += torch.sigmoid(x32 @ shared_gate.float().reshape(H, 1)) * y
+    return out
+
+
 def moe_prefill_scalar(x, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, return_parts=False, act="silu"):
     """FP8 MoE prefill with per-expert scalar scales, fp32 throughout
     (S/csrc/moe_prefill/moe_prefill_fp8.sycl:616-649; gate/up scales separate, :196-199):

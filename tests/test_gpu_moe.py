@@ -529,3 +529,54 @@ def test_moe_gemm_grouped_argument_errors(v, dev):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(K, 0))
     with pytest.raises(RuntimeError):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 3))
+
+
+# ----------------------------------------------------------------- per-tensor decode op on K-major routed weights
+def _kmajor_case(T, E, H, I, k, seed, dtype, shared=True):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=g) * 0.3).to(dtype)
+    logits = torch.randn(T, E, generator=g).to(dtype)
+    w13 = O.e4m3_quantize(torch.randn(E, H, 2 * I, generator=g))
+    w2 = O.e4m3_quantize(torch.randn(E, I, H, generator=g))
+    s13 = (0.004 * (1 + torch.rand(E, generator=g))).float()
+    s2 = (0.004 * (1 + torch.rand(E, generator=g))).float()
+    if not shared:
+        return x, logits, w13, s13, None, None, w2, s2, None, None, None
+    sw13 = O.e4m3_quantize(torch.randn(1, 2 * I, H, generator=g))
+    sw2 = O.e4m3_quantize(torch.randn(1, H, I, generator=g))
+    ss13, ss2 = torch.tensor([0.0051]), torch.tensor([0.0047])
+    gate = (torch.randn(1, H, generator=g) * 0.05).to(dtype)
+    return x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate
+
+
+@pytest.mark.parametrize("T,E,H,I,k,dtype", [(1, 512, 2048, 512, 10, torch.float16), (1, 16, 256, 128, 4, torch.bfloat16),
+                                             (3, 16, 1056, 288, 2, torch.float16), (9, 8, 2048, 768, 3, torch.float16)])
+def test_moe_forward_full_kmajor(v, dev, T, E, H, I, k, dtype):
+    """Qwen3-Next decode sizes (512 experts, top 10, H 2048, I 512), sizes that are not multiples of the
+    1024-column block or of the 8-row batch, and several tokens; shared expert included."""
+    case = _kmajor_case(T, E, H, I, k, 700 + T, dtype)
+    want = O.moe_forward_full_kmajor(*case, k)
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate = case
+    args = (x.to(dev), logits.to(dev), f8(w13), s13.to(dev), f8(sw13), ss13.to(dev), f8(w2), s2.to(dev), f8(sw2),
+            ss2.to(dev), gate.to(dev), k, 1, E)
+    got = torch.ops.moe_ops.moe_forward_full(*args)
+    assert got.shape == (T, H) and got.dtype == dtype
+    # the op rounds the routed and the shared intermediates to the activation type (w8a16 chain):
+    # the mean-based bar of the reference's block-FP8 test plus a max bar three roundings wide
+    diff = (got.cpu().float() - want).abs()
+    assert (diff.mean() / want.abs().mean()).item() < 3e-3
+    assert O.max_rel_err(got.cpu().float(), want) < 3 * TOL
+    again = torch.ops.moe_ops.moe_forward_full_v2(*args)
+    assert torch.equal(again.cpu(), got.cpu())                  # fixed summation order
+
+
+def test_moe_forward_full_kmajor_no_shared_expert(v, dev):
+    T, E, H, I, k = 2, 8, 512, 256, 2
+    x, logits, w13, s13, _, _, w2, s2, _, _, _ = _kmajor_case(T, E, H, I, k, 41, torch.float16, shared=False)
+    want = O.moe_forward_full_kmajor(x, logits, w13, s13, None, None, w2, s2, None, None, None, k)
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    e = torch.empty(0, device=dev)
+    got = torch.ops.moe_ops.moe_forward_full(x.to(dev), logits.to(dev), f8(w13), s13.to(dev), e, e, f8(w2), s2.to(dev), e, e,
+                                             e, k, 0, E)
+    assert O.max_rel_err(got.cpu().float(), want) < 2 * TOL

@@ -434,3 +434,27 @@ def test_gelu_tanh_mul_closed_form():
     exp = 0.5 * g * (1 + (e - 1) / (e + 1)) * gu[0, 4:].double()
     assert torch.allclose(out[0].double(), exp, rtol=1e-6, atol=1e-7)
     assert out[0, 0] == 0 and abs(out[0, 1].item() - 0.8411920 * 2.0) < 1e-5    # gelu_tanh(1) = 0.841192
+
+
+def test_moe_forward_full_kmajor_against_block_oracle():
+    """The K-major per-tensor forward equals the (separately pinned) block-scaled forward on the
+    transposed weights with every block of expert e carrying scale[e]: a transposed index, a scale
+    taken from the wrong expert or a gate / up swap fails this."""
+    g = torch.Generator().manual_seed(6)
+    T, E, H, I, k = 4, 6, 256, 128, 2
+    x = (torch.randn(T, H, generator=g) * 0.2).half()
+    logits = (torch.randn(T, E, generator=g) * 0.4).half()
+    w13 = O.e4m3_quantize(torch.randn(E, H, 2 * I, generator=g))           # K-major
+    w2 = O.e4m3_quantize(torch.randn(E, I, H, generator=g))
+    s13 = 0.01 * (1 + torch.rand(E, generator=g))
+    s2 = 0.01 * (1 + torch.rand(E, generator=g))
+    sw13 = O.e4m3_quantize(torch.randn(2 * I, H, generator=g))
+    sw2 = O.e4m3_quantize(torch.randn(H, I, generator=g))
+    ss13, ss2 = torch.tensor([0.013]), torch.tensor([0.017])
+    gate = (torch.randn(1, H, generator=g) * 0.1).half()
+    got = O.moe_forward_full_kmajor(x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate, k)
+    blk = lambda sc, n, kk: sc.reshape(-1, 1, 1).expand(-1, n // 128, kk // 128).contiguous()
+    want = O.moe_forward_full(x, logits, w13.transpose(1, 2).contiguous(), blk(s13, 2 * I, H), sw13,
+                              ss13.expand(2 * I // 128, H // 128).contiguous(), w2.transpose(1, 2).contiguous(),
+                              blk(s2, H, I), sw2, ss2.expand(H // 128, I // 128).contiguous(), gate, k)
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
