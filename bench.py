@@ -338,6 +338,49 @@ def wl_moe_gelu(dev):
                 kernel="moe_gemm_kernel", cpu=cpu, cpu_scale=n_cpu / T)
 
 
+def wl_moe_forward_full(dev):
+    """Per-tensor FP8 MoE decode step at Qwen3-Next sizes: one token, 512 experts, top 10, one shared
+    expert; routed weights K-major (moe_forward_full, vllm/custom-esimd-kernels-vllm/csrc/moe_batch/moe.sycl:1855).
+    Each launch routes to ten other experts and another copy of the shared expert, so nothing is
+    served from the Infinity Cache."""
+    import custom_esimd_kernels_vllm  # noqa: F401
+    from oracle import qlinear_oracle as O
+    T, E, K, H, I = 1, 512, 10, 2048, 512
+    g = torch.Generator(device=dev).manual_seed(98)
+    f8 = lambda *shape: ((torch.randn(*shape, generator=g, device=dev)).clamp(-3, 3) * 100).to(torch.float8_e4m3fn)
+    x = (torch.randn(T, H, generator=g, device=dev) * 0.3).half()
+    w13, w2 = f8(E, H, 2 * I), f8(E, I, H)
+    s13 = torch.full((E,), 2e-4, device=dev)
+    s2 = torch.full((E,), 2e-4, device=dev)
+    R = 96
+    sw13 = [f8(1, 2 * I, H) for _ in range(R)]
+    sw2 = [f8(1, H, I) for _ in range(R)]
+    ss = torch.full((1,), 2e-4, device=dev)
+    gate = (torch.randn(1, H, generator=g, device=dev) * 0.05).half()
+    sets = E // K
+    logits = []
+    for i in range(sets):                            # launch i prefers experts [i*K, (i+1)*K)
+        l = torch.randn(T, E, generator=g, device=dev) * 0.1
+        l[:, i * K:(i + 1) * K] += 8.0
+        logits.append(l.half())
+
+    def launch(i):
+        torch.ops.moe_ops.moe_forward_full(x, logits[i % sets], w13, s13, sw13[i % R], ss, w2, s2, sw2[i % R], ss, gate,
+                                           K, 1, E)
+
+    def cpu():
+        u8 = lambda t: t.view(torch.uint8).cpu()
+        return O.moe_forward_full_kmajor(x.cpu(), logits[0].cpu(), u8(w13), s13.cpu(), u8(sw13[0]), ss.cpu(), u8(w2),
+                                         s2.cpu(), u8(sw2[0]), ss.cpu(), gate.cpu(), K)
+
+    alg_bytes = (K + 1) * 3 * H * I + 2 * T * E + 4 * T * H
+    flops = 2 * T * (K + 1) * 3 * H * I
+    return dict(launch=launch, R=sets, bytes=alg_bytes, flops=flops, bound="hbm", dtype="fp16",
+                name=f"next: per-tensor FP8 MoE decode step, K-major routed weights (topk+up+down+shared+finalize) "
+                     f"T={T} E={E} top{K} H={H} I={I} fp16 (w8a16)",
+                kernel="km_up_kernel", cpu=cpu)
+
+
 WORKLOADS = {
     "cfg1_m1": lambda dev: wl_fp8_pern(1, dev),
     "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
@@ -355,6 +398,7 @@ WORKLOADS = {
     "next_q4_0_quantize": wl_q4_0_quantize,
     "next_resadd_norm_gemv": wl_resadd_norm_gemv,
     "next_moe_gelu_grouped": wl_moe_gelu,
+    "next_moe_forward_full_t1": wl_moe_forward_full,
 }
 HEADLINE = "cfg1_m1"
 

@@ -123,51 +123,103 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_down_kernel(const float* __r
   const int k_hi = min(I, k_lo + rows_per_split);
   const float se = up_scale[e];
   const float* up = up_partial + (size_t)route * up_splits * 2 * I;
-  for (int i = threadIdx.x; i < k_hi - k_lo; i += kKmWaves * 64) {
+  // gate / up sums over the up partials: nq threads share one row (each a strided subset of the
+  // splits, eight loads in flight), and the nq sub-sums are added in a fixed order
+  __shared__ float gsum[kKmWaves * 64], usum[kKmWaves * 64];
+  const int rows = k_hi - k_lo;
+  const int nq = rows > 0 && rows <= kKmWaves * 32 ? (kKmWaves * 64) / rows : 1;
+  for (int i0 = 0; i0 < rows; i0 += kKmWaves * 64) {
+    const int i = i0 + (nq > 1 ? (int)threadIdx.x % rows : (int)threadIdx.x);
+    const int q = nq > 1 ? (int)threadIdx.x / rows : 0;
+    const bool mine = i < rows && q < nq;
     float g = 0.f, u = 0.f;
-    for (int s = 0; s < up_splits; ++s) {
-      g += up[(size_t)s * 2 * I + k_lo + i];
-      u += up[(size_t)s * 2 * I + I + k_lo + i];
+    if (mine) {
+      for (int s0 = q; s0 < up_splits; s0 += 8 * nq) {
+        float gv[8], uv[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+          const bool ok = s0 + b * nq < up_splits;
+          const size_t row = (size_t)(ok ? s0 + b * nq : 0) * 2 * I + k_lo + i;
+          gv[b] = ok ? up[row] : 0.f;
+          uv[b] = ok ? up[row + I] : 0.f;
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b) { g += gv[b]; u += uv[b]; }
+      }
     }
-    g *= se;
-    u *= se;
-    float a;
-    if (gelu) {
-      float two_z = 2.0f * (0.7978845608f * (g + 0.044715f * (g * g * g)));
-      two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
-      const float ex = __expf(two_z);
-      a = 0.5f * g * (1.0f + (ex - 1.0f) / (ex + 1.0f));
-    } else {
-      a = g / (1.0f + __expf(-g));
+    if (nq > 1) {
+      gsum[threadIdx.x] = g;
+      usum[threadIdx.x] = u;
+      __syncthreads();
+      if (q == 0 && i < rows) {
+        for (int qq = 1; qq < nq; ++qq) { g += gsum[qq * rows + i]; u += usum[qq * rows + i]; }
+      }
     }
-    mult[i] = Act::to_f32(Act::from_f32(a * u));
+    if (q == 0 && i < rows) {
+      g *= se;
+      u *= se;
+      float a;
+      if (gelu) {
+        float two_z = 2.0f * (0.7978845608f * (g + 0.044715f * (g * g * g)));
+        two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
+        const float ex = __expf(two_z);
+        a = 0.5f * g * (1.0f + (ex - 1.0f) / (ex + 1.0f));
+      } else {
+        a = g / (1.0f + __expf(-g));
+      }
+      mult[i] = Act::to_f32(Act::from_f32(a * u));
+    }
   }
   __syncthreads();
   km_stream(w2 + (size_t)e * I * H, mult, red, partial + ((size_t)route * splits + sp) * H, k_lo, k_hi, H, cb * 1024);
 }
 
 // out[t][h] = sum_j w[t][j] * s2[e(t,j)] * sum_s partial[(t,j)][s][h]  (+ gate[t] * shared[t][h])
+// One workgroup per (token, 256 columns): lane = 4 columns, the (route, split) pairs are dealt
+// round-robin to the sixteen wavefronts (eight independent loads in flight each), whose sums are
+// added in wave order through LDS, so the result does not depend on timing.
+constexpr int kKmFinWaves = 16;
 template <class Act>
-__global__ __launch_bounds__(256) void km_finalize_kernel(const float* __restrict__ partial, int splits,
-                                                          const float* __restrict__ down_scale,
-                                                          const int32_t* __restrict__ route_expert,
-                                                          const typename Act::elem* __restrict__ top_w,
-                                                          const typename Act::elem* __restrict__ shared,
-                                                          const float* __restrict__ gate,
-                                                          typename Act::elem* __restrict__ out, int T, int top_k,
-                                                          int H) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const int h4 = H >> 2;
-  if (idx >= (size_t)T * h4) return;
-  const int t = (int)(idx / h4), h = (int)(idx % h4) * 4;
-  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-  for (int j = 0; j < top_k; ++j) {
-    const int route = t * top_k + j;
-    f32x4 r = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < splits; ++s)
-      r += *reinterpret_cast<const f32x4*>(partial + ((size_t)route * splits + s) * H + h);
-    sum += r * (Act::to_f32(top_w[route]) * down_scale[route_expert[route]]);
+__global__ __launch_bounds__(kKmFinWaves * 64) void km_finalize_kernel(
+    const float* __restrict__ partial, int splits, const float* __restrict__ down_scale,
+    const int32_t* __restrict__ route_expert, const typename Act::elem* __restrict__ top_w,
+    const typename Act::elem* __restrict__ shared, const float* __restrict__ gate, typename Act::elem* __restrict__ out,
+    int T, int top_k, int H, int cblocks) {
+  __shared__ f32x4 red[kKmFinWaves][64];
+  __shared__ float coef[64];                          // routing weight x down scale per route (top_k <= 64)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int t = blockIdx.x / cblocks;
+  const int h = ((blockIdx.x % cblocks) * 64 + lane) * 4;
+  const bool live = h < H;
+  if ((int)threadIdx.x < top_k) {
+    const int route = t * top_k + threadIdx.x;
+    coef[threadIdx.x] = Act::to_f32(top_w[route]) * down_scale[route_expert[route]];
   }
+  __syncthreads();
+  const int pairs = top_k * splits;
+  const float* base = partial + (size_t)t * pairs * H + (live ? h : 0);
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+  for (int p0 = wave; p0 < pairs; p0 += kKmFinWaves * 8) {
+    f32x4 v[8];
+    float c[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int p = p0 + kKmFinWaves * b;
+      const bool ok = p < pairs;
+      const int pc = ok ? p : 0;
+      v[b] = *reinterpret_cast<const f32x4*>(base + (size_t)pc * H);
+      c[b] = ok ? coef[pc / splits] : 0.f;
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) sum += v[b] * c[b];
+  }
+  red[wave][lane] = sum;
+  __syncthreads();
+  if (wave != 0 || !live) return;
+  sum = red[0][lane];
+#pragma unroll
+  for (int w = 1; w < kKmFinWaves; ++w) sum += red[w][lane];
   if (shared) {
     const float gt = gate ? gate[t] : 1.0f;
 #pragma unroll
@@ -236,17 +288,17 @@ int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_s
                            int H, int act_dtype, void* stream) {
   if (!partial || !down_scale || !route_expert || !top_w || !out) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (T < 0 || top_k <= 0 || H <= 0 || (H % 4) || splits <= 0) return MI_ERR_SHAPE;
+  if (T < 0 || top_k <= 0 || top_k > 64 || H <= 0 || (H % 4) || splits <= 0) return MI_ERR_SHAPE;
   if (!T) return MI_OK;
-  const size_t n = (size_t)T * (H / 4);
-  const dim3 grid((unsigned)((n + 255) / 256));
+  const int cblocks = (H + 255) / 256;
+  const dim3 grid((unsigned)T * cblocks);
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == DT_F16)
-    hipLaunchKernelGGL(km_finalize_kernel<ActF16>, grid, dim3(256), 0, st, partial, splits, down_scale, route_expert,
-                       (const _Float16*)top_w, (const _Float16*)shared, gate, (_Float16*)out, T, top_k, H);
+    hipLaunchKernelGGL(km_finalize_kernel<ActF16>, grid, dim3(kKmFinWaves * 64), 0, st, partial, splits, down_scale, route_expert,
+                       (const _Float16*)top_w, (const _Float16*)shared, gate, (_Float16*)out, T, top_k, H, cblocks);
   else
-    hipLaunchKernelGGL(km_finalize_kernel<ActBF16>, grid, dim3(256), 0, st, partial, splits, down_scale, route_expert,
-                       (const __bf16*)top_w, (const __bf16*)shared, gate, (__bf16*)out, T, top_k, H);
+    hipLaunchKernelGGL(km_finalize_kernel<ActBF16>, grid, dim3(kKmFinWaves * 64), 0, st, partial, splits, down_scale, route_expert,
+                       (const __bf16*)top_w, (const __bf16*)shared, gate, (__bf16*)out, T, top_k, H, cblocks);
   return launch_status();
 }
 
