@@ -381,6 +381,28 @@ def wl_moe_forward_full(dev):
                 kernel="km_up_kernel", cpu=cpu)
 
 
+def wl_gemv_fp16(dev):
+    """16-bit weight GEMV at the reference test's largest router shape (tests/test_gemv_fp16.py:62-71)."""
+    import custom_esimd_kernels_vllm as v
+    M, N, K = 8, 256, 2048
+    g = torch.Generator().manual_seed(99)
+    x = (torch.randn(M, K, generator=g) * 0.1).half()
+    per = N * K * 2
+    R = _copies(per)
+    W = [(torch.randn(N, K, generator=g) * 0.05).half().to(dev) for _ in range(R)]
+    xd = x.to(dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        v.esimd_gemv_fp16(xd, W[i % R], out)
+
+    def cpu():
+        return (x.float() @ W[0].cpu().float().t()).half()
+
+    return dict(launch=launch, R=R, bytes=per + 2 * M * K + 2 * M * N, flops=2 * M * N * K, bound="hbm", dtype="f16",
+                name=f"next: 16-bit weight GEMV (router) M={M} K={K} N={N} fp16", kernel="gemv_w16_kernel", cpu=cpu)
+
+
 WORKLOADS = {
     "cfg1_m1": lambda dev: wl_fp8_pern(1, dev),
     "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
@@ -399,6 +421,7 @@ WORKLOADS = {
     "next_resadd_norm_gemv": wl_resadd_norm_gemv,
     "next_moe_gelu_grouped": wl_moe_gelu,
     "next_moe_forward_full_t1": wl_moe_forward_full,
+    "next_gemv_fp16_router": wl_gemv_fp16,
 }
 HEADLINE = "cfg1_m1"
 

@@ -343,6 +343,15 @@ int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_s
                            const void* top_w, const void* shared, const float* gate, void* out, int T, int top_k,
                            int H, int act_dtype, void* stream);
 
+/* ---- 16-bit (unquantized) weight GEMV for the small projections beside the quantized ones
+ * out[M, N] = x[M, K] @ w[N, K]^T, w in the activation type; K % 8 == 0.  gelu_mul = 1: w is
+ * [2N, K] (gate rows first) and out = gelu_tanh(x @ gate^T) * (x @ up^T).
+ * Replaces esimd_gemv_fp16 and esimd_gemv_fp16_gelu_mul (V/csrc/xpu/torch_extension.cc:27-34)
+ * and the fp16 half of esimd_gemv_fp8_blockscale_fp16_fused2 (torch_extension_gemm.cc:37-41,
+ * V/csrc/xpu/esimd_kernels/fp8_GEMM_blockscale.h:228-446). */
+int mi_gemv_w16(const void* x, const void* w, void* out, int M, int N, int K, int gelu_mul, int act_dtype,
+                void* stream);
+
 #ifdef __cplusplus
 }
 #endif

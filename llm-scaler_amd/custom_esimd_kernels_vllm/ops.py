@@ -50,6 +50,20 @@ def esimd_gemv_fp8_blockscale_fused2(input, w0, s0, o0, w1, s1, o1, block_n=128,
     return _ops.esimd_gemv_fp8_blockscale_fused2(input, w0, s0, o0, w1, s1, o1, block_n, block_k)
 
 
+def esimd_gemv_fp8_blockscale_fp16_fused2(input, w0, s0, o0, w1, o1, block_n=128, block_k=128):
+    return _ops.esimd_gemv_fp8_blockscale_fp16_fused2(input, w0, s0, o0, w1, o1, block_n, block_k)
+
+
+def esimd_gemv_fp16(input, weight, output):
+    """input [M, K], weight [N, K] (16-bit, contiguous), output [M, N]."""
+    return _ops.esimd_gemv_fp16(input, weight, output)
+
+
+def esimd_gemv_fp16_gelu_mul(input, weight, output):
+    """weight [2N, K], gate rows first; output [M, N] = gelu_tanh(gate) * up."""
+    return _ops.esimd_gemv_fp16_gelu_mul(input, weight, output)
+
+
 def esimd_gemv_int4(input, weight, weight_scale, output):
     """weight [N, K/2] uint8 (or [N, K/8] int32), low nibble = even k, stored value + 8;
     weight_scale [N, K/128] fp16."""

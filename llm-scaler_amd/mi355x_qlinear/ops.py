@@ -171,6 +171,44 @@ def esimd_gemv_fp8_blockscale_fused2(input, w0, s0, o0, w1, s1, o1, block_n, blo
 
 
 # --------------------------------------------------------------------------
+# 16-bit weights beside the quantized ones (esimd_gemv_fp16, _gelu_mul, the fp16 half of
+# esimd_gemv_fp8_blockscale_fp16_fused2)
+# --------------------------------------------------------------------------
+def _gemv_w16(x, w, out, gelu, who):
+    _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, f"{who}: input [M, K], weight [N, K], output [M, N]")
+    _chk_act(x, out, who)
+    _chk(w.dtype == x.dtype and w.is_contiguous(), f"{who}: weight must be contiguous and share the input dtype")
+    M, K = x.shape
+    rows = w.shape[0]
+    _chk(w.shape[1] == K and K % 8 == 0, f"{who}: weight must be [N, K={K}] with K a multiple of 8")
+    _chk(not gelu or rows % 2 == 0, f"{who}: the gate-up weight must have an even number of rows")
+    N = rows // 2 if gelu else rows
+    _chk(tuple(out.shape) == (M, N), f"{who}: output must be [M, N] = {(M, N)}, got {tuple(out.shape)}")
+    capi.call("mi_gemv_w16", x, capi.ptr(x), capi.ptr(w), capi.ptr(out), M, N, K, 1 if gelu else 0, capi.act_dtype(x))
+    return out
+
+
+def esimd_gemv_fp16(input, weight, output):
+    """out = input @ weight^T on 16-bit weights (V/csrc/xpu/torch_extension.cc:27-28); bf16 accepted too."""
+    return _gemv_w16(input, weight, output, False, "esimd_gemv_fp16")
+
+
+def esimd_gemv_fp16_gelu_mul(input, weight, output):
+    """weight [2N, K], gate rows first: out = gelu_tanh(input @ gate^T) * (input @ up^T)
+    (V/csrc/xpu/torch_extension.cc:30-33)."""
+    return _gemv_w16(input, weight, output, True, "esimd_gemv_fp16_gelu_mul")
+
+
+def esimd_gemv_fp8_blockscale_fp16_fused2(input, w0, s0, o0, w1, o1, block_n, block_k):
+    """A block-scaled FP8 weight and a 16-bit weight sharing the input
+    (V/csrc/xpu/torch_extension_gemm.cc:37-41).  Two launches here: the formats do not share a kernel."""
+    who = "esimd_gemv_fp8_blockscale_fp16_fused2"
+    _fp8_block_multi(input, [w0], [s0], [o0], block_n, block_k, who)
+    _gemv_w16(input, w1, o1, False, who)
+    return o0
+
+
+# --------------------------------------------------------------------------
 # INT4 group-128  (esimd_gemv_int4, _fused2, esimd_gemm_int4_pgrp [+ _zp sibling])
 # --------------------------------------------------------------------------
 def _int4_nk(w: torch.Tensor, who: str):
@@ -1524,6 +1562,12 @@ def register():
                     "Tensor output) -> Tensor", esimd_gemm_fp8_pert, _ret(3))
         _define(ns, "esimd_gemm_fp8_blockscale(Tensor input, Tensor weight, Tensor weight_scale, "
                     "Tensor output, int block_n, int block_k) -> Tensor", esimd_gemm_fp8_blockscale, _ret(3))
+        _define(ns, "esimd_gemv_fp16(Tensor input, Tensor weight, Tensor output) -> Tensor", esimd_gemv_fp16, _ret(2))
+        _define(ns, "esimd_gemv_fp16_gelu_mul(Tensor input, Tensor weight, Tensor output) -> Tensor",
+                esimd_gemv_fp16_gelu_mul, _ret(2))
+        _define(ns, "esimd_gemv_fp8_blockscale_fp16_fused2(Tensor input, Tensor w0, Tensor s0, Tensor(a!) o0, "
+                    "Tensor w1, Tensor(b!) o1, int block_n, int block_k) -> Tensor(a!)",
+                esimd_gemv_fp8_blockscale_fp16_fused2, _ret(3))
         _define(ns, "esimd_gemv_fp8_blockscale_fused2(Tensor input, Tensor w0, Tensor s0, Tensor(a!) o0, "
                     "Tensor w1, Tensor s1, Tensor(b!) o1, int block_n, int block_k) -> Tensor(a!)",
                 esimd_gemv_fp8_blockscale_fused2, _ret(3))

@@ -602,3 +602,58 @@ def test_int4_small_n_many_rows(ops, dev):
     v, _ = ops
     assert _run_int4(v, dev, 48, 4096, 1536, torch.bfloat16, seed=77) < TOL
     assert _run_int4(v, dev, 64, 2048, 4096, torch.float16, seed=78) < TOL
+
+
+# ----------------------------------------------------------------- 16-bit weights beside the quantized ones
+@pytest.mark.parametrize("M,N,K", [(1, 128, 2816), (1, 128, 1408), (2, 32, 2048), (4, 32, 2048), (8, 32, 2048),
+                                   (2, 256, 2048), (8, 256, 2048), (11, 13, 264)])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_gemv_fp16(ops, dev, M, N, K, dt):
+    """The shapes of V/tests/test_gemv_fp16.py:62-71 (routers, the GDN b/a projection) plus a ragged one,
+    against the fp32 product of the same 16-bit operands."""
+    v, _ = ops
+    g = torch.Generator().manual_seed(M * 100 + N)
+    x = (torch.randn(M, K, generator=g) * 0.1).to(dt)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dt)
+    out = torch.full((M, N), float("nan"), dtype=dt, device=dev)
+    r = v.esimd_gemv_fp16(x.to(dev), w.to(dev), out)
+    assert r.data_ptr() == out.data_ptr()
+    ref = x.float() @ w.float().t()
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+    assert (out.cpu().float() - ref).abs().max().item() < 5e-2           # the reference test's bar
+
+
+def test_gemv_fp16_gelu_mul_and_errors(ops, dev):
+    v, _ = ops
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 3, 96, 1024
+    x = (torch.randn(M, K, generator=g) * 0.3).half()
+    w = (torch.randn(2 * N, K, generator=g) * 0.1).half()
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    v.esimd_gemv_fp16_gelu_mul(x.to(dev), w.to(dev), out)
+    ref = O.gelu_tanh_mul(x.float() @ w.float().t())
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+    xd, wd = x.to(dev), w[:N].contiguous().to(dev)
+    o = torch.empty(M, N, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError):                                     # mixed dtypes
+        v.esimd_gemv_fp16(xd.to(torch.bfloat16), wd, o)
+    with pytest.raises(RuntimeError):                                     # non-contiguous input
+        v.esimd_gemv_fp16(torch.randn(K, M, dtype=torch.float16, device=dev).t(), wd, o)
+    with pytest.raises(RuntimeError):                                     # wrong output shape
+        v.esimd_gemv_fp16(xd, wd, torch.empty(M, N - 1, dtype=torch.float16, device=dev))
+
+
+def test_fp8_blockscale_fp16_fused2(ops, dev):
+    """Block-scaled qkvz weight + 16-bit b/a weight on one input (V/tests/test_fp8_blockscale_fusions.py)."""
+    v, _ = ops
+    M, K, N0, N1 = 1, 2048, 1024, 64
+    x, w8, s = O.make_fp8_block_case(M, K, N0, seed=21, act_dtype=torch.float16)
+    g = torch.Generator().manual_seed(22)
+    w1 = (torch.randn(N1, K, generator=g) * 0.05).half()
+    o0 = torch.empty(M, N0, dtype=torch.float16, device=dev)
+    o1 = torch.empty(M, N1, dtype=torch.float16, device=dev)
+    r = v.esimd_gemv_fp8_blockscale_fp16_fused2(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), s.to(dev), o0,
+                                                w1.to(dev), o1)
+    assert r.data_ptr() == o0.data_ptr()
+    assert O.max_rel_err(o0.cpu(), O.matmul_ref(x, O.fp8_dequant_block(w8, s))) < TOL
+    assert O.max_rel_err(o1.cpu(), x.float() @ w1.float().t()) < TOL
