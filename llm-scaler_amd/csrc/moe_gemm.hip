@@ -40,7 +40,7 @@ struct MoeGemmArgs {
   const void* row_weight;     // optional, activation dtype: factor per row of `out`
   int out_f32;
   int gelu;                   // fused epilogue: tanh-GELU instead of SiLU
-  int s_e, s_nb, s_g;         // w_scale strides: expert, 128-row block, granule (0, 0 = per expert)
+  int scale_per_expert;       // w_scale is [E] instead of block scales
   int E, N, K;                // N = weight rows per expert
   int n_out;                  // output columns (N, or N/2 with the fused SiLU*mul)
   int tiles_per_expert;       // workgroups per expert
@@ -73,7 +73,7 @@ constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of
 // The weights are the MFMA A operand and the activations the B operand, so a lane
 // ends up holding ONE activation row (16 w + j) and four consecutive weight rows
 // (4 g + v): the per-row activation scale is a single value per lane and granule.
-template <class Act, bool A8, bool SILU, int RT, int D>
+template <class Act, bool A8, bool SILU, int RT, int D, bool PE>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, const float* __restrict__ w_scale,
                                                         const int32_t* __restrict__ expert_start) {
   static_assert(RT == 2 || RT == 4 || RT == 8, "two, four or eight weight tiles");
@@ -134,8 +134,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   const int Nb = (N + 127) >> 7;
   // read through a restrict kernel argument so the (uniform) scale loads stay on the
   // scalar unit and do not queue behind the vector prefetch
-  const float* __restrict__ wsc = w_scale + (size_t)e * p.s_e;
-  const int s_nb = p.s_nb, s_g = p.s_g;
+  // PE: one scale per expert, read once; otherwise the block scales of this expert
+  const float* __restrict__ wsc = PE ? w_scale + e : w_scale + (size_t)e * Nb * Kb;
+  const float ws_expert = PE ? wsc[0] : 1.0f;
   const uint32_t tg_stride = (uint32_t)kCols * (uint32_t)K;   // weight bytes between tile groups
 
   struct Regs {                                       // one granule in flight
@@ -176,7 +177,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
     auto load_granule = [&](Regs& r, int tg, int gi) {
       const uint32_t dead = tg < ntg ? 0u : 0x80000000u;
       const uint32_t wso = (uint32_t)tg * tg_stride + (uint32_t)gi * 128u;
-      const int kext = gi == G - 1 ? ktail : 128;     // uniform
+      // quantised activations come in whole 128-groups: no partial granule there
+      const int kext = (!A8 && gi == G - 1) ? ktail : 128;   // uniform
 #pragma unroll
       for (int i = 0; i < WL; ++i) {
         const bool ok = wcol[i] + tg * kCols < limit && wch[i] < kext;
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
           float sc[RT];
 #pragma unroll
           for (int t = 0; t < RT; ++t) {
-            const float ws = wsc[nb[t] * s_nb + gi * s_g];
+            const float ws = PE ? ws_expert : wsc[(size_t)nb[t] * Kb + gi];
             sc[t] = A8 ? xs_now * ws : ws;
           }
           // prefetch D granules ahead, across the tile-group boundary
@@ -340,6 +342,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
 
 template <class Act, bool A8, bool SILU, int RT, int D>
 static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
+  // quantised activations only come with block scales (the per-expert form is the reference's w8a16 mode)
+  constexpr bool kHasPE = !A8;
   const int cols = SILU ? p.N / 2 : p.N;
   const int cols_per_group = SILU ? (RT / 2) * 16 : RT * 16;
   const int groups = (cols + cols_per_group - 1) / cols_per_group;
@@ -348,7 +352,14 @@ static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
   p.n_out = cols;
   const long wgs = (long)p.E * p.tiles_per_expert;
   if (wgs <= 0) return MI_OK;
-  hipLaunchKernelGGL((moe_gemm_kernel<Act, A8, SILU, RT, D>), dim3((unsigned)wgs), dim3(256), 0, st, p,
+  if constexpr (kHasPE) {
+    if (p.scale_per_expert) {
+      hipLaunchKernelGGL((moe_gemm_kernel<Act, A8, SILU, RT, D, true>), dim3((unsigned)wgs), dim3(256), 0, st, p,
+                         p.w_scale, p.start);
+      return launch_status();
+    }
+  }
+  hipLaunchKernelGGL((moe_gemm_kernel<Act, A8, SILU, RT, D, false>), dim3((unsigned)wgs), dim3(256), 0, st, p,
                      p.w_scale, p.start);
   return launch_status();
 }
@@ -400,9 +411,8 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
   p.out_map = out_map; p.row_weight = row_weight;
   p.out_f32 = out_f32;
   p.gelu = fuse_act == 2;
-  const int Kb = (K + 127) / 128, Nb = (N + 127) / 128;
-  if (scale_per_expert) { p.s_e = 1; p.s_nb = 0; p.s_g = 0; }
-  else { p.s_e = Nb * Kb; p.s_nb = Kb; p.s_g = 1; }
+  if (a_scale && scale_per_expert) return MI_ERR_ARG;
+  p.scale_per_expert = scale_per_expert ? 1 : 0;
   hipStream_t st = (hipStream_t)stream;
   if (a_scale) {
     return act_dtype == DT_F16 ? dispatch_moe<ActF16, true>(p, fuse_act, st)
