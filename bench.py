@@ -388,7 +388,7 @@ def wl_gemv_fp16(dev):
     g = torch.Generator().manual_seed(99)
     x = (torch.randn(M, K, generator=g) * 0.1).half()
     per = N * K * 2
-    R = _copies(per)
+    R = 320                                      # 335 MB of distinct weights: more than the Infinity Cache
     W = [(torch.randn(N, K, generator=g) * 0.05).half().to(dev) for _ in range(R)]
     xd = x.to(dev)
     out = torch.empty(M, N, dtype=torch.float16, device=dev)
