@@ -35,8 +35,12 @@ __device__ __forceinline__ void km_fma16(float (&acc)[16], const u32x4 v, const 
 
 // Rows [k_lo, k_hi) of one expert's [K, N] matrix against the multipliers in LDS
 // (mult[k - k_lo]); columns [c0 + 16 lane, +16).  The partial row goes to `dst` (fp32, N wide).
+// `fill` computes the multipliers into `mult` (it ends with a workgroup barrier); it runs after
+// the first batch of weight loads has been issued, so that its own loads wait together with
+// them instead of in front of them.
+template <class Fill>
 __device__ __forceinline__ void km_stream(const uint8_t* __restrict__ wexp, const float* mult, float* red,
-                                          float* __restrict__ dst, int k_lo, int k_hi, int N, int c0) {
+                                          float* __restrict__ dst, int k_lo, int k_hi, int N, int c0, Fill&& fill) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = c0 + lane * 16;
@@ -46,20 +50,27 @@ __device__ __forceinline__ void km_stream(const uint8_t* __restrict__ wexp, cons
   float acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  for (int k0 = k_lo + wave * kKmBatch; k0 < k_hi; k0 += kKmWaves * kKmBatch) {
-    u32x4 v[kKmBatch];
+  auto load_batch = [&](u32x4 (&v)[kKmBatch], int k0) {
 #pragma unroll
     for (int b = 0; b < kKmBatch; ++b) {
       const int k = k0 + b;
       const uint32_t off = k < k_hi ? ((uint32_t)k * (uint32_t)N + (uint32_t)col) | dead : 0x80000000u;
       v[b] = __builtin_amdgcn_raw_buffer_load_b128(wr, off, 0, 2);
     }
+  };
+  u32x4 v[kKmBatch];
+  int k0 = k_lo + wave * kKmBatch;
+  load_batch(v, k0);
+  __builtin_amdgcn_sched_barrier(0);
+  fill();
+  for (; k0 < k_hi; k0 += kKmWaves * kKmBatch) {
 #pragma unroll
     for (int b = 0; b < kKmBatch; ++b) {
       const int k = k0 + b;
       const float a = k < k_hi ? mult[k - k_lo] : 0.f;
       km_fma16(acc, v[b], a);
     }
+    if (k0 + kKmWaves * kKmBatch < k_hi) load_batch(v, k0 + kKmWaves * kKmBatch);
   }
   // reduce the four wavefronts' partial rows through LDS: red[wave][i][lane]
 #pragma unroll
@@ -97,10 +108,11 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_up_kernel(const typename Act
   const int k_lo = sp * rows_per_split;
   const int k_hi = min(H, k_lo + rows_per_split);
   const typename Act::elem* xr = x + (size_t)(route / top_k) * H;
-  for (int i = threadIdx.x; i < k_hi - k_lo; i += kKmWaves * 64) mult[i] = Act::to_f32(xr[k_lo + i]);
-  __syncthreads();
   km_stream(w + (size_t)e * H * two_i, mult, red, partial + ((size_t)route * splits + sp) * two_i, k_lo, k_hi, two_i,
-            cb * 1024);
+            cb * 1024, [&]() {
+              for (int i = threadIdx.x; i < k_hi - k_lo; i += kKmWaves * 64) mult[i] = Act::to_f32(xr[k_lo + i]);
+              __syncthreads();
+            });
 }
 
 // grid = routes * splits * column blocks.  The multipliers are the route's intermediate
@@ -123,6 +135,7 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_down_kernel(const float* __r
   const int k_hi = min(I, k_lo + rows_per_split);
   const float se = up_scale[e];
   const float* up = up_partial + (size_t)route * up_splits * 2 * I;
+  auto fill = [&]() {
   // gate / up sums over the up partials: nq threads share one row (each a strided subset of the
   // splits, eight loads in flight), and the nq sub-sums are added in a fixed order
   __shared__ float gsum[kKmWaves * 64], usum[kKmWaves * 64];
@@ -171,7 +184,8 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_down_kernel(const float* __r
     }
   }
   __syncthreads();
-  km_stream(w2 + (size_t)e * I * H, mult, red, partial + ((size_t)route * splits + sp) * H, k_lo, k_hi, H, cb * 1024);
+  };
+  km_stream(w2 + (size_t)e * I * H, mult, red, partial + ((size_t)route * splits + sp) * H, k_lo, k_hi, H, cb * 1024, fill);
 }
 
 // out[t][h] = sum_j w[t][j] * s2[e(t,j)] * sum_s partial[(t,j)][s][h]  (+ gate[t] * shared[t][h])

@@ -1443,7 +1443,9 @@ def _km_splits(routes, K, N, dev):
     cblocks = (N + 1023) // 1024
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     want = -(-2 * cus // max(1, routes * cblocks))
-    return max(min(want, max(1, K // 32)), -(-K // 1024))
+    # whole batches of 32 rows (8 per wavefront): a workgroup then waits for memory once per batch
+    rows = min(1024, max(32, (K // want) // 32 * 32))
+    return -(-K // rows)
 
 
 def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight, shared_gate_up_scale,
