@@ -332,16 +332,16 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
  * mi_moe_kmajor_finalize: out[t][:] = sum_j top_w[t][j] * s2[e] * sum_s partial[r][s][:]
  *                     + gate[t] * shared[t][:] (shared / gate optional), rounded once.
  * `splits` (K split over workgroups, rows per split = ceil(K / splits) rounded up to 8, at most
- * 1024) is the caller's choice: about two workgroups per compute unit over
+ * 1024) is the caller's choice; a route whose expert id is outside [0, num_experts) contributes zeros: about two workgroups per compute unit over
  * routes * ceil(N / 1024) column blocks fills the device. */
 int mi_moe_kmajor_up(const void* x, const void* w, const int32_t* route_expert, float* partial, int routes,
-                     int top_k, int H, int two_i, int splits, int act_dtype, void* stream);
+                     int top_k, int num_experts, int H, int two_i, int splits, int act_dtype, void* stream);
 int mi_moe_kmajor_down(const float* up_partial, int up_splits, const float* up_scale, const void* w2,
-                       const int32_t* route_expert, float* partial, int routes, int I, int H, int splits,
-                       int gelu, int act_dtype, void* stream);
+                       const int32_t* route_expert, float* partial, int routes, int num_experts, int I, int H,
+                       int splits, int gelu, int act_dtype, void* stream);
 int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_scale, const int32_t* route_expert,
                            const void* top_w, const void* shared, const float* gate, void* out, int T, int top_k,
-                           int H, int act_dtype, void* stream);
+                           int num_experts, int H, int act_dtype, void* stream);
 
 /* ---- 16-bit (unquantized) weight GEMV for the small projections beside the quantized ones
  * out[M, N] = x[M, K] @ w[N, K]^T, w in the activation type; K % 8 == 0.  gelu_mul = 1: w is

@@ -98,15 +98,18 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_up_kernel(const typename Act
                                                               const uint8_t* __restrict__ w,
                                                               const int32_t* __restrict__ route_expert,
                                                               float* __restrict__ partial, int top_k, int H,
-                                                              int two_i, int splits, int rows_per_split, int cblocks) {
+                                                              int two_i, int splits, int rows_per_split, int cblocks,
+                                                              int E) {
   __shared__ float mult[1024];
   __shared__ float red[kKmWaves * 16 * 64];
   const int cb = blockIdx.x % cblocks;
   const int sp = (blockIdx.x / cblocks) % splits;
   const int route = blockIdx.x / (cblocks * splits);
-  const int e = route_expert[route];
+  int e = route_expert[route];
+  const bool valid = (unsigned)e < (unsigned)E;       // an id outside [0, E) contributes zeros
+  if (!valid) e = 0;
   const int k_lo = sp * rows_per_split;
-  const int k_hi = min(H, k_lo + rows_per_split);
+  const int k_hi = valid ? min(H, k_lo + rows_per_split) : k_lo;
   const typename Act::elem* xr = x + (size_t)(route / top_k) * H;
   km_stream(w + (size_t)e * H * two_i, mult, red, partial + ((size_t)route * splits + sp) * two_i, k_lo, k_hi, two_i,
             cb * 1024, [&]() {
@@ -124,15 +127,17 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_down_kernel(const float* __r
                                                                 const uint8_t* __restrict__ w2,
                                                                 const int32_t* __restrict__ route_expert,
                                                                 float* __restrict__ partial, int I, int H, int splits,
-                                                                int rows_per_split, int cblocks, int gelu) {
+                                                                int rows_per_split, int cblocks, int gelu, int E) {
   __shared__ float mult[1024];
   __shared__ float red[kKmWaves * 16 * 64];
   const int cb = blockIdx.x % cblocks;
   const int sp = (blockIdx.x / cblocks) % splits;
   const int route = blockIdx.x / (cblocks * splits);
-  const int e = route_expert[route];
+  int e = route_expert[route];
+  const bool valid = (unsigned)e < (unsigned)E;
+  if (!valid) e = 0;
   const int k_lo = sp * rows_per_split;
-  const int k_hi = min(I, k_lo + rows_per_split);
+  const int k_hi = valid ? min(I, k_lo + rows_per_split) : k_lo;
   const float se = up_scale[e];
   const float* up = up_partial + (size_t)route * up_splits * 2 * I;
   auto fill = [&]() {
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(kKmFinWaves * 64) void km_finalize_kernel(
     const float* __restrict__ partial, int splits, const float* __restrict__ down_scale,
     const int32_t* __restrict__ route_expert, const typename Act::elem* __restrict__ top_w,
     const typename Act::elem* __restrict__ shared, const float* __restrict__ gate, typename Act::elem* __restrict__ out,
-    int T, int top_k, int H, int cblocks) {
+    int T, int top_k, int H, int cblocks, int E) {
   __shared__ f32x4 red[kKmFinWaves][64];
   __shared__ float coef[64];                          // routing weight x down scale per route (top_k <= 64)
   const int lane = threadIdx.x & 63;
@@ -208,7 +213,8 @@ __global__ __launch_bounds__(kKmFinWaves * 64) void km_finalize_kernel(
   const bool live = h < H;
   if ((int)threadIdx.x < top_k) {
     const int route = t * top_k + threadIdx.x;
-    coef[threadIdx.x] = Act::to_f32(top_w[route]) * down_scale[route_expert[route]];
+    const int e = route_expert[route];
+    coef[threadIdx.x] = (unsigned)e < (unsigned)E ? Act::to_f32(top_w[route]) * down_scale[e] : 0.f;
   }
   __syncthreads();
   const int pairs = top_k * splits;
@@ -255,10 +261,10 @@ using namespace qlin;
 extern "C" {
 
 int mi_moe_kmajor_up(const void* x, const void* w, const int32_t* route_expert, float* partial, int routes,
-                     int top_k, int H, int two_i, int splits, int act_dtype, void* stream) {
+                     int top_k, int num_experts, int H, int two_i, int splits, int act_dtype, void* stream) {
   if (!x || !w || !route_expert || !partial) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (routes < 0 || top_k <= 0 || H <= 0 || two_i <= 0 || (two_i % 32) || splits <= 0) return MI_ERR_SHAPE;
+  if (routes < 0 || top_k <= 0 || num_experts <= 0 || H <= 0 || two_i <= 0 || (two_i % 32) || splits <= 0) return MI_ERR_SHAPE;
   if ((uint64_t)H * (uint64_t)two_i >= (1ull << 31)) return MI_ERR_SHAPE;
   const int rows = km_rows_per_split(H, splits);
   if (rows > 1024) return MI_ERR_SHAPE;
@@ -268,19 +274,19 @@ int mi_moe_kmajor_up(const void* x, const void* w, const int32_t* route_expert, 
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == DT_F16)
     hipLaunchKernelGGL(km_up_kernel<ActF16>, grid, dim3(kKmWaves * 64), 0, st, (const _Float16*)x, (const uint8_t*)w,
-                       route_expert, partial, top_k, H, two_i, splits, rows, cblocks);
+                       route_expert, partial, top_k, H, two_i, splits, rows, cblocks, num_experts);
   else
     hipLaunchKernelGGL(km_up_kernel<ActBF16>, grid, dim3(kKmWaves * 64), 0, st, (const __bf16*)x, (const uint8_t*)w,
-                       route_expert, partial, top_k, H, two_i, splits, rows, cblocks);
+                       route_expert, partial, top_k, H, two_i, splits, rows, cblocks, num_experts);
   return launch_status();
 }
 
 int mi_moe_kmajor_down(const float* up_partial, int up_splits, const float* up_scale, const void* w2,
-                       const int32_t* route_expert, float* partial, int routes, int I, int H, int splits,
-                       int gelu, int act_dtype, void* stream) {
+                       const int32_t* route_expert, float* partial, int routes, int num_experts, int I, int H,
+                       int splits, int gelu, int act_dtype, void* stream) {
   if (!up_partial || !up_scale || !w2 || !route_expert || !partial) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (routes < 0 || up_splits <= 0 || I <= 0 || H <= 0 || (H % 16) || splits <= 0) return MI_ERR_SHAPE;
+  if (routes < 0 || num_experts <= 0 || up_splits <= 0 || I <= 0 || H <= 0 || (H % 16) || splits <= 0) return MI_ERR_SHAPE;
   if ((uint64_t)H * (uint64_t)I >= (1ull << 31)) return MI_ERR_SHAPE;
   const int rows = km_rows_per_split(I, splits);
   if (rows > 1024) return MI_ERR_SHAPE;
@@ -290,29 +296,29 @@ int mi_moe_kmajor_down(const float* up_partial, int up_splits, const float* up_s
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == DT_F16)
     hipLaunchKernelGGL(km_down_kernel<ActF16>, grid, dim3(kKmWaves * 64), 0, st, up_partial, up_splits, up_scale,
-                       (const uint8_t*)w2, route_expert, partial, I, H, splits, rows, cblocks, gelu);
+                       (const uint8_t*)w2, route_expert, partial, I, H, splits, rows, cblocks, gelu, num_experts);
   else
     hipLaunchKernelGGL(km_down_kernel<ActBF16>, grid, dim3(kKmWaves * 64), 0, st, up_partial, up_splits, up_scale,
-                       (const uint8_t*)w2, route_expert, partial, I, H, splits, rows, cblocks, gelu);
+                       (const uint8_t*)w2, route_expert, partial, I, H, splits, rows, cblocks, gelu, num_experts);
   return launch_status();
 }
 
 int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_scale, const int32_t* route_expert,
                            const void* top_w, const void* shared, const float* gate, void* out, int T, int top_k,
-                           int H, int act_dtype, void* stream) {
+                           int num_experts, int H, int act_dtype, void* stream) {
   if (!partial || !down_scale || !route_expert || !top_w || !out) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (T < 0 || top_k <= 0 || top_k > 64 || H <= 0 || (H % 4) || splits <= 0) return MI_ERR_SHAPE;
+  if (T < 0 || top_k <= 0 || top_k > 64 || num_experts <= 0 || H <= 0 || (H % 4) || splits <= 0) return MI_ERR_SHAPE;
   if (!T) return MI_OK;
   const int cblocks = (H + 255) / 256;
   const dim3 grid((unsigned)T * cblocks);
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == DT_F16)
     hipLaunchKernelGGL(km_finalize_kernel<ActF16>, grid, dim3(kKmFinWaves * 64), 0, st, partial, splits, down_scale, route_expert,
-                       (const _Float16*)top_w, (const _Float16*)shared, gate, (_Float16*)out, T, top_k, H, cblocks);
+                       (const _Float16*)top_w, (const _Float16*)shared, gate, (_Float16*)out, T, top_k, H, cblocks, num_experts);
   else
     hipLaunchKernelGGL(km_finalize_kernel<ActBF16>, grid, dim3(kKmFinWaves * 64), 0, st, partial, splits, down_scale, route_expert,
-                       (const __bf16*)top_w, (const __bf16*)shared, gate, (__bf16*)out, T, top_k, H, cblocks);
+                       (const __bf16*)top_w, (const __bf16*)shared, gate, (__bf16*)out, T, top_k, H, cblocks, num_experts);
   return launch_status();
 }
 

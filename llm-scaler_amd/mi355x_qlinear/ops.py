@@ -1477,11 +1477,11 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
     s_up = _km_splits(P, H, 2 * I, dev)
     up_part = torch.empty(P, s_up, 2 * I, dtype=torch.float32, device=dev)
     capi.call("mi_moe_kmajor_up", x, capi.ptr(x), capi.ptr(gate_up_weight), capi.ptr(route_expert), capi.ptr(up_part), P, k,
-              H, 2 * I, s_up, adt)
+              E, H, 2 * I, s_up, adt)
     s_dn = _km_splits(P, I, H, dev)
     dn_part = torch.empty(P, s_dn, H, dtype=torch.float32, device=dev)
     capi.call("mi_moe_kmajor_down", x, capi.ptr(up_part), s_up, capi.ptr(gate_up_scale.contiguous()), capi.ptr(down_weight),
-              capi.ptr(route_expert), capi.ptr(dn_part), P, I, H, s_dn, 0, adt)
+              capi.ptr(route_expert), capi.ptr(dn_part), P, E, I, H, s_dn, 0, adt)
     shared = gate = None
     if S > 0:
         _chk(S == 1, f"{who}: one shared expert is supported")
@@ -1503,7 +1503,7 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
         capi.call("mi_moe_shared_gate", x, capi.ptr(x), capi.ptr(shared_expert_gate_weight.contiguous()), capi.ptr(gate), T, H, adt)
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     capi.call("mi_moe_kmajor_finalize", x, capi.ptr(dn_part), s_dn, capi.ptr(down_scale.contiguous()), capi.ptr(route_expert),
-              capi.ptr(top_w), capi.ptr(shared), capi.ptr(gate), capi.ptr(out), T, k, H, adt)
+              capi.ptr(top_w), capi.ptr(shared), capi.ptr(gate), capi.ptr(out), T, k, E, H, adt)
     return out
 
 

@@ -580,3 +580,37 @@ def test_moe_forward_full_kmajor_no_shared_expert(v, dev):
     got = torch.ops.moe_ops.moe_forward_full(x.to(dev), logits.to(dev), f8(w13), s13.to(dev), e, e, f8(w2), s2.to(dev), e, e,
                                              e, k, 0, E)
     assert O.max_rel_err(got.cpu().float(), want) < 2 * TOL
+
+
+def test_kmajor_out_of_range_expert_ids_contribute_zero(v, dev):
+    """Routes whose expert id is not in [0, E) must not be dereferenced: their partial rows are zero and
+    they add nothing to the output (the host forces the condition; every kernel exits normally)."""
+    from mi355x_qlinear import capi
+    g = torch.Generator().manual_seed(8)
+    E, H, I, k = 2, 256, 64, 3
+    x = (torch.randn(1, H, generator=g) * 0.3).half()
+    w13 = O.e4m3_quantize(torch.randn(E, H, 2 * I, generator=g))
+    w2 = O.e4m3_quantize(torch.randn(E, I, H, generator=g))
+    s13 = torch.tensor([0.01, 0.02])
+    s2 = torch.tensor([0.03, 0.015])
+    ids = torch.tensor([1, -1, 99], dtype=torch.int32)
+    tw = torch.tensor([[0.5, 0.3, 0.2]]).half()
+    d = lambda t: t.to(dev)
+    xd, w13d, w2d, idd, twd, s13d, s2d = d(x), d(w13), d(w2), d(ids), d(tw), d(s13), d(s2)
+    su, sd = 2, 2
+    up = torch.full((k, su, 2 * I), float("nan"), device=dev)
+    capi.call("mi_moe_kmajor_up", xd, capi.ptr(xd), capi.ptr(w13d), capi.ptr(idd), capi.ptr(up), k, k, E, H, 2 * I, su,
+              capi.DT_F16)
+    assert torch.isfinite(up).all() and (up[1:] == 0).all() and (up[0] != 0).any()
+    dn = torch.full((k, sd, H), float("nan"), device=dev)
+    capi.call("mi_moe_kmajor_down", xd, capi.ptr(up), su, capi.ptr(s13d), capi.ptr(w2d), capi.ptr(idd), capi.ptr(dn), k, E, I, H,
+              sd, 0, capi.DT_F16)
+    assert torch.isfinite(dn).all() and (dn[1:] == 0).all()
+    out = torch.empty(1, H, dtype=torch.float16, device=dev)
+    capi.call("mi_moe_kmajor_finalize", xd, capi.ptr(dn), sd, capi.ptr(s2d), capi.ptr(idd), capi.ptr(twd), None, None,
+              capi.ptr(out), 1, k, E, H, capi.DT_F16)
+    d13 = O.e4m3_decode(w13[1].reshape(-1, 2 * I)).reshape(H, 2 * I)
+    gu = (x.float()[0] @ d13) * s13[1]
+    inter = (torch.nn.functional.silu(gu[:I]) * gu[I:]).half().float()
+    want = 0.5 * s2[1] * (inter @ O.e4m3_decode(w2[1].reshape(-1, H)).reshape(I, H))
+    assert O.max_rel_err(out.cpu().float()[0], want) < TOL
