@@ -290,10 +290,10 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
 
       // ---- epilogue of this tile group: lane holds row 16 w + j, weight rows 4 g + v ----
       const int m = mc + wave * 16 + j;
-      if (active && m < cnt) {
+      const int dst = (active && m < cnt) ? (p.out_map ? p.out_map[r0 + m] : r0 + m) : -1;
+      if ((unsigned)dst < (unsigned)p.total_rows) {    // a mapped row outside the output is dropped
         Elem* out = (Elem*)p.out;
         float* out32 = (float*)p.out;
-        const int dst = p.out_map ? p.out_map[r0 + m] : r0 + m;
         const size_t orow = (size_t)dst * p.n_out;
         const float rw = p.row_weight ? Act::to_f32(((const Elem*)p.row_weight)[dst]) : 1.0f;
         constexpr int NO = SILU ? RT / 2 : RT;
