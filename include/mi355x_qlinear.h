@@ -8,7 +8,9 @@
  *
  *   - every pointer is device memory; outputs are pre-allocated by the caller;
  *   - the call enqueues on `stream` (a hipStream_t, 0 = the null stream) and
- *     returns without synchronising; nothing is allocated or freed;
+ *     returns without synchronising; nothing is allocated or freed, except by the
+ *     entries that say so (mi_gemm_int4: a grow-only scratch buffer; mi_norm_gemv: a
+ *     2 KiB counter block per device and stream, on first use);
  *   - tensors are dense row-major;
  *   - act_dtype: 0 = fp16, 1 = bf16 (inputs and outputs share it);
  *   - return value: 0 on success, MI_ERR_ARG (-1) for a null pointer or bad
@@ -268,8 +270,9 @@ int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weig
  *   block scale, 2 = INT4 group 128 (scale[i] fp16 [N, K/128]).  residual (in place),
  *   gate and normed_out may be null.  Every workgroup normalises its own copy of the
  *   row; the in-place residual and normed_out are written by the workgroup that
- *   arrives last at a per-stream device counter, after all others have read their
- *   inputs.  Rows longer than 16384 fall back to mi_rmsnorm + the GEMV (normed_out
+ *   arrives last at a per-stream device counter (2 KiB, allocated and zeroed by the
+ *   first call on a device and stream: not while that stream is being captured), after
+ *   all others have read their inputs.  Rows longer than 16384 fall back to mi_rmsnorm + the GEMV (normed_out
  *   is then required).  Replaces the launch of esimd_resadd_norm_gemv_{int4,fp8}_pert,
  *   esimd_resadd_norm_gemv2_fp8_pert, esimd_norm_gemv_{int4,fp8}_pert and
  *   esimd_norm_gemv_fp8_blockscale (V/csrc/xpu/torch_extension.cc:103-133,
