@@ -68,6 +68,9 @@ struct RowsArgs {
 enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2, RF_Q40 = 3, RF_Q80 = 4, RF_Q5K = 5, RF_Q6K = 6 };
 constexpr bool rows_byte_fmt(int fmt) { return fmt == RF_FP8 || fmt == RF_Q80; }   // one byte per weight
 enum : int { RS_PERN = 0, RS_PERT = 1, RS_BLOCK = 2 };
+// INT4 reuses the scale-mode slot of the template: RS_ZP = the weights come with zero-points
+// (their byte is then loaded per group; without them no load is issued at all).
+enum : int { RS_ZP = 1 };
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
@@ -201,7 +204,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
           int gi = chunk >> 2;
           gi = gi < Kg ? gi : Kg - 1;
           b.s[r][sp] = s16u[(size_t)nc * Kg + gi];
-          b.z[r][sp] = zsrc[(size_t)nc * Kg + gi];      // no zero-points: a dummy byte, replaced by 8 at use
+          if constexpr (SC == RS_ZP) b.z[r][sp] = zsrc[(size_t)nc * Kg + gi];
         } else if constexpr (FMT == RF_Q4K || FMT == RF_Q5K) {
           const int Kc = K >> 5;
           const int ci = chunk < Kc ? chunk : Kc - 1;
@@ -526,7 +529,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
 
-  const bool has_zp = FMT == RF_INT4 && a.z[0] != nullptr;   // zero-points come for all matrices or for none
+  constexpr bool has_zp = FMT == RF_INT4 && SC == RS_ZP;     // zero-points come for all matrices or for none
   auto compute = [&](const Batch& b, int sb) {
 #pragma unroll
     for (int sp = 0; sp < SPU; ++sp) {
@@ -672,11 +675,12 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
   // (see the loop): stores and loads retire through one in-order counter, so reusing a
   // store's data register any earlier would make the compiler wait for every load in flight.
   using Elem = typename Act::elem;
-  uint32_t stored[RW][MR];
+  // The RW rows of a batch are adjacent outputs: lane r keeps row r's value and one store per
+  // activation row writes them all (a store costs the memory pipeline an instruction slot, like
+  // a load, whatever its size).
+  uint32_t stored[MR];
 #pragma unroll
-  for (int r = 0; r < RW; ++r)
-#pragma unroll
-    for (int m = 0; m < MR; ++m) stored[r][m] = 0u;
+  for (int m = 0; m < MR; ++m) stored[m] = 0u;
   auto finish = [&](const Batch& b, int g) {
     int mat, row0;
     locate(g, mat, row0);
@@ -684,7 +688,6 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
     Elem* out = (Elem*)QLIN_PICK(out, mat);
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
-      const int n = row0 + r;
       float os = 1.0f;
       if constexpr (kFp8 && SC == RS_PERN)
         os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)b.os_lo[r])
@@ -694,10 +697,13 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       for (int m = 0; m < MR; ++m) {
         const float v = wave_sum(acc[r][m]);
         acc[r][m] = 0.f;
-        stored[r][m] = (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(v * os));
-        asm volatile("" : "+v"(stored[r][m]));        // the store below reads exactly this register
-        if (lane == 0 && n < N && m < M)
-          out[(size_t)m * N + n] = __builtin_bit_cast(Elem, (uint16_t)stored[r][m]);
+        const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(v * os));
+        stored[m] = lane == r ? bits : stored[m];
+        if (r == RW - 1) {
+          asm volatile("" : "+v"(stored[m]));         // the store below reads exactly this register
+          if (lane < RW && row0 + lane < N && m < M)
+            out[(size_t)m * N + row0 + lane] = __builtin_bit_cast(Elem, (uint16_t)stored[m]);
+        }
       }
     }
   };
@@ -717,9 +723,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       // the fence the compiler rotates the loop (compute first), which halves the prefetch
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int r = 0; r < RW; ++r)
-#pragma unroll
-        for (int m = 0; m < MR; ++m) asm volatile("" ::"v"(stored[r][m]));
+      for (int m = 0; m < MR; ++m) asm volatile("" ::"v"(stored[m]));
       advance(g_next, sb_next);
       if (gq[i] < ngroups) {                          // uniform; rejoins before the next loads
         compute(buf[i], sq[i]);
@@ -822,7 +826,7 @@ static void launch_rows(RowsArgs a, hipStream_t st) {
   constexpr int span_k = 64 * ppl * 8;
   constexpr int SPU = kByte ? 4 : 2;
   constexpr bool kRegOk = MR <= 2;
-  constexpr int RW2 = kHigh ? 1 : 2, RW4 = kHigh ? 2 : 4;
+  constexpr int RW2 = kHigh ? 1 : 2;
   a.nspan = (a.K + span_k - 1) / span_k;
   // Few rows (fewer than about four per wavefront): one row per batch.  A wavefront then walks
   // several small batches, so the next one loads while the current one is consumed and the work
@@ -854,8 +858,13 @@ static void launch_rows(RowsArgs a, hipStream_t st) {
     if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, RW2, SPU, true>(a, st); }
     launch_rows_rw<Act, FMT, SC, MR, RW2, SPU, false>(a, st);
   } else {
-    if constexpr (kRegOk) { if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, RW4, SPU, true>(a, st); }
-    launch_rows_rw<Act, FMT, SC, MR, RW4, SPU, false>(a, st);
+    // rows of one span: two per batch (four were 15-30 % slower up to N = 16384 and equal
+    // beyond), one when there are few rows
+    if constexpr (kRegOk) {
+      if (one_batch && few) return launch_rows_rw<Act, FMT, SC, MR, 1, SPU, true>(a, st);
+      if (one_batch) return launch_rows_rw<Act, FMT, SC, MR, 2, SPU, true>(a, st);
+    }
+    launch_rows_rw<Act, FMT, SC, MR, 2, SPU, false>(a, st);
   }
 }
 

@@ -31,7 +31,15 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     for (int i = 0; i < a.nmat; ++i) {
       r.w[i] = a.w[i]; r.s[i] = a.s[i]; r.z[i] = a.z[i]; r.out[i] = a.out[i]; r.N[i] = a.N[i];
     }
-    if (FMT == 2 || act_dtype == DT_F16)
+    if constexpr (FMT == 1) {                          // int4: the zero-point load is a template choice
+      if (a.z[0]) {
+        if (act_dtype == DT_F16) launch_rows_m<ActF16, RF_INT4, RS_ZP>(r, st);
+        else launch_rows_m<ActBF16, RF_INT4, RS_ZP>(r, st);
+      } else {
+        if (act_dtype == DT_F16) launch_rows_m<ActF16, RF_INT4, RS_PERN>(r, st);
+        else launch_rows_m<ActBF16, RF_INT4, RS_PERN>(r, st);
+      }
+    } else if (FMT == 2 || act_dtype == DT_F16)
       launch_rows_m<ActF16, FMT, SC>(r, st);
     else
       launch_rows_m<ActBF16, FMT, SC>(r, st);
