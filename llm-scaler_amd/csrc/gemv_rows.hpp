@@ -845,6 +845,24 @@ static void launch_rows(RowsArgs a, hipStream_t st) {
     // K = 5120: five spans in registers instead of two batches (4 + 1) through LDS
     if (a.nspan == 5 && ntot >= 4096) return launch_rows_rw<Act, FMT, SC, MR, 1, 5, true>(a, st);
   }
+  if constexpr (kRegOk) {
+    // Rows shorter than the widest batch get a batch of exactly their own spans: an empty span
+    // slot would still cost a (dead) load instruction and a pass of arithmetic on zeros.
+    if (a.nspan == 1) {
+      if (few) return launch_rows_rw<Act, FMT, SC, MR, 1, 1, true>(a, st);
+      return launch_rows_rw<Act, FMT, SC, MR, 2, 1, true>(a, st);
+    }
+    if constexpr (kByte) {
+      if (a.nspan == 2) {
+        if (few) return launch_rows_rw<Act, FMT, SC, MR, 1, 2, true>(a, st);
+        return launch_rows_rw<Act, FMT, SC, MR, 2, 2, true>(a, st);
+      }
+      if (a.nspan == 3) {
+        if (few) return launch_rows_rw<Act, FMT, SC, MR, 1, 3, true>(a, st);
+        return launch_rows_rw<Act, FMT, SC, MR, 2, 3, true>(a, st);
+      }
+    }
+  }
   const int per_batch = a.nspan < SPU ? a.nspan : SPU;     // loads per row per batch
   const bool one_batch = kRegOk && a.nspan <= SPU;
   if (per_batch >= 4) {

@@ -657,3 +657,28 @@ def test_fp8_blockscale_fp16_fused2(ops, dev):
     assert r.data_ptr() == o0.data_ptr()
     assert O.max_rel_err(o0.cpu(), O.matmul_ref(x, O.fp8_dequant_block(w8, s))) < TOL
     assert O.max_rel_err(o1.cpu(), x.float() @ w1.float().t()) < TOL
+
+
+# ----------------------------------------------------------------- short rows: batches of exactly 1, 2, 3 spans
+@pytest.mark.parametrize("N", [520, 9000])          # few rows per wavefront / many: one or two rows per batch
+@pytest.mark.parametrize("K", [1024, 2048, 3072])
+@pytest.mark.parametrize("M", [1, 2])
+def test_short_rows_fp8_and_int4(ops, dev, N, K, M):
+    v, _ = ops
+    x, w8, s = O.make_fp8_pern_case(M, K, N, seed=N + K + M, act_dtype=torch.float16)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    v.esimd_gemv_fp8_pern(x.to(dev), w8.to(dev), s.to(dev), out, N, K)
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))) < TOL
+    st = torch.tensor([3.0e-4])
+    v.esimd_gemv_fp8_pert(x.to(dev), w8.to(dev), st.to(dev), out)
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, O.fp8_dequant_per_tensor(w8, st))) < TOL
+    if K % 128 == 0:
+        assert _run_int4(v, dev, M, K, N, torch.float16, seed=N + K) < TOL
+        # bf16: the decode kernel keeps (nib - 8) * s in fp32 as the reference's GEMV does
+        # (V/csrc/xpu/esimd_kernels/int4_GEMV.h:91-107); weights rounded to bf16 first differ by up to
+        # 2^-9 each, which over 18000 outputs reaches 1.1e-2 of the error measure
+        xb, packed, scale, _ = O.make_int4_case(M, K, N, seed=N + K + 1, act_dtype=torch.bfloat16)
+        outb = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        v.esimd_gemv_int4(xb.to(dev), packed.to(dev), scale.to(dev), outb)
+        ref = O.matmul_ref(xb, O.int4_dequant(packed, scale, out_dtype=torch.float32))
+        assert O.max_rel_err(outb.cpu(), ref) < TOL
