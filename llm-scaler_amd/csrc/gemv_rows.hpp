@@ -894,6 +894,26 @@ static void launch_rows_norm(RowsArgs a, hipStream_t st) {
   constexpr int span_k = 64 * ppl * 8;
   constexpr int SPU = kByte ? 4 : 2;
   a.nspan = (a.K + span_k - 1) / span_k;
+  long ntot = 0;
+  for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
+  const bool few = ntot < 4L * device_cu_count() * 8;
+  // short rows: batches of exactly their own spans, one row per batch when there are few rows
+  if (a.nspan == 1) {
+    if (few) return launch_rows_rw<Act, FMT, SC, 1, 1, 1, false, true>(a, st);
+    return launch_rows_rw<Act, FMT, SC, 1, 2, 1, false, true>(a, st);
+  }
+  if constexpr (kByte) {
+    if (a.nspan == 2) {
+      if (few) return launch_rows_rw<Act, FMT, SC, 1, 1, 2, false, true>(a, st);
+      return launch_rows_rw<Act, FMT, SC, 1, 2, 2, false, true>(a, st);
+    }
+    if (a.nspan == 3) {
+      if (few) return launch_rows_rw<Act, FMT, SC, 1, 1, 3, false, true>(a, st);
+      return launch_rows_rw<Act, FMT, SC, 1, 2, 3, false, true>(a, st);
+    }
+  } else {
+    if (a.nspan == 2 && few) return launch_rows_rw<Act, FMT, SC, 1, 1, 2, false, true>(a, st);
+  }
   const int per_batch = a.nspan < SPU ? a.nspan : SPU;
   if (per_batch >= 4)
     launch_rows_rw<Act, FMT, SC, 1, 1, SPU, false, true>(a, st);
