@@ -425,7 +425,8 @@ static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
     } else if (rpw <= 32) {
       if (a.M <= 16) launch_one<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
       else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
-      else launch_one<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
+      else if constexpr (FMT == 0 || FMT == 4) launch_one<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
+      else launch_one<Act, FMT, SC, 4, 2, 8, 1>(a, rpw, st);   // nibble formats: eight waves' tiles fit the LDS
     } else {
       if (a.M <= 16) launch_one<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
       else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 4, 8, 1>(a, rpw, st);
