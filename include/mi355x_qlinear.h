@@ -332,6 +332,10 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
  *                     the up partials in split order and the product rounded to the activation
  *                     type; partial[r][s][:] = sum over split s's rows i of inter[i] * W2[e][i][:]
  *                     (fp32 [routes, splits, H], unscaled); gelu = 0: SiLU, 1: tanh-GELU; H % 16 == 0.
+ * mi_moe_kmajor_act:  inter[r][i] (activation type, [routes, I]) = the same act(..) * (..) product,
+ *                     written out for a caller whose down projection is N-major
+ *                     (moe_forward_full_silu_routed, S/csrc/moe_batch/moe.sycl:2022-2077: K-major
+ *                     gate_up, [E, H, I] down).
  * mi_moe_kmajor_finalize: out[t][:] = sum_j top_w[t][j] * s2[e] * sum_s partial[r][s][:]
  *                     + gate[t] * shared[t][:] (shared / gate optional), rounded once.
  * `splits` (K split over workgroups, rows per split = ceil(K / splits) rounded up to 8, at most
@@ -342,6 +346,8 @@ int mi_moe_kmajor_up(const void* x, const void* w, const int32_t* route_expert, 
 int mi_moe_kmajor_down(const float* up_partial, int up_splits, const float* up_scale, const void* w2,
                        const int32_t* route_expert, float* partial, int routes, int num_experts, int I, int H,
                        int splits, int gelu, int act_dtype, void* stream);
+int mi_moe_kmajor_act(const float* up_partial, int up_splits, const float* up_scale, const int32_t* route_expert,
+                      void* inter, int routes, int num_experts, int I, int gelu, int act_dtype, void* stream);
 int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_scale, const int32_t* route_expert,
                            const void* top_w, const void* shared, const float* gate, void* out, int T, int top_k,
                            int num_experts, int H, int act_dtype, void* stream);

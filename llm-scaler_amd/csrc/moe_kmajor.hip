@@ -118,6 +118,42 @@ __global__ __launch_bounds__(kKmWaves * 64) void km_up_kernel(const typename Act
             });
 }
 
+// Activation between a K-major up projection and an N-major down projection:
+// inter[route][i] = act(s_e * gate[i]) * (s_e * up[i]), gate / up summed over the up partials in
+// split order, the product rounded once to the activation type.  One thread per (route, i).
+template <class Act>
+__global__ __launch_bounds__(256) void km_act_kernel(const float* __restrict__ up_partial, int up_splits,
+                                                      const float* __restrict__ up_scale,
+                                                      const int32_t* __restrict__ route_expert,
+                                                      typename Act::elem* __restrict__ inter, int I, int iblocks,
+                                                      int gelu, int E) {
+  const int route = blockIdx.x / iblocks;
+  const int i = (blockIdx.x - route * iblocks) * 256 + (int)threadIdx.x;
+  if (i >= I) return;
+  const int e = route_expert[route];
+  float g = 0.f, u = 0.f;
+  if ((unsigned)e < (unsigned)E) {                    // a route outside [0, E) yields zeros
+    const float* up = up_partial + (size_t)route * up_splits * 2 * I;
+    for (int s = 0; s < up_splits; ++s) {
+      g += up[(size_t)s * 2 * I + i];
+      u += up[(size_t)s * 2 * I + I + i];
+    }
+    const float se = up_scale[e];
+    g *= se;
+    u *= se;
+  }
+  float a;
+  if (gelu) {
+    float two_z = 2.0f * (0.7978845608f * (g + 0.044715f * (g * g * g)));
+    two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
+    const float ex = __expf(two_z);
+    a = 0.5f * g * (1.0f + (ex - 1.0f) / (ex + 1.0f));
+  } else {
+    a = g / (1.0f + __expf(-g));
+  }
+  inter[(size_t)route * I + i] = Act::from_f32(a * u);
+}
+
 // grid = routes * splits * column blocks.  The multipliers are the route's intermediate
 // values inter[i] = act(s_e * gate[i]) * (s_e * up[i]), gate / up summed over the up partials,
 // rounded to the activation type.  partial[route][split][H] (unscaled by the down scale).
@@ -300,6 +336,24 @@ int mi_moe_kmajor_down(const float* up_partial, int up_splits, const float* up_s
   else
     hipLaunchKernelGGL(km_down_kernel<ActBF16>, grid, dim3(kKmWaves * 64), 0, st, up_partial, up_splits, up_scale,
                        (const uint8_t*)w2, route_expert, partial, I, H, splits, rows, cblocks, gelu, num_experts);
+  return launch_status();
+}
+
+int mi_moe_kmajor_act(const float* up_partial, int up_splits, const float* up_scale, const int32_t* route_expert,
+                      void* inter, int routes, int num_experts, int I, int gelu, int act_dtype, void* stream) {
+  if (!up_partial || !up_scale || !route_expert || !inter) return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (routes < 0 || num_experts <= 0 || up_splits <= 0 || I <= 0) return MI_ERR_SHAPE;
+  if (!routes) return MI_OK;
+  const int iblocks = (I + 255) / 256;
+  const dim3 grid((unsigned)routes * iblocks);
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(km_act_kernel<ActF16>, grid, dim3(256), 0, st, up_partial, up_splits, up_scale, route_expert,
+                       (_Float16*)inter, I, iblocks, gelu, num_experts);
+  else
+    hipLaunchKernelGGL(km_act_kernel<ActBF16>, grid, dim3(256), 0, st, up_partial, up_splits, up_scale, route_expert,
+                       (__bf16*)inter, I, iblocks, gelu, num_experts);
   return launch_status();
 }
 

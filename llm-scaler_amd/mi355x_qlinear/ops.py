@@ -1405,6 +1405,63 @@ def moe_forward_full_gelu_tanh_routed_no_accum(x, topk_weights, topk_indices, ga
                             top_k, _ACT_GELU_TANH, False, "moe_forward_full_gelu_tanh_routed_no_accum")
 
 
+def moe_forward_full_silu_routed_sglang(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight,
+                                        down_scale, top_k, n_routed_experts):
+    """SiLU form of moe_forward_full_gelu_tanh_routed on N-major weights gate_up [E, 2*I, H] / down [E, H, I],
+    one fp32 scale per expert (S/csrc/moe_batch/moe.sycl:1953-2007)."""
+    return _moe_pert_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                            top_k, _ACT_SILU, True, "moe_forward_full_silu_routed_sglang")
+
+
+def moe_forward_full_silu_routed(x, topk_weights, topk_indices, gate_up_weight, gate_up_scale, down_weight, down_scale,
+                                 top_k, n_routed_experts):
+    """The same forward with the up projection K-major: gate_up [E, H, 2*I] (the caller transposes w13),
+    down [E, H, I] (S/csrc/moe_batch/moe.sycl:2022-2077).  The up projection runs on the K-major
+    streaming kernel (fp32 split partials), the activation kernel rounds SiLU(gate) * up once to the
+    activation dtype in pair order, and the down projection is the grouped GEMM over expert-sorted
+    pairs with fp32 rows summed per token."""
+    who = "moe_forward_full_silu_routed"
+    _chk(x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(),
+         f"{who}: x must be contiguous fp16 [T, H]")
+    _chk(topk_weights.dtype == x.dtype, f"{who}: topk_weights must be fp16 (the activation dtype) [T, top_k]")
+    _chk(topk_indices.dtype == torch.int32, f"{who}: topk_indices must be int32 [T, top_k]")
+    _chk_fp8(gate_up_weight, who)
+    _chk_fp8(down_weight, who)
+    T, H = x.shape
+    k = int(top_k)
+    P = T * k
+    _chk(gate_up_weight.dim() == 3 and gate_up_weight.shape[1] == H and gate_up_weight.shape[2] % 32 == 0 and
+         gate_up_weight.is_contiguous(),
+         f"{who}: gate_up_weight must be [E, hidden, 2*intermediate] - transpose w13 before calling")
+    E = gate_up_weight.shape[0]
+    I = gate_up_weight.shape[2] // 2
+    _chk(tuple(down_weight.shape) == (E, H, I) and down_weight.is_contiguous(), f"{who}: down_weight must be [E, H, I]")
+    _chk(gate_up_scale.dtype == torch.float32 and gate_up_scale.numel() >= E and down_scale.dtype == torch.float32 and
+         down_scale.numel() >= E, f"{who}: scales must be float32 [E]")
+    _chk(topk_weights.numel() == P and topk_indices.numel() == P, f"{who}: routing tensors must be [T, top_k]")
+    dev = x.device
+    adt = capi.act_dtype(x)
+    ids = topk_indices.contiguous().reshape(T, k)
+    top_w = topk_weights.contiguous().reshape(T, k)
+    route_expert = ids.reshape(-1)
+    s_up = _km_splits(P, H, 2 * I, dev)
+    up_part = torch.empty(P, s_up, 2 * I, dtype=torch.float32, device=dev)
+    capi.call("mi_moe_kmajor_up", x, capi.ptr(x), capi.ptr(gate_up_weight), capi.ptr(route_expert), capi.ptr(up_part), P, k,
+              E, H, 2 * I, s_up, adt)
+    inter = torch.empty(P, I, dtype=x.dtype, device=dev)
+    capi.call("mi_moe_kmajor_act", x, capi.ptr(up_part), s_up, capi.ptr(gate_up_scale.contiguous()), capi.ptr(route_expert),
+              capi.ptr(inter), P, E, I, 0, adt)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    start = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    moe_sort(ids, E, sorted_pairs, start, inv, None, None)
+    y = torch.empty(P, H, dtype=torch.float32, device=dev)
+    _moe_gemm(inter, None, sorted_pairs, down_weight, down_scale.contiguous(), start, y, E, H, I, _ACT_NONE, who,
+              per_expert=True)
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    return moe_combine(y, inv, top_w, out, k)
+
+
 def moe_forward_full_gelu_tanh(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
                                n_routed_experts):
     """Softmax top-k with renormalisation, then moe_forward_full_gelu_tanh_routed
@@ -1674,6 +1731,10 @@ def register():
             lambda x, *a: torch.empty_like(x))
     for name, fn in (("moe_forward_full_gelu_tanh_routed", moe_forward_full_gelu_tanh_routed),
                      ("moe_forward_full_gelu_tanh_routed_decode", moe_forward_full_gelu_tanh_routed_decode)):
+        _define("moe_ops", name + "(Tensor x, Tensor topk_weights, Tensor topk_indices, " + _pert, fn,
+                lambda x, *a: torch.empty_like(x))
+    for name, fn in (("moe_forward_full_silu_routed", moe_forward_full_silu_routed),
+                     ("moe_forward_full_silu_routed_sglang", moe_forward_full_silu_routed_sglang)):
         _define("moe_ops", name + "(Tensor x, Tensor topk_weights, Tensor topk_indices, " + _pert, fn,
                 lambda x, *a: torch.empty_like(x))
     _define("moe_ops", "moe_forward_full_gelu_tanh_routed_no_accum(Tensor x, Tensor topk_weights, Tensor topk_indices, "

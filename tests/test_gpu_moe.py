@@ -433,6 +433,33 @@ def _pert_case(T, E, H, I, k, seed, dtype):
     return x, logits, tw.to(dtype), ti, w13, s13, w2, s2
 
 
+@pytest.mark.parametrize("T,E,H,I,k,dtype", [(1, 16, 2048, 768, 8, torch.float16), (8, 8, 512, 256, 2, torch.float16),
+                                             (3, 4, 384, 80, 2, torch.bfloat16), (40, 8, 256, 144, 2, torch.float16)])
+def test_moe_silu_routed(v, dev, T, E, H, I, k, dtype):
+    """moe_forward_full_silu_routed_sglang (N-major w13) and moe_forward_full_silu_routed (w13 transposed to
+    [E, H, 2I]) against the per-route loop with the intermediate rounded to the activation dtype."""
+    x, logits, tw, ti, w13, s13, w2, s2 = _pert_case(T, E, H, I, k, 900 + T, dtype)
+    want, inter_ref, y_ref = O.moe_prefill_scalar(x, tw, ti, w13, s13, w2, s2, return_parts=True, act="silu")
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    d = lambda t: t.to(dev)
+    ids = ti.reshape(-1).long()
+    d2 = O.e4m3_decode(w2.reshape(-1, I)).reshape(E, H, I)
+    y_r = torch.einsum("pi,phi->ph", inter_ref.to(dtype).float(), d2[ids]) * s2[ids].view(-1, 1)
+    want_r = (tw.float().reshape(T, k, 1) * y_r.reshape(T, k, H)).sum(1)
+    import custom_esimd_kernels_sglang.moe_ops as sg_moe
+    got = sg_moe.moe_forward_full_silu_routed_sglang(d(x), d(tw), d(ti), f8(w13), d(s13), f8(w2), d(s2), k, E)
+    assert got.shape == (T, H) and got.dtype == dtype
+    assert O.max_rel_err(got.cpu().float(), want_r) < TOL
+    assert ((got.cpu().float() - want).abs().mean() / want.abs().mean()).item() < 5e-3
+    w13_km = w13.transpose(1, 2).contiguous()          # [E, H, 2I]
+    got2 = sg_moe.moe_forward_full_silu_routed(d(x), d(tw), d(ti), f8(w13_km), d(s13), f8(w2), d(s2), k, E)
+    assert got2.shape == (T, H) and got2.dtype == dtype
+    assert O.max_rel_err(got2.cpu().float(), want_r) < TOL
+    if 2 * I != H:
+      with pytest.raises(RuntimeError):                # N-major w13 handed to the K-major op
+        sg_moe.moe_forward_full_silu_routed(d(x), d(tw), d(ti), f8(w13), d(s13), f8(w2), d(s2), k, E)
+
+
 @pytest.mark.parametrize("T,E,H,I,k,dtype", [(2, 16, 2816, 704, 8, torch.float16), (40, 8, 256, 144, 2, torch.float16),
                                              (1, 16, 512, 256, 4, torch.float16), (70, 4, 384, 80, 2, torch.bfloat16)])
 def test_moe_gelu_tanh_family(v, dev, T, E, H, I, k, dtype):
