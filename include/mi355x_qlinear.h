@@ -209,7 +209,8 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
  *   scattered_w[pos] = top_w[sorted_pairs[pos]]   (esimd_moe_scatter, moe_ops.h:522-569).
  * mi_moe_combine: out[t] = sum_j w * y[inv[t*topk + j]], weights indexed by sorted
  *   position (weights_by_position = 1, esimd_moe_gather, moe_ops.h:627-676) or by
- *   pair; y is in the activation dtype, or fp32 when y_f32 = 1.
+ *   pair; y is in the activation dtype, or fp32 when y_f32 = 1.  w may be null: the rows are
+ *   summed unweighted (moe_accumulate, V/csrc/moe_batch/moe.sycl:1177-1230).
  *   inv may be null: y is then already in pair order (row t*topk + j), as
  *   moe_prefill_accumulate_forward_fp8 takes it
  *   (S/csrc/moe_prefill/moe_prefill_fp8.sycl:413-436).

@@ -414,7 +414,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < topk; ++j) {
     const int pos = inv ? inv[(size_t)t * topk + j] : t * topk + j;   // no map: y is in pair order
-    const float wj = Act::to_f32(w[by_pos ? pos : t * topk + j]);
+    const float wj = w ? Act::to_f32(w[by_pos ? pos : t * topk + j]) : 1.0f;   // no weights: plain sum
     if constexpr (Y32) {
       const f32x4* y = (const f32x4*)yv;
       const f32x4 a = y[((size_t)pos * H8 + c) * 2], b = y[((size_t)pos * H8 + c) * 2 + 1];
@@ -623,7 +623,7 @@ int mi_moe_scatter(const void* hidden, const void* top_w, const int32_t* sorted_
 int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void* out, const void* shared,
                           const float* gate, int H, int topk, int T, int weights_by_position, int act_dtype,
                           int y_f32, void* stream) {
-  if (!y || !w || !out) return MI_ERR_ARG;
+  if (!y || !out) return MI_ERR_ARG;
   if (gate && !shared) return MI_ERR_ARG;
   if (H <= 0 || (H % 8) || topk < 1 || T < 0) return MI_ERR_SHAPE;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;

@@ -644,6 +644,46 @@ def moe_topk(logits, top_k, norm):
     return w, ids
 
 
+def topk_v2(router_logits, top_values, top_indices, T, num_experts, topk):
+    """esimd_topk_v2::topk_v2: esimd_moe_topk with the expert and route counts passed explicitly
+    (V/csrc/xpu/torch_extension_topk_v2.cc:12-16)."""
+    who = "topk_v2"
+    _chk(router_logits.dim() == 2 and router_logits.shape[1] == int(num_experts), f"{who}: router_logits must be [T, num_experts]")
+    _chk(top_values.dim() == 2 and top_values.shape[1] == int(topk), f"{who}: top_values must be [T, topk]")
+    return esimd_moe_topk(router_logits, top_values, top_indices, T)
+
+
+def moe_router_forward(x, weight, scale):
+    """logits[T, E] = x[T, H] @ (scale[0] * e4m3(weight[E, H]))^T in x's dtype
+    (V/csrc/moe_batch/moe.sycl:302-358); runs on the per-tensor FP8 GEMV / small-batch GEMM."""
+    who = "moe_router_forward"
+    _chk(x.dim() == 2 and x.is_contiguous() and x.dtype in (torch.float16, torch.bfloat16), f"{who}: x must be contiguous fp16 [T, H]")
+    _chk(scale.dtype == torch.float32 and scale.numel() >= 1, f"{who}: scale must be float32")
+    _chk_fp8(weight, who)
+    _chk(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.is_contiguous(), f"{who}: weight must be [num_experts, hidden]")
+    out = torch.empty(x.shape[0], weight.shape[0], dtype=x.dtype, device=x.device)
+    return esimd_gemm_fp8_pert(x, weight, scale.reshape(-1)[:1], out)
+
+
+def moe_accumulate(partials, top_k, num_shared_experts):
+    """out[t] = sum of the top_k + num_shared_experts consecutive rows of token t, added in fp32 and
+    rounded once (V/csrc/moe_batch/moe.sycl:1177-1230)."""
+    who = "moe_accumulate"
+    _chk(partials.dim() == 2 and partials.is_contiguous() and partials.dtype in (torch.float16, torch.bfloat16),
+         f"{who}: partials must be contiguous fp16 [T * rows_per_token, H]")
+    rows = int(top_k) + int(num_shared_experts)
+    _chk(rows >= 1 and partials.shape[0] % rows == 0, f"{who}: the row count must be a multiple of top_k + num_shared_experts")
+    H = partials.shape[1]
+    _chk(H % 8 == 0, f"{who}: hidden size must be a multiple of 8")
+    T = partials.shape[0] // rows
+    out = torch.empty(T, H, dtype=partials.dtype, device=partials.device)
+    if T == 0:
+        return out
+    capi.call("mi_moe_combine", partials, capi.ptr(partials), None, None, capi.ptr(out), H, rows, T, 0,
+              capi.act_dtype(partials), 0)
+    return out
+
+
 def moe_sort(top_ids, num_experts, sorted_pairs, expert_start, inv, sorted_token=None, max_count=None):
     """Stable expert sort of the flattened (token, route) pairs; all outputs int32, written in place."""
     who = "moe_sort"
@@ -1725,6 +1765,12 @@ def register():
                        "Tensor down_weight, Tensor down_scale, Tensor shared_down_weight, Tensor shared_down_scale, "
                        "Tensor shared_expert_gate_weight, int top_k, int num_shared_experts, "
                        "int n_routed_experts) -> Tensor(a!)", moe_forward_full_fp8_block, _ret(2))
+    _define("esimd_topk_v2", "topk_v2(Tensor router_logits, Tensor top_values, Tensor top_indices, int T, "
+            "int num_experts, int topk) -> Tensor", topk_v2, _ret(1))
+    _define("moe_ops", "moe_router_forward(Tensor x, Tensor weight, Tensor scale) -> Tensor", moe_router_forward,
+            lambda x, w, s: x.new_empty(x.shape[0], w.shape[0]))
+    _define("moe_ops", "moe_accumulate(Tensor partials, int top_k, int num_shared_experts) -> Tensor", moe_accumulate,
+            lambda p, k, n: p.new_empty(p.shape[0] // (k + n), p.shape[1]))
     _pert = ("Tensor gate_up_weight, Tensor gate_up_scale, Tensor down_weight, Tensor down_scale, "
              "int top_k, int n_routed_experts) -> Tensor")
     _define("moe_ops", "moe_forward_full_gelu_tanh(Tensor x, Tensor logits, " + _pert, moe_forward_full_gelu_tanh,

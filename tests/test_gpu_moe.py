@@ -48,6 +48,45 @@ def test_topk_ids_exact_weights_close(v, dev, T, E, K, dt):
     assert torch.equal(i2.cpu(), ri) and torch.equal(w2, tw)
 
 
+def test_topk_v2_matches_topk(v, dev):
+    T, E, K = 9, 128, 8
+    logits = torch.randn(T, E, generator=torch.Generator().manual_seed(5)).half().to(dev)
+    tw = torch.empty(T, K, dtype=torch.float16, device=dev)
+    ti = torch.empty(T, K, dtype=torch.int32, device=dev)
+    r = torch.ops.esimd_topk_v2.topk_v2(logits, tw, ti, T, E, K)
+    assert r.data_ptr() == tw.data_ptr()
+    rw, ri = O.moe_topk(logits.cpu(), K)
+    assert torch.equal(ti.cpu(), ri)
+    assert ((tw.cpu().float() - rw.float()).abs() <= 2 * 2.0 ** -11 * rw.float().abs() + 1e-7).all()
+    with pytest.raises(RuntimeError):
+        torch.ops.esimd_topk_v2.topk_v2(logits, tw, ti, T, E + 1, K)
+
+
+@pytest.mark.parametrize("T,E,H,dt", [(1, 128, 2048, torch.float16), (4, 64, 512, torch.float16), (12, 256, 1024, torch.bfloat16)])
+def test_moe_router_forward(v, dev, T, E, H, dt):
+    """logits = x @ (scale * e4m3(w))^T (V/csrc/moe_batch/moe.sycl:302-358)."""
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, H, generator=g).to(dt)
+    w8 = O.e4m3_quantize(torch.randn(E, H, generator=g).clamp(-3, 3) / 3)
+    sc = torch.tensor([0.037], dtype=torch.float32)
+    got = torch.ops.moe_ops.moe_router_forward(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev))
+    assert got.shape == (T, E) and got.dtype == dt
+    want = (x.float() @ O.e4m3_decode(w8).t()) * sc[0]
+    assert O.max_rel_err(got.cpu().float(), want) < TOL
+
+
+@pytest.mark.parametrize("T,k,ns,H,dt", [(1, 8, 1, 2048, torch.float16), (5, 2, 0, 136, torch.bfloat16), (0, 4, 1, 64, torch.float16)])
+def test_moe_accumulate(v, dev, T, k, ns, H, dt):
+    """Unweighted fp32 sum over each token's top_k + shared rows, one rounding
+    (V/csrc/moe_batch/moe.sycl:1177-1230)."""
+    rows = k + ns
+    p = torch.randn(T * rows, H, generator=torch.Generator().manual_seed(T + H)).to(dt)
+    got = torch.ops.moe_ops.moe_accumulate(p.to(dev), k, ns)
+    assert got.shape == (T, H) and got.dtype == dt
+    want = p.float().reshape(T, rows, H).sum(1).to(dt)
+    assert torch.equal(got.cpu(), want) or (got.cpu().float() - want.float()).abs().max() <= 2.0 ** -7 * want.float().abs().max()
+
+
 @pytest.mark.parametrize("T,E,K", [(512, 128, 8), (1, 8, 2), (37, 16, 4), (4096, 128, 8), (300, 1000, 6),
                                    (2500, 64, 2), (0, 8, 2)])
 def test_sort_bit_exact(v, dev, T, E, K):
