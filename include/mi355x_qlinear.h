@@ -264,6 +264,16 @@ int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weig
                int weight_len, float eps, int act_dtype,
                float residual_scale, void* stream);
 
+/* Two chained norms around a residual add, per token:
+ *   h2 = sum of rows_per_token consecutive rows of src (fp32; 1: the row itself),
+ *   h1 <- h2 * rsqrt(mean(h2^2) + eps1) * w1 + h1 (in place),
+ *   out = h1 * rsqrt(mean(h1^2) + eps2) * w2, the second mean over the unrounded h1.
+ * Replaces esimd_norm_add_norm (rows_per_token = 1) and esimd_accum_norm_add_norm
+ * (rows_per_token = top_k) (V/csrc/xpu/torch_extension.cc:168-175,
+ * esimd_kernels/norm_add_norm.h:46-86, accum_norm_add_norm.h). */
+int mi_norm_add_norm(const void* src, int rows_per_token, void* h1, const void* w1, const void* w2, void* out,
+                     int T, int K, float eps1, float eps2, int act_dtype, void* stream);
+
 /* The same normalisation fused into the decode GEMV (one launch, M == 1):
  *   x' = rmsnorm(x (+ residual)) (* silu(gate)) per head of norm_len elements
  *   (norm_len == K: the whole row), out[i] = x' @ dequant(w[i])^T for nmat <= 3
@@ -282,6 +292,13 @@ int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* no
                  void* normed_out, int norm_len, float eps, int fmt, int nmat, const void* const* w,
                  const void* const* scale, void* const* out, const int* N, int K, int act_dtype,
                  void* stream);
+/* The same with x + residual multiplied by residual_scale before it is stored and normalised
+ * (unrounded into the norm, as the reference does): replaces esimd_scaled_resadd_norm_gemv_fp8_pert
+ * (V/csrc/xpu/torch_extension.cc:163-166, esimd_kernels/scaled_resadd_norm_gemv_fp8.h:70-100). */
+int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const void* norm_weight,
+                        void* normed_out, int norm_len, float eps, float residual_scale, int fmt, int nmat,
+                        const void* const* w, const void* const* scale, void* const* out, const int* N, int K,
+                        int act_dtype, void* stream);
 
 /* ---- MoE grouped FP8 block-scaled GEMM ----------------------------------------
  * out[r, :] = a[src(r), :] @ dequant(w[e])^T for the rows r of expert e,

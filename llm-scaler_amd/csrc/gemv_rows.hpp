@@ -63,6 +63,7 @@ struct RowsArgs {
   unsigned int* n_arrive;      // zeroed counter; the kernel leaves it at zero again
   int n_len;
   float n_eps;
+  float n_rscale;              // factor on x + residual before it is stored and normalised
 };
 
 enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2, RF_Q40 = 3, RF_Q80 = 4, RF_Q5K = 5, RF_Q6K = 6 };
@@ -414,7 +415,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       for (int e = 0; e < 8; ++e) {
         const E h = __builtin_bit_cast(E, (uint16_t)(xpre[t][e >> 1] >> (16 * (e & 1))));
         const E r = __builtin_bit_cast(E, (uint16_t)(nres[t][e >> 1] >> (16 * (e & 1))));
-        av[t][e] = Act::to_f32(h) + Act::to_f32(r);
+        av[t][e] = (Act::to_f32(h) + Act::to_f32(r)) * a.n_rscale;
         ssp[t] += av[t][e] * av[t][e];
       }
     }

@@ -498,6 +498,48 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const typename Act::elem* 
   }
 }
 
+// h2 = sum of `nsum` consecutive rows of src (fp32; nsum = 1: the row itself);
+// h1 <- h2 * rsqrt(mean(h2^2) + eps1) * w1 + h1 (stored rounded, its fp32 value feeds the
+// second mean); out = round(h1_stored * rsqrt(mean(h1_new^2) + eps2) * w2).  One workgroup per
+// token; each thread re-reads only elements it wrote itself.
+template <class Act>
+__global__ __launch_bounds__(256) void norm_add_norm_kernel(const typename Act::elem* __restrict__ src, int nsum,
+                                                            typename Act::elem* h1,
+                                                            const typename Act::elem* __restrict__ w1,
+                                                            const typename Act::elem* __restrict__ w2,
+                                                            typename Act::elem* out, int K, float eps1, float eps2) {
+  __shared__ float wsum[2][4];
+  const size_t sbase = (size_t)blockIdx.x * nsum * K;
+  const size_t base = (size_t)blockIdx.x * K;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  auto h2_at = [&](int i) {
+    float v = 0.f;
+    for (int r = 0; r < nsum; ++r) v += Act::to_f32(src[sbase + (size_t)r * K + i]);
+    return v;
+  };
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < K; i += 256) {
+    const float v = h2_at(i);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  if (lane == 0) wsum[0][wave] = ss;
+  __syncthreads();
+  const float inv1 = rsqrtf(((wsum[0][0] + wsum[0][1]) + (wsum[0][2] + wsum[0][3])) / (float)K + eps1);
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < K; i += 256) {
+    const float v = h2_at(i) * inv1 * Act::to_f32(w1[i]) + Act::to_f32(h1[base + i]);
+    h1[base + i] = Act::from_f32(v);
+    ss2 += v * v;
+  }
+  ss2 = wave_sum(ss2);
+  if (lane == 0) wsum[1][wave] = ss2;
+  __syncthreads();
+  const float inv2 = rsqrtf(((wsum[1][0] + wsum[1][1]) + (wsum[1][2] + wsum[1][3])) / (float)K + eps2);
+  for (int i = threadIdx.x; i < K; i += 256)
+    out[base + i] = Act::from_f32(Act::to_f32(h1[base + i]) * inv2 * Act::to_f32(w2[i]));
+}
+
 static inline dim3 grid1d(size_t n, int bs = 256) { return dim3((unsigned)((n + bs - 1) / bs)); }
 
 }  // namespace qlin
@@ -673,6 +715,22 @@ int mi_rmsnorm(const void* x, void* residual, const void* gate, const void* weig
   else
     hipLaunchKernelGGL(rmsnorm_kernel<ActBF16>, dim3(rows), dim3(256), 0, st, (const __bf16*)x, (__bf16*)residual,
                        (const __bf16*)gate, (const __bf16*)weight, (__bf16*)out, L, weight_len, eps, residual_scale);
+  return launch_status();
+}
+
+int mi_norm_add_norm(const void* src, int rows_per_token, void* h1, const void* w1, const void* w2, void* out,
+                     int T, int K, float eps1, float eps2, int act_dtype, void* stream) {
+  if (!src || !h1 || !w1 || !w2 || !out) return MI_ERR_ARG;
+  if (T < 0 || K <= 0 || rows_per_token < 1) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (!T) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16)
+    hipLaunchKernelGGL(norm_add_norm_kernel<ActF16>, dim3(T), dim3(256), 0, st, (const _Float16*)src, rows_per_token,
+                       (_Float16*)h1, (const _Float16*)w1, (const _Float16*)w2, (_Float16*)out, K, eps1, eps2);
+  else
+    hipLaunchKernelGGL(norm_add_norm_kernel<ActBF16>, dim3(T), dim3(256), 0, st, (const __bf16*)src, rows_per_token,
+                       (__bf16*)h1, (const __bf16*)w1, (const __bf16*)w2, (__bf16*)out, K, eps1, eps2);
   return launch_status();
 }
 

@@ -18,6 +18,14 @@ extern "C" {
 int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
                  int norm_len, float eps, int fmt, int nmat, const void* const* w, const void* const* scale,
                  void* const* out, const int* N, int K, int act_dtype, void* stream) {
+  return mi_norm_gemv_scaled(x, residual, gate, norm_weight, normed_out, norm_len, eps, 1.0f, fmt, nmat, w, scale, out,
+                             N, K, act_dtype, stream);
+}
+
+int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
+                        int norm_len, float eps, float residual_scale, int fmt, int nmat, const void* const* w,
+                        const void* const* scale, void* const* out, const int* N, int K, int act_dtype,
+                        void* stream) {
   if (!x || !norm_weight || !w || !scale || !out || !N) return MI_ERR_ARG;
   if (nmat < 1 || nmat > kRowsMaxMat) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
@@ -38,7 +46,7 @@ int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* no
     // two kernels: the norm writes the row (into normed_out, or over x's scratch copy), then the GEMV
     if (!normed_out) return MI_ERR_ARG;
     const int rc = mi_rmsnorm(x, residual, gate, norm_weight, normed_out, K / norm_len, norm_len, norm_len, eps,
-                              act_dtype, 1.0f, stream);
+                              act_dtype, residual_scale, stream);
     if (rc != MI_OK) return rc;
     const float* const* fs = reinterpret_cast<const float* const*>(scale);
     if (fmt == 0) return mi_gemm_fp8_pert_multi(normed_out, nmat, w, fs, out, N, 1, K, act_dtype, stream);
@@ -46,7 +54,7 @@ int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* no
     return mi_gemv_int4_multi(normed_out, nmat, w, scale, nullptr, out, N, 1, K, act_dtype, stream);
   }
   r.n_res = residual; r.n_gate = gate; r.n_weight = norm_weight; r.n_out = normed_out;
-  r.n_len = norm_len; r.n_eps = eps;
+  r.n_len = norm_len; r.n_eps = eps; r.n_rscale = residual_scale;
   r.n_arrive = arrival_counter_get(st);
   if (!r.n_arrive) return MI_ERR_LAUNCH;
   const bool f16 = act_dtype == DT_F16;

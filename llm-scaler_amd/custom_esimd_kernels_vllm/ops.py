@@ -281,6 +281,20 @@ def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s
     return _ops.esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps)
 
 
+def esimd_scaled_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, qkv_weight, qkv_scale, qkv_out, eps,
+                                           scalar):
+    return _ops.esimd_scaled_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, qkv_weight, qkv_scale,
+                                                       qkv_out, eps, scalar)
+
+
+def esimd_norm_add_norm(h2_raw, h1, w1, w2, out, eps1, eps2):
+    return _ops.esimd_norm_add_norm(h2_raw, h1, w1, w2, out, eps1, eps2)
+
+
+def esimd_accum_norm_add_norm(routed_output, h1, w1, w2, out, top_k, eps1, eps2):
+    return _ops.esimd_accum_norm_add_norm(routed_output, h1, w1, w2, out, top_k, eps1, eps2)
+
+
 def esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
     return _ops.esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)
 

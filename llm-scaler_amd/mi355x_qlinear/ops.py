@@ -1069,7 +1069,7 @@ def esimd_rms_norm(input, output, weight, eps):
 _NORM_FP8_PERT, _NORM_FP8_BLOCK, _NORM_INT4 = 0, 1, 2
 
 
-def _norm_gemv(x, residual, gate, norm_weight, normed_out, norm_len, eps, fmt, ws, ss, outs, who):
+def _norm_gemv(x, residual, gate, norm_weight, normed_out, norm_len, eps, fmt, ws, ss, outs, who, residual_scale=1.0):
     """One launch: RMS norm (+ residual add / SiLU gate) of the single activation row, fused
     into the decode GEMV over `ws`.  More than one row takes the norm kernel + GEMV route."""
     _chk(x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(), f"{who}: activations must be contiguous fp16/bf16")
@@ -1092,7 +1092,7 @@ def _norm_gemv(x, residual, gate, norm_weight, normed_out, norm_len, eps, fmt, w
         _chk(normed_out.numel() >= x.numel(), f"{who}: normed output is too small")
     if rows != 1:
         normed = normed_out if normed_out is not None else torch.empty_like(x)
-        _rmsnorm(x, residual, gate, norm_weight, normed, x.numel() // norm_len, norm_len, eps, who)
+        _rmsnorm(x, residual, gate, norm_weight, normed, x.numel() // norm_len, norm_len, eps, who, residual_scale)
         xin = normed.view(rows, K)
         if fmt == _NORM_INT4:
             return _int4_multi(xin, ws, ss, [None] * len(ws), outs, who)
@@ -1119,8 +1119,8 @@ def _norm_gemv(x, residual, gate, norm_weight, normed_out, norm_len, eps, fmt, w
                      f"{who}: gemv_scale must be contiguous fp32 [ceil(N/128), K/128]")
         _chk(o.numel() == w.shape[0], f"{who}: output has {o.numel()} elements, expected N={w.shape[0]}")
         Ns.append(w.shape[0])
-    capi.call("mi_norm_gemv", x, capi.ptr(x), capi.ptr(residual), capi.ptr(gate), capi.ptr(norm_weight),
-              capi.ptr(normed_out), norm_len, float(eps), fmt, len(ws), capi.ptr_array(ws), capi.ptr_array(ss),
+    capi.call("mi_norm_gemv_scaled", x, capi.ptr(x), capi.ptr(residual), capi.ptr(gate), capi.ptr(norm_weight),
+              capi.ptr(normed_out), norm_len, float(eps), float(residual_scale), fmt, len(ws), capi.ptr_array(ws), capi.ptr_array(ss),
               capi.ptr_array(outs), capi.int_array(Ns), K, capi.act_dtype(x))
     return outs[0]
 
@@ -1140,6 +1140,43 @@ def esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_w
     K = hidden_states.shape[-1]
     return _norm_gemv(hidden_states, residual, None, norm_weight, normed_out, K, eps, _NORM_FP8_PERT,
                       [gemv_weight], [gemv_scale], [output], "esimd_resadd_norm_gemv_fp8_pert")
+
+
+def esimd_scaled_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, qkv_weight, qkv_scale, qkv_out, eps,
+                                           scalar):
+    """residual <- (hidden_states + residual) * scalar (in place); qkv_out = (rmsnorm(residual) * norm_weight)
+    @ (qkv_scale * e4m3(qkv_weight))^T in one launch (V/csrc/xpu/esimd_kernels/scaled_resadd_norm_gemv_fp8.h)."""
+    K = hidden_states.shape[-1]
+    # rows beyond the fused kernel's 16384 elements go through the norm kernel and need a buffer for its output
+    normed = torch.empty_like(hidden_states) if K > 16384 else None
+    _norm_gemv(hidden_states, residual, None, norm_weight, normed, K, eps, _NORM_FP8_PERT, [qkv_weight], [qkv_scale],
+               [qkv_out], "esimd_scaled_resadd_norm_gemv_fp8_pert", residual_scale=float(scalar))
+
+
+def _norm_add_norm(src, rows_per_token, h1, w1, w2, out, eps1, eps2, who):
+    _chk(src.dtype in (torch.float16, torch.bfloat16), f"{who}: activations must be fp16 or bf16")
+    for name, t in (("input", src), ("h1", h1), ("w1", w1), ("w2", w2), ("out", out)):
+        _chk(t.dtype == src.dtype and t.is_contiguous() and t.device == src.device,
+             f"{who}: {name} must be contiguous and share dtype and device")
+    K = h1.shape[-1]
+    T = h1.numel() // K
+    _chk(w1.numel() == K and w2.numel() == K and out.numel() == T * K and src.numel() == T * rows_per_token * K,
+         f"{who}: sizes must be h1/out [T, K], w1/w2 [K], input [T * rows, K]")
+    capi.call("mi_norm_add_norm", src, capi.ptr(src), int(rows_per_token), capi.ptr(h1), capi.ptr(w1), capi.ptr(w2),
+              capi.ptr(out), T, K, float(eps1), float(eps2), capi.act_dtype(src))
+
+
+def esimd_norm_add_norm(h2_raw, h1, w1, w2, out, eps1, eps2):
+    """h1 <- rmsnorm(h2_raw, eps1) * w1 + h1 (in place); out = rmsnorm(h1, eps2) * w2
+    (V/csrc/xpu/esimd_kernels/norm_add_norm.h:46-86)."""
+    _norm_add_norm(h2_raw, 1, h1, w1, w2, out, eps1, eps2, "esimd_norm_add_norm")
+
+
+def esimd_accum_norm_add_norm(routed_output, h1, w1, w2, out, top_k, eps1, eps2):
+    """The same with h2 = the sum of each token's top_k rows of routed_output
+    (V/csrc/xpu/esimd_kernels/accum_norm_add_norm.h)."""
+    _chk(int(top_k) >= 1, "esimd_accum_norm_add_norm: top_k must be positive")
+    _norm_add_norm(routed_output, int(top_k), h1, w1, w2, out, eps1, eps2, "esimd_accum_norm_add_norm")
 
 
 def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps):
@@ -1686,6 +1723,13 @@ def register():
         _define(ns, "esimd_resadd_norm_gemv_fp8_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
                     "Tensor gemv_weight, Tensor gemv_scale, Tensor output, Tensor normed_out, float eps) -> Tensor",
                 esimd_resadd_norm_gemv_fp8_pert, _ret(5))
+        _define(ns, "esimd_scaled_resadd_norm_gemv_fp8_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
+                    "Tensor qkv_weight, Tensor qkv_scale, Tensor qkv_out, float eps, float scalar) -> ()",
+                esimd_scaled_resadd_norm_gemv_fp8_pert, lambda *a: None)
+        _define(ns, "esimd_norm_add_norm(Tensor h2_raw, Tensor h1, Tensor w1, Tensor w2, Tensor out, float eps1, "
+                    "float eps2) -> ()", esimd_norm_add_norm, lambda *a: None)
+        _define(ns, "esimd_accum_norm_add_norm(Tensor routed_output, Tensor h1, Tensor w1, Tensor w2, Tensor out, "
+                    "int top_k, float eps1, float eps2) -> ()", esimd_accum_norm_add_norm, lambda *a: None)
         _define(ns, "esimd_resadd_norm_gemv2_fp8_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
                     "Tensor w0, Tensor s0, Tensor o0, Tensor w1, Tensor s1, Tensor o1, float eps) -> Tensor",
                 esimd_resadd_norm_gemv2_fp8_pert, _ret(5))

@@ -580,6 +580,64 @@ def test_norm_only_ops(ops, dev, dt):
     assert _ulp_close(out.cpu().float(), ref, dt)
 
 
+@pytest.mark.parametrize("N,K,dt", [(256, 2048, torch.float16), (96, 2816, torch.bfloat16), (64, 20480, torch.float16)])
+def test_scaled_resadd_norm_gemv_fp8(ops, dev, N, K, dt):
+    """residual <- (h + r) * scalar; qkv = rmsnorm(residual) @ W^T (V/csrc/xpu/esimd_kernels/scaled_resadd_norm_gemv_fp8.h:70-100);
+    K = 20480 takes the two-kernel route."""
+    v, _ = ops
+    g = torch.Generator().manual_seed(N + K)
+    eps, scalar = 1e-6, 0.70703125
+    hidden = torch.randn(1, K, generator=g).to(dt)
+    residual = torch.randn(1, K, generator=g).to(dt)
+    nw = (torch.randn(K, generator=g) * 0.1 + 1.0).to(dt)
+    w8 = O.e4m3_quantize((torch.randn(N, K, generator=g) * 100).clamp(-448, 448))
+    sc = torch.tensor([3.0e-3])
+    out = torch.empty(1, N, dtype=dt, device=dev)
+    res_d = residual.to(dev).clone()
+    r = v.esimd_scaled_resadd_norm_gemv_fp8_pert(hidden.to(dev), res_d, nw.to(dev), w8.view(torch.float8_e4m3fn).to(dev),
+                                                 sc.to(dev), out, eps, scalar)
+    assert r is None
+    a = (hidden.float() + residual.float()) * scalar
+    assert torch.equal(res_d.cpu().view(torch.int16), a.to(dt).view(torch.int16))
+    normed = a * torch.rsqrt(a.pow(2).mean(dim=-1, keepdim=True) + eps) * nw.float()
+    full = normed @ O.fp8_dequant_per_tensor(w8, sc).float().t()
+    assert ((out.cpu().float() - full).abs().mean() / full.abs().mean()).item() < 5e-3
+    assert O.max_rel_err(out.cpu(), O.matmul_ref(normed.to(dt), O.fp8_dequant_per_tensor(w8, sc))) < 2 * TOL
+
+
+@pytest.mark.parametrize("T,K,k,dt", [(1, 2816, 8, torch.float16), (3, 2048, 2, torch.bfloat16), (1, 136, 1, torch.float16)])
+def test_norm_add_norm(ops, dev, T, K, k, dt):
+    """esimd_norm_add_norm / esimd_accum_norm_add_norm (V/csrc/xpu/esimd_kernels/norm_add_norm.h:46-86)."""
+    v, _ = ops
+    g = torch.Generator().manual_seed(T + K)
+    eps1, eps2 = 1e-6, 1e-5
+    routed = torch.randn(T * k, K, generator=g).to(dt)
+    h1 = torch.randn(T, K, generator=g).to(dt)
+    w1 = (torch.randn(K, generator=g) * 0.1 + 1.0).to(dt)
+    w2 = (torch.randn(K, generator=g) * 0.1 + 1.0).to(dt)
+
+    def ref(h2):
+        h2n = h2 * torch.rsqrt(h2.pow(2).mean(-1, keepdim=True) + eps1) * w1.float()
+        h1n = h2n + h1.float()
+        stored = h1n.to(dt)
+        return stored, stored.float() * torch.rsqrt(h1n.pow(2).mean(-1, keepdim=True) + eps2) * w2.float()
+
+    # accumulate form: h2 = sum of each token's k rows
+    h1_d = h1.to(dev).clone()
+    out = torch.empty(T, K, dtype=dt, device=dev)
+    assert v.esimd_accum_norm_add_norm(routed.to(dev), h1_d, w1.to(dev), w2.to(dev), out, k, eps1, eps2) is None
+    st, o = ref(routed.float().reshape(T, k, K).sum(1))
+    assert _ulp_close(h1_d.cpu().float(), st.float(), dt)
+    assert _ulp_close(out.cpu().float(), o, dt, ulps=3)
+    # plain form on the first row of each token
+    h2 = routed.reshape(T, k, K)[:, 0].contiguous()
+    h1_d = h1.to(dev).clone()
+    assert v.esimd_norm_add_norm(h2.to(dev), h1_d, w1.to(dev), w2.to(dev), out, eps1, eps2) is None
+    st, o = ref(h2.float())
+    assert _ulp_close(h1_d.cpu().float(), st.float(), dt)
+    assert _ulp_close(out.cpu().float(), o, dt, ulps=3)
+
+
 # ----------------------------------------------------------------- few weight rows, many activation rows
 @pytest.mark.parametrize("M,K,N,dt", [(64, 4096, 1024, torch.bfloat16), (17, 8192, 512, torch.float16),
                                       (40, 4096, 2000, torch.float16), (64, 2176, 72, torch.bfloat16)])
