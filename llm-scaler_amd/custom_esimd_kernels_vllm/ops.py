@@ -287,6 +287,10 @@ def esimd_scaled_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight,
                                                        qkv_out, eps, scalar)
 
 
+def esimd_norm_gemv_norm_fp16(residual, scale_with_root, proj_w, pre_ff_w, router_logits, moe_input, eps):
+    return _ops.esimd_norm_gemv_norm_fp16(residual, scale_with_root, proj_w, pre_ff_w, router_logits, moe_input, eps)
+
+
 def esimd_norm_add_norm(h2_raw, h1, w1, w2, out, eps1, eps2):
     return _ops.esimd_norm_add_norm(h2_raw, h1, w1, w2, out, eps1, eps2)
 

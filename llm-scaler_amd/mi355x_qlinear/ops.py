@@ -1179,6 +1179,22 @@ def esimd_accum_norm_add_norm(routed_output, h1, w1, w2, out, top_k, eps1, eps2)
     _norm_add_norm(routed_output, int(top_k), h1, w1, w2, out, eps1, eps2, "esimd_accum_norm_add_norm")
 
 
+def esimd_norm_gemv_norm_fp16(residual, scale_with_root, proj_w, pre_ff_w, router_logits, moe_input, eps):
+    """router_logits = (rmsnorm(residual) * scale_with_root) @ proj_w^T and moe_input = rmsnorm(residual) * pre_ff_w
+    (V/csrc/xpu/esimd_kernels/norm_gemv_norm_fp16.h:1-40).  Runs the three launches the reference's fusion
+    replaces (norm, 16-bit GEMV, norm); the router's input is rounded to the activation dtype in between."""
+    who = "esimd_norm_gemv_norm_fp16"
+    _chk(residual.dtype in (torch.float16, torch.bfloat16) and residual.is_contiguous(), f"{who}: residual must be contiguous fp16")
+    K = residual.shape[-1]
+    _chk(scale_with_root.numel() == K and pre_ff_w.numel() == K and moe_input.numel() == residual.numel(),
+         f"{who}: scale_with_root / pre_ff_w must be [K], moe_input must match residual")
+    rows = residual.numel() // K
+    tmp = torch.empty_like(residual)
+    _rmsnorm(residual, None, None, scale_with_root, tmp, rows, K, eps, who)
+    _gemv_w16(tmp.view(rows, K), proj_w, router_logits, False, who)
+    _rmsnorm(residual, None, None, pre_ff_w, moe_input, rows, K, eps, who)
+
+
 def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps):
     """Residual add + RMS norm feeding two per-tensor FP8 GEMVs in one launch (resadd_norm_gemv2_fused.h)."""
     K = hidden_states.shape[-1]
@@ -1726,6 +1742,8 @@ def register():
         _define(ns, "esimd_scaled_resadd_norm_gemv_fp8_pert(Tensor hidden_states, Tensor residual, Tensor norm_weight, "
                     "Tensor qkv_weight, Tensor qkv_scale, Tensor qkv_out, float eps, float scalar) -> ()",
                 esimd_scaled_resadd_norm_gemv_fp8_pert, lambda *a: None)
+        _define(ns, "esimd_norm_gemv_norm_fp16(Tensor residual, Tensor scale_with_root, Tensor proj_w, Tensor pre_ff_w, "
+                    "Tensor router_logits, Tensor moe_input, float eps) -> ()", esimd_norm_gemv_norm_fp16, lambda *a: None)
         _define(ns, "esimd_norm_add_norm(Tensor h2_raw, Tensor h1, Tensor w1, Tensor w2, Tensor out, float eps1, "
                     "float eps2) -> ()", esimd_norm_add_norm, lambda *a: None)
         _define(ns, "esimd_accum_norm_add_norm(Tensor routed_output, Tensor h1, Tensor w1, Tensor w2, Tensor out, "

@@ -638,6 +638,25 @@ def test_norm_add_norm(ops, dev, T, K, k, dt):
     assert _ulp_close(out.cpu().float(), o, dt, ulps=3)
 
 
+@pytest.mark.parametrize("K,N,dt", [(2816, 128, torch.float16), (512, 24, torch.bfloat16)])
+def test_norm_gemv_norm_fp16(ops, dev, K, N, dt):
+    """Router logits and the MoE input from one shared RMS norm (V/csrc/xpu/esimd_kernels/norm_gemv_norm_fp16.h:1-40)."""
+    v, _ = ops
+    g = torch.Generator().manual_seed(K + N)
+    eps = 1e-6
+    res = torch.randn(1, K, generator=g).to(dt)
+    swr = (torch.rand(K, generator=g) * 0.05).to(dt)
+    pw = (torch.randn(N, K, generator=g) * 0.5).to(dt)
+    fw = (torch.randn(K, generator=g) * 0.1 + 1.0).to(dt)
+    logits = torch.empty(1, N, dtype=dt, device=dev)
+    moe_in = torch.empty(1, K, dtype=dt, device=dev)
+    assert v.esimd_norm_gemv_norm_fp16(res.to(dev), swr.to(dev), pw.to(dev), fw.to(dev), logits, moe_in, eps) is None
+    normed = res.float() * torch.rsqrt(res.float().pow(2).mean(-1, keepdim=True) + eps)
+    assert _ulp_close(moe_in.cpu().float(), normed * fw.float(), dt)
+    want = (normed * swr.float()).to(dt).float() @ pw.float().t()
+    assert O.max_rel_err(logits.cpu(), want) < TOL
+
+
 # ----------------------------------------------------------------- few weight rows, many activation rows
 @pytest.mark.parametrize("M,K,N,dt", [(64, 4096, 1024, torch.bfloat16), (17, 8192, 512, torch.float16),
                                       (40, 4096, 2000, torch.float16), (64, 2176, 72, torch.bfloat16)])
