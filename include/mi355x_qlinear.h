@@ -155,6 +155,19 @@ int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int
  *   layout mi_gemv_int4 reads.  GGML's quantize_row_q4_0 rule on 128-wide blocks;
  *   replaces q4_0_quantize (V/csrc/xpu/torch_extension_q4_0.cc:27-75,
  *   V/csrc/xpu/q4_0_quant.sycl:30-120).  K % 128 == 0. */
+/* Routed decode GEMVs of a GGUF MoE layer, one launch over all routes r = t * top_k + j:
+ *   out[i][r, :] = route_weight[r] * (x[r / x_div, :] @ dequant(W_i[route_expert[r]])^T), i < nmat <= 2,
+ * W_i = the per-expert stack [E, N, ...] of the repacked representation the dense GEMVs read
+ * (fmt 2 = Q4_K: ql, scale, qmin; 5 = Q5_K: + qh; 6 = Q6_K: ql, qh, scale), fp16, rows of out
+ * out_stride elements apart, route_weight (fp16) optional, expert ids clamped into [0, E).
+ * Replaces the launches of esimd_moe_up_q4k (two matrices: gate and up halves of one buffer,
+ * x_div = top_k; SiLU * up follows as mi_moe_silu_mul) and esimd_moe_down_q5k / _q6k
+ * (x = the intermediate in route order, x_div = 1, route_weight = topk_w)
+ * (S/csrc/xpu/torch_extension.cc:86-101, S/csrc/xpu/esimd_kernels/moe_kquant_GEMV.h). */
+int mi_moe_gguf_gemv(int fmt, const void* x, int x_div, int nmat, const void* const* ql, const void* const* qh,
+                     const void* const* scale, const void* const* qmin, void* const* out, long long out_stride,
+                     const int32_t* route_expert, const void* route_weight, int routes, int num_experts, int N,
+                     int K, void* stream);
 int mi_q4_0_repack(const void* raw, void* packed, void* scale, int N, int K, void* stream);
 int mi_q8_0_repack(const void* raw, void* qs, void* scale, int N, int K, void* stream);
 int mi_q5k_repack(const void* raw, void* ql, void* qh, void* scale, void* qmin, int N, int K,

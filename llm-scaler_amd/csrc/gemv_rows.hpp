@@ -64,6 +64,16 @@ struct RowsArgs {
   int n_len;
   float n_eps;
   float n_rscale;              // factor on x + residual before it is stored and normalised
+  // Routed launch (ROUTED kernels, M == 1): blockIdx.y is a route r with expert
+  // e = r_expert[r] (ids outside [0, r_num_experts) are clamped into range); the matrices of
+  // expert e start e * r_*_stride[i] bytes into w / s / z / h, the activation row is row
+  // r / r_x_div of x, the output row is r (r_out_stride elements apart) and is multiplied by
+  // r_out_mul[r] when that is given.
+  const int32_t* r_expert;
+  const void* r_out_mul;
+  int r_num_experts, r_x_div;
+  long long r_out_stride;
+  long long r_w_stride[kRowsMaxMat], r_s_stride[kRowsMaxMat], r_z_stride[kRowsMaxMat], r_h_stride[kRowsMaxMat];
 };
 
 enum : int { RF_FP8 = 0, RF_INT4 = 1, RF_Q4K = 2, RF_Q40 = 3, RF_Q80 = 4, RF_Q5K = 5, RF_Q6K = 6 };
@@ -111,9 +121,31 @@ __device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_
 // consumed (two register buffers).  Weight loads carry the non-temporal hint:
 // every byte is used exactly once.
 template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI, bool XREG,
-          bool NORM = false>
-__global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
+          bool NORM = false, bool ROUTED = false>
+__global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in) {
   static_assert(!NORM || (MR == 1 && !XREG), "the fused norm stages one activation row through LDS");
+  static_assert(!ROUTED || (MR == 1 && !NORM), "routed launches take one activation row per route");
+  // ROUTED: a private copy of the arguments with this route's bases; otherwise `a` is the
+  // kernel argument itself.
+  [[maybe_unused]] RowsArgs a_route;
+  [[maybe_unused]] float route_mul = 1.0f;
+  if constexpr (ROUTED) {
+    a_route = a_in;
+    const int r = blockIdx.y;
+    int e = a_in.r_expert[r];
+    e = e < 0 ? 0 : (e >= a_in.r_num_experts ? a_in.r_num_experts - 1 : e);
+#pragma unroll
+    for (int i = 0; i < kRowsMaxMat; ++i) {
+      a_route.w[i] = (const char*)a_in.w[i] + (long long)e * a_in.r_w_stride[i];
+      a_route.s[i] = a_in.s[i] ? (const char*)a_in.s[i] + (long long)e * a_in.r_s_stride[i] : nullptr;
+      a_route.z[i] = a_in.z[i] ? (const char*)a_in.z[i] + (long long)e * a_in.r_z_stride[i] : nullptr;
+      a_route.h[i] = a_in.h[i] ? (const char*)a_in.h[i] + (long long)e * a_in.r_h_stride[i] : nullptr;
+      a_route.out[i] = a_in.out[i] ? (char*)a_in.out[i] + (long long)r * a_in.r_out_stride * 2 : nullptr;
+    }
+    a_route.x = (const char*)a_in.x + (long long)(r / a_in.r_x_div) * a_in.K * 2;
+    if (a_in.r_out_mul) route_mul = Act::to_f32(((const typename Act::elem*)a_in.r_out_mul)[r]);
+  }
+  const RowsArgs& a = ROUTED ? a_route : a_in;
   constexpr bool kFp8 = FMT == RF_FP8;
   constexpr bool kByte = rows_byte_fmt(FMT);
   constexpr bool kNib = !kByte;
@@ -698,7 +730,7 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a) {
       for (int m = 0; m < MR; ++m) {
         const float v = wave_sum(acc[r][m]);
         acc[r][m] = 0.f;
-        const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(v * os));
+        const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, Act::from_f32(ROUTED ? v * os * route_mul : v * os));
         stored[m] = lane == r ? bits : stored[m];
         if (r == RW - 1) {
           asm volatile("" : "+v"(stored[m]));         // the store below reads exactly this register
@@ -784,8 +816,8 @@ static inline int device_cu_count() {
   return cus;
 }
 
-template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG, bool NORM = false>
-static void launch_rows_rw(RowsArgs a, hipStream_t st) {
+template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG, bool NORM = false, bool ROUTED = false>
+static void launch_rows_rw(RowsArgs a, hipStream_t st, int routes = 1) {
   constexpr int NWV = 8;
   constexpr int NBUF = 2;
   int groups = 0;
@@ -809,11 +841,24 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st) {
   a.total_waves = wgs * NWV;
   const size_t lds = XREG ? 0 : rows_lds_bytes(FMT, MR, a.K) + (NORM ? rows_norm_lds_bytes(a.K) : 0);
   if (a.nmat == 1)
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false, XREG, NORM>), dim3(wgs),
-                       dim3(NWV * 64), lds, st, a);
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false, XREG, NORM, ROUTED>),
+                       dim3(wgs, ROUTED ? routes : 1), dim3(NWV * 64), lds, st, a);
   else
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG, NORM>), dim3(wgs),
-                       dim3(NWV * 64), lds, st, a);
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG, NORM, ROUTED>),
+                       dim3(wgs, ROUTED ? routes : 1), dim3(NWV * 64), lds, st, a);
+}
+
+// Routed launch (one activation row per route, expert-indexed matrices): one row per batch,
+// activations staged through LDS; the routes are the grid's second dimension.
+template <class Act, int FMT>
+static void launch_rows_routed(RowsArgs a, int routes, hipStream_t st) {
+  constexpr bool kByte = rows_byte_fmt(FMT);
+  constexpr int ppl = kByte ? 2 : 4;
+  constexpr int span_k = 64 * ppl * 8;
+  constexpr int SPU = kByte ? 4 : 2;
+  a.nspan = (a.K + span_k - 1) / span_k;
+  if (a.nspan == 1) return launch_rows_rw<Act, FMT, 0, 1, 1, 1, false, false, true>(a, st, routes);
+  launch_rows_rw<Act, FMT, 0, 1, 1, SPU, false, false, true>(a, st, routes);
 }
 
 // Batch shape by row length.  Rows of up to one batch (fp8: 4 spans = 4096 k,

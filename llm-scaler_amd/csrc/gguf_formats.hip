@@ -355,11 +355,53 @@ static int run_gguf_gemv(RowsArgs r, int M, hipStream_t st) {
   return launch_status();
 }
 
+// Routed decode GEMVs of a GGUF MoE layer: one launch over all (token, expert) routes.
+template <int FMT>
+static int run_gguf_routed(RowsArgs r, int routes, hipStream_t st) {
+  if (rows_lds_bytes(FMT, 1, r.K) > 64 * 1024) return MI_ERR_SHAPE;
+  launch_rows_routed<ActF16, FMT>(r, routes, st);
+  return launch_status();
+}
+
 }  // namespace qlin
 
 using namespace qlin;
 
 extern "C" {
+
+int mi_moe_gguf_gemv(int fmt, const void* x, int x_div, int nmat, const void* const* ql, const void* const* qh,
+                     const void* const* scale, const void* const* qmin, void* const* out, long long out_stride,
+                     const int32_t* route_expert, const void* route_weight, int routes, int num_experts, int N,
+                     int K, void* stream) {
+  if (!x || !ql || !scale || !out || !route_expert) return MI_ERR_ARG;
+  if (fmt != RF_Q4K && fmt != RF_Q5K && fmt != RF_Q6K) return MI_ERR_ARG;
+  if (nmat < 1 || nmat > 2 || x_div < 1 || num_experts < 1) return MI_ERR_ARG;
+  if (routes < 0 || N < 0 || K <= 0 || out_stride < N) return MI_ERR_SHAPE;
+  if (fmt == RF_Q4K ? (K % 32) : (K % 512)) return MI_ERR_SHAPE;
+  if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || routes > 65535) return MI_ERR_SHAPE;
+  if (!routes || !N) return MI_OK;
+  RowsArgs r{};
+  r.x = x; r.nmat = nmat; r.M = 1; r.K = K;
+  r.r_expert = route_expert; r.r_out_mul = route_weight; r.r_num_experts = num_experts; r.r_x_div = x_div;
+  r.r_out_stride = out_stride;
+  const long long nk = (long long)N * K;
+  for (int i = 0; i < nmat; ++i) {
+    if (!ql[i] || !scale[i] || !out[i]) return MI_ERR_ARG;
+    if (fmt != RF_Q6K && (!qmin || !qmin[i])) return MI_ERR_ARG;
+    if (fmt != RF_Q4K && (!qh || !qh[i])) return MI_ERR_ARG;
+    r.w[i] = ql[i]; r.s[i] = scale[i]; r.out[i] = out[i]; r.N[i] = N;
+    r.z[i] = fmt != RF_Q6K ? qmin[i] : nullptr;
+    r.h[i] = fmt != RF_Q4K ? qh[i] : nullptr;
+    r.r_w_stride[i] = nk / 2;
+    r.r_s_stride[i] = fmt == RF_Q6K ? nk / 16 * 2 : nk / 32 * 2;
+    r.r_z_stride[i] = nk / 32 * 2;
+    r.r_h_stride[i] = fmt == RF_Q5K ? nk / 8 : nk / 4;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (fmt == RF_Q4K) return run_gguf_routed<RF_Q4K>(r, routes, st);
+  if (fmt == RF_Q5K) return run_gguf_routed<RF_Q5K>(r, routes, st);
+  return run_gguf_routed<RF_Q6K>(r, routes, st);
+}
 
 int mi_q4_0_repack(const void* raw, void* packed, void* scale, int N, int K, void* stream) {
   if (!raw || !packed || !scale) return MI_ERR_ARG;

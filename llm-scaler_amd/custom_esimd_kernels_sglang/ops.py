@@ -116,3 +116,19 @@ _moe_fp8_prefill = torch.ops.moe_fp8_prefill_ops
 def moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, top_k, num_experts):
     return _moe_fp8_prefill.moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale,
                                                  top_k, num_experts)
+
+
+# fused GGUF k-quant MoE decode stages, S/python/custom_esimd_kernels_sglang/ops.py:250-298
+def esimd_moe_up_q4k(x, gate_ql, gate_sc, gate_mn, up_ql, up_sc, up_mn, sel, inter, n_tokens, hidden, intermediate,
+                     top_k):
+    return _ops.esimd_moe_up_q4k(x, gate_ql, gate_sc, gate_mn, up_ql, up_sc, up_mn, sel, inter, n_tokens, hidden,
+                                 intermediate, top_k)
+
+
+def esimd_moe_down_q5k(inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
+    return _ops.esimd_moe_down_q5k(inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate,
+                                   top_k)
+
+
+def esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
+    return _ops.esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k)

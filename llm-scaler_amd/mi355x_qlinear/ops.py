@@ -413,6 +413,88 @@ def esimd_gemv_q5_k(input, ql, qh, weight_scale, weight_min, output):
     return output
 
 
+# routed decode GEMVs of a GGUF MoE layer (esimd_moe_up_q4k, esimd_moe_down_q5k / _q6k)
+def _chk_moe_gguf(x, sel, n_tokens, top_k, who):
+    _chk(x.dtype == torch.float16 and x.is_contiguous(), f"{who}: activations must be contiguous fp16")
+    _chk(sel.dtype == torch.int32 and sel.is_contiguous() and sel.numel() >= int(n_tokens) * int(top_k),
+         f"{who}: sel must be contiguous int32 [n_tokens * top_k]")
+    _chk(int(n_tokens) * int(top_k) <= 65535, f"{who}: at most 65535 routes per call")
+
+
+def _chk_stack(t, dtype, shape, name, who):
+    _chk(t.dtype == dtype and t.is_contiguous() and tuple(t.shape) == tuple(shape),
+         f"{who}: {name} must be contiguous {dtype} {list(shape)}, got {t.dtype} {list(t.shape)}")
+
+
+def esimd_moe_up_q4k(x, gate_ql, gate_sc, gate_mn, up_ql, up_sc, up_mn, sel, inter, n_tokens, hidden, intermediate,
+                     top_k):
+    """inter[r] = silu(x[t] @ Wg[e]^T) * (x[t] @ Wu[e]^T), r = t * top_k + j, e = sel[r]; Q4_K stacks
+    gate_ql / up_ql [E, I, H/2] uint8, scale / min [E, I, H/32] fp16
+    (S/csrc/xpu/torch_extension.cc:86-91).  One routed GEMV launch over both matrices, then SiLU * up on
+    their fp16 results."""
+    who = "esimd_moe_up_q4k"
+    T, H, I, k = int(n_tokens), int(hidden), int(intermediate), int(top_k)
+    _chk_moe_gguf(x, sel, T, k, who)
+    _chk(gate_ql.dim() == 3 and H % 32 == 0, f"{who}: gate_ql must be [E, I, H/2], H a multiple of 32")
+    E = gate_ql.shape[0]
+    for q, sc, mn, nm in ((gate_ql, gate_sc, gate_mn, "gate"), (up_ql, up_sc, up_mn, "up")):
+        _chk_stack(q, torch.uint8, (E, I, H // 2), nm + "_ql", who)
+        _chk_stack(sc, torch.float16, (E, I, H // 32), nm + "_sc", who)
+        _chk_stack(mn, torch.float16, (E, I, H // 32), nm + "_mn", who)
+    P = T * k
+    _chk(x.numel() >= T * H and inter.dtype == torch.float16 and inter.is_contiguous() and inter.numel() >= P * I,
+         f"{who}: x must be [n_tokens, hidden], inter fp16 [n_tokens * top_k, intermediate]")
+    if P == 0:
+        return inter
+    gu = torch.empty(P, 2 * I, dtype=torch.float16, device=x.device)
+    capi.call("mi_moe_gguf_gemv", x, 2, capi.ptr(x), k, 2, capi.ptr_array([gate_ql, up_ql]), None,
+              capi.ptr_array([gate_sc, up_sc]), capi.ptr_array([gate_mn, up_mn]), capi.ptr_array([gu, gu[:, I:]]),
+              2 * I, capi.ptr(sel), None, P, E, I, H)
+    capi.call("mi_moe_silu_mul", gu, capi.ptr(gu), capi.ptr(inter), 2 * I, I, P, capi.DT_F16)
+    return inter
+
+
+def _moe_down_gguf(fmt, inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k, who):
+    T, H, I, k = int(n_tokens), int(hidden), int(intermediate), int(top_k)
+    _chk_moe_gguf(inter, sel, T, k, who)
+    _chk(ql.dim() == 3 and I % 512 == 0, f"{who}: ql must be [E, hidden, intermediate/2], intermediate a multiple of 512")
+    E = ql.shape[0]
+    _chk_stack(ql, torch.uint8, (E, H, I // 2), "ql", who)
+    if fmt == 5:
+        _chk_stack(qh, torch.uint8, (E, H, I // 8), "qh", who)
+        _chk_stack(sc, torch.float16, (E, H, I // 32), "sc", who)
+        _chk_stack(mn, torch.float16, (E, H, I // 32), "mn", who)
+    else:
+        _chk_stack(qh, torch.uint8, (E, H, I // 4), "qh", who)
+        _chk_stack(sc, torch.float16, (E, H, I // 16), "sc", who)
+    P = T * k
+    _chk(inter.numel() >= P * I and topk_w.dtype == torch.float16 and topk_w.is_contiguous() and topk_w.numel() >= P,
+         f"{who}: inter must be [n_tokens * top_k, intermediate], topk_w fp16 [n_tokens * top_k]")
+    _chk(out_partial.dtype == torch.float16 and out_partial.is_contiguous() and out_partial.numel() >= P * H,
+         f"{who}: out_partial must be contiguous fp16 [n_tokens * top_k, hidden]")
+    if P == 0:
+        return out_partial
+    capi.call("mi_moe_gguf_gemv", inter, fmt, capi.ptr(inter), 1, 1, capi.ptr_array([ql]), capi.ptr_array([qh]),
+              capi.ptr_array([sc]), capi.ptr_array([mn]) if mn is not None else None, capi.ptr_array([out_partial]),
+              H, capi.ptr(sel), capi.ptr(topk_w), P, E, H, I)
+    return out_partial
+
+
+def esimd_moe_down_q5k(inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
+    """out_partial[r] = topk_w[r] * (inter[r] @ Wd[sel[r]]^T) on the Q5_K stack ql [E, H, I/2], qh [E, H, I/8]
+    (tile-shuffled fifth bits), scale / min [E, H, I/32] fp16 (S/csrc/xpu/torch_extension.cc:93-97);
+    the caller sums each token's top_k rows."""
+    return _moe_down_gguf(5, inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k,
+                          "esimd_moe_down_q5k")
+
+
+def esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
+    """The same on the Q6_K stack ql [E, H, I/2], qh [E, H, I/4], scale [E, H, I/16] fp16
+    (S/csrc/xpu/torch_extension.cc:98-101)."""
+    return _moe_down_gguf(6, inter, ql, qh, sc, None, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k,
+                          "esimd_moe_down_q6k")
+
+
 def _gemv_q6_k(input, ql, qh, weight_scale, output, who):
     _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be contiguous uint8 [N, K/2]")
     N, K = ql.shape[0], ql.shape[1] * 2
@@ -1774,6 +1856,15 @@ def register():
             esimd_gemv_q8_0, _ret(3))
     _define(_S, "esimd_gemv_q8_0_m(Tensor input, Tensor weight, Tensor weight_scale, Tensor output) -> Tensor",
             esimd_gemv_q8_0_m, _ret(3))
+    _define(_S, "esimd_moe_up_q4k(Tensor x, Tensor gate_ql, Tensor gate_sc, Tensor gate_mn, Tensor up_ql, Tensor up_sc, "
+                "Tensor up_mn, Tensor sel, Tensor inter, int n_tokens, int hidden, int intermediate, int top_k) -> Tensor",
+            esimd_moe_up_q4k, _ret(8))
+    _define(_S, "esimd_moe_down_q5k(Tensor inter, Tensor ql, Tensor qh, Tensor sc, Tensor mn, Tensor sel, Tensor topk_w, "
+                "Tensor out_partial, int n_tokens, int hidden, int intermediate, int top_k) -> Tensor",
+            esimd_moe_down_q5k, _ret(7))
+    _define(_S, "esimd_moe_down_q6k(Tensor inter, Tensor ql, Tensor qh, Tensor sc, Tensor sel, Tensor topk_w, "
+                "Tensor out_partial, int n_tokens, int hidden, int intermediate, int top_k) -> Tensor",
+            esimd_moe_down_q6k, _ret(6))
     _define(_S, "esimd_gemv_q5_k(Tensor input, Tensor ql, Tensor qh, Tensor weight_scale, Tensor weight_min, "
                 "Tensor output) -> Tensor", esimd_gemv_q5_k, _ret(5))
     _define(_S, "esimd_gemv_q6_k(Tensor input, Tensor ql, Tensor qh, Tensor weight_scale, Tensor output) -> Tensor",

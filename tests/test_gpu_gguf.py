@@ -146,6 +146,52 @@ def test_gemv(ops, dev, kind, M, N, K):
     assert O.max_rel_err(out.cpu(), ref) < TOL
 
 
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 8, 4, 2048, 512), (3, 16, 2, 512, 1024), (2, 4, 4, 5120, 512)])
+def test_moe_gguf_routed_stages(ops, dev, T, E, k, H, I):
+    """esimd_moe_up_q4k -> esimd_moe_down_q5k / _q6k (S/csrc/xpu/torch_extension.cc:86-101): per-route
+    GEMVs on expert stacks of the repacked representations, against the per-route loop on the oracle's
+    dequantized weights."""
+    _, s = ops
+    rng = np.random.default_rng(T + E + H)
+    g = torch.Generator().manual_seed(H + I)
+    x = (torch.randn(T, H, generator=g) * 0.1).half()   # keeps silu(gate) * up inside fp16 range
+    sel = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).reshape(-1)
+    P = T * k
+    stack = lambda a: _t(a).reshape(E, -1, a.shape[-1]).to(dev)
+    # gate / up: Q4_K stacks [E, I, ...]
+    reps, deq = [], []
+    for seed in (11, 12):
+        _, raw = O.make_q4k_case(1, H, E * I, seed=seed + H)
+        rep = O.q4k_repack(raw)
+        reps.append([stack(a) for a in rep])
+        deq.append(torch.from_numpy(O.q4k_dequant(*rep).astype(np.float32)).reshape(E, I, H))
+    inter = torch.empty(P, I, dtype=torch.float16, device=dev)
+    ret = s.esimd_moe_up_q4k(x.to(dev), *reps[0], *reps[1], sel.to(dev), inter, T, H, I, k)
+    assert ret.data_ptr() == inter.data_ptr()
+    tok = torch.arange(P) // k
+    e_of = sel.long()
+    gate = torch.einsum("ph,pih->pi", x.float()[tok], deq[0][e_of])
+    up = torch.einsum("ph,pih->pi", x.float()[tok], deq[1][e_of])
+    want = torch.nn.functional.silu(gate.half().float()) * up.half().float()
+    assert O.max_rel_err(inter.cpu(), want) < 2 * TOL           # gate / up are rounded to fp16 before SiLU * up
+    free = torch.nn.functional.silu(gate) * up
+    assert ((inter.cpu().float() - free).abs().mean() / free.abs().mean()).item() < 5e-3
+    # down: Q5_K and Q6_K stacks [E, H, ...] on an intermediate of a size that keeps fp16 outputs finite
+    tw = torch.rand(P, generator=g).half()
+    inter = (torch.randn(P, I, generator=g) * 0.1).half().to(dev)
+    for kind in ("q5_k", "q6_k"):
+        raw = _raw_case(kind, E * H, I, seed=31 + I)
+        rep = _repack_oracle(kind, raw)
+        wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32)).reshape(E, H, I)
+        out = torch.empty(P, H, dtype=torch.float16, device=dev)
+        args = [stack(a) for a in rep]
+        fn = s.esimd_moe_down_q5k if kind == "q5_k" else s.esimd_moe_down_q6k
+        ret = fn(inter, *args, sel.to(dev), tw.to(dev), out, T, H, I, k)
+        assert ret.data_ptr() == out.data_ptr()
+        ref = torch.einsum("pi,phi->ph", inter.cpu().float(), wd[e_of]) * tw.float().view(-1, 1)
+        assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
 @pytest.mark.parametrize("name,kind", [("esimd_gemm_q4_0", "q4_0"), ("esimd_gemv_q8_0_m", "q8_0"), ("esimd_gemv_q6_k_m", "q6_k")])
 def test_small_m_variants(ops, dev, name, kind):
     _, s = ops
