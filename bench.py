@@ -171,6 +171,37 @@ def wl_gguf(kind: str, M: int, dev):
                 name=f"next: GGUF {kind} (repacked) decode GEMV M={M} K={K} N={N} fp16", kernel="gemv_rows_kernel", cpu=cpu)
 
 
+def wl_moe_gguf(dev):
+    """One decode token through the routed GGUF MoE stages (next-row workload): Q4_K gate / up,
+    SiLU * up, Q6_K down over top-8 of 256 experts, H = 2048, I = 1024.  Consecutive launches route to
+    consecutive groups of eight experts, so 32 launches walk the whole 1.2 GB stack once.  The stacks
+    hold random codes and scales (timing only; parity is tests/test_gpu_gguf.py)."""
+    import custom_esimd_kernels_sglang as s
+    E, k, H, I = 256, 8, 2048, 1024
+    g = torch.Generator(device="cpu").manual_seed(97)
+    u8 = lambda *shape: torch.randint(0, 256, shape, dtype=torch.uint8, generator=g).to(dev)
+    f16 = lambda hi, *shape: (torch.rand(*shape, generator=g) * hi).half().to(dev)
+    gq, uq = u8(E, I, H // 2), u8(E, I, H // 2)
+    gs, gm, us, um = f16(0.01, E, I, H // 32), f16(0.005, E, I, H // 32), f16(0.01, E, I, H // 32), f16(0.005, E, I, H // 32)
+    dq, dh, ds = u8(E, H, I // 2), u8(E, H, I // 4), f16(0.002, E, H, I // 16)
+    x = (torch.randn(1, H, generator=g) * 0.1).half().to(dev)
+    tw = torch.full((k,), 1.0 / k, dtype=torch.float16, device=dev)
+    R = E // k
+    sels = [(torch.arange(k, dtype=torch.int32) + k * i).to(dev) for i in range(R)]
+    inter = torch.empty(k, I, dtype=torch.float16, device=dev)
+    out = torch.empty(k, H, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        sel = sels[i % R]
+        s.esimd_moe_up_q4k(x, gq, gs, gm, uq, us, um, sel, inter, 1, H, I, k)
+        s.esimd_moe_down_q6k(inter, dq, dh, ds, sel, tw, out, 1, H, I, k)
+
+    per = k * (2 * (I * H // 2 + 2 * I * (H // 32) * 2) + H * I // 2 + H * I // 4 + H * (I // 16) * 2)
+    return dict(launch=launch, R=R, bytes=per + 2 * H + 2 * k * (3 * I + H) * 2, flops=2 * k * 3 * I * H, bound="hbm",
+                dtype="f16", name=f"next: GGUF MoE decode stages T=1 top-{k} of {E} experts H={H} I={I} "
+                                   "(Q4_K gate, Q4_K up, SiLU*up, Q6_K down: 4 launches)", kernel="gemv_rows_kernel", cpu=lambda: None)
+
+
 def wl_q4_0_quantize(dev):
     """On-device group-128 Q4_0 quantization of a [14336, 4096] bf16 weight (next-row workload)."""
     import custom_esimd_kernels_vllm as v
@@ -422,6 +453,7 @@ WORKLOADS = {
     "next_moe_gelu_grouped": wl_moe_gelu,
     "next_moe_forward_full_t1": wl_moe_forward_full,
     "next_gemv_fp16_router": wl_gemv_fp16,
+    "next_moe_gguf_t1": wl_moe_gguf,
 }
 HEADLINE = "cfg1_m1"
 

@@ -160,6 +160,7 @@ int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int
  * W_i = the per-expert stack [E, N, ...] of the repacked representation the dense GEMVs read
  * (fmt 2 = Q4_K: ql, scale, qmin; 5 = Q5_K: + qh; 6 = Q6_K: ql, qh, scale), fp16, rows of out
  * out_stride elements apart, route_weight (fp16) optional, expert ids clamped into [0, E).
+ * One kernel launch per matrix.
  * Replaces the launches of esimd_moe_up_q4k (two matrices: gate and up halves of one buffer,
  * x_div = top_k; SiLU * up follows as mi_moe_silu_mul) and esimd_moe_down_q5k / _q6k
  * (x = the intermediate in route order, x_div = 1, route_weight = topk_w)

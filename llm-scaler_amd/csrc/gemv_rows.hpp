@@ -837,7 +837,13 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st, int routes = 1) {
     if (eff > best_eff + 1e-9) { best_eff = eff; best_wgs = cus * per_cu; }
   }
   const int needed = (groups + NWV - 1) / NWV;
-  const int wgs = needed < best_wgs ? needed : best_wgs;
+  int wgs = needed < best_wgs ? needed : best_wgs;
+  if constexpr (ROUTED) {
+    // the routes share the device: about two workgroups per CU over all of them, so that a
+    // wavefront walks several rows and the next row loads while the current one is consumed
+    const int cap = (2 * cus + routes - 1) / routes;
+    if (wgs > cap) wgs = cap;
+  }
   a.total_waves = wgs * NWV;
   const size_t lds = XREG ? 0 : rows_lds_bytes(FMT, MR, a.K) + (NORM ? rows_norm_lds_bytes(a.K) : 0);
   if (a.nmat == 1)
