@@ -444,6 +444,8 @@ WORKLOADS = {
     "cfg3": wl_moe,
     "cfg4_m1": lambda dev: wl_q4k(1, dev),
     "cfg4_m64": lambda dev: wl_q4k(64, dev),
+    "next_q4k_m8": lambda dev: wl_q4k(8, dev),
+    "next_q4k_m32": lambda dev: wl_q4k(32, dev),
     "next_q4_0_m1": lambda dev: wl_gguf("q4_0", 1, dev),
     "next_q8_0_m1": lambda dev: wl_gguf("q8_0", 1, dev),
     "next_q5_k_m1": lambda dev: wl_gguf("q5_k", 1, dev),

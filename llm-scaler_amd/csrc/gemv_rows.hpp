@@ -846,12 +846,12 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st, int routes = 1) {
   }
   a.total_waves = wgs * NWV;
   const size_t lds = XREG ? 0 : rows_lds_bytes(FMT, MR, a.K) + (NORM ? rows_norm_lds_bytes(a.K) : 0);
-  if (a.nmat == 1)
+  if (a.nmat == 1 || ROUTED)                          // routed launches take one matrix
     hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, false, XREG, NORM, ROUTED>),
                        dim3(wgs, ROUTED ? routes : 1), dim3(NWV * 64), lds, st, a);
-  else
-    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG, NORM, ROUTED>),
-                       dim3(wgs, ROUTED ? routes : 1), dim3(NWV * 64), lds, st, a);
+  else if constexpr (!ROUTED)
+    hipLaunchKernelGGL((gemv_rows_kernel<Act, FMT, SC, MR, NWV, RW, SPU, NBUF, true, XREG, NORM, false>), dim3(wgs),
+                       dim3(NWV * 64), lds, st, a);
 }
 
 // Routed launch (one activation row per route, expert-indexed matrices): one row per batch,

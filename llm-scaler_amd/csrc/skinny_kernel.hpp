@@ -51,7 +51,10 @@ enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
 // 4 = Q8_0, 5 = Q5_K, 6 = Q6_K (the GGUF formats in their repacked representation, fp16).
 // MT = 16-row activation tiles (M <= 16 MT), RT = 16-row weight tiles per
 // workgroup, NW = wavefronts splitting K, UN = granules in flight per wave.
-template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
+// SL: the per-32 scales (and mins) of the workgroup's rows are staged once in LDS instead of
+// being fetched per tile and granule with scattered 16-bit loads (Q4_K, Q5_K, Q4_0, Q8_0;
+// needs K % 256 == 0 and room beside the staging tiles).
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   using V8 = typename Act::v8;
   using Elem = typename Act::elem;
@@ -65,6 +68,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr bool kByteW = kIsFp8 || kIsQ80;           // one byte per weight: 128 bytes per row and granule
   constexpr bool kHigh = kIsQ5K || kIsQ6K;            // extra high bits per weight
   constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
+  constexpr bool kSide32 = kIsQ4K || kIsQ5K || kIsQ40 || kIsQ80;   // one fp16 scale per 32 k
+  constexpr bool kHasMin = kIsQ4K || kIsQ5K;
+  static_assert(!SL || kSide32, "LDS-staged scales are for the formats with per-32 scales");
 
   // wave-private staging tiles for the weights (one 16-row tile = 16 rows of one
   // granule, padded pitch); the cross-wave reduction buffer overlays them at the end
@@ -73,6 +79,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr int kXP = 256 + 16;                       // activation tile pitch
   constexpr bool kXLds = MT >= 4;                     // stage the activations through LDS too
   constexpr int kWStage = NW * RT * 16 * kWP;         // activation tiles follow the weight tiles
+  constexpr int kTiles = kWStage + (kXLds ? NW * MT * 16 * kXP : 0);   // SL: the scale tables follow
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
 
@@ -167,6 +174,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
         if constexpr (kIsInt4) {
           st.sc[u][t] = s16u[(size_t)nc * Kg + gic];
           st.zz[u][t] = zsrc[(size_t)nc * Kg + gic];
+        } else if constexpr (SL) {
+          // read from the LDS tables when the stage is consumed
         } else if constexpr (kIsQ4K || kIsQ5K) {
           const int sb = gic * 4 + g;
           const int sbc = sb < Kb32 ? sb : Kb32 - 1;
@@ -245,6 +254,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
           *reinterpret_cast<u32x4*>(wl + (lane >> 2) * kWP + (lane & 3) * 16) = wa;
           wa = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 16);
         }
+        if constexpr (SL) {
+          const int gi_here = gbase_of_stage + u * NW;
+          const int sb = min(gi_here * 4 + g, Kb32 - 1);
+          const uint16_t* tab = reinterpret_cast<const uint16_t*>(smem + kTiles);
+          st.sc[u][t] = tab[(t * 16 + j) * Kb32 + sb];
+          if constexpr (kHasMin) st.zz[u][t] = tab[(RT * 16 + t * 16 + j) * Kb32 + sb];
+        }
         V8 b[4];
         float scf = 0.f;
         if constexpr (kIsFp8) {
@@ -319,6 +335,37 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     }
   };
 
+  if constexpr (SL) {
+    // tables [RT * 16 rows][K / 32] of scales, then of mins; rows past the workgroup's range are zeros
+    const __amdgpu_buffer_rsrc_t sr = make_rsrc(a.s[mat], (uint32_t)N * (uint32_t)Kb32 * 2u);
+    const __amdgpu_buffer_rsrc_t mr = make_rsrc(a.z[mat], kHasMin ? (uint32_t)N * (uint32_t)Kb32 * 2u : 0u);
+    const int cpr = Kb32 >> 3;                        // 16-byte chunks per row
+    u32x4* tab = reinterpret_cast<u32x4*>(smem + kTiles);
+    const int total = RT * 16 * cpr;
+    constexpr int FI = 4;                             // chunks in flight per thread and table
+    for (int c0 = 0; c0 < total; c0 += NW * 64 * FI) {
+      u32x4 sv[FI], mv[FI];
+#pragma unroll
+      for (int i = 0; i < FI; ++i) {
+        const int c = c0 + i * NW * 64 + (int)threadIdx.x;
+        const int r = c / cpr, cc = c - r * cpr;
+        const int n = n0 + r;
+        const uint32_t off = (c < total && n < nend) ? ((uint32_t)n * (uint32_t)Kb32 + (uint32_t)cc * 8u) * 2u : kOOB;
+        sv[i] = buf_load16(sr, off);
+        if constexpr (kHasMin) mv[i] = buf_load16(mr, off);
+      }
+#pragma unroll
+      for (int i = 0; i < FI; ++i) {
+        const int c = c0 + i * NW * 64 + (int)threadIdx.x;
+        if (c < total) {
+          tab[c] = sv[i];
+          if constexpr (kHasMin) tab[total + c] = mv[i];
+        }
+      }
+    }
+    __syncthreads();
+  }
+
   if constexpr (UN >= 2) {
     // two-stage ring; the only exit is at the bottom (stages past the end load zeros)
     Stage s0, s1;
@@ -377,7 +424,15 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   }
 }
 
-template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
+// Bytes of the LDS scale tables of an SL instantiation (0: the format has none).
+template <int FMT, int RT>
+static inline int skinny_table_bytes(int K) {
+  const bool side32 = FMT == 2 || FMT == 5 || FMT == 3 || FMT == 4;
+  if (!side32) return 0;
+  return RT * 16 * (K / 32) * 2 * ((FMT == 2 || FMT == 5) ? 2 : 1);
+}
+
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false>
 static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
   int tiles = 0;
   a.rpw = rpw;
@@ -388,17 +443,37 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
   if (tiles == 0) return;
   constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
   constexpr int kRed = (NW - 1) * RT * MT * 1024;
-  constexpr int lds = kStage > kRed ? kStage : kRed;
-  static_assert(lds <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
-  auto kern = skinny_kernel<Act, FMT, SC, MT, RT, NW, UN>;
+  static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
+  const int with_tables = kStage + (SL ? skinny_table_bytes<FMT, RT>(a.K) : 0);
+  const int lds = with_tables > kRed ? with_tables : kRed;
+  auto kern = skinny_kernel<Act, FMT, SC, MT, RT, NW, UN, SL>;
   if (lds > 64 * 1024) {
-    static bool raised = false;                       // opt in to > 64 KiB of dynamic LDS once
-    if (!raised) {
+    static int raised = 0;                            // opt in to > 64 KiB of dynamic LDS (grows with K)
+    if (raised < lds) {
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      raised = true;
+      raised = lds;
     }
   }
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(NW * 64), lds, st, a);
+}
+
+// The SL instantiation when the format has per-32 scales, K allows whole 16-byte chunks per row
+// and the tables fit beside the staging tiles; the plain one otherwise.
+template <int FMT, int MT, int RT, int NW>
+static inline bool skinny_tables_fit(int K) {
+  if constexpr (FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
+    constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
+    return K % 256 == 0 && kStage + skinny_table_bytes<FMT, RT>(K) <= 160 * 1024;
+  }
+  return false;
+}
+
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
+static void launch_pick(const SkinnyArgs& a, int rpw, hipStream_t st) {
+  if constexpr (FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
+    if (skinny_tables_fit<FMT, MT, RT, NW>(a.K)) return launch_one<Act, FMT, SC, MT, RT, NW, UN, true>(a, rpw, st);
+  }
+  launch_one<Act, FMT, SC, MT, RT, NW, UN, false>(a, rpw, st);
 }
 
 template <class Act, int FMT, int SC>
@@ -419,18 +494,20 @@ static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
     rpw = (FMT == 0 && SC == SC_BLOCK) ? ((rpw + 15) & ~15) : ((rpw + 7) & ~7);
     if (rpw > 64) rpw = 64;
     if (rpw <= 16) {
-      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 1, 8, 4>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 1, 8, 2>(a, rpw, st);
-      else launch_one<Act, FMT, SC, 4, 1, 8, 1>(a, rpw, st);
+      if (a.M <= 16) launch_pick<Act, FMT, SC, 1, 1, 8, 4>(a, rpw, st);
+      else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 1, 8, 2>(a, rpw, st);
+      else launch_pick<Act, FMT, SC, 4, 1, 8, 1>(a, rpw, st);
     } else if (rpw <= 32) {
-      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
-      else if constexpr (FMT == 0 || FMT == 4) launch_one<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
+      if (a.M <= 16) launch_pick<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
+      else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
+      else if constexpr (FMT == 0 || FMT == 4) launch_pick<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
+      else if (skinny_tables_fit<FMT, 4, 2, 6>(a.K)) launch_pick<Act, FMT, SC, 4, 2, 6, 1>(a, rpw, st);
       else launch_one<Act, FMT, SC, 4, 2, 8, 1>(a, rpw, st);   // nibble formats: eight waves' tiles fit the LDS
+      // (cfg4 M=64, Q4_K: 24.1 us with four waves, 21.9 with eight, 18.6 with six + the LDS tables)
     } else {
-      if (a.M <= 16) launch_one<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
-      else if (a.M <= 32) launch_one<Act, FMT, SC, 2, 4, 8, 1>(a, rpw, st);
-      else launch_one<Act, FMT, SC, 4, 4, 4, 1>(a, rpw, st);
+      if (a.M <= 16) launch_pick<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
+      else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 4, 8, 1>(a, rpw, st);
+      else launch_pick<Act, FMT, SC, 4, 4, 4, 1>(a, rpw, st);
     }
   }
   return launch_status();
