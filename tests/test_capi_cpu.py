@@ -39,6 +39,28 @@ REFERENCE_SCHEMAS = {
     "custom_esimd_kernels_vllm::esimd_gemm_fp8_blockscale": ["input", "weight", "weight_scale", "output", "block_n", "block_k"],
     "custom_esimd_kernels_sglang::esimd_gemv_q4_k": ["input", "weight", "weight_scale", "weight_min", "output"],
     "custom_esimd_kernels::esimd_gemm_fp8_pert": ["input", "weight", "weight_scale", "output"],
+    # sglang/custom-esimd-kernels/csrc/xpu/torch_extension.cc:86-101
+    "custom_esimd_kernels_sglang::esimd_moe_up_q4k": ["x", "gate_ql", "gate_sc", "gate_mn", "up_ql", "up_sc", "up_mn", "sel",
+                                                      "inter", "n_tokens", "hidden", "intermediate", "top_k"],
+    "custom_esimd_kernels_sglang::esimd_moe_down_q5k": ["inter", "ql", "qh", "sc", "mn", "sel", "topk_w", "out_partial",
+                                                        "n_tokens", "hidden", "intermediate", "top_k"],
+    "custom_esimd_kernels_sglang::esimd_moe_down_q6k": ["inter", "ql", "qh", "sc", "sel", "topk_w", "out_partial",
+                                                        "n_tokens", "hidden", "intermediate", "top_k"],
+    # sglang/custom-esimd-kernels/csrc/moe_batch/moe.sycl:2156-2167
+    "moe_ops::moe_forward_full_silu_routed": ["x", "topk_weights", "topk_indices", "gate_up_weight", "gate_up_scale",
+                                              "down_weight", "down_scale", "top_k", "n_routed_experts"],
+    "moe_ops::moe_forward_full_silu_routed_sglang": ["x", "topk_weights", "topk_indices", "gate_up_weight", "gate_up_scale",
+                                                     "down_weight", "down_scale", "top_k", "n_routed_experts"],
+    "moe_ops::moe_router_forward": ["x", "weight", "scale"],
+    "moe_ops::moe_accumulate": ["partials", "top_k", "num_shared_experts"],
+    # vllm/custom-esimd-kernels-vllm/csrc/xpu/torch_extension_topk_v2.cc:13-14, torch_extension.cc:158-175
+    "esimd_topk_v2::topk_v2": ["router_logits", "top_values", "top_indices", "T", "num_experts", "topk"],
+    "custom_esimd_kernels_vllm::esimd_norm_gemv_norm_fp16": ["residual", "scale_with_root", "proj_w", "pre_ff_w",
+                                                             "router_logits", "moe_input", "eps"],
+    "custom_esimd_kernels_vllm::esimd_scaled_resadd_norm_gemv_fp8_pert": ["hidden_states", "residual", "norm_weight",
+                                                                          "qkv_weight", "qkv_scale", "qkv_out", "eps", "scalar"],
+    "custom_esimd_kernels_vllm::esimd_norm_add_norm": ["h2_raw", "h1", "w1", "w2", "out", "eps1", "eps2"],
+    "custom_esimd_kernels_vllm::esimd_accum_norm_add_norm": ["routed_output", "h1", "w1", "w2", "out", "top_k", "eps1", "eps2"],
 }
 
 
