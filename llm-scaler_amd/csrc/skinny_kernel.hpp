@@ -51,9 +51,10 @@ enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
 // 4 = Q8_0, 5 = Q5_K, 6 = Q6_K (the GGUF formats in their repacked representation, fp16).
 // MT = 16-row activation tiles (M <= 16 MT), RT = 16-row weight tiles per
 // workgroup, NW = wavefronts splitting K, UN = granules in flight per wave.
-// SL: the per-32 scales (and mins) of the workgroup's rows are staged once in LDS instead of
-// being fetched per tile and granule with scattered 16-bit loads (Q4_K, Q5_K, Q4_0, Q8_0;
-// needs K % 256 == 0 and room beside the staging tiles).
+// SL: the scales (and mins / zero-points) of the workgroup's rows are staged once in LDS instead
+// of being fetched per tile and granule with scattered 16-bit loads: per-32 tables for Q4_K,
+// Q5_K, Q4_0, Q8_0 (needs K % 256 == 0), per-128 tables for INT4; chosen when the tables fit
+// beside the staging tiles.
 template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   using V8 = typename Act::v8;
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
   constexpr bool kSide32 = kIsQ4K || kIsQ5K || kIsQ40 || kIsQ80;   // one fp16 scale per 32 k
   constexpr bool kHasMin = kIsQ4K || kIsQ5K;
-  static_assert(!SL || kSide32, "LDS-staged scales are for the formats with per-32 scales");
+  static_assert(!SL || kSide32 || kIsInt4, "LDS-staged scales are for the formats with per-32 or per-128 scales");
 
   // wave-private staging tiles for the weights (one 16-row tile = 16 rows of one
   // granule, padded pitch); the cross-wave reduction buffer overlays them at the end
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
         }
         // side data stays raw until it is used: a conversion here would wait for the load,
         // and with it for every older load in flight
-        if constexpr (kIsInt4) {
+        if constexpr (kIsInt4 && !SL) {
           st.sc[u][t] = s16u[(size_t)nc * Kg + gic];
           st.zz[u][t] = zsrc[(size_t)nc * Kg + gic];
         } else if constexpr (SL) {
@@ -254,7 +255,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
           *reinterpret_cast<u32x4*>(wl + (lane >> 2) * kWP + (lane & 3) * 16) = wa;
           wa = *reinterpret_cast<const u32x4*>(wl + j * kWP + g * 16);
         }
-        if constexpr (SL) {
+        if constexpr (SL && kIsInt4) {
+          const int gq = min(gbase_of_stage + u * NW, Kg - 1);
+          const uint16_t* ts = reinterpret_cast<const uint16_t*>(smem + kTiles);
+          const uint8_t* tz = reinterpret_cast<const uint8_t*>(ts + RT * 16 * Kg);
+          st.sc[u][t] = ts[(t * 16 + j) * Kg + gq];
+          st.zz[u][t] = tz[(t * 16 + j) * Kg + gq];
+        } else if constexpr (SL) {
           const int gi_here = gbase_of_stage + u * NW;
           const int sb = min(gi_here * 4 + g, Kb32 - 1);
           const uint16_t* tab = reinterpret_cast<const uint16_t*>(smem + kTiles);
@@ -335,7 +342,35 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     }
   };
 
-  if constexpr (SL) {
+  if constexpr (SL && kIsInt4) {
+    // tables [RT * 16 rows][K / 128]: fp16 scales, then zero-point bytes; rows past the range are zeros
+    uint16_t* ts = reinterpret_cast<uint16_t*>(smem + kTiles);
+    uint8_t* tz = reinterpret_cast<uint8_t*>(ts + RT * 16 * Kg);
+    const int total = RT * 16 * Kg;
+    constexpr int FI = 4;
+    for (int c0 = 0; c0 < total; c0 += NW * 64 * FI) {
+      uint16_t sv[FI];
+      uint8_t zv[FI];
+#pragma unroll
+      for (int i = 0; i < FI; ++i) {
+        const int c = c0 + i * NW * 64 + (int)threadIdx.x;
+        const int r = min(c, total - 1) / Kg, cc = min(c, total - 1) - r * Kg;
+        const int n = min(n0 + r, N - 1);
+        sv[i] = s16u[(size_t)n * Kg + cc];
+        zv[i] = zsrc[(size_t)n * Kg + cc];
+      }
+#pragma unroll
+      for (int i = 0; i < FI; ++i) {
+        const int c = c0 + i * NW * 64 + (int)threadIdx.x;
+        if (c < total) {
+          const bool ok = n0 + c / Kg < nend;
+          ts[c] = ok ? sv[i] : (uint16_t)0;
+          tz[c] = ok ? zv[i] : (uint8_t)0;
+        }
+      }
+    }
+    __syncthreads();
+  } else if constexpr (SL) {
     // tables [RT * 16 rows][K / 32] of scales, then of mins; rows past the workgroup's range are zeros
     const __amdgpu_buffer_rsrc_t sr = make_rsrc(a.s[mat], (uint32_t)N * (uint32_t)Kb32 * 2u);
     const __amdgpu_buffer_rsrc_t mr = make_rsrc(a.z[mat], kHasMin ? (uint32_t)N * (uint32_t)Kb32 * 2u : 0u);
@@ -427,6 +462,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 // Bytes of the LDS scale tables of an SL instantiation (0: the format has none).
 template <int FMT, int RT>
 static inline int skinny_table_bytes(int K) {
+  if (FMT == 1) return (RT * 16 * (K / 128) * 3 + 15) & ~15;   // fp16 scales + zero-point bytes
   const bool side32 = FMT == 2 || FMT == 5 || FMT == 3 || FMT == 4;
   if (!side32) return 0;
   return RT * 16 * (K / 32) * 2 * ((FMT == 2 || FMT == 5) ? 2 : 1);
@@ -461,16 +497,16 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
 // and the tables fit beside the staging tiles; the plain one otherwise.
 template <int FMT, int MT, int RT, int NW>
 static inline bool skinny_tables_fit(int K) {
-  if constexpr (FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
+  if constexpr (FMT == 1 || FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
     constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
-    return K % 256 == 0 && kStage + skinny_table_bytes<FMT, RT>(K) <= 160 * 1024;
+    return (FMT == 1 || K % 256 == 0) && kStage + skinny_table_bytes<FMT, RT>(K) <= 160 * 1024;
   }
   return false;
 }
 
 template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN>
 static void launch_pick(const SkinnyArgs& a, int rpw, hipStream_t st) {
-  if constexpr (FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
+  if constexpr (FMT == 1 || FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
     if (skinny_tables_fit<FMT, MT, RT, NW>(a.K)) return launch_one<Act, FMT, SC, MT, RT, NW, UN, true>(a, rpw, st);
   }
   launch_one<Act, FMT, SC, MT, RT, NW, UN, false>(a, rpw, st);
