@@ -1094,6 +1094,22 @@ def moe_prefill_gather_forward_fp8(selected_experts, num_experts):
     moe_sort(sel, E, tokens, start, perm, None, None)
     return [start[:E], tokens, perm, start[1:] - start[:E]]
 
+def moe_prefill_gather_forward_v2(selected_experts, num_experts):
+    """moe_int4_prefill_ops::moe_prefill_gather_forward_v2: the same grouping under the name the FP8
+    grouped path of the patched vLLM calls (V/csrc/moe_prefill/moe_prefill_int4.sycl:458-486,
+    vllm/patches/vllm_for_multi_arc.patch:8228-8230)."""
+    return moe_prefill_gather_forward_fp8(selected_experts, num_experts)
+
+
+def moe_topk_softmax(router_logits, top_k, num_experts):
+    """-> [weights [T, top_k] (renormalised, logits dtype), ids [T, top_k] int32]
+    (V/csrc/moe_prefill/moe_prefill_int4.sycl:869-920)."""
+    _chk(router_logits.dim() == 2 and router_logits.shape[1] == int(num_experts),
+         "moe_topk_softmax: router_logits.size(1) must equal num_experts")
+    w, ids = moe_topk(router_logits, int(top_k), True)
+    return [w, ids]
+
+
 # --------------------------------------------------------------------------
 # decode fusions: RMS norm (+ residual add / + SiLU gate) in front of a GEMV
 # (V/csrc/xpu/torch_extension.cc:103-140).  Two launches here: the norm kernel,
@@ -1918,6 +1934,12 @@ def register():
                        "Tensor down_weight, Tensor down_scale, Tensor shared_down_weight, Tensor shared_down_scale, "
                        "Tensor shared_expert_gate_weight, int top_k, int num_shared_experts, "
                        "int n_routed_experts) -> Tensor(a!)", moe_forward_full_fp8_block, _ret(2))
+    _define("moe_int4_prefill_ops", "moe_prefill_gather_forward_v2(Tensor selected_experts, int num_experts) -> Tensor[]",
+            moe_prefill_gather_forward_v2,
+            lambda sel, e: [sel.new_empty(e), sel.new_empty(sel.numel()), sel.new_empty(sel.numel()), sel.new_empty(e)])
+    _define("moe_int4_prefill_ops", "moe_topk_softmax(Tensor router_logits, int top_k, int num_experts) -> Tensor[]",
+            moe_topk_softmax,
+            lambda l, k, e: [l.new_empty(l.shape[0], k), l.new_empty(l.shape[0], k, dtype=torch.int32)])
     _define("esimd_topk_v2", "topk_v2(Tensor router_logits, Tensor top_values, Tensor top_indices, int T, "
             "int num_experts, int topk) -> Tensor", topk_v2, _ret(1))
     _define("moe_ops", "moe_router_forward(Tensor x, Tensor weight, Tensor scale) -> Tensor", moe_router_forward,

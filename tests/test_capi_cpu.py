@@ -54,6 +54,9 @@ REFERENCE_SCHEMAS = {
     "moe_ops::moe_router_forward": ["x", "weight", "scale"],
     "moe_ops::moe_accumulate": ["partials", "top_k", "num_shared_experts"],
     # vllm/custom-esimd-kernels-vllm/csrc/xpu/torch_extension_topk_v2.cc:13-14, torch_extension.cc:158-175
+    # vllm/custom-esimd-kernels-vllm/csrc/moe_prefill/moe_prefill_int4.sycl:996-1013
+    "moe_int4_prefill_ops::moe_prefill_gather_forward_v2": ["selected_experts", "num_experts"],
+    "moe_int4_prefill_ops::moe_topk_softmax": ["router_logits", "top_k", "num_experts"],
     "esimd_topk_v2::topk_v2": ["router_logits", "top_values", "top_indices", "T", "num_experts", "topk"],
     "custom_esimd_kernels_vllm::esimd_norm_gemv_norm_fp16": ["residual", "scale_with_root", "proj_w", "pre_ff_w",
                                                              "router_logits", "moe_input", "eps"],

@@ -547,6 +547,28 @@ def test_moe_gelu_tanh_family(v, dev, T, E, H, I, k, dtype):
     assert O.max_rel_err(full.cpu().float(), want_r) < TOL
 
 
+def test_moe_fp8_grouped_vllm_call_chain(v, dev):
+    """The call sequence of the patched vLLM's grouped FP8 MoE forward
+    (vllm/patches/vllm_for_multi_arc.patch:8216-8246): module import, softmax top-k, gather v2 of the
+    moe_int4_prefill_ops namespace, grouped up / down on uint8 views, sum over the routes."""
+    import custom_esimd_kernels_vllm.moe_int4_prefill_ops  # noqa: F401  (registers the gather)
+    T, E, H, I, k = 20, 16, 512, 256, 4
+    x, logits, tw, ti, w13, s13, w2, s2 = _pert_case(T, E, H, I, k, 77, torch.float16)
+    d = lambda t: t.to(dev)
+    weights, indices = torch.ops.moe_int4_prefill_ops.moe_topk_softmax(d(logits), k, E)
+    assert torch.equal(indices.cpu(), ti)
+    go = torch.ops.moe_int4_prefill_ops.moe_prefill_gather_forward_v2(indices.contiguous(), E)
+    expert_offsets, expert_tokens = go[0], go[1]
+    assert len(go) == 4 and expert_offsets.numel() == E and expert_tokens.numel() == T * k
+    w13u, w2u = d(w13).view(torch.uint8), d(w2).view(torch.uint8)
+    rw_flat = weights.reshape(-1).contiguous()
+    inter = torch.ops.moe_ops.moe_up_fp8_grouped(d(x), w13u, d(s13), expert_offsets, expert_tokens, k, E)
+    outp = torch.ops.moe_ops.moe_down_fp8_grouped(inter, w2u, d(s2), rw_flat, expert_offsets, expert_tokens, k, E)
+    out = outp.view(T, k, -1).sum(1)
+    want = O.moe_prefill_scalar(x, weights.cpu(), ti, w13, s13, w2, s2, act="gelu_tanh")
+    assert ((out.cpu().float() - want).abs().mean() / want.abs().mean()).item() < 1e-2
+
+
 def test_moe_fp8_grouped_reference_shape(v, dev):
     """E=128, top_k=8, H=2816, I=704, T=256 (V/tests/test_moe_fp8_grouped.py:16-37): the three routes through
     the kernels agree, and a sample of tokens matches the fp32 per-route loop."""
