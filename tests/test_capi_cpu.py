@@ -74,6 +74,20 @@ def test_schema_matches_reference(qual):
     assert [a.name for a in op._schema.arguments] == REFERENCE_SCHEMAS[qual]
 
 
+def test_extension_module_stand_ins_import():
+    """The patched callers import the reference's compiled extension modules by name for their
+    registration side effect (vllm/patches/vllm_for_multi_arc.patch:8218,
+    sglang/patches/sglang_for_multi_arc.patch:1181, :1414); each stand-in resolves its ops."""
+    import custom_esimd_kernels_vllm.moe_int4_prefill_ops as a
+    import custom_esimd_kernels_vllm.moe_ops as b
+    from custom_esimd_kernels_sglang import moe_fp8_prefill_ops as c
+    from custom_esimd_kernels_sglang import moe_ops as d
+    assert a.moe_prefill_gather_forward_v2 is not None and b.moe_forward_full_v2 is not None
+    assert c.moe_prefill_full_fp8 is not None and d.moe_forward_full_silu_routed_sglang is not None
+    with pytest.raises(AttributeError):
+        d.moe_forward_full_silu_routed_e5m2          # not built: the caller's try / except falls back
+
+
 def test_no_cpu_fallback():
     x = torch.zeros(1, 128, dtype=torch.float16)
     w = torch.zeros(16, 64, dtype=torch.uint8)
