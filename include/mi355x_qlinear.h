@@ -157,9 +157,14 @@ int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int
  *   V/csrc/xpu/q4_0_quant.sycl:30-120).  K % 128 == 0. */
 /* Routed decode GEMVs of a GGUF MoE layer, one launch over all routes r = t * top_k + j:
  *   out[i][r, :] = route_weight[r] * (x[r / x_div, :] @ dequant(W_i[route_expert[r]])^T), i < nmat <= 2,
- * W_i = the per-expert stack [E, N, ...] of the repacked representation the dense GEMVs read
+ * W_i = the per-expert stack [E, N, ...] of the repacked representation
  * (fmt 2 = Q4_K: ql, scale, qmin; 5 = Q5_K: + qh; 6 = Q6_K: ql, qh, scale), fp16, rows of out
  * out_stride elements apart, route_weight (fp16) optional, expert ids clamped into [0, E).
+ * The high bits of the Q5_K / Q6_K stacks are in ELEMENT order, not tile-shuffled as for the
+ * dense GEMVs: Q5_K qh [E,N,K/8], bit b of byte j = fifth bit of element 8j+b; Q6_K qh
+ * [E,N,K/4], 2-bit field p of byte j = top bits of element 4j+p (moe_kquant_GEMV.h:109-116,
+ * 159-166; built by _xpu_repack_q5_k_plain / _q6_k_plain, sglang_for_multi_arc.patch:2736-2765,
+ * here mi_q5k_repack_plain / mi_q6k_repack_plain).  K % 32 == 0 for every format.
  * One kernel launch per matrix.
  * Replaces the launches of esimd_moe_up_q4k (two matrices: gate and up halves of one buffer,
  * x_div = top_k; SiLU * up follows as mi_moe_silu_mul) and esimd_moe_down_q5k / _q6k
@@ -174,6 +179,11 @@ int mi_q8_0_repack(const void* raw, void* qs, void* scale, int N, int K, void* s
 int mi_q5k_repack(const void* raw, void* ql, void* qh, void* scale, void* qmin, int N, int K,
                   void* stream);
 int mi_q6k_repack(const void* raw, void* ql, void* qh, void* scale, int N, int K, void* stream);
+/* The same with qh in element order (the MoE down stacks, see mi_moe_gguf_gemv); K % 256 == 0.
+ * Replace _xpu_repack_q5_k_plain / _xpu_repack_q6_k_plain (sglang_for_multi_arc.patch:2736-2765). */
+int mi_q5k_repack_plain(const void* raw, void* ql, void* qh, void* scale, void* qmin, int N, int K,
+                        void* stream);
+int mi_q6k_repack_plain(const void* raw, void* ql, void* qh, void* scale, int N, int K, void* stream);
 int mi_dequant_q4_0(const void* packed, const void* scale, void* out, int N, int K, void* stream);
 int mi_dequant_q8_0(const void* qs, const void* scale, void* out, int N, int K, void* stream);
 int mi_dequant_q5k(const void* ql, const void* qh, const void* scale, const void* qmin, void* out,

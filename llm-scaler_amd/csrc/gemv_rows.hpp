@@ -24,7 +24,9 @@
 //   Q4_K  : same planting; acc += s * (dot - C1) - min * C2;
 //   Q4_0  : the Q4_K path with min = 8 s (32-wide groups, w = (nib - 8) s);
 //   Q5_K  : Q4_K plus the fifth bit, OR-ed into the planted constant (bit 4 for
-//           even, bit 8 for odd nibbles) from the tile-shuffled qh bytes;
+//           even, bit 8 for odd nibbles) from the tile-shuffled qh bytes (dense GEMV) or
+//           from element-order qh (routed launches: byte j bit b = element 8j + b for
+//           Q5_K, byte j field p = element 4j + p for Q6_K, any K % 32 == 0);
 //   Q6_K  : two high bits OR-ed in the same way, the constant and the zero point
 //           32 removed exactly in 16 bit before the dot product, one scale per 16;
 //   Q8_0  : bytes planted as 0x6400 | (q ^ 0x80) = 1152 + q, 1152 removed exactly
@@ -43,7 +45,7 @@ struct RowsArgs {
   const void* w[kRowsMaxMat];
   const void* s[kRowsMaxMat];
   const void* z[kRowsMaxMat];
-  const void* h[kRowsMaxMat];     // Q5_K / Q6_K high bits (tile-shuffled)
+  const void* h[kRowsMaxMat];     // Q5_K / Q6_K high bits (tile-shuffled; element order in routed launches)
   void* out[kRowsMaxMat];
   int N[kRowsMaxMat];
   int groups[kRowsMaxMat];     // row groups (RW rows each) per matrix
@@ -273,7 +275,20 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
         const uint32_t dead = (uint32_t)(!(live && (row0 + r < N) && (kb < wrow))) << 31;
         b.w[r][sp] = __builtin_amdgcn_raw_buffer_load_b128(
             wr, ((uint32_t)(row0 + r) * wrow + kb) | dead, 0, 2 /* nt */);
-        if constexpr (kHigh) {
+        if constexpr (kHigh && ROUTED) {
+          // element-order high bits: the lane's 32 consecutive k are 4 (Q5_K) or 8 (Q6_K)
+          // consecutive bytes of the row
+          const uint32_t hrow = FMT == RF_Q5K ? ((uint32_t)K >> 3) : ((uint32_t)K >> 2);
+          const uint32_t hb = FMT == RF_Q5K ? kb >> 2 : kb >> 1;
+          const uint32_t ho = ((uint32_t)(row0 + r) * hrow + hb) | dead;
+          b.h[r][sp][1] = u32x4{0u, 0u, 0u, 0u};
+          if constexpr (FMT == RF_Q5K) {
+            b.h[r][sp][0] = u32x4{__builtin_amdgcn_raw_buffer_load_b32(hr, ho, 0, 2), 0u, 0u, 0u};
+          } else {
+            const u32x2 two = __builtin_amdgcn_raw_buffer_load_b64(hr, ho, 0, 2);
+            b.h[r][sp][0] = u32x4{two[0], two[1], 0u, 0u};
+          }
+        } else if constexpr (kHigh) {
           // per 512-k tile the high bits of element b*64 + t (Q5_K, 1 bit) or
           // p*128 + t (Q6_K, 2 bits) sit in byte t: the lane's 32 consecutive k
           // are 32 consecutive bytes, one bit field
@@ -644,7 +659,25 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
                 t2 = ((w[d] >> 8) & 0x000F000Fu) | 0x43004300u;
                 t3 = ((w[d] >> 12) & 0x000F000Fu) | 0x43004300u;
               }
-              if constexpr (kHigh && Act::dt == DT_F16) {
+              if constexpr (kHigh && ROUTED && Act::dt == DT_F16) {
+                if constexpr (FMT == RF_Q5K) {
+                  // byte d of the lane's word: bit e = fifth bit of element 8d + e.  A second copy
+                  // 12 bits up puts bits 4..7 at 16..19, beside the upper halves' nibbles.
+                  const uint32_t hb = (b.h[r][sp][0][0] >> (8 * d)) & 0xFFu;
+                  const uint32_t spv = hb | (hb << 12);
+                  t0 |= (spv << 4) & 0x00100010u;          // elements 0, 4 -> bits 4, 20
+                  t1 |= (spv << 7) & 0x01000100u;          // elements 1, 5 -> bits 8, 24
+                  t2 |= (spv << 2) & 0x00100010u;          // elements 2, 6
+                  t3 |= (spv << 5) & 0x01000100u;          // elements 3, 7
+                } else {
+                  // 16 bits per 8 elements, field e at bits 2e: low byte -> byte 0, high byte -> byte 2
+                  const uint32_t spv = __builtin_amdgcn_perm(0u, b.h[r][sp][0][d >> 1], (d & 1) ? 0x0C030C02u : 0x0C010C00u);
+                  t0 |= (spv << 4) & 0x00300030u;          // fields 0, 4 -> bits 4..5, 20..21
+                  t1 |= (spv << 6) & 0x03000300u;          // fields 1, 5 -> bits 8..9, 24..25
+                  t2 |= spv & 0x00300030u;                 // fields 2, 6
+                  t3 |= (spv << 2) & 0x03000300u;          // fields 3, 7
+                }
+              } else if constexpr (kHigh && Act::dt == DT_F16) {
                 // elements 8d .. 8d+3 have their high bits in bytes of hA, 8d+4 .. 8d+7 in hB;
                 // pair (i, i+4) takes byte i of each, moved to bit 4 (even) / bit 8 (odd nibbles)
                 const uint32_t hA = (b.h[r][sp][d >> 1][(d & 1) * 2] >> hshift) & hmask;

@@ -107,6 +107,21 @@ __global__ __launch_bounds__(256) void q5k_repack_qh_kernel(const uint8_t* __res
   qh[i] = (uint8_t)byte;
 }
 
+// element-order qh (what the MoE down stacks carry): bit b of byte j = fifth bit of element 8j + b
+__global__ __launch_bounds__(256) void q5k_repack_qh_plain_kernel(const uint8_t* __restrict__ raw,
+                                                                  uint8_t* __restrict__ qh, int N, int K) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t total = (size_t)N * (K >> 3);
+  if (i >= total) return;
+  const int per = K >> 3, nsb = K >> 8;
+  const int n = (int)(i / per), j = (int)(i % per);
+  const uint8_t* sb = raw + ((size_t)n * nsb + (j >> 5)) * 176;
+  uint32_t byte = 0;
+#pragma unroll
+  for (int b = 0; b < 8; ++b) byte |= ((q5k_value(sb, ((8 * j) & 255) + b) >> 4) & 1u) << b;
+  qh[i] = (uint8_t)byte;
+}
+
 // scale = fp16(f32(d) * sc6), min = fp16(f32(dmin) * mn6); RAWB = 144 (Q4_K) or 176 (Q5_K)
 __global__ __launch_bounds__(256) void kquant_scale_min_kernel(const uint8_t* __restrict__ raw, int rawb,
                                                                _Float16* __restrict__ scale,
@@ -162,6 +177,21 @@ __global__ __launch_bounds__(256) void q6k_repack_qh_kernel(const uint8_t* __res
     const uint8_t* sb = raw + ((size_t)n * nsb + (e >> 8)) * 210;
     byte |= ((q6k_value(sb, e & 255) >> 4) & 3u) << (2 * p);
   }
+  qh[i] = (uint8_t)byte;
+}
+
+// element-order qh: 2-bit field p of byte j = top bits of element 4j + p
+__global__ __launch_bounds__(256) void q6k_repack_qh_plain_kernel(const uint8_t* __restrict__ raw,
+                                                                  uint8_t* __restrict__ qh, int N, int K) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t total = (size_t)N * (K >> 2);
+  if (i >= total) return;
+  const int per = K >> 2, nsb = K >> 8;
+  const int n = (int)(i / per), j = (int)(i % per);
+  const uint8_t* sb = raw + ((size_t)n * nsb + (j >> 6)) * 210;
+  uint32_t byte = 0;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) byte |= ((q6k_value(sb, ((4 * j) & 255) + p) >> 4) & 3u) << (2 * p);
   qh[i] = (uint8_t)byte;
 }
 
@@ -377,7 +407,7 @@ int mi_moe_gguf_gemv(int fmt, const void* x, int x_div, int nmat, const void* co
   if (fmt != RF_Q4K && fmt != RF_Q5K && fmt != RF_Q6K) return MI_ERR_ARG;
   if (nmat < 1 || nmat > 2 || x_div < 1 || num_experts < 1) return MI_ERR_ARG;
   if (routes < 0 || N < 0 || K <= 0 || out_stride < N) return MI_ERR_SHAPE;
-  if (fmt == RF_Q4K ? (K % 32) : (K % 512)) return MI_ERR_SHAPE;
+  if (K % 32) return MI_ERR_SHAPE;
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || routes > 65535) return MI_ERR_SHAPE;
   if (!routes || !N) return MI_OK;
   const long long nk = (long long)N * K;
@@ -451,6 +481,34 @@ int mi_q6k_repack(const void* raw, void* ql, void* qh, void* scale, int N, int K
                      (uint8_t*)ql, N, K);
   hipLaunchKernelGGL(q6k_repack_qh_kernel, grid_for((size_t)N * (K >> 2)), dim3(256), 0, st, (const uint8_t*)raw,
                      (uint8_t*)qh, N, K);
+  hipLaunchKernelGGL(q6k_scale_kernel, grid_for((size_t)N * (K >> 4)), dim3(256), 0, st, (const uint8_t*)raw,
+                     (_Float16*)scale, N, K);
+  return launch_status();
+}
+
+int mi_q5k_repack_plain(const void* raw, void* ql, void* qh, void* scale, void* qmin, int N, int K, void* stream) {
+  if (!raw || !ql || !qh || !scale || !qmin) return MI_ERR_ARG;
+  if (N < 0 || K <= 0 || (K % 256)) return MI_ERR_SHAPE;
+  if (N == 0) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(q5k_repack_ql_kernel, grid_for((size_t)N * (K >> 1)), dim3(256), 0, st, (const uint8_t*)raw,
+                     (uint8_t*)ql, N, K);
+  hipLaunchKernelGGL(q5k_repack_qh_plain_kernel, grid_for((size_t)N * (K >> 3)), dim3(256), 0, st,
+                     (const uint8_t*)raw, (uint8_t*)qh, N, K);
+  hipLaunchKernelGGL(kquant_scale_min_kernel, grid_for((size_t)N * (K >> 5)), dim3(256), 0, st, (const uint8_t*)raw,
+                     176, (_Float16*)scale, (_Float16*)qmin, N, K);
+  return launch_status();
+}
+
+int mi_q6k_repack_plain(const void* raw, void* ql, void* qh, void* scale, int N, int K, void* stream) {
+  if (!raw || !ql || !qh || !scale) return MI_ERR_ARG;
+  if (N < 0 || K <= 0 || (K % 256)) return MI_ERR_SHAPE;
+  if (N == 0) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(q6k_repack_ql_kernel, grid_for((size_t)N * (K >> 1)), dim3(256), 0, st, (const uint8_t*)raw,
+                     (uint8_t*)ql, N, K);
+  hipLaunchKernelGGL(q6k_repack_qh_plain_kernel, grid_for((size_t)N * (K >> 2)), dim3(256), 0, st,
+                     (const uint8_t*)raw, (uint8_t*)qh, N, K);
   hipLaunchKernelGGL(q6k_scale_kernel, grid_for((size_t)N * (K >> 4)), dim3(256), 0, st, (const uint8_t*)raw,
                      (_Float16*)scale, N, K);
   return launch_status();

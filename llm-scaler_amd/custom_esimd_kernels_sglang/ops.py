@@ -68,6 +68,14 @@ def q6_k_repack(qweight, ql, qh, weight_scale):
     return _ops.q6_k_repack(qweight, ql, qh, weight_scale)
 
 
+def q5_k_repack_plain(qweight, ql, qh, weight_scale, weight_min):
+    return _ops.q5_k_repack_plain(qweight, ql, qh, weight_scale, weight_min)
+
+
+def q6_k_repack_plain(qweight, ql, qh, weight_scale):
+    return _ops.q6_k_repack_plain(qweight, ql, qh, weight_scale)
+
+
 def q4_0_dequant(weight, weight_scale, output):
     return _ops.q4_0_dequant(weight, weight_scale, output)
 

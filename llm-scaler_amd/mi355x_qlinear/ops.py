@@ -457,7 +457,7 @@ def esimd_moe_up_q4k(x, gate_ql, gate_sc, gate_mn, up_ql, up_sc, up_mn, sel, int
 def _moe_down_gguf(fmt, inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k, who):
     T, H, I, k = int(n_tokens), int(hidden), int(intermediate), int(top_k)
     _chk_moe_gguf(inter, sel, T, k, who)
-    _chk(ql.dim() == 3 and I % 512 == 0, f"{who}: ql must be [E, hidden, intermediate/2], intermediate a multiple of 512")
+    _chk(ql.dim() == 3 and I % 32 == 0, f"{who}: ql must be [E, hidden, intermediate/2], intermediate a multiple of 32")
     E = ql.shape[0]
     _chk_stack(ql, torch.uint8, (E, H, I // 2), "ql", who)
     if fmt == 5:
@@ -482,15 +482,17 @@ def _moe_down_gguf(fmt, inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_token
 
 def esimd_moe_down_q5k(inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
     """out_partial[r] = topk_w[r] * (inter[r] @ Wd[sel[r]]^T) on the Q5_K stack ql [E, H, I/2], qh [E, H, I/8]
-    (tile-shuffled fifth bits), scale / min [E, H, I/32] fp16 (S/csrc/xpu/torch_extension.cc:93-97);
+    in ELEMENT order (byte j bit b = fifth bit of element 8j + b; not the tile shuffle of the dense GEMV),
+    scale / min [E, H, I/32] fp16 (S/csrc/xpu/torch_extension.cc:93-97, moe_kquant_GEMV.h:109-157); I % 32 == 0;
     the caller sums each token's top_k rows."""
     return _moe_down_gguf(5, inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k,
                           "esimd_moe_down_q5k")
 
 
 def esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
-    """The same on the Q6_K stack ql [E, H, I/2], qh [E, H, I/4], scale [E, H, I/16] fp16
-    (S/csrc/xpu/torch_extension.cc:98-101)."""
+    """The same on the Q6_K stack ql [E, H, I/2], qh [E, H, I/4] in ELEMENT order (byte j 2-bit field p = top
+    bits of element 4j + p), scale [E, H, I/16] fp16 (S/csrc/xpu/torch_extension.cc:98-101,
+    moe_kquant_GEMV.h:159-209)."""
     return _moe_down_gguf(6, inter, ql, qh, sc, None, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k,
                           "esimd_moe_down_q6k")
 
@@ -566,6 +568,32 @@ def q6_k_repack(qweight, ql, qh, weight_scale):
     _chk_u8(qh, (N, K // 4), "qh", who)
     _chk_f16(weight_scale, N * (K // 16), "weight_scale", who)
     capi.call("mi_q6k_repack", qweight, capi.ptr(qweight), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale), N, K)
+    return ql
+
+
+def q5_k_repack_plain(qweight, ql, qh, weight_scale, weight_min):
+    """Raw GGML q5_K rows -> (ql, element-order qh [N, K/8]: byte j bit b = element 8j + b, scale, min): the
+    representation of the MoE down stacks (sglang_for_multi_arc.patch:2736-2750).  K % 256 == 0."""
+    who = "q5_k_repack_plain"
+    N, K = _raw_rows(qweight, 176, 256, who)
+    _chk_u8(ql, (N, K // 2), "ql", who)
+    _chk_u8(qh, (N, K // 8), "qh", who)
+    _chk_f16(weight_scale, N * (K // 32), "weight_scale", who)
+    _chk_f16(weight_min, N * (K // 32), "weight_min", who)
+    capi.call("mi_q5k_repack_plain", qweight, capi.ptr(qweight), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale),
+              capi.ptr(weight_min), N, K)
+    return ql
+
+
+def q6_k_repack_plain(qweight, ql, qh, weight_scale):
+    """Raw GGML q6_K rows -> (ql, element-order qh [N, K/4]: byte j field p = element 4j + p, scale [N, K/16])
+    (sglang_for_multi_arc.patch:2753-2765).  K % 256 == 0."""
+    who = "q6_k_repack_plain"
+    N, K = _raw_rows(qweight, 210, 256, who)
+    _chk_u8(ql, (N, K // 2), "ql", who)
+    _chk_u8(qh, (N, K // 4), "qh", who)
+    _chk_f16(weight_scale, N * (K // 16), "weight_scale", who)
+    capi.call("mi_q6k_repack_plain", qweight, capi.ptr(qweight), capi.ptr(ql), capi.ptr(qh), capi.ptr(weight_scale), N, K)
     return ql
 
 
@@ -1893,6 +1921,10 @@ def register():
                 "Tensor(d!) weight_min) -> Tensor(a!)", q5_k_repack, _ret(1))
     _define(_S, "q6_k_repack(Tensor qweight, Tensor(a!) ql, Tensor(b!) qh, Tensor(c!) weight_scale) -> Tensor(a!)",
             q6_k_repack, _ret(1))
+    _define(_S, "q5_k_repack_plain(Tensor qweight, Tensor(a!) ql, Tensor(b!) qh, Tensor(c!) weight_scale, "
+                "Tensor(d!) weight_min) -> Tensor(a!)", q5_k_repack_plain, _ret(1))
+    _define(_S, "q6_k_repack_plain(Tensor qweight, Tensor(a!) ql, Tensor(b!) qh, Tensor(c!) weight_scale) -> Tensor(a!)",
+            q6_k_repack_plain, _ret(1))
     _define(_S, "q4_0_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output) -> Tensor(a!)", q4_0_dequant, _ret(2))
     _define(_S, "q8_0_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output) -> Tensor(a!)", q8_0_dequant, _ret(2))
     _define(_S, "q5_k_dequant(Tensor ql, Tensor qh, Tensor weight_scale, Tensor weight_min, Tensor(a!) output) -> Tensor(a!)",

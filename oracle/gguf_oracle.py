@@ -21,6 +21,10 @@ Pinning status:
   * Q4_0, Q8_0, Q5_K, Q6_K repack / dequant: the two routes above, hand-built
     single-block fixtures, all 64x64 (sc6, mn6) encodings for Q5_K (shared with
     Q4_K), every 2-bit / 1-bit high field position of a 512-tile.
+  * Q5_K / Q6_K element-order ("plain") high bits of the MoE down stacks
+    (q5k_repack_plain, q6k_repack_plain + the *_dequant_plain element decodes): against the
+    raw-block walk, against the tile-shuffled route, and hand-built single-element blocks
+    that fix byte and bit position.
   * q4_0_quantize: GGML's published quantize_row_q4_0 rule restated; pinned by
     the reference's known-answer block (7, -7, 3, -3 -> scale -0.875,
     V/tests/test_gemv_int4.py:360-414), by the error envelope the reference's
@@ -261,6 +265,40 @@ def q5k_dequant(ql, qh, scale, minv) -> np.ndarray:
     return (prod - _f16(minv)[:, :, None]).astype(np.float16).reshape(N, K)
 
 
+def q5k_repack_plain(raw: np.ndarray):
+    """SP:2736-2750 (`_xpu_repack_q5_k_plain`), the representation the MoE down kernels read
+    (S/csrc/xpu/esimd_kernels/moe_kquant_GEMV.h:109-116): ql [N, K/2] interleaved nibbles,
+    qh [N, K/8] in ELEMENT order (byte j bit b = element 8j + b), scale / min [N, K/32] fp16.
+    Any K that is a multiple of 256 (the super-block)."""
+    v5, scale, minv = q5k_elem(raw)
+    N, K = v5.shape
+    hbit = ((v5 >> 4) & 1).reshape(N, K // 8, 8)
+    weights = (1 << np.arange(8, dtype=np.int32))
+    qh = (hbit * weights).sum(axis=2).astype(np.uint8)
+    return (pack_nibble_interleaved(v5), np.ascontiguousarray(qh),
+            np.ascontiguousarray(scale), np.ascontiguousarray(minv))
+
+
+def q5k_dequant_plain(ql, qh, scale, minv) -> np.ndarray:
+    """Element decode of the MoE down kernel, moe_kquant_GEMV.h:136-151: per 32-element block the
+    fifth bit of element e is bit e of the little-endian 4-byte qh word; v5 = nibble + 16 bit;
+    w = v5 * scale - min, here with the two fp16 roundings of the dense dequant (SP:2952-2970)
+    so that both representations of one tensor give the same fp16 weights."""
+    N = ql.shape[0]
+    K = ql.shape[1] * 2
+    words = np.ascontiguousarray(qh).view("<u4").reshape(N, K // 32)
+    out = np.empty((N, K), dtype=np.float16)
+    for blk in range(K // 32):
+        w32 = words[:, blk].astype(np.int64)
+        for e in range(32):
+            byte = ql[:, blk * 16 + e // 2].astype(np.int32)
+            nib = (byte >> 4) if (e & 1) else (byte & 0xF)
+            v = nib + (((w32 >> e) & 1) << 4).astype(np.int32)
+            prod = (v.astype(np.float16) * _f16(scale[:, blk])).astype(np.float16)
+            out[:, blk * 32 + e] = (prod - _f16(minv[:, blk])).astype(np.float16)
+    return out
+
+
 def _scale_min_k4(j: int, sc) -> tuple:
     if j < 4:
         return int(sc[j]) & 63, int(sc[j + 4]) & 63
@@ -361,6 +399,39 @@ def q6k_dequant(ql, qh, scale) -> np.ndarray:
     nb = scale.shape[1]
     w = ((v.astype(np.float16).reshape(N, nb, 16) - np.float16(32)) * _f16(scale)[:, :, None]).astype(np.float16)
     return w.reshape(N, K)
+
+
+def q6k_repack_plain(raw: np.ndarray):
+    """SP:2753-2765 (`_xpu_repack_q6_k_plain`), read by moe_kquant_GEMV.h:159-166: ql [N, K/2]
+    interleaved nibbles, qh [N, K/4] in ELEMENT order (byte j 2-bit field p = element 4j + p),
+    scale [N, K/16] fp16."""
+    u6, scale = q6k_elem(raw)
+    N, K = u6.shape
+    h2 = ((u6 >> 4) & 3).reshape(N, K // 4, 4)
+    shifts = 2 * np.arange(4, dtype=np.int32)
+    qh = (h2 << shifts).sum(axis=2).astype(np.uint8)
+    return pack_nibble_interleaved(u6), np.ascontiguousarray(qh), np.ascontiguousarray(scale)
+
+
+def q6k_dequant_plain(ql, qh, scale) -> np.ndarray:
+    """Element decode of moe_kquant_GEMV.h:185-203: per 32-element block two little-endian words,
+    element e of the first 16 = bits [2e, 2e+1] of w0, of the second 16 of w1; v6 = nibble + 16 h;
+    w = (v6 - 32) * scale[k / 16], one fp16 rounding as in the dense dequant (SP:3011-3026)."""
+    N = ql.shape[0]
+    K = ql.shape[1] * 2
+    words = np.ascontiguousarray(qh).view("<u4").reshape(N, K // 16)
+    out = np.empty((N, K), dtype=np.float16)
+    for blk in range(K // 32):
+        for half in range(2):
+            w32 = words[:, 2 * blk + half].astype(np.int64)
+            s16 = _f16(scale[:, 2 * blk + half])
+            for e in range(16):
+                k = blk * 32 + half * 16 + e
+                byte = ql[:, k // 2].astype(np.int32)
+                nib = (byte >> 4) if (k & 1) else (byte & 0xF)
+                v = nib + (((w32 >> (2 * e)) & 3) << 4).astype(np.int32)
+                out[:, k] = ((v.astype(np.float16) - np.float16(32)) * s16).astype(np.float16)
+    return out
 
 
 def q6k_dequant_from_raw(raw: np.ndarray) -> np.ndarray:

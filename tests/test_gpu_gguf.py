@@ -146,7 +146,29 @@ def test_gemv(ops, dev, kind, M, N, K):
     assert O.max_rel_err(out.cpu(), ref) < TOL
 
 
-@pytest.mark.parametrize("T,E,k,H,I", [(1, 8, 4, 2048, 512), (3, 16, 2, 512, 1024), (2, 4, 4, 5120, 512)])
+@pytest.mark.parametrize("kind", ["q5_k", "q6_k"])
+@pytest.mark.parametrize("N,K", [(3, 256), (40, 768), (17, 2048)])
+def test_repack_plain_bit_exact(ops, dev, kind, N, K):
+    # element-order high bits of the MoE down stacks (sglang_for_multi_arc.patch:2736-2765)
+    _, s = ops
+    raw = _raw_case(kind, N, K, seed=3 * N + K)
+    r = _t(raw).to(dev)
+    u8 = lambda *sh: torch.empty(*sh, dtype=torch.uint8, device=dev)
+    f16 = lambda *sh: torch.empty(*sh, dtype=torch.float16, device=dev)
+    if kind == "q5_k":
+        ref = G.q5k_repack_plain(raw)
+        got = (u8(N, K // 2), u8(N, K // 8), f16(N, K // 32), f16(N, K // 32))
+        s.q5_k_repack_plain(r, *got)
+    else:
+        ref = G.q6k_repack_plain(raw)
+        got = (u8(N, K // 2), u8(N, K // 4), f16(N, K // 16))
+        s.q6_k_repack_plain(r, *got)
+    for g_, r_ in zip(got, ref):
+        assert _same(g_, r_)
+
+
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 8, 4, 2048, 512), (3, 16, 2, 512, 1024), (2, 4, 4, 5120, 512),
+                                       (1, 128, 8, 2048, 768), (5, 6, 3, 512, 96), (2, 8, 2, 256, 2080)])
 def test_moe_gguf_routed_stages(ops, dev, T, E, k, H, I):
     """esimd_moe_up_q4k -> esimd_moe_down_q5k / _q6k (S/csrc/xpu/torch_extension.cc:86-101): per-route
     GEMVs on expert stacks of the repacked representations, against the per-route loop on the oracle's
@@ -157,19 +179,24 @@ def test_moe_gguf_routed_stages(ops, dev, T, E, k, H, I):
     x = (torch.randn(T, H, generator=g) * 0.1).half()   # keeps silu(gate) * up inside fp16 range
     sel = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).reshape(-1)
     P = T * k
-    stack = lambda a: _t(a).reshape(E, -1, a.shape[-1]).to(dev)
+    # Large expert counts: U distinct experts are generated and decoded on the CPU, and the
+    # device stack of E experts repeats them through a scrambled map (expert e holds distinct
+    # expert (7e + 3) % U), so the operands keep their full [E, ...] shape.
+    U = min(E, 16)
+    emap = (7 * torch.arange(E) + 3) % U if U < E else torch.arange(E)
+    stack = lambda a: _t(a).reshape(U, -1, a.shape[-1]).to(dev)[emap.to(dev)].contiguous()
     # gate / up: Q4_K stacks [E, I, ...]
     reps, deq = [], []
     for seed in (11, 12):
-        _, raw = O.make_q4k_case(1, H, E * I, seed=seed + H)
+        _, raw = O.make_q4k_case(1, H, U * I, seed=seed + H)
         rep = O.q4k_repack(raw)
         reps.append([stack(a) for a in rep])
-        deq.append(torch.from_numpy(O.q4k_dequant(*rep).astype(np.float32)).reshape(E, I, H))
+        deq.append(torch.from_numpy(O.q4k_dequant(*rep).astype(np.float32)).reshape(U, I, H))
     inter = torch.empty(P, I, dtype=torch.float16, device=dev)
     ret = s.esimd_moe_up_q4k(x.to(dev), *reps[0], *reps[1], sel.to(dev), inter, T, H, I, k)
     assert ret.data_ptr() == inter.data_ptr()
     tok = torch.arange(P) // k
-    e_of = sel.long()
+    e_of = emap[sel.long()]
     gate = torch.einsum("ph,pih->pi", x.float()[tok], deq[0][e_of])
     up = torch.einsum("ph,pih->pi", x.float()[tok], deq[1][e_of])
     want = torch.nn.functional.silu(gate.half().float()) * up.half().float()
@@ -180,9 +207,17 @@ def test_moe_gguf_routed_stages(ops, dev, T, E, k, H, I):
     tw = torch.rand(P, generator=g).half()
     inter = (torch.randn(P, I, generator=g) * 0.1).half().to(dev)
     for kind in ("q5_k", "q6_k"):
-        raw = _raw_case(kind, E * H, I, seed=31 + I)
-        rep = _repack_oracle(kind, raw)
-        wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32)).reshape(E, H, I)
+        # element-order ("plain") high bits: the representation the reference's down kernels
+        # read and the patched loader passes (moe_kquant_GEMV.h:109-116, 159-166)
+        Ip = (I + 255) // 256 * 256                       # raw super-blocks hold 256 elements
+        raw = _raw_case(kind, U * H, Ip, seed=31 + I)
+        full = G.q5k_repack_plain(raw) if kind == "q5_k" else G.q6k_repack_plain(raw)
+        if Ip != I:                                       # K % 32 == 0: cut every row to its first I elements
+            per = (2, 8, 32, 32) if kind == "q5_k" else (2, 4, 16)
+            full = tuple(np.ascontiguousarray(a[:, :I // d]) for a, d in zip(full, per))
+        rep = full
+        deq = G.q5k_dequant_plain(*rep) if kind == "q5_k" else G.q6k_dequant_plain(*rep)
+        wd = torch.from_numpy(deq.astype(np.float32)).reshape(U, H, I)
         out = torch.empty(P, H, dtype=torch.float16, device=dev)
         args = [stack(a) for a in rep]
         fn = s.esimd_moe_down_q5k if kind == "q5_k" else s.esimd_moe_down_q6k

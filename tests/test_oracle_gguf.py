@@ -170,6 +170,56 @@ def test_q6k_single_element():
         assert np.array_equal(w, exp)
 
 
+# ---------------------------------- element-order high bits (MoE down stacks) ----
+@pytest.mark.parametrize("K", [768, 1024, 256])
+def test_plain_high_bits_routes_agree(K):
+    # the element-order representation, decoded the way the MoE down kernels index it, equals
+    # the raw-block walk and the tile-shuffled route; K = 768 and 256 are not whole 512-tiles
+    rng = _rng(5 + K)
+    N = 3
+    v5, _, _, raw5, _, _ = _q5k_case(rng, N, K)
+    ql, qh, s, m = G.q5k_repack_plain(raw5)
+    assert ql.shape == (N, K // 2) and qh.shape == (N, K // 8) and s.shape == m.shape == (N, K // 32)
+    w = G.q5k_dequant_plain(ql, qh, s, m)
+    assert np.array_equal(w.view(np.uint16), G.q5k_dequant_from_raw(raw5).view(np.uint16))
+    nsb = K // 256
+    v6 = rng.integers(0, 64, size=(N, K))
+    raw6 = G.q6k_build_raw(v6, rng.integers(-128, 128, size=(N, nsb, 16)).astype(np.int8), _f16u(rng, (N, nsb), 0.0005, 0.005))
+    ql6, qh6, s6 = G.q6k_repack_plain(raw6)
+    assert ql6.shape == (N, K // 2) and qh6.shape == (N, K // 4) and s6.shape == (N, K // 16)
+    w6 = G.q6k_dequant_plain(ql6, qh6, s6)
+    assert np.array_equal(w6.view(np.uint16), G.q6k_dequant_from_raw(raw6).view(np.uint16))
+    if K % 512 == 0:
+        # same nibbles, scales and decoded weights as the tile-shuffled representation
+        t5 = G.q5k_repack(raw5)
+        assert np.array_equal(t5[0], ql) and np.array_equal(t5[2], s) and np.array_equal(t5[3], m)
+        assert np.array_equal(G.q5k_dequant(*t5).view(np.uint16), w.view(np.uint16))
+        t6 = G.q6k_repack(raw6)
+        assert np.array_equal(t6[0], ql6) and np.array_equal(t6[2], s6)
+        assert np.array_equal(G.q6k_dequant(*t6).view(np.uint16), w6.view(np.uint16))
+
+
+def test_plain_high_bits_positions():
+    # one element with high bits set: Q5_K byte e // 8 bit e % 8; Q6_K byte e // 4 field e % 4
+    N, K = 1, 768
+    for e in (0, 7, 8, 33, 255, 256 + 77, 511, 512 + 130, 767):
+        v5 = np.zeros((N, K), dtype=np.int64)
+        v5[0, e] = 16
+        raw = G.q5k_build_raw(v5, np.zeros((N, 3, 12), np.uint8), np.ones((N, 3), np.float16), np.ones((N, 3), np.float16))
+        ql, qh, _, _ = G.q5k_repack_plain(raw)
+        assert qh[0, e // 8] == (1 << (e % 8)) and qh.astype(np.int64).sum() == (1 << (e % 8)) and ql.sum() == 0
+        v6 = np.zeros((N, K), dtype=np.int64)
+        v6[0, e] = 0b100000 | 0b0101          # high field 2, nibble 5
+        raw = G.q6k_build_raw(v6, np.ones((N, 3, 16), np.int8), np.ones((N, 3), np.float16))
+        ql, qh, _ = G.q6k_repack_plain(raw)
+        assert qh[0, e // 4] == (2 << (2 * (e % 4))) and qh.astype(np.int64).sum() == (2 << (2 * (e % 4)))
+        assert ql[0, e // 2] == (5 << 4 if e & 1 else 5) and ql.astype(np.int64).sum() == ql[0, e // 2]
+        w = G.q6k_dequant_plain(ql, qh, np.ones((N, K // 16), np.float16))
+        exp = np.full((N, K), -32.0, dtype=np.float16)
+        exp[0, e] = 37.0 - 32.0
+        assert np.array_equal(w, exp)
+
+
 # ------------------------------------------------------- Q4_0 quantizer ----
 def test_q4_0_quantize_known_answer():
     # V/tests/test_gemv_int4.py:360-414: 7, -7, 3, -3 in an otherwise zero block -> scale -0.875
