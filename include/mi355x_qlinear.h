@@ -15,7 +15,8 @@
  *   - act_dtype: 0 = fp16, 1 = bf16 (inputs and outputs share it);
  *   - return value: 0 on success, MI_ERR_ARG (-1) for a null pointer or bad
  *     enum, MI_ERR_SHAPE (-2) for a shape the kernels do not cover,
- *     MI_ERR_LAUNCH (-3) if the launch itself failed.
+ *     MI_ERR_LAUNCH (-3) if the launch itself failed, MI_ERR_LIMIT (-4) for a size
+ *     beyond the fixed capacity of an entry point that allocates nothing.
  */
 #ifndef MI355X_QLINEAR_H_
 #define MI355X_QLINEAR_H_
@@ -320,6 +321,22 @@ int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* no
  * (unrounded into the norm, as the reference does): replaces esimd_scaled_resadd_norm_gemv_fp8_pert
  * (V/csrc/xpu/torch_extension.cc:163-166, esimd_kernels/scaled_resadd_norm_gemv_fp8.h:70-100). */
 int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const void* norm_weight,
+                        void* normed_out, int norm_len, float eps, float residual_scale, int fmt, int nmat,
+                        const void* const* w, const void* const* scale, void* const* out, const int* N, int K,
+                        int act_dtype, void* stream);
+/* mi_norm_gemv_scaled for callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+ * arguments and results; the arrival counters live in a 2 KiB static device array inside the
+ * library (one copy per GPU, held until the process ends) instead of a per-stream hipMalloc,
+ * and the call allocates and frees nothing.  Only the fused single launch is covered: rows
+ * beyond its limit (K > 16384, or K whose staged row exceeds 64 KiB of LDS) return
+ * MI_ERR_LIMIT (-4) instead of taking the two-kernel route.  All calls on one GPU share the
+ * counters: the kernel leaves them at zero when it ends, so back-to-back calls on one stream
+ * are fine, while calls that overlap on one GPU (different streams) race.
+ * mi_static_scratch_setup resolves the array's address on the current device (the first call
+ * of mi_norm_gemv_static on a device does the same); call it once per device before capturing. */
+int mi_static_scratch_setup(void);
+int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const void* norm_weight,
                         void* normed_out, int norm_len, float eps, float residual_scale, int fmt, int nmat,
                         const void* const* w, const void* const* scale, void* const* out, const int* N, int K,
                         int act_dtype, void* stream);

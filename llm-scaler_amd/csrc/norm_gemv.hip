@@ -11,9 +11,66 @@
 #include "scratch.hpp"
 #include "../../include/mi355x_qlinear.h"
 
+#include <mutex>
+
 using namespace qlin;
 
+// ---- arrival counters that live in the library image ---------------------------
+// mi_norm_gemv_static counts arriving workgroups in this array instead of a buffer
+// from hipMalloc.  Every GPU the library runs on holds its own copy at its own
+// address; host code never uses the name below as an address, only the per-device
+// pointer that hipGetSymbolAddress returns.  The loader zero-fills it and the kernel
+// leaves every counter at zero when it ends, so one call finds what the previous one
+// left: zeros.  Calls that overlap on one GPU (two streams) would share the counters
+// and race; calls on one stream are ordered by the stream.
+constexpr int kStaticCounterWords = 512;                       // 2 KiB, the size the kernel indexes into
+static __device__ __align__(256) unsigned int scratch[kStaticCounterWords];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mu;
+unsigned int* g_static_ptr[kMaxDevices];                       // per device, resolved once
+
+// MI_OK and *out = the current device's copy of `scratch`
+int static_counters(unsigned int** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
+    g_static_ptr[dev] = static_cast<unsigned int*>(p);
+  }
+  *out = g_static_ptr[dev];
+  return MI_OK;
+}
+
+// Shared body.  counters == nullptr: take the per-stream counters (allocated on first use) and
+// fall back to two kernels for rows the fused staging cannot hold; otherwise use `counters` and
+// refuse those rows.
+int norm_gemv_run(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
+                  int norm_len, float eps, float residual_scale, int fmt, int nmat, const void* const* w,
+                  const void* const* scale, void* const* out, const int* N, int K, int act_dtype, void* stream,
+                  unsigned int* counters);
+}  // namespace
+
 extern "C" {
+
+int mi_static_scratch_setup(void) {
+  unsigned int* p = nullptr;
+  return static_counters(&p);
+}
+
+int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
+                        int norm_len, float eps, float residual_scale, int fmt, int nmat, const void* const* w,
+                        const void* const* scale, void* const* out, const int* N, int K, int act_dtype,
+                        void* stream) {
+  unsigned int* counters = nullptr;
+  const int rc = static_counters(&counters);
+  if (rc != MI_OK) return rc;
+  return norm_gemv_run(x, residual, gate, norm_weight, normed_out, norm_len, eps, residual_scale, fmt, nmat, w, scale,
+                       out, N, K, act_dtype, stream, counters);
+}
 
 int mi_norm_gemv(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
                  int norm_len, float eps, int fmt, int nmat, const void* const* w, const void* const* scale,
@@ -26,6 +83,18 @@ int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const v
                         int norm_len, float eps, float residual_scale, int fmt, int nmat, const void* const* w,
                         const void* const* scale, void* const* out, const int* N, int K, int act_dtype,
                         void* stream) {
+  return norm_gemv_run(x, residual, gate, norm_weight, normed_out, norm_len, eps, residual_scale, fmt, nmat, w, scale,
+                       out, N, K, act_dtype, stream, nullptr);
+}
+
+}  // extern "C"
+
+namespace {
+
+int norm_gemv_run(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
+                  int norm_len, float eps, float residual_scale, int fmt, int nmat, const void* const* w,
+                  const void* const* scale, void* const* out, const int* N, int K, int act_dtype, void* stream,
+                  unsigned int* counters) {
   if (!x || !norm_weight || !w || !scale || !out || !N) return MI_ERR_ARG;
   if (nmat < 1 || nmat > kRowsMaxMat) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
@@ -42,6 +111,7 @@ int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const v
   }
   const int rfmt = fmt == 2 ? RF_INT4 : RF_FP8;
   const bool fused = K <= kRowsNormMaxK && rows_lds_bytes(rfmt, 1, K) + rows_norm_lds_bytes(K) <= 64 * 1024;
+  if (!fused && counters) return MI_ERR_LIMIT;          // the no-allocation entry covers the fused launch only
   if (!fused) {
     // two kernels: the norm writes the row (into normed_out, or over x's scratch copy), then the GEMV
     if (!normed_out) return MI_ERR_ARG;
@@ -55,7 +125,7 @@ int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const v
   }
   r.n_res = residual; r.n_gate = gate; r.n_weight = norm_weight; r.n_out = normed_out;
   r.n_len = norm_len; r.n_eps = eps; r.n_rscale = residual_scale;
-  r.n_arrive = arrival_counter_get(st);
+  r.n_arrive = counters ? counters : arrival_counter_get(st);
   if (!r.n_arrive) return MI_ERR_LAUNCH;
   const bool f16 = act_dtype == DT_F16;
   if (fmt == 0) {
@@ -68,4 +138,4 @@ int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const v
   return launch_status();
 }
 
-}  // extern "C"
+}  // namespace

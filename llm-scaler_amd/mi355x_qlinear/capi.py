@@ -19,7 +19,8 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libmi355x_qlinear.so")
 
 MI_ERRORS = {-1: "invalid argument (null pointer or bad enum)",
              -2: "unsupported shape or divisibility",
-             -3: "kernel launch failed"}
+             -3: "kernel launch failed",
+             -4: "size beyond the fixed capacity of this no-allocation entry point"}
 
 DT_F16, DT_BF16 = 0, 1
 _ACT_DT = {torch.float16: DT_F16, torch.bfloat16: DT_BF16}
@@ -36,6 +37,8 @@ def parse_header(path: str = HEADER):
         types = []
         for p in params.split(","):
             p = " ".join(p.split())
+            if p == "void":                       # f(void): no parameters
+                continue
             if "*" in p:
                 types.append(ctypes.c_void_p)
             elif p.startswith("long long") or p.startswith("int64_t"):
