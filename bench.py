@@ -1,21 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--all]
 
 A step is one launch of the hot-path op on one batch of seeded synthetic input.
 The headline workload (default) is the second benchmark configuration: FP8 per-channel
 weight-only GEMV, M=1, K=4096, N=14336, bf16 activations.  Each step uses the
 next of R distinct weight copies (R x weight bytes >> the 256 MB Infinity Cache)
 so the figure is HBM bandwidth, not cache bandwidth.  The K timed steps are
-issued back to back on one stream as replays of a HIP graph holding R launches,
-bracketed by a device synchronise on both sides; HIP events recorded on that same
-stream give the average per-launch duration used for the roofline fraction.
+exactly K launches, all of them nodes of HIP graphs replayed back to back on one
+stream and bracketed by a device synchronise on both sides; HIP events recorded
+on that same stream give the average per-launch duration used for the roofline
+fraction.
 
 Prints ONE JSON line.  `value` is the algorithmic bytes moved per second with
-inputs resident in HBM.  `cpu_baseline` times the reference's CPU path (torch
-dequant + fp32 matmul, restated in oracle/) on this host's cores on a bounded
-sample.
+inputs resident in HBM.  `cases` holds the other benchmark configurations (W4A16
+GEMV, FP8 GEMV at M = 8 / 32, W4A16 prefill GEMM, block-FP8 MoE forward, Q4_K at
+M = 1 / 64), each timed the same way with its own `roofline` and `cpu_baseline`;
+`--only` leaves them out, `--all` adds the workloads beyond the configurations.
+`cpu_baseline` times the reference's CPU path (torch dequant + fp32 matmul,
+restated in oracle/) on this host's cores on a bounded sample.
 """
 from __future__ import annotations
 
@@ -39,6 +43,9 @@ CACHE_BUST_BYTES = 1 << 30       # rotate over >= 1 GiB of distinct weights (4 x
 # ----------------------------------------------------------------------------
 # workloads: each returns (launch(i), alg_bytes, alg_flops, bound, dtype, descr, cpu_fn)
 # ----------------------------------------------------------------------------
+_CACHE = {}
+
+
 def _copies(nbytes: int) -> int:
     return max(2, -(-CACHE_BUST_BYTES // nbytes))
 
@@ -47,13 +54,16 @@ def wl_fp8_pern(M: int, dev):
     import custom_esimd_kernels_vllm as v
     from oracle import qlinear_oracle as O
     K, N = 4096, 14336
-    x, w8, s = O.make_fp8_pern_case(M, K, N)
     R = _copies(N * K)
-    g = torch.Generator().manual_seed(99)
-    ws = [w8.to(dev)]
-    for _ in range(R - 1):          # distinct contents per copy, same distribution (row permutation)
-        ws.append(w8[torch.randperm(N, generator=g)].to(dev))
-    ws = [w.view(torch.float8_e4m3fn) for w in ws]
+    if "fp8_pern" not in _CACHE:    # the three M of this configuration share the weights
+        _, w8, s = O.make_fp8_pern_case(1, K, N)
+        g = torch.Generator().manual_seed(99)
+        ws = [w8.to(dev)]
+        for _ in range(R - 1):      # distinct contents per copy, same distribution (row permutation)
+            ws.append(w8[torch.randperm(N, generator=g)].to(dev))
+        _CACHE["fp8_pern"] = (w8, s, [w.view(torch.float8_e4m3fn) for w in ws])
+    w8, s, ws = _CACHE["fp8_pern"]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(1235)).to(torch.bfloat16)
     xd, sd = x.to(dev), s.to(dev)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
 
@@ -116,13 +126,16 @@ def wl_q4k(M: int, dev):
         a, b, c = W[i % R]
         s.esimd_gemv_q4_k(xd, a, b, c, out)
 
+    n_cpu = N                                     # weight rows of the CPU sample (all of them)
+
     def cpu():
-        return O.matmul_ref(x, torch.from_numpy(O.q4k_dequant(ql, sc, mn))).to(torch.float16)
+        return O.matmul_ref(x, torch.from_numpy(O.q4k_dequant(ql[:n_cpu], sc[:n_cpu], mn[:n_cpu]))).to(torch.float16)
 
     alg_bytes = per + 2 * M * K + 2 * M * N
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="f16",
                 name=f"cfg4 GGUF Q4_K (repacked) dequant-matmul M={M} K={K} N={N} fp16",
-                kernel="gemv_rows_kernel" if M <= 4 else "skinny_kernel", cpu=cpu)
+                kernel="gemv_rows_kernel" if M <= 4 else "skinny_kernel", cpu=cpu, cpu_scale=n_cpu / N,
+                cpu_what=f"{n_cpu} of the {N} weight rows")
 
 
 def wl_gguf(kind: str, M: int, dev):
@@ -268,13 +281,12 @@ def wl_gemm_w4a16(dev):
         v.esimd_gemm_int4_pgrp_zp(xd, wd, sd, zd, out)
 
     def cpu():
-        # bounded sample: 256 of the 2048 rows (the dequant of the whole weight is in every pass)
-        return O.matmul_ref(x[:256], O.int4_dequant(packed, scale, out_dtype=torch.bfloat16, zp=zp)).to(torch.bfloat16)
+        return O.matmul_ref(x, O.int4_dequant(packed, scale, out_dtype=torch.bfloat16, zp=zp)).to(torch.bfloat16)
 
     alg_bytes = N * K // 2 + N * (K // 128) * 3 + 2 * M * K + 2 * M * N
     return dict(launch=launch, R=1, bytes=alg_bytes, flops=2 * M * N * K, bound="mfma", dtype="bf16",
                 name=f"cfg2 W4A16 asymmetric group-128 prefill GEMM M={M} K={K} N={N} bf16",
-                kernel="gemm_w4a16_kernel", cpu=cpu, cpu_scale=256 / M)
+                kernel="gemm_w4a16_kernel", cpu=cpu)
 
 
 def wl_copy(dev):
@@ -309,9 +321,12 @@ def wl_moe(dev):
         a, b, c, d = W[i % R]
         v.moe_forward_fp8_block(xd, ld, a, b, c, d, out, K, True)
 
+    e_cpu, t_cpu = 64, 256                        # CPU sample: half of the experts and of the tokens, 32 rows per expert as in the whole
+
     def cpu():
-        tw, ti = O.moe_topk(logits, K)
-        return O.moe_forward_grouped(x, tw, ti, w13q, w13s, w2q, w2s, E, act_quant=True).to(torch.bfloat16)
+        tw, ti = O.moe_topk(logits[:t_cpu, :e_cpu], K)
+        return O.moe_forward_grouped(x[:t_cpu], tw, ti, w13q[:e_cpu], w13s[:e_cpu], w2q[:e_cpu], w2s[:e_cpu], e_cpu,
+                                     act_quant=True).to(torch.bfloat16)
 
     P = T * K
     # algorithmic bytes: every expert's weights + block scales once, x and logits in, output out
@@ -320,7 +335,8 @@ def wl_moe(dev):
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=flops, bound="hbm", dtype="fp8",
                 name=f"cfg3 FP8 128x128-block MoE forward (topk+sort+quant+gate_up/SiLU+quant+down+combine) "
                      f"T={T} E={E} top{K} H={H} I={I} bf16, fp8 activations",
-                kernel="moe_gemm_kernel", cpu=cpu)
+                kernel="moe_gemm_kernel", cpu=cpu, cpu_scale=e_cpu / E,
+                cpu_what=f"{e_cpu} of the {E} experts and {t_cpu} of the {T} tokens (32 rows per expert, as in the whole)")
 
 
 def wl_moe_gelu(dev):
@@ -458,13 +474,19 @@ WORKLOADS = {
     "next_moe_gguf_t1": wl_moe_gguf,
 }
 HEADLINE = "cfg1_m1"
+# the other benchmark configurations: reported as `cases` of the default run
+BASELINE_CASES = ["cfg0", "cfg1_m8", "cfg1_m32", "cfg2", "cfg3", "cfg4_m1", "cfg4_m64"]
+CASE_MIN_STEPS = 200             # a case is timed over at least this many launches
 
 
 # ----------------------------------------------------------------------------
 def run_gpu(wl, steps: int, warmup: int):
-    """-> (wall seconds for `steps` launches, event ms for the same region)"""
+    """Times exactly `steps` launches, every one a node of a replayed HIP graph.
+    -> (wall seconds for the timed region, event ms for the same region)"""
     R = wl["R"]
     launch = wl["launch"]
+    G = min(steps, max(R, 128))                 # launches per graph
+    reps, rem = divmod(steps, G)
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for i in range(max(warmup, 1)):
@@ -472,10 +494,17 @@ def run_gpu(wl, steps: int, warmup: int):
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            for i in range(R):
+            for i in range(G):
                 launch(i)
-        reps, rem = divmod(steps, R)
-        graph.replay()                      # one untimed replay: graph upload
+        tail = None
+        if rem:
+            tail = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(tail, stream=stream):
+                for i in range(rem):
+                    launch(G + i)
+        graph.replay()                      # untimed replays: graph upload
+        if tail is not None:
+            tail.replay()
         stream.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
@@ -484,8 +513,8 @@ def run_gpu(wl, steps: int, warmup: int):
         e0.record(stream)
         for _ in range(reps):
             graph.replay()
-        for i in range(rem):
-            launch(i)
+        if tail is not None:
+            tail.replay()
         e1.record(stream)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
@@ -501,7 +530,7 @@ def measured_traffic(workload_id):
         return None
 
 
-def summarize(wl, steps, wall_s, ev_ms):
+def summarize(wl, wid, steps, warmup, wall_s, ev_ms):
     per_launch_s = ev_ms * 1e-3 / steps
     if wl["bound"] == "hbm":
         achieved = wl["bytes"] / per_launch_s / 1e9
@@ -510,26 +539,34 @@ def summarize(wl, steps, wall_s, ev_ms):
         achieved = wl["flops"] / per_launch_s / 1e12
         peak, unit = MFMA_PEAK_TFLOPS[wl["dtype"]], "TFLOP/s"
     return {
+        "id": wid,
         "workload": wl["name"],
+        "dtype": wl["dtype"],
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": wall_s * 1e3 / steps,
         "us_per_launch_events": per_launch_s * 1e6,
         "GBps": wl["bytes"] / per_launch_s / 1e9,
         "TFLOPs": wl["flops"] / per_launch_s / 1e12,
         "roofline": {"bound": wl["bound"], "achieved": achieved, "peak": peak, "unit": unit,
-                     "frac": achieved / peak, "traffic": None, "kernel": wl["kernel"],
+                     "frac": achieved / peak, "traffic": measured_traffic(wid), "kernel": wl["kernel"],
                      "alg_bytes_per_launch": wl["bytes"], "alg_flops_per_launch": wl["flops"]},
     }
 
 
 def cpu_baseline(wl, budget_s: float = 20.0):
-    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    """The oracle's torch dequant + fp32 matmul on this host's cores, on a bounded sample."""
+    host = os.cpu_count() or 1
+    # the GPU box exports OMP_NUM_THREADS = its CPU share for one GPU; never more threads than that
+    torch.set_num_threads(min(host, int(os.environ.get("OMP_NUM_THREADS", "16"))))
     cores = torch.get_num_threads()
     times = []
     t_start = time.perf_counter()
     n = 0
     while True:
         t0 = time.perf_counter()
-        wl["cpu"]()
+        if wl["cpu"]() is None:                     # this workload has no CPU leg
+            return None
         dt = time.perf_counter() - t0
         n += 1
         if n > 2:
@@ -543,11 +580,21 @@ def cpu_baseline(wl, budget_s: float = 20.0):
         value, unit = wl["bytes"] * frac / med / 1e9, "GB/s"
     else:
         value, unit = wl["flops"] * frac / med / 1e12, "TFLOP/s"
-    what = "the full workload" if frac == 1.0 else f"{frac:.3f} of the workload's rows"
-    return {"value": value, "unit": unit, "cores": cores, "kind": "port",
+    what = "the full workload" if frac == 1.0 else wl.get("cpu_what", f"{frac:.3f} of the workload")
+    return {"value": value, "unit": unit, "cores": cores, "host_cpu_count": host, "kind": "port",
             "seconds_per_pass": med,
             "sample": f"{len(times)} timed passes (after 2 warm-ups) over {what}: torch dequant of the "
-                      f"whole weight + fp32 matmul, {wl['name']}"}
+                      f"sampled weight + fp32 matmul, {wl['name']}"}
+
+
+def run_case(wid, dev, steps, warmup, with_cpu, cpu_budget_s):
+    wl = WORKLOADS[wid](dev)
+    wall, ev = run_gpu(wl, steps, warmup)
+    c = summarize(wl, wid, steps, warmup, wall, ev)
+    c["cpu_baseline"] = cpu_baseline(wl, cpu_budget_s) if with_cpu else None
+    del wl
+    torch.cuda.empty_cache()
+    return c
 
 
 def main():
@@ -556,8 +603,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
-    ap.add_argument("--all", action="store_true", help="also time the other single-GPU workloads")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", action="store_true", help="time --workload alone (no `cases`)")
+    ap.add_argument("--all", action="store_true", help="also time the workloads beyond the benchmark configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path has no multi-GPU leg "
@@ -569,26 +617,18 @@ def main():
     import mi355x_qlinear  # noqa: F401  (raises if the HIP library is not built)
     dev = torch.device("cuda:0")
 
-    wl = WORKLOADS[args.workload](dev)
-    wall, ev = run_gpu(wl, args.steps, args.warmup)
-    head = summarize(wl, args.steps, wall, ev)
-    head["roofline"]["traffic"] = measured_traffic(args.workload)
-    cpu = None if args.no_cpu else cpu_baseline(wl)
-    del wl
-    torch.cuda.empty_cache()
+    head = run_case(args.workload, dev, args.steps, args.warmup, not args.no_cpu, 10.0)
 
     cases = []
-    if args.all:
-        for name in sorted(WORKLOADS):
-            if name == args.workload:
-                continue
-            w = WORKLOADS[name](dev)
-            wa, e = run_gpu(w, args.steps, args.warmup)
-            c = summarize(w, args.steps, wa, e)
-            c["id"] = name
-            cases.append(c)
-            del w
-            torch.cuda.empty_cache()
+    if not args.only:
+        ids = [w for w in BASELINE_CASES if w != args.workload]
+        if args.workload != HEADLINE:
+            ids.insert(0, HEADLINE)
+        if args.all:
+            ids += [w for w in sorted(WORKLOADS) if w not in ids and w != args.workload and w != "copy"]
+        for wid in ids:
+            cases.append(run_case(wid, dev, max(args.steps, CASE_MIN_STEPS), max(args.warmup, 20),
+                                  not args.no_cpu and wid in BASELINE_CASES + [HEADLINE], 5.0))
 
     line = {
         "metric": "HBM GB/s (GEMV) and TFLOP/s (GEMM) as % of MI355X roofline, 1 GPU",
@@ -601,12 +641,12 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": head["dtype"],
         "data": "synthetic (seeded; weights rotate over >=1 GiB of distinct copies)",
         "config": {"workload": head["workload"], "id": args.workload,
-                   "timing": "HIP-graph replays of back-to-back launches on one stream"},
+                   "timing": "exactly `steps` launches, all HIP-graph nodes replayed back to back on one stream"},
         "roofline": head["roofline"],
-        "cpu_baseline": cpu,
+        "cpu_baseline": head["cpu_baseline"],
     }
     if cases:
         line["cases"] = cases
