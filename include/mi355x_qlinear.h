@@ -306,9 +306,10 @@ int mi_norm_add_norm(const void* src, int rows_per_token, void* h1, const void* 
  *   block scale, 2 = INT4 group 128 (scale[i] fp16 [N, K/128]).  residual (in place),
  *   gate and normed_out may be null.  Every workgroup normalises its own copy of the
  *   row; the in-place residual and normed_out are written by the workgroup that
- *   arrives last at a per-stream device counter (2 KiB, allocated and zeroed by the
- *   first call on a device and stream: not while that stream is being captured), after
- *   all others have read their inputs.  Rows longer than 16384 fall back to mi_rmsnorm + the GEMV (normed_out
+ *   arrives last at a per-stream device counter (2 KiB, from a pool of 64 blocks that the
+ *   first call on a device allocates and zeroes: that one call must not run under stream
+ *   capture; later streams take a block without allocating), after all others have read
+ *   their inputs.  Rows longer than 16384 fall back to mi_rmsnorm + the GEMV (normed_out
  *   is then required).  Replaces the launch of esimd_resadd_norm_gemv_{int4,fp8}_pert,
  *   esimd_resadd_norm_gemv2_fp8_pert, esimd_norm_gemv_{int4,fp8}_pert and
  *   esimd_norm_gemv_fp8_blockscale (V/csrc/xpu/torch_extension.cc:103-133,

@@ -102,7 +102,12 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
 // ---------------------------------------------------------------- sort
 // Stable counting sort of the flattened (token, route) pairs by expert, in one
 // workgroup, deterministic.  Inside an expert the pairs keep their pair-index
-// order.  Because a token's K experts are distinct, the rank of pair (t, j) in
+// order.  Precondition (what a top-k selection produces): a token's K expert ids
+// are distinct and lie in [0, E).  Ids outside the range are held into it, and a
+// repeated id within a token makes its pairs share one position; in both cases
+// the token's result is unspecified, but every index written stays valid (the
+// positions no pair claimed hold pair 0 / token 0), so nothing downstream reads
+// out of bounds.  Because a token's K experts are distinct, the rank of pair (t, j) in
 // expert e equals the number of tokens t' < t that selected e: a per-expert
 // bitmap over tokens (built with order-independent LDS atomic ORs) plus popcounts
 // gives the rank without any ordered atomics.
@@ -114,6 +119,12 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
 // then one bitmap pass per chunk of tokens.
 constexpr int kSortThreads = 1024;
 constexpr int kSortWords = 4096;                     // bitmap words in LDS
+
+// Expert id of pair q, held into [0, E): an id outside the range would index the LDS tables out of bounds.
+__device__ __forceinline__ int sort_expert(const int32_t* __restrict__ top_ids, int q, int E) {
+  const int e = top_ids[q];
+  return e < 0 ? 0 : (e >= E ? E - 1 : e);
+}
 
 // inclusive scan of one value per thread over the 1024-thread workgroup
 __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* wave_tot, int tid) {
@@ -165,7 +176,7 @@ __device__ __forceinline__ void moe_sort_body(
 #pragma unroll
     for (int i = 0; i < kCache; ++i) {
       const int q = tid + i * kSortThreads;
-      ecache[i] = q < P ? top_ids[q] : -1;
+      ecache[i] = q < P ? sort_expert(top_ids, q, E) : -1;
     }
     __syncthreads();
 #pragma unroll
@@ -175,7 +186,7 @@ __device__ __forceinline__ void moe_sort_body(
     }
     for (int q = tid + kCache * kSortThreads; q < P; q += kSortThreads) {
       const int tl = q / K;
-      atomicOr(&bitmap[top_ids[q] * wpe + (tl >> 5)], 1u << (tl & 31));
+      atomicOr(&bitmap[sort_expert(top_ids, q, E) * wpe + (tl >> 5)], 1u << (tl & 31));
     }
     __syncthreads();
     uint32_t pc[WPT], tot = 0;
@@ -206,7 +217,12 @@ __device__ __forceinline__ void moe_sort_body(
       const int q = tid + i * kSortThreads;
       if (q < P) place(q, ecache[i]);
     }
-    for (int q = tid + kCache * kSortThreads; q < P; q += kSortThreads) place(q, top_ids[q]);
+    for (int q = tid + kCache * kSortThreads; q < P; q += kSortThreads) place(q, sort_expert(top_ids, q, E));
+    // positions no pair claimed (only with repeated ids inside a token): valid indices
+    for (int pos = (int)wordpre[kSortWords] + tid; pos < P; pos += kSortThreads) {
+      sorted_pairs[pos] = 0;
+      if (sorted_token) sorted_token[pos] = 0;
+    }
     if (max_count) {
       __syncthreads();
       if (tid == 0) max_count[0] = mx;
@@ -216,8 +232,14 @@ __device__ __forceinline__ void moe_sort_body(
 
   // ---- chunked path ----
   if (tid < E) { count[tid] = 0; base[tid] = 0; }
+  // every position starts as a valid index: with repeated ids inside a token some positions of
+  // an expert's range are claimed by no pair (ordered before the placement by the barriers below)
+  for (int pos = tid; pos < P; pos += kSortThreads) {
+    sorted_pairs[pos] = 0;
+    if (sorted_token) sorted_token[pos] = 0;
+  }
   __syncthreads();
-  for (int p = tid; p < P; p += kSortThreads) atomicAdd(&count[top_ids[p]], 1);
+  for (int p = tid; p < P; p += kSortThreads) atomicAdd(&count[sort_expert(top_ids, p, E)], 1);
   __syncthreads();
   // exclusive prefix over experts (Hillis-Steele on up to 1024 entries)
   if (tid < E) start[tid + 1] = count[tid];
@@ -245,7 +267,7 @@ __device__ __forceinline__ void moe_sort_body(
     __syncthreads();
     for (int q = tid; q < tn * K; q += kSortThreads) {
       const int tl = q / K;
-      const int e = top_ids[(size_t)t0 * K + q];
+      const int e = sort_expert(top_ids, t0 * K + q, E);
       atomicOr(&bitmap[e * wpe + (tl >> 5)], 1u << (tl & 31));
     }
     __syncthreads();
@@ -261,7 +283,7 @@ __device__ __forceinline__ void moe_sort_body(
     for (int q = tid; q < tn * K; q += kSortThreads) {
       const int tl = q / K;
       const int p = t0 * K + q;
-      const int e = top_ids[p];
+      const int e = sort_expert(top_ids, p, E);
       const uint32_t word = bitmap[e * wpe + (tl >> 5)];
       const int rank = base[e] + (int)wordpre[e * wpe + (tl >> 5)] +
                        __popc(word & ((1u << (tl & 31)) - 1u));

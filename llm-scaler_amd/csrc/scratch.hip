@@ -32,16 +32,36 @@ void* scratch_get(hipStream_t stream, size_t bytes) {
   return p;
 }
 
+// One pool of counter blocks per device, handed out to streams in order: only the first call on a
+// device allocates (and clears) anything, so a stream first seen while it is being captured still
+// gets its block without an allocation.
+namespace {
+constexpr int kCounterBlockBytes = 2048;
+constexpr int kCounterBlocksPerPool = 64;
+struct CounterPool {
+  unsigned char* base = nullptr;
+  int used = 0;
+};
+std::map<int, CounterPool> g_pools;
+}  // namespace
+
 unsigned int* arrival_counter_get(hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
   std::lock_guard<std::mutex> lock(g_mu);
   unsigned int*& c = g_counters[{dev, stream}];
   if (c) return c;
-  void* p = nullptr;
-  if (hipMalloc(&p, 2048) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-  if (hipMemset(p, 0, 2048) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(p); return nullptr; }
-  c = static_cast<unsigned int*>(p);
+  CounterPool& pool = g_pools[dev];
+  if (!pool.base || pool.used == kCounterBlocksPerPool) {
+    // a fresh pool (the exhausted one stays allocated: its blocks are in use)
+    void* p = nullptr;
+    const size_t bytes = (size_t)kCounterBlockBytes * kCounterBlocksPerPool;
+    if (hipMalloc(&p, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    if (hipMemset(p, 0, bytes) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(p); return nullptr; }
+    pool.base = static_cast<unsigned char*>(p);
+    pool.used = 0;
+  }
+  c = reinterpret_cast<unsigned int*>(pool.base + (size_t)kCounterBlockBytes * pool.used++);
   return c;
 }
 

@@ -21,8 +21,10 @@ namespace qlin {
 void* scratch_get(hipStream_t stream, size_t bytes);
 
 // A zero-initialised block of 512 32-bit counters per (device, stream) for kernels that
-// count arriving workgroups and leave the counters at zero again when they finish.
-// Allocated and cleared on first use (not under stream capture); nullptr on failure.
+// count arriving workgroups and leave the counters at zero again when they finish.  The
+// blocks come from a pool of 64 that the first call on a device allocates and clears (not
+// possible under stream capture); later streams take the next block without allocating.
+// nullptr on failure.
 unsigned int* arrival_counter_get(hipStream_t stream);
 
 }  // namespace qlin

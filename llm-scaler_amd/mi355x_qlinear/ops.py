@@ -34,10 +34,14 @@ def _library(ns: str) -> torch.library.Library:
     return _libs[ns]
 
 
+_DEFINED = {}        # namespace -> names of the operators defined here
+
+
 def _define(ns: str, schema: str, impl, meta=None):
     lib = _library(ns)
     lib.define(schema)
     name = schema.split("(", 1)[0]
+    _DEFINED.setdefault(ns, []).append(name)
     lib.impl(name, impl, "CUDA")
     if meta is not None:
         lib.impl(name, meta, "Meta")
@@ -1931,7 +1935,8 @@ def register():
             q5_k_dequant, _ret(4))
     _define(_S, "q6_k_dequant(Tensor ql, Tensor qh, Tensor weight_scale, Tensor(a!) output) -> Tensor(a!)",
             q6_k_dequant, _ret(3))
-    _define(_V, "q4_0_quantize(Tensor input, Tensor(a!) out_qweight, Tensor(b!) out_scale) -> ()", q4_0_quantize, None)
+    _define(_V, "q4_0_quantize(Tensor input, Tensor(a!) out_qweight, Tensor(b!) out_scale) -> ()", q4_0_quantize,
+            lambda *a: None)
     _define(_V, "int4_dequant(Tensor weight, Tensor weight_scale, Tensor? weight_zp, "
                 "Tensor(a!) output) -> Tensor(a!)", int4_dequant, _ret(3))
     _define(_V, "fp8_dequant(Tensor weight, Tensor weight_scale, Tensor(a!) output, str mode) -> Tensor(a!)",
@@ -2012,7 +2017,8 @@ def register():
             "Tensor down_weight, Tensor down_scale, Tensor routing_weights, Tensor expert_offsets, Tensor expert_tokens, "
             "int top_k, int n_routed_experts) -> Tensor", moe_forward_full_fp8_grouped, lambda x, *a: torch.empty_like(x))
     _define("moe_fp8_prefill_ops", "moe_prefill_gather_forward_fp8(Tensor selected_experts, int num_experts) -> Tensor[]",
-            moe_prefill_gather_forward_fp8)
+            moe_prefill_gather_forward_fp8,
+            lambda sel, e: [sel.new_empty(e), sel.new_empty(sel.numel()), sel.new_empty(sel.numel()), sel.new_empty(e)])
     _define("moe_fp8_prefill_ops", "moe_prefill_full_fp8(Tensor hidden_states, Tensor topk_weights, Tensor topk_ids, "
             "Tensor w13, Tensor w13_scale, Tensor w2, Tensor w2_scale, int top_k, int num_experts) -> Tensor",
             moe_prefill_full_fp8, lambda h, *a: torch.empty_like(h))

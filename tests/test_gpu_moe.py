@@ -112,6 +112,35 @@ def test_sort_bit_exact(v, dev, T, E, K):
     assert int(mx.cpu()) == int((rs[1:] - rs[:-1]).max())
 
 
+@pytest.mark.parametrize("T,E,K", [(40, 16, 4), (3000, 32, 2)])
+def test_sort_bad_ids_stay_in_bounds(v, dev, T, E, K):
+    # ids a top-k selection never produces (out of range, repeated inside a token) give unspecified
+    # results for their tokens, but every index the sort writes stays valid and the other tokens'
+    # experts keep their pairs (single-pass and chunked path)
+    g = torch.Generator().manual_seed(T)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    ids[1, 0] = -7
+    ids[2, 1] = E + 100
+    ids[3, :] = 5                                   # one expert K times
+    ids[T - 1, 0] = ids[T - 1, 1]
+    P = T * K
+    sp = torch.full((P,), -1, dtype=torch.int32, device=dev)
+    st = torch.full((E + 1,), -1, dtype=torch.int32, device=dev)
+    inv = torch.full((P,), -1, dtype=torch.int32, device=dev)
+    tok = torch.full((P,), -1, dtype=torch.int32, device=dev)
+    v.moe_sort(ids.to(dev), E, sp, st, inv, tok)
+    sp, st, inv, tok = sp.cpu(), st.cpu(), inv.cpu(), tok.cpu()
+    assert st[0] == 0 and bool((st[1:] >= st[:-1]).all()) and int(st[E]) <= P
+    assert bool(((sp >= 0) & (sp < P)).all()) and bool(((inv >= 0) & (inv < P)).all())
+    assert bool(((tok >= 0) & (tok < T)).all())
+    good = [t for t in range(T) if t not in (1, 2, 3, T - 1)]
+    for t in good[:64]:
+        for j in range(K):
+            pos = int(inv[t * K + j])
+            e = int(ids[t, j])
+            assert int(st[e]) <= pos < int(st[e + 1]) and int(sp[pos]) == t * K + j and int(tok[pos]) == t
+
+
 def test_sort_golden_fixture(v, dev):
     import json
     import os
