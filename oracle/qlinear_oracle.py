@@ -557,6 +557,17 @@ def max_rel_err(out: torch.Tensor, ref: torch.Tensor) -> float:
     return float(((o - r).abs() / r.abs().clamp(min=float(floor))).max())
 
 
+def max_rel_err_abs_floor(out: torch.Tensor, ref: torch.Tensor, floor: float = 1e-3) -> float:
+    """max |out - ref| / max(|ref|, floor): the reference's own element-wise form
+    (`ref.abs().clamp(min=1e-3)`, V/tests/test_fp8_blockscale_gemm.py:55).  Stricter than
+    max_rel_err on the outputs that sit near zero: there the error of a K-long dot product
+    (rounding of the 16-bit output, summation order, weights kept unrounded by a kernel) is
+    judged against 1e-3 instead of against the tensor's typical magnitude."""
+    o = out.to(torch.float32)
+    r = ref.to(torch.float32)
+    return float(((o - r).abs() / r.abs().clamp(min=floor)).max())
+
+
 def moe_forward_full(x, logits, w13, s13, shared_w13, shared_s13, w2, s2, shared_w2, shared_s2, shared_gate, top_k):
     """Small-batch fused MoE decode step with one shared expert, fp32 throughout.
     Follows the per-token loop of V/tests/test_moe_forward_full_fp8_block.py:49-80:

@@ -136,9 +136,30 @@ def _run_int4(v, dev, M, K, N, dt, seed=1234):
     return O.max_rel_err(out.cpu(), ref)
 
 
+def _both(name, out, ref):
+    """Both forms of the maximum relative error: denominator floored at mean |ref| (the bar of this
+    suite) and at 1e-3 absolute (the reference's own form, V/tests/test_fp8_blockscale_gemm.py:55)."""
+    a, b = O.max_rel_err(out, ref), O.max_rel_err_abs_floor(out, ref)
+    print(f"{name}: max-rel (mean floor) {a:.3e}, (1e-3 floor) {b:.3e}", flush=True)
+    return a, b
+
+
 def test_cfg0_w4a16_gemv(ops, dev):
     v, _ = ops
-    assert _run_int4(v, dev, 1, 4096, 4096, torch.float16) < TOL
+    M, K, N = 1, 4096, 4096
+    x, packed, scale, _ = O.make_int4_case(M, K, N)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    v.esimd_gemv_int4(x.to(dev), packed.to(dev), scale.to(dev), out)
+    a, b = _both("cfg0 vs fp16-rounded weights", out.cpu(), O.matmul_ref(x, O.int4_dequant(packed, scale)))
+    assert a < TOL
+    # With the 1e-3 floor an output near zero is judged on its absolute error.  The decode GEMV keeps
+    # (nib - 8) * s unrounded, so against the fp16-ROUNDED weights every output carries the K-long sum
+    # of those roundings (about 5e-3 absolute at a typical |out| of 3); against the unrounded weights
+    # what is left is the rounding of the fp16 output itself.
+    assert b < 0.25
+    a32, b32 = _both("cfg0 vs unrounded weights", out.cpu(),
+                     O.matmul_ref(x, O.int4_dequant(packed, scale, out_dtype=torch.float32)))
+    assert a32 < TOL and b32 < 2e-2
 
 
 @pytest.mark.parametrize("M,K,N,dt", [
@@ -176,7 +197,8 @@ def test_cfg1_fp8_pern(ops, dev, M):
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     v.esimd_gemv_fp8_pern(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), s.to(dev), out, N, K)
     ref = O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))
-    assert O.max_rel_err(out.cpu(), ref) < TOL
+    a, b = _both(f"cfg1 M={M}", out.cpu(), ref)
+    assert a < TOL and b < TOL                     # both forms: the E4M3 decode is exact, only the bf16 output rounds
 
 
 @pytest.mark.parametrize("M,K,N,dt,s16", [
@@ -278,7 +300,12 @@ def test_cfg4_q4k(ops, dev, M):
     s.esimd_gemv_q4_k(x.to(dev), torch.from_numpy(ql).to(dev), torch.from_numpy(sc).to(dev),
                       torch.from_numpy(mn).to(dev), out)
     w = torch.from_numpy(O.q4k_dequant(ql, sc, mn))
-    assert O.max_rel_err(out.cpu(), O.matmul_ref(x, w)) < TOL
+    a, b = _both(f"cfg4 M={M}", out.cpu(), O.matmul_ref(x, w))
+    assert a < TOL
+    # 1e-3 floor: outputs here have a typical magnitude of 100 (K = 5120 products of order 1), so a
+    # near-zero output is judged on an absolute error of 0.05-0.2: the unrounded weights of the row
+    # kernel (M = 1) or the fp32 accumulation order of the matrix-core kernel (M = 64)
+    assert b < (0.6 if M == 1 else 0.1)
 
 
 @pytest.mark.parametrize("M,K,N", [(1, 256, 3), (5, 768, 100), (40, 512, 33)])
@@ -374,7 +401,8 @@ def test_cfg2_w4a16_prefill_gemm(ops, dev):
     rows = torch.arange(0, M, 37)
     cols = torch.arange(0, N, 29)
     ref = O.matmul_ref(x[rows], wd[cols])
-    assert O.max_rel_err(o[rows][:, cols], ref) < TOL
+    a, b = _both("cfg2", o[rows][:, cols], ref)
+    assert a < TOL and b < TOL                     # both forms hold: the kernel uses the bf16-rounded weights
     # size-independent property: linearity in x.  out(2x) == 2 out(x) exactly (power of two)
     out2 = torch.empty_like(out)
     v.esimd_gemm_int4_pgrp_zp((x * 2).to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out2)

@@ -341,6 +341,9 @@ def _check_forward(v, dev, T, E, K, H, I, aq, seed):
     # stage 3: down GEMM, stage 4: weighted combine
     assert O.max_rel_err(g["y"].cpu(), ref_y) < TOL
     assert O.max_rel_err(g["out"].cpu(), ref) < TOL
+    # the reference's 1e-3-floor form on the same teacher-forced output (near-zero outputs are judged on
+    # the absolute error of an 8-expert weighted sum rounded to 16 bit)
+    assert O.max_rel_err_abs_floor(g["out"].cpu(), ref) < 3e-2
     # the fused op runs the same kernels; with fused SiLU (act-quant mode) it is bit-identical
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     r = v.moe_forward_fp8_block(x.to(dev), logits.to(dev), w13q.view(torch.float8_e4m3fn).to(dev), w13s.to(dev),
@@ -353,6 +356,12 @@ def _check_forward(v, dev, T, E, K, H, I, aq, seed):
     mean_rel = ((o - free).abs().mean() / free.abs().mean()).item()
     cos = torch.nn.functional.cosine_similarity(o.flatten(), free.flatten(), dim=0).item()
     assert mean_rel < 1e-2 and cos > 0.9995, (mean_rel, cos)
+    # recorded, not asserted (re-quantising the intermediate is discontinuous): the free-running
+    # maximum under both denominators, and the staged (teacher-forced) output under the reference's floor
+    print(f"moe forward T={T} E={E} aq={aq}: staged out max-rel (mean floor) {O.max_rel_err(g['out'].cpu(), ref):.3e}, "
+          f"(1e-3 floor) {O.max_rel_err_abs_floor(g['out'].cpu(), ref):.3e}; free-running max-rel (mean floor) "
+          f"{O.max_rel_err(out.cpu(), free):.3e}, (1e-3 floor) {O.max_rel_err_abs_floor(out.cpu(), free):.3e}, "
+          f"mean-rel {mean_rel:.3e}, cos {cos:.6f}", flush=True)
     return out
 
 
@@ -364,6 +373,8 @@ def test_moe_forward_small(v, dev, T, E, K, H, I, aq):
 
 
 def test_cfg3_moe_forward(v, dev):
+    # the stage-wise 1e-2 bars (mean floor) are inside _check_forward; it also prints the staged and the
+    # free-running maxima under both denominators (free-running, this shape: 4e-2 with the mean floor)
     out = _check_forward(v, dev, 512, 128, 8, 2048, 768, True, seed=1237)
     assert torch.isfinite(out.float()).all()
 
