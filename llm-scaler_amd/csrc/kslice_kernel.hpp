@@ -1,0 +1,268 @@
+// Small-M FP8 weight-only GEMM with the activations resident in registers.
+//
+// Regime: 5 <= M <= 32 rows against an [N, K] FP8 weight, M * K small enough that a
+// workgroup can hold all of x in its register file (x is the matrix-core operand that never
+// changes while the weight streams past).  One workgroup owns up to 64 weight rows; its 8
+// wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
+//   - a wavefront loads its slice of x ONCE, straight into operand layout, before any weight
+//     load is issued (x comes from L2; the vector-memory counter retires in order, so these
+//     loads never queue behind the weight stream),
+//   - the loop is weight loads -> wave-private LDS transpose -> E4M3 decode -> MFMA, with the
+//     next 16-row tile in flight while the current one is consumed: no barrier, no x traffic,
+//   - the 8 partial tiles meet once, at the end, in LDS.
+// Weight loads are row-contiguous (one instruction reads 1 KiB of consecutive slice bytes, row
+// after row: operand-layout loads whose lanes read 64-byte pieces of 16 rows were measured
+// about 3 us slower on a 56 MB weight); the wavefront's own LDS tile (pitch + 16 bytes) turns
+// them into operand layout.
+//
+// k assignment inside a slice: read q (0 .. NQ-1) of lane (j = lane % 16, g = lane / 16) holds
+// bytes [64 q + 16 g, +16) of weight row n0 + 16 t + j; MFMA 2 q + h consumes bytes 8 h .. 8 h + 7
+// of it against x[j][slice + 64 q + 16 g + 8 h .. + 7].
+#pragma once
+#include "skinny_kernel.hpp"
+
+namespace qlin {
+
+constexpr int kKsliceWaves = 8;
+constexpr int kKsliceMaxTiles = 4;                    // 16-row weight tiles per workgroup
+
+template <int MT, int NQ>
+constexpr int kslice_lds_bytes() {
+  return kKsliceWaves * 16 * (64 * NQ + 16) + kKsliceWaves * kKsliceMaxTiles * MT * 1024;
+}
+
+// MT = 16-row activation tiles (M <= 16 MT), NQ = 16-byte loads per lane, row tile and slice
+// (slice = 64 NQ k), BLOCK = 128x128 block scales (otherwise one scale per output channel or
+// per tensor, applied to the finished sum).
+template <class Act, bool BLOCK, int MT, int NQ>
+__global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const SkinnyArgs a, const int scale_mode) {
+  using V8 = typename Act::v8;
+  using Elem = typename Act::elem;
+  constexpr int NW = kKsliceWaves;
+  constexpr int kMaxTiles = kKsliceMaxTiles;
+  constexpr int kSliceB = 64 * NQ;                    // bytes of one weight row inside a slice
+  constexpr int kPitch = kSliceB + 16;                // LDS row pitch: operand reads hit distinct banks
+  constexpr int kStage = 16 * kPitch;                 // one wavefront's staging tile
+  constexpr int kCPR = kSliceB / 16;                  // 16-byte chunks per row of the slice
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // the partial tiles live beside the staging tiles
+  f32x4 (*red)[kMaxTiles][MT][64] = reinterpret_cast<f32x4 (*)[kMaxTiles][MT][64]>(smem + NW * kStage);
+
+  int tile = blockIdx.x;
+  int mat = 0;
+#pragma unroll
+  for (int i = 0; i + 1 < kMaxMat; ++i) {
+    if (mat == i && i + 1 < a.nmat && tile >= a.tiles[i]) { tile -= a.tiles[i]; mat = i + 1; }
+  }
+  const int N = a.N[mat];
+  const int K = a.K, M = a.M;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, g = lane >> 4;
+  const int n0 = tile * a.rpw;
+  const int nend = min(N, n0 + a.rpw);
+  const int ntiles = (nend - n0 + 15) >> 4;           // <= kMaxTiles
+  const int kbase = wave * kSliceB;                   // first k of this wavefront's slice
+
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * (uint32_t)K);
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+
+  // ---- x: the wavefront's slice of every row, once ----
+  u32x4 xq[MT][NQ][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int m = mt * 16 + j;
+        const int k = kbase + 64 * q + 16 * g + 8 * h;
+        xq[mt][q][h] = buf_load16(xr, (m < M && k < K) ? ((uint32_t)m * (uint32_t)K + (uint32_t)k) * 2u : kOOB);
+      }
+
+  // ---- weights: two 16-row tiles in flight in registers ----
+  // The 64 NQ chunks of a tile's slice (16 rows x kCPR chunks) are walked row-major: load i takes
+  // chunks 64 i .. 64 i + 63, i.e. 1 KiB of consecutive slice bytes, row after row.
+  auto chunk_of = [&](int i, int& r, int& c) {
+    const int f = i * 64 + lane;
+    r = f / kCPR;
+    c = f - r * kCPR;
+  };
+  auto load_tile = [&](u32x4 (&w)[NQ], int t) {
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      int r, c;
+      chunk_of(i, r, c);
+      const int n = n0 + t * 16 + r;
+      const int k = kbase + 16 * c;
+      const bool ok = t < ntiles && n < nend && k < K;
+      w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, ok ? (uint32_t)n * (uint32_t)K + (uint32_t)k : kOOB, 0, 2 /* nt */);
+    }
+  };
+  unsigned char* stage = smem + wave * kStage;
+  // registers (row-contiguous) -> this wavefront's LDS tile -> registers (operand layout)
+  auto transpose_tile = [&](u32x4 (&w)[NQ]) {
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      int r, c;
+      chunk_of(i, r, c);
+      *reinterpret_cast<u32x4*>(stage + r * kPitch + c * 16) = w[i];
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) w[q] = *reinterpret_cast<const u32x4*>(stage + j * kPitch + 64 * q + 16 * g);
+  };
+  const float* s32 = (const float*)a.s[mat];
+  const int Kb = (K + 127) >> 7;
+  auto compute_tile = [&](u32x4 (&w)[NQ], int t) {
+    transpose_tile(w);
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (BLOCK) {
+      // two reads = one 128-wide scale block; its partial sum is scaled before it joins the total
+      const int nb = min(n0 + t * 16, N - 1) >> 7;
+#pragma unroll
+      for (int q2 = 0; q2 < NQ / 2; ++q2) {
+        const int kb = min((kbase >> 7) + q2, Kb - 1);
+        const float sc = s32[(size_t)nb * Kb + kb];
+        f32x4 part[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq) {
+          const int q = q2 * 2 + qq;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const V8 b = fp8x8_to_act<Act>(w[q][2 * h], w[q][2 * h + 1]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) part[mt] = Act::mfma(as_v8<V8>(xq[mt][q][h]), b, part[mt]);
+          }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt] += part[mt] * sc;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const V8 b = fp8x8_to_act<Act>(w[q][2 * h], w[q][2 * h + 1]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt] = Act::mfma(as_v8<V8>(xq[mt][q][h]), b, acc[mt]);
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[wave][t][mt][lane] = acc[mt];
+  };
+
+  u32x4 w0[NQ], w1[NQ];
+  load_tile(w0, 0);
+  load_tile(w1, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  // Tiles 0 .. 3 with static register slots.  Every load is issued unconditionally (a tile past
+  // the workgroup's range loads nothing), so the wait counts stay exact on every path; only the
+  // arithmetic of a missing tile is skipped.
+  compute_tile(w0, 0);
+  load_tile(w0, 2);
+  __builtin_amdgcn_sched_barrier(0);
+  if (ntiles > 1) compute_tile(w1, 1);
+  load_tile(w1, 3);
+  __builtin_amdgcn_sched_barrier(0);
+  if (ntiles > 2) compute_tile(w0, 2);
+  if (ntiles > 3) compute_tile(w1, 3);
+
+  // ---- the 8 slices meet: wavefront w finishes output tile (t, mt) = w ----
+  __syncthreads();
+  for (int o = wave; o < ntiles * MT; o += NW) {
+    const int t = o / MT, mt = o - t * MT;
+    f32x4 sum = red[0][t][mt][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[w][t][mt][lane];
+    // D layout: lane holds output column n0 + 16 t + j, rows 16 mt + 4 g + v
+    const int n = n0 + t * 16 + j;
+    if (n < nend) {
+      float os = 1.0f;
+      if constexpr (!BLOCK) {
+        if (scale_mode == SC_PERT) os = s32[0];
+        else os = a.scale_f16 ? (float)((const _Float16*)a.s[mat])[n] : s32[n];
+      }
+      Elem* out = (Elem*)a.out[mat];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = mt * 16 + g * 4 + v;
+        if (m < M) out[(size_t)m * N + n] = Act::from_f32(sum[v] * os);
+      }
+    }
+  }
+}
+
+// Whether the register-resident path covers a problem: FP8, 5 .. 32 rows, the slice of x within
+// 128 registers per lane, 16-byte aligned rows.
+static inline int kslice_loads(int M, int K) {
+  if (M < 5 || M > 32 || (K % 16)) return 0;
+  const int mt = M <= 16 ? 1 : 2;
+  int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // loads per lane to cover K with 8 slices
+  nq = (nq + 1) & ~1;                                            // even: whole 128-wide scale blocks
+  const int choices[] = {2, 4, 6, 8, 10, 12};          // 16 loads spill
+  for (int c : choices)
+    if (c >= nq) return (mt * c <= 16) ? c : 0;                 // x registers: mt * c * 8 <= 128
+  return 0;
+}
+
+template <class Act, bool BLOCK, int MT>
+static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_mode, hipStream_t st) {
+  const dim3 grid(tiles), block(kKsliceWaves * 64);
+#define QLIN_KSLICE(NQ_)                                                                                       \
+  case NQ_:                                                                                                    \
+    if constexpr (MT * NQ_ <= 16)                                                                              \
+    {                                                                                                          \
+      auto kern = kslice_fp8_kernel<Act, BLOCK, MT, NQ_>;                                                      \
+      constexpr int lds = kslice_lds_bytes<MT, NQ_>();                                                         \
+      static_assert(lds <= 160 * 1024, "staging tiles exceed the LDS");                                        \
+      static bool raised = false;                                                                              \
+      if (lds > 64 * 1024 && !raised) {                                                                        \
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
+        raised = true;                                                                                         \
+      }                                                                                                        \
+      hipLaunchKernelGGL(kern, grid, block, lds, st, a, scale_mode);                                           \
+    }         \
+    break;
+  switch (nq) {
+    QLIN_KSLICE(2) QLIN_KSLICE(4) QLIN_KSLICE(6) QLIN_KSLICE(8) QLIN_KSLICE(10) QLIN_KSLICE(12)
+    default: break;
+  }
+#undef QLIN_KSLICE
+}
+
+// scale_mode: SC_PERN / SC_PERT / SC_BLOCK.  Rows per workgroup as in the skinny kernel: one
+// workgroup per CU and round, a multiple of 16 rows, at most 64.
+template <class Act>
+static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
+  long ntot = 0;
+  for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
+  const int cus = device_cu_count();
+  int rounds = (int)((ntot + (long)cus * 64 - 1) / ((long)cus * 64));
+  if (rounds < 1) rounds = 1;
+  int rpw = (int)((ntot + (long)cus * rounds - 1) / ((long)cus * rounds));
+  rpw = scale_mode == SC_BLOCK ? ((rpw + 15) & ~15) : ((rpw + 7) & ~7);
+  if (rpw > 64) rpw = 64;
+  if (rpw < 8) rpw = 8;
+  a.rpw = rpw;
+  int tiles = 0;
+  for (int i = 0; i < a.nmat; ++i) {
+    a.tiles[i] = (a.N[i] + rpw - 1) / rpw;
+    tiles += a.tiles[i];
+  }
+  if (!tiles) return MI_OK;
+  const bool block = scale_mode == SC_BLOCK;
+  if (a.M <= 16) {
+    if (block) kslice_launch_nq<Act, true, 1>(a, nq, tiles, scale_mode, st);
+    else kslice_launch_nq<Act, false, 1>(a, nq, tiles, scale_mode, st);
+  } else {
+    if (block) kslice_launch_nq<Act, true, 2>(a, nq, tiles, scale_mode, st);
+    else kslice_launch_nq<Act, false, 2>(a, nq, tiles, scale_mode, st);
+  }
+  return launch_status();
+}
+
+}  // namespace qlin

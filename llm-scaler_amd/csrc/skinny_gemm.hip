@@ -2,6 +2,7 @@
 // 128x128 block), INT4 group 128 and GGUF Q4_K: M <= 4 takes the one-wavefront-per-row
 // kernel (gemv_rows.hpp), larger M the MFMA kernel (skinny_kernel.hpp).
 #include "skinny_kernel.hpp"
+#include "kslice_kernel.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -47,6 +48,16 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     else
       launch_rows_m<ActBF16, FMT, SC>(r, st);
     return launch_status();
+  }
+  // few rows whose slice of x fits the register file: activations resident, weights streamed
+  if constexpr (FMT == 0) {
+    long ntot = 0;
+    for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
+    // measured against the granule-interleaved kernel (M = 5 .. 32): ahead by 5-35 % when a workgroup
+    // owns at least two 16-row tiles or rows are short, behind by 10-25 % for one tile of long rows
+    const bool pays = ntot > 16L * device_cu_count() || a.K <= 2048;
+    if (const int nq = pays ? kslice_loads(a.M, a.K) : 0)
+      return act_dtype == DT_F16 ? kslice_launch<ActF16>(a, SC, nq, st) : kslice_launch<ActBF16>(a, SC, nq, st);
   }
   const int M = a.M;
   const size_t esz = 2;

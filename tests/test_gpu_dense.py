@@ -216,6 +216,37 @@ def test_fp8_pern_shapes(ops, dev, M, K, N, dt, s16):
     assert O.max_rel_err(out.cpu(), ref) < TOL
 
 
+@pytest.mark.parametrize("M,K,N,dt,mode", [
+    (5, 4096, 8200, torch.bfloat16, "pern"), (16, 2048, 333, torch.float16, "pern"), (17, 4096, 9000, torch.float16, "pern"),
+    (32, 4096, 8192, torch.bfloat16, "pert"), (9, 5120, 5120, torch.float16, "block"), (24, 1024, 4160, torch.bfloat16, "block"),
+    (31, 3584, 9216, torch.float16, "block"), (8, 6144, 8448, torch.bfloat16, "pern"), (12, 1056, 520, torch.float16, "pern"),
+    (6, 6112, 8300, torch.float16, "pert")])
+def test_fp8_register_resident_activations(ops, dev, M, K, N, dt, mode):
+    # 5 .. 32 rows with x held in registers and K split over the wavefronts in slices: slices that
+    # end inside K (3584, 1056, 6112), row counts off the 16-row tiles, every scale mode
+    v, _ = ops
+    if mode == "block":
+        x, w8, s = O.make_fp8_block_case(M, K, (N + 127) // 128 * 128, seed=M + K, act_dtype=dt, std=0.3)
+        w8 = w8[:N].contiguous()
+        ref = O.matmul_ref(x, O.fp8_dequant_block(w8, s))
+    else:
+        x, w8, s = O.make_fp8_pern_case(M, K, N, seed=M + K, act_dtype=dt)
+        if mode == "pert":
+            s = torch.tensor([3.0e-4])
+            ref = O.matmul_ref(x, O.fp8_dequant_per_tensor(w8, s))
+        else:
+            ref = O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))
+    out = torch.empty(M, N, dtype=dt, device=dev)
+    xd, wd, sd = x.to(dev), w8.to(dev), s.to(dev)
+    if mode == "block":
+        v.esimd_gemm_fp8_blockscale(xd, wd, sd, out)
+    elif mode == "pert":
+        v.esimd_gemm_fp8_pert(xd, wd, sd, out)
+    else:
+        v.esimd_gemv_fp8_pern(xd, wd, sd, out, N, K)
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+
+
 def test_fp8_pern_fused3_equals_separate(ops, dev):
     v, _ = ops
     K = 2048
