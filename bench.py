@@ -289,6 +289,61 @@ def wl_gemm_w4a16(dev):
                 kernel="gemm_w4a16_kernel", cpu=cpu)
 
 
+def wl_fp8_prefill(dev, mode="pern"):
+    """FP8 weight-only prefill GEMM at the cfg1 shape with 2048 rows (workload beyond the configurations):
+    the tiled matrix-core GEMM with the FP8 weight staged through LDS."""
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    M, K, N = 2048, 4096, 14336
+    g = torch.Generator().manual_seed(1241)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    if mode == "block":
+        _, w8, s = O.make_fp8_block_case(1, K, N, seed=1241)
+    else:
+        _, w8, s = O.make_fp8_pern_case(1, K, N, seed=1241)
+    xd, wd, sd = x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), s.to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+    def launch(i):
+        if mode == "block":
+            v.esimd_gemm_fp8_blockscale(xd, wd, sd, out)
+        else:
+            v.esimd_gemv_fp8_pern(xd, wd, sd, out, N, K)
+
+    def cpu():
+        wdq = O.fp8_dequant_block(w8, s) if mode == "block" else O.fp8_dequant_per_channel(w8, s)
+        return O.matmul_ref(x[:256], wdq).to(torch.bfloat16)
+
+    alg_bytes = N * K + 4 * N + 2 * M * K + 2 * M * N
+    return dict(launch=launch, R=1, bytes=alg_bytes, flops=2 * M * N * K, bound="mfma", dtype="bf16",
+                name=f"next: FP8 e4m3 {'128x128-block' if mode == 'block' else 'per-channel'} weight-only prefill GEMM "
+                     f"M={M} K={K} N={N} bf16", kernel="gemm_tiled_kernel", cpu=cpu, cpu_scale=256 / M,
+                cpu_what=f"256 of the {M} activation rows (the whole weight is dequantized in every pass)")
+
+
+def wl_q4k_prefill(dev):
+    """Q4_K prefill at the cfg4 shape with 2048 rows (workload beyond the configurations)."""
+    import custom_esimd_kernels_sglang as s
+    from oracle import qlinear_oracle as O
+    M, K, N = 2048, 5120, 5120
+    x, raw = O.make_q4k_case(M, K, N, seed=1242)
+    ql, sc, mn = O.q4k_repack(raw)
+    W = (torch.from_numpy(ql).to(dev), torch.from_numpy(sc).to(dev), torch.from_numpy(mn).to(dev))
+    xd = x.to(dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        s.esimd_gemv_q4_k(xd, *W, out)
+
+    def cpu():
+        return O.matmul_ref(x[:256], torch.from_numpy(O.q4k_dequant(ql, sc, mn))).to(torch.float16)
+
+    alg_bytes = N * K // 2 + 2 * N * (K // 32) * 2 + 2 * M * K + 2 * M * N
+    return dict(launch=launch, R=1, bytes=alg_bytes, flops=2 * M * N * K, bound="mfma", dtype="f16",
+                name=f"next: GGUF Q4_K (repacked) prefill GEMM M={M} K={K} N={N} fp16", kernel="gemm_tiled_kernel",
+                cpu=cpu, cpu_scale=256 / M, cpu_what=f"256 of the {M} activation rows")
+
+
 def wl_copy(dev):
     """Plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
     n = 256 << 20
@@ -460,6 +515,9 @@ WORKLOADS = {
     "cfg3": wl_moe,
     "cfg4_m1": lambda dev: wl_q4k(1, dev),
     "cfg4_m64": lambda dev: wl_q4k(64, dev),
+    "next_fp8_prefill_m2048": wl_fp8_prefill,
+    "next_fp8_block_prefill_m2048": lambda dev: wl_fp8_prefill(dev, "block"),
+    "next_q4k_prefill_m2048": wl_q4k_prefill,
     "next_q4k_m8": lambda dev: wl_q4k(8, dev),
     "next_q4k_m32": lambda dev: wl_q4k(32, dev),
     "next_q4_0_m1": lambda dev: wl_gguf("q4_0", 1, dev),

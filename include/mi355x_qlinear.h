@@ -342,6 +342,25 @@ int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const v
                         const void* const* w, const void* const* scale, void* const* out, const int* N, int K,
                         int act_dtype, void* stream);
 
+/* ---- prefill (M > 64) on FP8 and Q4_K weights: the tiled matrix-core GEMM ---------
+ * The same results as mi_gemm_fp8_pern / _pert / _blockscale and mi_gemv_q4k, computed by the
+ * 256 x 256 (224, 128) tiled GEMM that also serves mi_gemm_int4, so that a weight byte is read
+ * once per 256 activation rows.  scale_mode 0 = per output channel (fp32, or fp16 with
+ * scale_is_f16), 1 = per tensor (fp32 [1]), 2 = 128 x 128 blocks (fp32 [ceil(N/128), K/128],
+ * folded into the weight before its rounding to the activation type).  K % 128 == 0.
+ * workspace: mi_gemm_tiled_workspace(M, K) bytes for the re-tiled activations.  The entry points
+ * above take this route themselves for M > 64 (with the per-stream scratch buffer); the torch
+ * ops pass a workspace from the caching allocator.  Reference: the M > 64 dispatch of
+ * GEMM_fp8_pert_dispatch (V/csrc/xpu/esimd_kernels/fp8_GEMM_pert.h:4030-4075), the M >= 16 torch
+ * route of the block-scaled linear (vllm/patches/vllm_for_multi_arc.patch:2671-2691) and the
+ * M > 1 dense route of Q4_K (sglang/patches/sglang_for_multi_arc.patch:3211-3213). */
+int mi_gemm_tiled_workspace(int M, int K, long long* bytes);
+int mi_gemm_fp8_tiled_ws(const void* x, const void* w, const void* scale, int scale_mode, int scale_is_f16,
+                         void* out, void* workspace, long long workspace_bytes, int M, int N, int K,
+                         int act_dtype, void* stream);
+int mi_gemm_q4k_tiled_ws(const void* x, const void* ql, const void* scale, const void* qmin, void* out,
+                         void* workspace, long long workspace_bytes, int M, int N, int K, void* stream);
+
 /* ---- MoE grouped FP8 block-scaled GEMM ----------------------------------------
  * out[r, :] = a[src(r), :] @ dequant(w[e])^T for the rows r of expert e,
  * expert_start[e] <= r < expert_start[e+1]; src(r) = row_map[r] if row_map else r.

@@ -3,6 +3,7 @@
 // kernel (gemv_rows.hpp), larger M the MFMA kernel (skinny_kernel.hpp).
 #include "skinny_kernel.hpp"
 #include "kslice_kernel.hpp"
+#include "scratch.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -58,6 +59,23 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     const bool pays = ntot > 16L * device_cu_count() || a.K <= 2048;
     if (const int nq = pays ? kslice_loads(a.M, a.K) : 0)
       return act_dtype == DT_F16 ? kslice_launch<ActF16>(a, SC, nq, st) : kslice_launch<ActBF16>(a, SC, nq, st);
+  }
+  // prefill: the tiled matrix-core GEMM reads the weight once per 256 rows instead of once per 64
+  if constexpr (FMT == 0 || FMT == 2) {
+    if (a.M > 64 && a.K % 128 == 0) {
+      long long bytes = 0;
+      if (mi_gemm_tiled_workspace(a.M, a.K, &bytes) != MI_OK) return MI_ERR_SHAPE;
+      void* ws = scratch_get(st, (size_t)bytes);
+      if (!ws) return MI_ERR_LAUNCH;
+      for (int i = 0; i < a.nmat; ++i) {
+        const int rc = FMT == 0 ? mi_gemm_fp8_tiled_ws(a.x, a.w[i], a.s[i], SC, a.scale_f16, a.out[i], ws, bytes, a.M,
+                                                       a.N[i], a.K, act_dtype, st)
+                                : mi_gemm_q4k_tiled_ws(a.x, a.w[i], a.s[i], a.z[i], a.out[i], ws, bytes, a.M, a.N[i],
+                                                       a.K, st);
+        if (rc != MI_OK) return rc;
+      }
+      return MI_OK;
+    }
   }
   const int M = a.M;
   const size_t esz = 2;

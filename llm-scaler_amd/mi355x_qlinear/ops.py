@@ -65,6 +65,34 @@ def _chk_act(x: torch.Tensor, out: torch.Tensor, who: str):
 
 
 # --------------------------------------------------------------------------
+# Prefill route (M > 64, K % 128 == 0) of the FP8 and Q4_K ops: the tiled matrix-core GEMM.  The
+# re-tiled activations live in a workspace from torch's caching allocator, so that the op stays
+# capturable in a HIP graph.
+# --------------------------------------------------------------------------
+_SC_PERN, _SC_PERT, _SC_BLOCK = 0, 1, 2
+
+
+def _tiled_workspace(x, M, K):
+    need = ctypes.c_longlong(0)
+    rc = capi.lib().mi_gemm_tiled_workspace(M, K, ctypes.byref(need))
+    if rc != 0:
+        raise RuntimeError(f"mi_gemm_tiled_workspace: {capi.MI_ERRORS.get(rc, rc)}")
+    return torch.empty(need.value, dtype=torch.uint8, device=x.device), need.value
+
+
+def _prefill_route(M, K):
+    return M > 64 and K % 128 == 0
+
+
+def _fp8_tiled_multi(x, ws, ss, os_, Ns, M, K, mode, scale_f16):
+    buf, nbytes = _tiled_workspace(x, M, K)
+    for w, s, o, N in zip(ws, ss, os_, Ns):
+        capi.call("mi_gemm_fp8_tiled_ws", x, capi.ptr(x), capi.ptr(w), capi.ptr(s), mode, 1 if scale_f16 else 0,
+                  capi.ptr(o), capi.ptr(buf), nbytes, M, int(N), K, capi.act_dtype(x))
+    return os_[0]
+
+
+# --------------------------------------------------------------------------
 # FP8 per-channel  (esimd_gemv_fp8_pern, _fused2, _fused3)
 # --------------------------------------------------------------------------
 def _fp8_pern_multi(x, ws, ss, os_, Ns, K, who):
@@ -80,6 +108,8 @@ def _fp8_pern_multi(x, ws, ss, os_, Ns, K, who):
              f"{who}: weight_scale must be fp16 or fp32 (all the same), got {s.dtype}")
         _chk(s.numel() == int(N), f"{who}: weight_scale must have N={int(N)} entries")
         _chk(o.numel() == M * int(N), f"{who}: output has {o.numel()} elements, expected M*N={M * int(N)}")
+    if _prefill_route(M, K):
+        return _fp8_tiled_multi(x, ws, ss, os_, Ns, M, K, _SC_PERN, sdt == torch.float16)
     capi.call("mi_gemm_fp8_pern_multi", x, capi.ptr(x), len(ws), capi.ptr_array(ws), capi.ptr_array(ss),
               capi.ptr_array(os_), capi.int_array(Ns), M, K, capi.act_dtype(x),
               1 if sdt == torch.float16 else 0)
@@ -115,6 +145,8 @@ def _fp8_pert_multi(x, ws, ss, os_, who):
         _chk(s.dtype == torch.float32 and s.numel() >= 1, f"{who}: weight_scale must be an fp32 scalar tensor")
         _chk(o.numel() == M * w.shape[0], f"{who}: output has {o.numel()} elements, expected {M * w.shape[0]}")
         Ns.append(w.shape[0])
+    if _prefill_route(M, K):
+        return _fp8_tiled_multi(x, ws, ss, os_, Ns, M, K, _SC_PERT, False)
     capi.call("mi_gemm_fp8_pert_multi", x, capi.ptr(x), len(ws), capi.ptr_array(ws), capi.ptr_array(ss),
               capi.ptr_array(os_), capi.int_array(Ns), M, K, capi.act_dtype(x))
     return os_[0]
@@ -159,6 +191,8 @@ def _fp8_block_multi(x, ws, ss, os_, block_n, block_k, who):
              f"{who}: weight_scale must be [ceil(N/128), K/128] = {((N + 127) // 128, K // 128)}, got {tuple(s.shape)}")
         _chk(o.numel() == M * N, f"{who}: output must be [M, N]")
         Ns.append(N)
+    if _prefill_route(M, K):
+        return _fp8_tiled_multi(x, ws, ss, os_, Ns, M, K, _SC_BLOCK, False)
     capi.call("mi_gemm_fp8_blockscale_multi", x, capi.ptr(x), len(ws), capi.ptr_array(ws), capi.ptr_array(ss),
               capi.ptr_array(os_), capi.int_array(Ns), M, K, capi.act_dtype(x))
     return os_[0]
@@ -305,6 +339,11 @@ def _chk_q4k(x, w, s, mn, o, who):
 
 def esimd_gemv_q4_k(input, weight, weight_scale, weight_min, output):
     M, N, K = _chk_q4k(input, weight, weight_scale, weight_min, output, "esimd_gemv_q4_k")
+    if _prefill_route(M, K):
+        buf, nbytes = _tiled_workspace(input, M, K)
+        capi.call("mi_gemm_q4k_tiled_ws", input, capi.ptr(input), capi.ptr(weight), capi.ptr(weight_scale),
+                  capi.ptr(weight_min), capi.ptr(output), capi.ptr(buf), nbytes, M, N, K)
+        return output
     capi.call("mi_gemv_q4k", input, capi.ptr(input), capi.ptr(weight), capi.ptr(weight_scale),
               capi.ptr(weight_min), capi.ptr(output), M, N, K)
     return output

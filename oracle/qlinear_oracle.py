@@ -145,15 +145,20 @@ def fp8_dequant_per_tensor(w8: torch.Tensor, scale: torch.Tensor) -> torch.Tenso
     return e4m3_decode(w8) * scale.to(torch.float32).reshape(())
 
 
-def fp8_dequant_block(w8: torch.Tensor, scale: torch.Tensor, bn=FP8_BLOCK, bk=FP8_BLOCK) -> torch.Tensor:
+def fp8_dequant_block(w8: torch.Tensor, scale: torch.Tensor, bn=FP8_BLOCK, bk=FP8_BLOCK, out_dtype=None) -> torch.Tensor:
     """[..., N, K] E4M3 + [..., ceil(N/bn), ceil(K/bk)] fp32 -> float32.
 
     V/tests/test_fp8_blockscale_gemm.py:31-36, V/tests/test_fp8_blockscale_moe_prefill.py:47-50.
+    out_dtype (fp16 / bf16): the fp32 product rounded once to that type and returned as float32 —
+    the dequantized weight of a prefill path that materialises 16-bit weights, as the reference's
+    caller does for M >= 16 (`B.to(fp16) * Bs.to(fp16)`, vllm/patches/vllm_for_multi_arc.patch:2680-2682;
+    here the scale stays fp32 and only the product is rounded).
     """
     n, k = w8.shape[-2:]
     wf = e4m3_decode(w8.reshape(-1, k)).reshape(w8.shape)
     full = scale.to(torch.float32).repeat_interleave(bn, -2).repeat_interleave(bk, -1)
-    return wf * full[..., :n, :k]
+    out = wf * full[..., :n, :k]
+    return out if out_dtype is None else out.to(out_dtype).to(torch.float32)
 
 
 def fp8_quantize_per_channel(w: torch.Tensor):

@@ -247,6 +247,70 @@ def test_fp8_register_resident_activations(ops, dev, M, K, N, dt, mode):
     assert O.max_rel_err(out.cpu(), ref) < TOL
 
 
+@pytest.mark.parametrize("M,K,N,dt,mode", [
+    (65, 1024, 520, torch.float16, "pern"), (200, 2048, 1000, torch.bfloat16, "pern"), (2048, 4096, 14336, torch.bfloat16, "pern"),
+    (130, 512, 64, torch.float16, "pern16"), (300, 1024, 777, torch.float16, "pert"), (65, 5120, 5120, torch.float16, "block"),
+    (200, 1024, 4160, torch.bfloat16, "block"), (2048, 5120, 5120, torch.bfloat16, "block"), (513, 768, 200, torch.bfloat16, "block")])
+def test_fp8_prefill_tiled_gemm(ops, dev, M, K, N, dt, mode):
+    # more than 64 rows: the tiled matrix-core GEMM (the weight is read once per 256 rows); the same
+    # bar as the small-M path, on a strided sample of rows and columns where the problem is large
+    v, _ = ops
+    if mode == "block":
+        x, w8, s = O.make_fp8_block_case(M, K, (N + 127) // 128 * 128, seed=M + K, act_dtype=dt, std=0.3)
+        w8 = w8[:N].contiguous()
+        # the block scale is folded into the weight before its rounding to the activation type (the
+        # accumulators cannot be rescaled per K block): the same dequantized weights for the oracle
+        wd = O.fp8_dequant_block(w8, s, out_dtype=dt)
+    else:
+        x, w8, s = O.make_fp8_pern_case(M, K, N, seed=M + K, act_dtype=dt)
+        if mode == "pert":
+            s = torch.tensor([3.0e-4])
+            wd = O.fp8_dequant_per_tensor(w8, s)
+        else:
+            if mode == "pern16":
+                s = s.to(torch.float16)
+            wd = O.fp8_dequant_per_channel(w8, s)
+    out = torch.empty(M, N, dtype=dt, device=dev)
+    xd, wdv, sd = x.to(dev), w8.to(dev), s.to(dev)
+    if mode == "block":
+        v.esimd_gemm_fp8_blockscale(xd, wdv, sd, out)
+    elif mode == "pert":
+        v.esimd_gemm_fp8_pert(xd, wdv, sd, out)
+    else:
+        v.esimd_gemv_fp8_pern(xd, wdv, sd, out, N, K)
+    o = out.cpu()
+    rows = torch.arange(0, M, 37 if M > 600 else 1)
+    cols = torch.arange(0, N, 29 if N > 6000 else 1)
+    assert O.max_rel_err(o[rows][:, cols], O.matmul_ref(x[rows], wd[cols])) < TOL
+    if mode == "block":
+        # against the unrounded fp32 weights the rounding of the scaled weight shows (bf16: 2^-9 each)
+        wd32 = O.fp8_dequant_block(w8, s)
+        assert O.max_rel_err(o[rows][:, cols], O.matmul_ref(x[rows], wd32[cols])) < 2 * TOL
+    if M == 2048:
+        # size-independent property at full size: exact linearity in x (a power of two)
+        out2 = torch.empty_like(out)
+        if mode == "block":
+            v.esimd_gemm_fp8_blockscale((x * 2).to(dev), wdv, sd, out2)
+        else:
+            v.esimd_gemv_fp8_pern((x * 2).to(dev), wdv, sd, out2, N, K)
+        assert torch.equal(out2.cpu().float(), 2 * o.float())
+
+
+def test_fp8_prefill_c_abi_scratch_route(ops, dev):
+    # the C entry point without a workspace argument takes the same route with the library's
+    # per-stream scratch buffer and gives the same bits as the op
+    from mi355x_qlinear import capi
+    v, _ = ops
+    M, K, N = 150, 1024, 640
+    x, w8, s = O.make_fp8_pern_case(M, K, N, seed=77, act_dtype=torch.float16)
+    xd, wdv, sd = x.to(dev), w8.to(dev), s.to(dev)
+    a = torch.empty(M, N, dtype=torch.float16, device=dev)
+    b = torch.empty_like(a)
+    v.esimd_gemv_fp8_pern(xd, wdv, sd, a, N, K)
+    capi.call("mi_gemm_fp8_pern", xd, capi.ptr(xd), capi.ptr(wdv), capi.ptr(sd), capi.ptr(b), M, N, K, capi.act_dtype(xd), 0)
+    assert torch.equal(a, b)
+
+
 def test_fp8_pern_fused3_equals_separate(ops, dev):
     v, _ = ops
     K = 2048
@@ -337,6 +401,22 @@ def test_cfg4_q4k(ops, dev, M):
     # near-zero output is judged on an absolute error of 0.05-0.2: the unrounded weights of the row
     # kernel (M = 1) or the fp32 accumulation order of the matrix-core kernel (M = 64)
     assert b < (0.6 if M == 1 else 0.1)
+
+
+@pytest.mark.parametrize("M,K,N", [(65, 512, 130), (200, 2048, 1000), (2048, 5120, 5120)])
+def test_q4k_prefill_tiled_gemm(ops, dev, M, K, N):
+    # M > 64: the tiled matrix-core GEMM with the two-rounding Q4_K dequantization staged through LDS
+    # (the reference dequantizes densely and calls a matmul, sglang_for_multi_arc.patch:3211-3213)
+    _, s = ops
+    x, raw = O.make_q4k_case(M, K, N, seed=M + N)
+    ql, sc, mn = O.q4k_repack(raw)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    s.esimd_gemv_q4_k(x.to(dev), torch.from_numpy(ql).to(dev), torch.from_numpy(sc).to(dev),
+                      torch.from_numpy(mn).to(dev), out)
+    w = torch.from_numpy(O.q4k_dequant(ql, sc, mn))
+    rows = torch.arange(0, M, 37 if M > 600 else 1)
+    cols = torch.arange(0, N, 13 if N > 4000 else 1)
+    assert O.max_rel_err(out.cpu()[rows][:, cols], O.matmul_ref(x[rows], w[cols])) < TOL
 
 
 @pytest.mark.parametrize("M,K,N", [(1, 256, 3), (5, 768, 100), (40, 512, 33)])
