@@ -357,10 +357,10 @@ def wl_copy(dev):
                 name="plain device copy, 256 MiB read + 256 MiB written", kernel="copy", cpu=lambda: None)
 
 
-def wl_moe(dev):
+def wl_moe(dev, T=512):
     import custom_esimd_kernels_vllm as v
     from oracle import qlinear_oracle as O
-    T, E, K, H, I = 512, 128, 8, 2048, 768
+    E, K, H, I = 128, 8, 2048, 768
     x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I)
     wbytes = E * (2 * I * H + H * I)
     R = _copies(wbytes)
@@ -372,9 +372,11 @@ def wl_moe(dev):
     xd, ld = x.to(dev), logits.to(dev)
     out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
 
+    aq = T <= 512              # the configuration quantises the activations; the 4096-token workload is w8a16 (the reference's mode)
+
     def launch(i):
         a, b, c, d = W[i % R]
-        v.moe_forward_fp8_block(xd, ld, a, b, c, d, out, K, True)
+        v.moe_forward_fp8_block(xd, ld, a, b, c, d, out, K, aq)
 
     e_cpu, t_cpu = 64, 256                        # CPU sample: half of the experts and of the tokens, 32 rows per expert as in the whole
 
@@ -387,9 +389,9 @@ def wl_moe(dev):
     # algorithmic bytes: every expert's weights + block scales once, x and logits in, output out
     alg_bytes = wbytes + 4 * E * ((2 * I // 128) * (H // 128) + (H // 128) * (I // 128)) + 2 * T * H + 2 * T * E + 2 * T * H
     flops = 2 * P * (2 * I * H + H * I)
-    return dict(launch=launch, R=R, bytes=alg_bytes, flops=flops, bound="hbm", dtype="fp8",
-                name=f"cfg3 FP8 128x128-block MoE forward (topk+sort+quant+gate_up/SiLU+quant+down+combine) "
-                     f"T={T} E={E} top{K} H={H} I={I} bf16, fp8 activations",
+    return dict(launch=launch, R=R, bytes=alg_bytes, flops=flops, bound="hbm" if T <= 512 else "mfma", dtype="fp8" if aq else "bf16",
+                name=f"{'cfg3' if T == 512 else 'next:'} FP8 128x128-block MoE forward (topk+sort+quant+gate_up/SiLU+quant+down+combine) "
+                     f"T={T} E={E} top{K} H={H} I={I} bf16, {'fp8 activations' if aq else '16-bit activations (w8a16)'}",
                 kernel="moe_gemm_kernel", cpu=cpu, cpu_scale=e_cpu / E,
                 cpu_what=f"{e_cpu} of the {E} experts and {t_cpu} of the {T} tokens (32 rows per expert, as in the whole)")
 
@@ -515,6 +517,7 @@ WORKLOADS = {
     "cfg3": wl_moe,
     "cfg4_m1": lambda dev: wl_q4k(1, dev),
     "cfg4_m64": lambda dev: wl_q4k(64, dev),
+    "next_moe_prefill_t4096": lambda dev: wl_moe(dev, 4096),
     "next_fp8_prefill_m2048": wl_fp8_prefill,
     "next_fp8_block_prefill_m2048": lambda dev: wl_fp8_prefill(dev, "block"),
     "next_q4k_prefill_m2048": wl_q4k_prefill,

@@ -342,6 +342,23 @@ int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const v
                         const void* const* w, const void* const* scale, void* const* out, const int* N, int K,
                         int act_dtype, void* stream);
 
+/* ---- MoE prefill: grouped FP8 GEMM on the tiled matrix-core kernel ---------------
+ * mi_moe_gemm_fp8_grouped in w8a16 mode (no a_scale, output in the activation type) for experts
+ * with hundreds of rows: a device-built table of M-tiles per expert, activations gathered and
+ * re-tiled per 16-row block, then the 256 x 256 (128 x 128) tiled GEMM with one weight matrix per
+ * expert, so that an expert's weights are read once per 256 of its rows.  Same arguments and
+ * results; K % 128 == 0, E <= 1024.  workspace: mi_moe_gemm_fp8_tiled_workspace bytes.
+ * mi_moe_gemm_fp8_grouped takes this route itself (per-stream scratch) when the experts average
+ * 96 rows or more.  Reference: the 64-row expert tiles with a device-built tile map of
+ * V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:83-120, 187-302 and the per-expert M-tiled
+ * GEMMs of S/csrc/moe_prefill/moe_prefill_fp8.sycl:167-410. */
+int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes);
+int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* w, const float* w_scale,
+                             int scale_per_expert, const int32_t* expert_start, void* out,
+                             const int32_t* out_map, const void* row_weight, int a_rows, int total_rows,
+                             int E, int N, int K, int fuse_act, int act_dtype, void* workspace,
+                             long long workspace_bytes, void* stream);
+
 /* ---- prefill (M > 64) on FP8 and Q4_K weights: the tiled matrix-core GEMM ---------
  * The same results as mi_gemm_fp8_pern / _pert / _blockscale and mi_gemv_q4k, computed by the
  * 256 x 256 (224, 128) tiled GEMM that also serves mi_gemm_int4, so that a weight byte is read

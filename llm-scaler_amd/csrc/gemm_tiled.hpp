@@ -42,6 +42,21 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int scale_mode;             // fp8: 0 = per output channel, 1 = per tensor
   int scale_f16;              // fp8 per channel: the scales are fp16 instead of fp32
+  // Grouped launch (GROUPED kernels): M-tile i of the grid belongs to expert g_tile[4 i] and covers
+  // the rows [g_tile[4 i + 1], + g_tile[4 i + 2]) of the expert-sorted order; its activations
+  // start at 16-row block g_tile[4 i + 3] of the re-tiled copy (every expert's rows are padded
+  // to whole blocks there).  g_count[0] = number of M-tiles; M = rows of x (all experts).
+  // The matrices of expert e start e * g_w_stride bytes into w and e * g_s_stride bytes into
+  // scale.  out rows: sorted position, or out_map[position]; optional factor row_weight[row].
+  const int32_t* g_tile;
+  const int32_t* g_count;
+  long long g_w_stride, g_s_stride;
+  const int32_t* out_map;
+  const void* row_weight;
+  int x_blocks;               // 16-row blocks in the re-tiled activations
+  int n_half;                 // FUSE: weight row n (gate) pairs with row n + n_half (up); N = 2 n_half
+  int gelu;                   // FUSE: tanh-GELU instead of SiLU
+  int out_rows;               // rows of out (bounds mapped rows)
 };
 
 // MFMA with the accumulator pinned to the AGPR half of the register file and updated in place.
@@ -94,7 +109,7 @@ struct WInt4 {
     u32x4 outv;
     float sf[B_CH], nzs[B_CH];                        // 512 * scale and -z * scale (exact)
   };
-  static __device__ __forceinline__ Res make(const GemmArgs& p) {
+  static __device__ __forceinline__ Res make(const GemmArgs& p, int = 0) {
     Res r;
     r.Kg = p.K >> 7;
     r.wr = make_rsrc(p.w, (uint32_t)p.N * ((uint32_t)p.K >> 1));
@@ -197,7 +212,7 @@ struct WQ4K {
     float sf[B_CH];                                   // 512 * scale
     f16x2 mv[B_CH];
   };
-  static __device__ __forceinline__ Res make(const GemmArgs& p) {
+  static __device__ __forceinline__ Res make(const GemmArgs& p, int = 0) {
     Res r;
     r.Kc = p.K >> 5;
     r.wr = make_rsrc(p.w, (uint32_t)p.N * ((uint32_t)p.K >> 1));
@@ -273,6 +288,7 @@ struct WFp8 {
   static constexpr bool kPermK = false;
   struct Res {
     __amdgpu_buffer_rsrc_t wr, sr;
+    const void* se;                                   // this expert's scales
     int Kb;
   };
   struct Stage {
@@ -282,11 +298,14 @@ struct WFp8 {
   struct Dq {
     u32x4 outv;
   };
-  static __device__ __forceinline__ Res make(const GemmArgs& p) {
+  // e: expert of a grouped launch (its matrices start e * stride bytes in)
+  static __device__ __forceinline__ Res make(const GemmArgs& p, int e = 0) {
     Res r;
     r.Kb = (p.K + 127) >> 7;
-    r.wr = make_rsrc(p.w, (uint32_t)p.N * (uint32_t)p.K);
-    r.sr = make_rsrc(p.scale, BLOCK ? (uint32_t)((p.N + 127) >> 7) * (uint32_t)r.Kb * 4u : 0u);
+    r.wr = make_rsrc((const char*)p.w + (long long)e * p.g_w_stride, (uint32_t)p.N * (uint32_t)p.K);
+    r.sr = make_rsrc((const char*)p.scale + (long long)e * p.g_s_stride,
+                     BLOCK ? (uint32_t)((p.N + 127) >> 7) * (uint32_t)r.Kb * 4u : 0u);
+    r.se = (const char*)p.scale + (long long)e * p.g_s_stride;
     return r;
   }
   static __device__ __forceinline__ void chunk_addr(const Res& r, int n, int kc, int K, uint32_t& boff, uint32_t& soff) {
@@ -340,14 +359,18 @@ struct WFp8 {
       }
     }
   }
-  static __device__ __forceinline__ float out_scale(const Res&, const GemmArgs& p, int n) {
-    if (p.scale_mode == 1) return ((const float*)p.scale)[0];
-    return p.scale_f16 ? (float)((const _Float16*)p.scale)[n] : ((const float*)p.scale)[n];
+  static __device__ __forceinline__ float out_scale(const Res& r, const GemmArgs& p, int n) {
+    if (p.scale_mode == 1) return ((const float*)r.se)[0];
+    return p.scale_f16 ? (float)((const _Float16*)r.se)[n] : ((const float*)r.se)[n];
   }
 };
 
 // ------------------------------------------------------------------ kernel
-template <class Act, class Fmt, int BM, int BN>
+// GROUPED: the M-tiles come from a device-built table of (expert, rows) instead of a regular grid
+// (MoE: rows sorted by expert, one weight matrix per expert).  FUSE: the tile's weight rows
+// alternate, 16 at a time, between a gate block and the up block n_half rows further on, and the
+// epilogue writes act(gate) * up (N / 2 output columns).
+template <class Act, class Fmt, int BM, int BN, bool GROUPED = false, bool FUSE = false>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   using Elem = typename Act::elem;
   constexpr int WM = BM / 2, WN = BN / 2;             // wave sub-tile
@@ -371,14 +394,28 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   // the 8 XCDs, which take workgroups round-robin, each keep re-using one slab of x
   const int tn = blockIdx.x / p.tiles_m;
   const int tm = blockIdx.x - tn * p.tiles_m;
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int M = p.M, N = p.N, K = p.K;
+  int m0 = tm * BM;
+  const int n0 = FUSE ? tn * (BN / 2) : tn * BN;      // FUSE: first gate row of the tile
+  int M = p.M;
+  const int N = p.N, K = p.K;
   const int KT = K / kBK;                             // 64-wide steps (even: K % 128 == 0)
   const int Q = K / 32;                               // 32-wide MFMA steps
+  int expert = 0, row0 = 0, xblk0 = 0;
+  if constexpr (GROUPED) {
+    if (tm >= p.g_count[0]) return;                   // the grid is an upper bound of the tile count
+    expert = p.g_tile[4 * tm];
+    row0 = p.g_tile[4 * tm + 1];
+    M = p.g_tile[4 * tm + 2];                         // rows of this tile
+    xblk0 = p.g_tile[4 * tm + 3];
+    m0 = 0;
+  }
 
-  const int Mp = (M + 15) & ~15;
-  const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x, (uint32_t)Mp * (uint32_t)K * 2u);
-  const typename Fmt::Res res = Fmt::make(p);
+  const int Mp = (p.M + 15) & ~15;
+  const uint32_t xtiles = GROUPED ? (uint32_t)p.x_blocks : (uint32_t)(Mp >> 4);
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x, xtiles * 16u * (uint32_t)K * 2u);
+  const typename Fmt::Res res = Fmt::make(p, expert);
+  // weight row of row r of the LDS tile
+  auto tile_row = [&](int r) { return FUSE ? n0 + (r >> 5) * 16 + (r & 15) + ((r >> 4) & 1) * p.n_half : n0 + r; };
 
   f32x4 acc[TN][TM];
 #pragma unroll
@@ -389,8 +426,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   // ---- activations: register ring.  Block (16-row tile t, 32-wide step q) of the
   // re-tiled x sits at (t * Q + q) * 1024; tile and step enter as a scalar offset.
   const uint32_t xlane = (uint32_t)lane * 16u;
-  const uint32_t xtile0 = (uint32_t)((m0 + wm0) >> 4);
-  const uint32_t xtiles = (uint32_t)(Mp >> 4);
+  const uint32_t xtile0 = (uint32_t)xblk0 + (uint32_t)((m0 + wm0) >> 4);
   u32x4 xring[4][TM];
   uint32_t xtoff[TM];                                 // scalar: byte offset of tile b's block row
 #pragma unroll
@@ -414,8 +450,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   for (int i = 0; i < B_CH; ++i) {
     const int c = tid + i * 256;
     const int row = c / CPR, kc = c % CPR;
-    const int n = n0 + row;
-    const uint32_t dead = (uint32_t)(!(n < N && row < BN)) << 31;
+    const int n = tile_row(row);
+    const bool live = FUSE ? (n0 + (row >> 5) * 16 + (row & 15) < p.n_half) : (n < N);
+    const uint32_t dead = (uint32_t)(!(live && row < BN)) << 31;
     Fmt::chunk_addr(res, n, kc, K, boff[i], soff[i]);
     boff[i] |= dead;
     soff[i] |= dead;
@@ -517,9 +554,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   // D = W-tile (rows n) x X-tile^T: lane holds n = 4 g + v (v = 0..3), m = j
   Elem* out = (Elem*)p.out;
+  const int n_out = FUSE ? p.n_half : N;              // output columns
+  // output row of this lane's row of activation tile b, or -1
+  int orow[TM];
+  float rw[TM];
 #pragma unroll
-  for (int a = 0; a < TN; ++a) {
-    const int n = n0 + wn0 + a * 16 + g * 4;
+  for (int b = 0; b < TM; ++b) {
+    const int m = m0 + wm0 + b * 16 + j;
+    orow[b] = m < M ? m : -1;
+    rw[b] = 1.0f;
+    if constexpr (GROUPED) {
+      if (m < M) {
+        const int pos = row0 + m;
+        const int dst = p.out_map ? p.out_map[pos] : pos;
+        orow[b] = (unsigned)dst < (unsigned)p.out_rows ? dst : -1;   // a mapped row outside the output is dropped
+        if (p.row_weight && orow[b] >= 0) rw[b] = Act::to_f32(((const Elem*)p.row_weight)[dst]);
+      }
+    }
+  }
+  constexpr int TNO = FUSE ? TN / 2 : TN;             // output column tiles of this wavefront
+#pragma unroll
+  for (int ao = 0; ao < TNO; ++ao) {
+    const int a = FUSE ? 2 * ao : ao;
+    // first of this lane's 4 output columns; FUSE: gate tile a pairs with up tile a + 1
+    const int n = FUSE ? n0 + (wn0 >> 1) + ao * 16 + g * 4 : n0 + wn0 + a * 16 + g * 4;
     float os[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     if constexpr (Fmt::kOutScale) {
 #pragma unroll
@@ -527,18 +585,34 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
     }
 #pragma unroll
     for (int b = 0; b < TM; ++b) {
-      const int m = m0 + wm0 + b * 16 + j;
-      if (m < M) {
+      if (orow[b] >= 0) {
         Elem v4[4];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) v4[v] = Act::from_f32(Fmt::kOutScale ? acc[a][b][v] * os[v] : acc[a][b][v]);
-        Elem* dst = out + (size_t)m * N + n;
-        if (n + 3 < N && (N & 3) == 0) {
+        for (int v = 0; v < 4; ++v) {
+          float r;
+          if constexpr (FUSE) {
+            // per-tensor / per-expert scale only: one factor for gate and up
+            const float gate = acc[a][b][v] * os[v], up = acc[a + 1][b][v] * os[v];
+            if (p.gelu) {
+              float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
+              two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
+              const float ex = __expf(two_z);
+              r = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up;
+            } else {
+              r = gate / (1.0f + __expf(-gate)) * up;
+            }
+          } else {
+            r = Fmt::kOutScale ? acc[a][b][v] * os[v] : acc[a][b][v];
+          }
+          v4[v] = Act::from_f32(GROUPED ? r * rw[b] : r);
+        }
+        Elem* dst = out + (size_t)orow[b] * n_out + n;
+        if (n + 3 < n_out && (n_out & 3) == 0) {
           *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(v4);
         } else {
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            if (n + v < N) dst[v] = v4[v];
+            if (n + v < n_out) dst[v] = v4[v];
         }
       }
     }

@@ -24,6 +24,7 @@
 // Output rows may be scattered through a map (sorted position -> destination row)
 // and scaled by a per-destination-row weight.
 #include "qlinear_common.hpp"
+#include "scratch.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -73,7 +74,10 @@ constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of
 // The weights are the MFMA A operand and the activations the B operand, so a lane
 // ends up holding ONE activation row (16 w + j) and four consecutive weight rows
 // (4 g + v): the per-row activation scale is a single value per lane and granule.
-template <class Act, bool A8, bool SILU, int RT, int D, bool PE>
+// MT = 16-row activation tiles per wavefront and pass (1: up to 64 rows per pass, the decode /
+// small-prefill case; 4: up to 256 rows per pass for experts with hundreds of rows, so that a
+// weight granule fetched once serves four times as many rows).
+template <class Act, bool A8, bool SILU, int RT, int D, bool PE, int MT = 1>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, const float* __restrict__ w_scale,
                                                         const int32_t* __restrict__ expert_start) {
   static_assert(RT == 2 || RT == 4 || RT == 8, "two, four or eight weight tiles");
@@ -85,7 +89,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   constexpr uint32_t AGran = A8 ? 128u : 256u;        // activation bytes per row per granule
   constexpr int kWBuf = RT * 16 * kWPitch;
   constexpr int kCols = SILU ? (RT / 2) * 16 : RT * 16;   // output columns per tile group
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kWBuf + 4 * 16 * APitch];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // 2 * kWBuf + 4 * MT * 16 * APitch
 
   const int e = blockIdx.x / p.tiles_per_expert;
   const int wg = blockIdx.x - e * p.tiles_per_expert;
@@ -124,7 +128,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
     wvoff[i] = (uint32_t)(tile_hi(t) + wcol[i]) * (uint32_t)K + (uint32_t)ch * 16u;
     wlds[i] = smem + row * kWPitch + ch * 16;
   }
-  unsigned char* al = smem + 2 * kWBuf + wave * 16 * APitch;
+  unsigned char* al = smem + 2 * kWBuf + wave * MT * 16 * APitch;
 
   const uint8_t* wexp = (const uint8_t*)p.w + (size_t)e * N * K;
   const __amdgpu_buffer_rsrc_t wr = make_rsrc(wexp, (uint32_t)N * (uint32_t)K);
@@ -141,37 +145,41 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
 
   struct Regs {                                       // one granule in flight
     u32x4 w[WL];
-    u32x4 a[NAI];
-    float xs;
+    u32x4 a[MT][NAI];
+    float xs[MT];
   };
+  constexpr int kPassRows = 64 * MT;                  // rows of the expert per pass over its weights
 
-  for (int mc = 0; mc < cnt; mc += 64) {
-    const int rows_here = min(64, cnt - mc);
-    const bool active = wave * 16 < rows_here;        // wave-uniform
+  for (int mc = 0; mc < cnt; mc += kPassRows) {
+    const int rows_here = min(kPassRows, cnt - mc);
+    const int wrow0 = wave * 16 * MT;                 // first row of this wavefront inside the pass
     // source row of this lane's activation row (MFMA layout) and staging slots
-    uint32_t xsoff;
-    {
-      const int m = mc + wave * 16 + j;
-      const bool ok = m < cnt;
-      const int pos = r0 + (ok ? m : 0);
-      const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
-      xsoff = (src * (uint32_t)Kb * 4u) | ((uint32_t)(!ok) << 31);
-    }
-    uint32_t aoff[NAI];
-    int ach[NAI];
-    unsigned char* alds[NAI];
+    uint32_t xsoff[MT];
 #pragma unroll
-    for (int i = 0; i < NAI; ++i) {
-      const int row = A8 ? (lane >> 3) + 8 * i : (lane >> 4) + 4 * i;
-      const int ch = A8 ? (lane & 7) : (lane & 15);
-      const int m = mc + wave * 16 + row;
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mc + wrow0 + mt * 16 + j;
       const bool ok = m < cnt;
       const int pos = r0 + (ok ? m : 0);
       const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
-      aoff[i] = (src * (uint32_t)K * a_esz + (uint32_t)ch * 16u) | ((uint32_t)(!ok) << 31);
-      alds[i] = al + row * APitch + ch * 16;
-      ach[i] = A8 ? ch * 16 : ch * 8;                 // first k of the chunk inside the granule
+      xsoff[mt] = (src * (uint32_t)Kb * 4u) | ((uint32_t)(!ok) << 31);
     }
+    uint32_t aoff[MT][NAI];
+    int ach[NAI];
+    unsigned char* alds[MT][NAI];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < NAI; ++i) {
+        const int row = A8 ? (lane >> 3) + 8 * i : (lane >> 4) + 4 * i;
+        const int ch = A8 ? (lane & 7) : (lane & 15);
+        const int m = mc + wrow0 + mt * 16 + row;
+        const bool ok = m < cnt;
+        const int pos = r0 + (ok ? m : 0);
+        const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
+        aoff[mt][i] = (src * (uint32_t)K * a_esz + (uint32_t)ch * 16u) | ((uint32_t)(!ok) << 31);
+        alds[mt][i] = al + (mt * 16 + row) * APitch + ch * 16;
+        ach[i] = A8 ? ch * 16 : ch * 8;               // first k of the chunk inside the granule
+      }
 
     // issue the loads of granule gi of tile group tg (dead beyond the last one)
     auto load_granule = [&](Regs& r, int tg, int gi) {
@@ -185,11 +193,15 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
         r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i] | dead | ((uint32_t)(!ok) << 31), wso, 2);
       }
 #pragma unroll
-      for (int i = 0; i < NAI; ++i)
-        r.a[i] = __builtin_amdgcn_raw_buffer_load_b128(ar, aoff[i] | dead | ((uint32_t)(ach[i] >= kext) << 31),
-                                                       (uint32_t)gi * AGran, 0);
-      if constexpr (A8)
-        r.xs = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xsr, xsoff | dead, (uint32_t)gi * 4u, 0));
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int i = 0; i < NAI; ++i)
+          r.a[mt][i] = __builtin_amdgcn_raw_buffer_load_b128(ar, aoff[mt][i] | dead | ((uint32_t)(ach[i] >= kext) << 31),
+                                                             (uint32_t)gi * AGran, 0);
+        if constexpr (A8)
+          r.xs[mt] = __builtin_bit_cast(float,
+                                        __builtin_amdgcn_raw_buffer_load_b32(xsr, xsoff[mt] | dead, (uint32_t)gi * 4u, 0));
+      }
     };
 
     Regs r[D];
@@ -201,11 +213,13 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       __builtin_amdgcn_sched_barrier(0);
     }
 
-    f32x4 acc[RT];
+    f32x4 acc[MT][RT];
     int odd_par = 0;
     for (int tg = 0; tg < ntg; ++tg) {
 #pragma unroll
-      for (int t = 0; t < RT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
       int nb[RT];
 #pragma unroll
       for (int t = 0; t < RT; ++t) nb[t] = min((tile_hi(t) + col0 + tg * kCols + tile_col(t)) >> 7, Nb - 1);
@@ -222,19 +236,22 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
 #pragma unroll
           for (int i = 0; i < WL; ++i) *reinterpret_cast<u32x4*>(wlds[i] + par * kWBuf) = r[s].w[i];
 #pragma unroll
-          for (int i = 0; i < NAI; ++i) *reinterpret_cast<u32x4*>(alds[i]) = r[s].a[i];
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < NAI; ++i) *reinterpret_cast<u32x4*>(alds[mt][i]) = r[s].a[mt][i];
           // The activation scale is taken out of the ring slot before the slot is reloaded
           // below.  Left to the scheduler, the multiply sinks under the reload, old and new
           // value overlap, and the loop latch gets a register copy of the NEW value, i.e. a
           // wait for every load in flight on each turn.
-          float xs_now = A8 ? r[s].xs : 1.0f;
-          asm volatile("" : "+v"(xs_now));
-          float sc[RT];
+          float xs_now[MT];
 #pragma unroll
-          for (int t = 0; t < RT; ++t) {
-            const float ws = PE ? ws_expert : wsc[(size_t)nb[t] * Kb + gi];
-            sc[t] = A8 ? xs_now * ws : ws;
+          for (int mt = 0; mt < MT; ++mt) {
+            xs_now[mt] = A8 ? r[s].xs[mt] : 1.0f;
+            asm volatile("" : "+v"(xs_now[mt]));
           }
+          float wsv[RT];
+#pragma unroll
+          for (int t = 0; t < RT; ++t) wsv[t] = PE ? ws_expert : wsc[(size_t)nb[t] * Kb + gi];
           // prefetch D granules ahead, across the tile-group boundary
           {
             int ngi = gi + D, ntgi = tg;
@@ -242,46 +259,50 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
             load_granule(r[s], ntgi, ngi);
           }
           __syncthreads();
-          if (active) {
+          if (wrow0 < rows_here) {                    // wave-uniform: this wavefront has rows in the pass
             u32x4 wf[RT][2];
 #pragma unroll
             for (int t = 0; t < RT; ++t)
 #pragma unroll
               for (int i = 0; i < 2; ++i)
                 wf[t][i] = *reinterpret_cast<const u32x4*>(wbuf + (t * 16 + j) * kWPitch + g * 32 + i * 16);
-            if constexpr (A8) {
-              const u32x4 x0 = *reinterpret_cast<const u32x4*>(al + j * APitch + g * 32);
-              const u32x4 x1 = *reinterpret_cast<const u32x4*>(al + j * APitch + g * 32 + 16);
-              const long xa = (long)(((uint64_t)x0[1] << 32) | x0[0]);
-              const long xb = (long)(((uint64_t)x0[3] << 32) | x0[2]);
-              const long xc = (long)(((uint64_t)x1[1] << 32) | x1[0]);
-              const long xd = (long)(((uint64_t)x1[3] << 32) | x1[2]);
 #pragma unroll
-              for (int t = 0; t < RT; ++t) {
-                const long w0 = (long)(((uint64_t)wf[t][0][1] << 32) | wf[t][0][0]);
-                const long w1 = (long)(((uint64_t)wf[t][0][3] << 32) | wf[t][0][2]);
-                const long w2 = (long)(((uint64_t)wf[t][1][1] << 32) | wf[t][1][0]);
-                const long w3 = (long)(((uint64_t)wf[t][1][3] << 32) | wf[t][1][2]);
-                f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-                tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, xa, tt, 0, 0, 0);
-                tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, xb, tt, 0, 0, 0);
-                tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, xc, tt, 0, 0, 0);
-                tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, xd, tt, 0, 0, 0);
-                acc[t] += tt * sc[t];
-              }
-            } else {
-              V8 xf[4];
+            for (int mt = 0; mt < MT; ++mt) {
+              if (MT > 1 && wrow0 + mt * 16 >= rows_here) continue;    // wave-uniform
+              const unsigned char* am = al + (mt * 16 + j) * APitch;
+              if constexpr (A8) {
+                const u32x4 x0 = *reinterpret_cast<const u32x4*>(am + g * 32);
+                const u32x4 x1 = *reinterpret_cast<const u32x4*>(am + g * 32 + 16);
+                const long xa = (long)(((uint64_t)x0[1] << 32) | x0[0]);
+                const long xb = (long)(((uint64_t)x0[3] << 32) | x0[2]);
+                const long xc = (long)(((uint64_t)x1[1] << 32) | x1[0]);
+                const long xd = (long)(((uint64_t)x1[3] << 32) | x1[2]);
 #pragma unroll
-              for (int i = 0; i < 4; ++i)
-                xf[i] = *reinterpret_cast<const V8*>(al + j * APitch + g * 64 + i * 16);
+                for (int t = 0; t < RT; ++t) {
+                  const long w0 = (long)(((uint64_t)wf[t][0][1] << 32) | wf[t][0][0]);
+                  const long w1 = (long)(((uint64_t)wf[t][0][3] << 32) | wf[t][0][2]);
+                  const long w2 = (long)(((uint64_t)wf[t][1][1] << 32) | wf[t][1][0]);
+                  const long w3 = (long)(((uint64_t)wf[t][1][3] << 32) | wf[t][1][2]);
+                  f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
+                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, xa, tt, 0, 0, 0);
+                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, xb, tt, 0, 0, 0);
+                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, xc, tt, 0, 0, 0);
+                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, xd, tt, 0, 0, 0);
+                  acc[mt][t] += tt * (xs_now[mt] * wsv[t]);
+                }
+              } else {
+                V8 xf[4];
 #pragma unroll
-              for (int t = 0; t < RT; ++t) {
-                f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-                tt = Act::mfma(fp8x8_to_act<Act>(wf[t][0][0], wf[t][0][1]), xf[0], tt);
-                tt = Act::mfma(fp8x8_to_act<Act>(wf[t][0][2], wf[t][0][3]), xf[1], tt);
-                tt = Act::mfma(fp8x8_to_act<Act>(wf[t][1][0], wf[t][1][1]), xf[2], tt);
-                tt = Act::mfma(fp8x8_to_act<Act>(wf[t][1][2], wf[t][1][3]), xf[3], tt);
-                acc[t] += tt * sc[t];
+                for (int i = 0; i < 4; ++i) xf[i] = *reinterpret_cast<const V8*>(am + g * 64 + i * 16);
+#pragma unroll
+                for (int t = 0; t < RT; ++t) {
+                  f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
+                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][0][0], wf[t][0][1]), xf[0], tt);
+                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][0][2], wf[t][0][3]), xf[1], tt);
+                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][1][0], wf[t][1][1]), xf[2], tt);
+                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][1][2], wf[t][1][3]), xf[3], tt);
+                  acc[mt][t] += tt * wsv[t];
+                }
               }
             }
           }
@@ -289,8 +310,10 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       }
 
       // ---- epilogue of this tile group: lane holds row 16 w + j, weight rows 4 g + v ----
-      const int m = mc + wave * 16 + j;
-      const int dst = (active && m < cnt) ? (p.out_map ? p.out_map[r0 + m] : r0 + m) : -1;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+      const int m = mc + wrow0 + mt * 16 + j;
+      const int dst = m < cnt ? (p.out_map ? p.out_map[r0 + m] : r0 + m) : -1;
       if ((unsigned)dst < (unsigned)p.total_rows) {    // a mapped row outside the output is dropped
         Elem* out = (Elem*)p.out;
         float* out32 = (float*)p.out;
@@ -305,7 +328,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             if constexpr (SILU) {
-              const float gate = acc[t][v], up = acc[t + 1][v];
+              const float gate = acc[mt][t][v], up = acc[mt][t + 1][v];
               if (p.gelu) {
                 // 0.5 g (1 + tanh z), tanh through exp(2z) with 2z held in [-30, 30]
                 float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
@@ -316,7 +339,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
                 v4[v] = gate / (1.0f + __expf(-gate)) * up * rw;
               }
             } else {
-              v4[v] = acc[t][v] * rw;
+              v4[v] = acc[mt][t][v] * rw;
             }
           }
           if (n + 3 < limit && (p.n_out & 3) == 0) {
@@ -335,12 +358,22 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
           }
         }
       }
+      }
     }
     __syncthreads();                                  // LDS is rewritten by the next pass
   }
 }
 
-template <class Act, bool A8, bool SILU, int RT, int D>
+template <class K>
+static void launch_moe_kernel(K kern, size_t lds, long wgs, const MoeGemmArgs& p, hipStream_t st, bool& raised) {
+  if (lds > 64 * 1024 && !raised) {                   // opt in to more than 64 KiB of dynamic LDS, once per kernel
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(256), lds, st, p, p.w_scale, p.start);
+}
+
+template <class Act, bool A8, bool SILU, int RT, int D, int MT = 1>
 static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
   // quantised activations only come with block scales (the per-expert form is the reference's w8a16 mode)
   constexpr bool kHasPE = !A8;
@@ -352,15 +385,15 @@ static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
   p.n_out = cols;
   const long wgs = (long)p.E * p.tiles_per_expert;
   if (wgs <= 0) return MI_OK;
+  const size_t lds = (size_t)2 * RT * 16 * kWPitch + (size_t)4 * MT * 16 * (A8 ? kWPitch : kA16Pitch);
+  static bool raised_pe = false, raised_block = false; // per instantiation of this function = per kernel
   if constexpr (kHasPE) {
     if (p.scale_per_expert) {
-      hipLaunchKernelGGL((moe_gemm_kernel<Act, A8, SILU, RT, D, true>), dim3((unsigned)wgs), dim3(256), 0, st, p,
-                         p.w_scale, p.start);
+      launch_moe_kernel(moe_gemm_kernel<Act, A8, SILU, RT, D, true, MT>, lds, wgs, p, st, raised_pe);
       return launch_status();
     }
   }
-  hipLaunchKernelGGL((moe_gemm_kernel<Act, A8, SILU, RT, D, false>), dim3((unsigned)wgs), dim3(256), 0, st, p,
-                     p.w_scale, p.start);
+  launch_moe_kernel(moe_gemm_kernel<Act, A8, SILU, RT, D, false, MT>, lds, wgs, p, st, raised_block);
   return launch_status();
 }
 
@@ -375,6 +408,9 @@ static int dispatch_moe2(const MoeGemmArgs& p, hipStream_t st) {
   // short K: walk two tile groups per workgroup so the prefetch pipeline stays filled
   const int tpw = (G < 16 && wgs_with(rt) >= 2048) ? 2 : 1;
   const bool d2 = (G % 2) == 0;                       // two granules in flight need an even count
+  // hundreds of rows per expert (prefill): 256 rows per pass over the weights instead of 64
+  if (rt == 8 && (long)p.total_rows > 96L * p.E)
+    return d2 ? launch_moe<Act, A8, SILU, 8, 2, 4>(p, 1, st) : launch_moe<Act, A8, SILU, 8, 1, 4>(p, 1, st);
   if (rt == 8) return d2 ? launch_moe<Act, A8, SILU, 8, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 8, 1>(p, tpw, st);
   if (rt == 4) return d2 ? launch_moe<Act, A8, SILU, 4, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 4, 1>(p, tpw, st);
   return d2 ? launch_moe<Act, A8, SILU, 2, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 2, 1>(p, tpw, st);
@@ -404,6 +440,15 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || (uint64_t)a_rows * (uint64_t)K * 2 >= (1ull << 31))
     return MI_ERR_SHAPE;
   if (!E || !total_rows) return MI_OK;
+  // prefill (experts averaging 96 rows or more, 16-bit activations and output): the tiled matrix-core GEMM
+  if (!a_scale && !out_f32 && (K % 128) == 0 && E <= 1024 && (long)total_rows >= 96L * E) {
+    long long bytes = 0;
+    if (mi_moe_gemm_fp8_tiled_workspace(total_rows, E, K, &bytes) != MI_OK) return MI_ERR_SHAPE;
+    void* ws = scratch_get((hipStream_t)stream, (size_t)bytes);
+    if (!ws) return MI_ERR_LAUNCH;
+    return mi_moe_gemm_fp8_tiled_ws(a, row_map, w, w_scale, scale_per_expert, expert_start, out, out_map, row_weight,
+                                    a_rows, total_rows, E, N, K, fuse_act, act_dtype, ws, bytes, stream);
+  }
   MoeGemmArgs p{};
   p.a = a; p.a_scale = a_scale; p.row_map = row_map; p.w = w; p.w_scale = w_scale;
   p.start = expert_start; p.out = out; p.E = E; p.N = N; p.K = K; p.a_rows = a_rows;

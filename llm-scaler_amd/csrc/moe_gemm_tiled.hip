@@ -1,0 +1,199 @@
+// Grouped (per-expert) FP8 weight GEMM for MoE prefill: experts with hundreds of rows.
+//
+// The weight-streaming grouped kernel (moe_gemm.hip) is built for a few dozen rows per expert;
+// with hundreds it is bound by LDS traffic, not by the matrix cores.  Here the expert-sorted rows
+// run through the tiled matrix-core GEMM of gemm_tiled.hpp instead (w8a16: fp16 / bf16
+// activations, FP8 weights with 128x128 block scales or one scale per expert):
+//   1. one small workgroup turns expert_start into a table of M-tiles (expert, first row, rows)
+//      and of 16-row activation blocks, every expert padded to whole blocks;
+//   2. the activations are gathered (row_map) and re-tiled into MFMA operand order per block;
+//   3. the GEMM runs one workgroup per (M-tile, N-tile); the grid is the host-side upper bound
+//      of the tile count and surplus workgroups exit at once.
+// Optional fused epilogue act(gate) * up (SiLU or tanh-GELU), output row map and per-row factor
+// as in the weight-streaming kernel.
+#include "gemm_tiled.hpp"
+#include "scratch.hpp"
+#include "../../include/mi355x_qlinear.h"
+
+namespace qlin {
+
+template <class Act, int BN> using WFp8PlainG = WFp8<Act, BN, false>;
+template <class Act, int BN> using WFp8BlockG = WFp8<Act, BN, true>;
+
+constexpr int kMapThreads = 1024;
+
+// exclusive scan of one value per thread over the 1024-thread workgroup
+__device__ __forceinline__ int map_scan(int v, int* tmp, int tid) {
+  tmp[tid] = v;
+  __syncthreads();
+  for (int off = 1; off < kMapThreads; off <<= 1) {
+    const int add = tid >= off ? tmp[tid - off] : 0;
+    __syncthreads();
+    tmp[tid] += add;
+    __syncthreads();
+  }
+  return tmp[tid] - v;
+}
+
+// g_tile[4 i] = {expert, first sorted row, rows, first activation block} per M-tile of `bm` rows;
+// blk[2 b] = {first sorted row, rows} per 16-row activation block; counts[0] = M-tiles,
+// counts[1] = blocks.  E <= 1024.
+__global__ __launch_bounds__(kMapThreads) void moe_tile_map_kernel(const int32_t* __restrict__ start, int E, int bm,
+                                                                   int32_t* __restrict__ g_tile,
+                                                                   int32_t* __restrict__ blk,
+                                                                   int32_t* __restrict__ counts) {
+  __shared__ int tmp[kMapThreads];
+  const int e = threadIdx.x;
+  const int r0 = e < E ? start[e] : 0;
+  const int cnt = e < E ? max(start[e + 1] - r0, 0) : 0;
+  const int nb = (cnt + 15) >> 4, nt = (cnt + bm - 1) / bm;
+  const int boff = map_scan(nb, tmp, e);
+  __syncthreads();
+  const int toff = map_scan(nt, tmp, e);
+  for (int i = 0; i < nt; ++i) {
+    int32_t* t = g_tile + 4 * (toff + i);
+    t[0] = e;
+    t[1] = r0 + i * bm;
+    t[2] = min(bm, cnt - i * bm);
+    t[3] = boff + i * (bm >> 4);
+  }
+  for (int b = 0; b < nb; ++b) {
+    blk[2 * (boff + b)] = r0 + 16 * b;
+    blk[2 * (boff + b) + 1] = min(16, cnt - 16 * b);
+  }
+  if (e == kMapThreads - 1) {                          // inclusive totals sit in the last thread
+    counts[0] = toff + nt;
+    counts[1] = boff + nb;
+  }
+}
+
+// Gather + re-tile: block b of the table -> MFMA operand order (see pack_x_kernel); rows past the
+// block's count are zero.  One workgroup writes four 32-wide steps of one block.
+__global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __restrict__ x,
+                                                             const int32_t* __restrict__ row_map,
+                                                             const int32_t* __restrict__ blk,
+                                                             const int32_t* __restrict__ counts,
+                                                             u32x4* __restrict__ xp, int a_rows, int K, int Q) {
+  const int b = blockIdx.y;
+  if (b >= counts[1]) return;
+  const int l = threadIdx.x & 63;
+  const int q = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (q >= Q) return;
+  const int r = l & 15;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (r < blk[2 * b + 1]) {
+    const int pos = blk[2 * b] + r;
+    const int src = row_map ? row_map[pos] : pos;
+    if ((unsigned)src < (unsigned)a_rows)
+      v = *reinterpret_cast<const u32x4*>(x + (size_t)src * K + q * 32 + (l >> 4) * 8);
+  }
+  xp[((size_t)b * Q + q) * 64 + l] = v;
+}
+
+struct TiledMoeLayout {
+  long long x_bytes, tile_off, blk_off, cnt_off, total;
+  int max_blocks, max_tiles;
+};
+static inline TiledMoeLayout tiled_moe_layout(int total_rows, int E, int K, int bm) {
+  TiledMoeLayout L;
+  L.max_blocks = total_rows / 16 + E;
+  L.max_tiles = total_rows / bm + E;
+  L.x_bytes = (long long)L.max_blocks * 16 * K * 2;
+  L.tile_off = (L.x_bytes + 255) & ~255LL;
+  L.blk_off = L.tile_off + (((long long)L.max_tiles * 16 + 255) & ~255LL);
+  L.cnt_off = L.blk_off + (((long long)L.max_blocks * 8 + 255) & ~255LL);
+  L.total = L.cnt_off + 256;
+  return L;
+}
+// rows per M-tile: 256 once the experts average enough rows to fill such tiles
+static inline int tiled_moe_bm(int total_rows, int E) { return (long)total_rows >= 160L * E ? 256 : 128; }
+
+template <class Act, template <class, int> class FMT, bool FUSE>
+static int launch_grouped(GemmArgs p, int bm, int max_tiles, hipStream_t st) {
+  p.tiles_m = max_tiles;
+  if (bm == 256) {
+    constexpr int BN = 256;
+    p.tiles_n = FUSE ? (p.n_half + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
+    using F = FMT<Act, BN>;
+    auto kern = gemm_tiled_kernel<Act, F, 256, BN, true, FUSE>;
+    const size_t lds = (size_t)2 * (F::B_CH * 256 / F::CPR) * kPitch * 2;
+    static bool raised = false;
+    if (lds > 64 * 1024 && !raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+          hipSuccess)
+        return MI_ERR_LAUNCH;
+      raised = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), lds, st, p);
+  } else {
+    constexpr int BN = 128;
+    p.tiles_n = FUSE ? (p.n_half + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
+    using F = FMT<Act, BN>;
+    const size_t lds = (size_t)2 * (F::B_CH * 256 / F::CPR) * kPitch * 2;
+    hipLaunchKernelGGL((gemm_tiled_kernel<Act, F, 128, BN, true, FUSE>), dim3((unsigned)(p.tiles_m * p.tiles_n)),
+                       dim3(256), lds, st, p);
+  }
+  return launch_status();
+}
+
+template <class Act>
+static int run_grouped(const GemmArgs& p, bool per_expert, int fuse, int bm, int max_tiles, hipStream_t st) {
+  if (per_expert)
+    return fuse ? launch_grouped<Act, WFp8PlainG, true>(p, bm, max_tiles, st)
+                : launch_grouped<Act, WFp8PlainG, false>(p, bm, max_tiles, st);
+  return fuse ? launch_grouped<Act, WFp8BlockG, true>(p, bm, max_tiles, st)
+              : launch_grouped<Act, WFp8BlockG, false>(p, bm, max_tiles, st);
+}
+
+}  // namespace qlin
+
+using namespace qlin;
+
+extern "C" {
+
+int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes) {
+  if (!bytes) return MI_ERR_ARG;
+  if (total_rows < 0 || E < 0 || E > kMapThreads || K <= 0) return MI_ERR_SHAPE;
+  *bytes = tiled_moe_layout(total_rows, E, K, 128).total;      // the larger of the two tile tables
+  return MI_OK;
+}
+
+int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* w, const float* w_scale,
+                             int scale_per_expert, const int32_t* expert_start, void* out, const int32_t* out_map,
+                             const void* row_weight, int a_rows, int total_rows, int E, int N, int K, int fuse_act,
+                             int act_dtype, void* workspace, long long workspace_bytes, void* stream) {
+  if (!a || !w || !w_scale || !expert_start || !out) return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (fuse_act < 0 || fuse_act > 2) return MI_ERR_ARG;
+  if (E < 0 || E > kMapThreads || N <= 0 || K <= 0 || (K % 128) || a_rows < 0 || total_rows < 0) return MI_ERR_SHAPE;
+  if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
+  if ((uint64_t)N * (uint64_t)K >= (1ull << 31)) return MI_ERR_SHAPE;
+  if (!E || !total_rows) return MI_OK;
+  const int bm = tiled_moe_bm(total_rows, E);
+  const TiledMoeLayout L = tiled_moe_layout(total_rows, E, K, bm);
+  if ((uint64_t)L.x_bytes >= (1ull << 31)) return MI_ERR_SHAPE;
+  if (!workspace || workspace_bytes < tiled_moe_layout(total_rows, E, K, 128).total) return MI_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  int32_t* g_tile = (int32_t*)(ws + L.tile_off);
+  int32_t* blk = (int32_t*)(ws + L.blk_off);
+  int32_t* counts = (int32_t*)(ws + L.cnt_off);
+  hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(kMapThreads), 0, st, expert_start, E, bm, g_tile, blk, counts);
+  const int Q = K / 32;
+  hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((Q + 3) / 4, L.max_blocks), dim3(256), 0, st, (const uint16_t*)a,
+                     row_map, blk, counts, (u32x4*)ws, a_rows, K, Q);
+  GemmArgs p{};
+  p.x = ws; p.w = w; p.scale = w_scale; p.out = out; p.M = total_rows; p.N = N; p.K = K;
+  p.scale_mode = scale_per_expert ? 1 : 2;
+  p.g_tile = g_tile; p.g_count = counts;
+  p.g_w_stride = (long long)N * K;
+  p.g_s_stride = scale_per_expert ? 4 : (long long)((N + 127) / 128) * (K / 128) * 4;
+  p.out_map = out_map; p.row_weight = row_weight;
+  p.x_blocks = L.max_blocks;
+  p.n_half = N / 2; p.gelu = fuse_act == 2;
+  p.out_rows = total_rows;
+  return act_dtype == DT_F16 ? run_grouped<ActF16>(p, scale_per_expert != 0, fuse_act, bm, L.max_tiles, st)
+                             : run_grouped<ActBF16>(p, scale_per_expert != 0, fuse_act, bm, L.max_tiles, st);
+}
+
+}  // extern "C"

@@ -970,6 +970,17 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
     if row_weight is not None:
         _chk(out.dtype != torch.float32 and row_weight.dtype == out.dtype and row_weight.is_contiguous() and
              row_weight.numel() >= total, f"{who}: row weights must share the output dtype, one per output row")
+    if a_scale is None and out.dtype != torch.float32 and K % 128 == 0 and E <= 1024 and total >= 96 * E:
+        # prefill: the tiled matrix-core GEMM, workspace from the caching allocator (graph-capturable)
+        need = ctypes.c_longlong(0)
+        rc = capi.lib().mi_moe_gemm_fp8_tiled_workspace(total, E, K, ctypes.byref(need))
+        if rc != 0:
+            raise RuntimeError(f"{who}: {capi.MI_ERRORS.get(rc, rc)}")
+        buf = torch.empty(need.value, dtype=torch.uint8, device=out.device)
+        capi.call("mi_moe_gemm_fp8_tiled_ws", out, capi.ptr(a), capi.ptr(row_map), capi.ptr(w), capi.ptr(w_scale),
+                  1 if per_expert else 0, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map), capi.ptr(row_weight),
+                  a_rows, total, E, N, K, fuse, adt, capi.ptr(buf), need.value)
+        return out
     capi.call("mi_moe_gemm_fp8_grouped", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), capi.ptr(w),
               capi.ptr(w_scale), 1 if per_expert else 0, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map),
               capi.ptr(row_weight), a_rows, total, E, N, K, fuse, adt, 1 if out.dtype == torch.float32 else 0)
@@ -1039,7 +1050,10 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
     inv = torch.empty(P, dtype=torch.int32, device=dev)
     sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
     inter = torch.empty(P, I, dtype=x.dtype, device=dev)
-    y = torch.empty(P, H, dtype=torch.float32, device=dev)      # fp32: the combine adds K rounded terms otherwise
+    # fp32 expert outputs (the combine adds K rounded terms otherwise); in the w8a16 prefill regime the
+    # tiled grouped GEMM takes over, which writes the activation type
+    prefill = (not act_quant) and P >= 96 * E
+    y = torch.empty(P, H, dtype=x.dtype if prefill else torch.float32, device=dev)
     if act_quant:
         xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
         xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)

@@ -285,6 +285,54 @@ def test_moe_gemm_skewed_experts(v, dev, counts, a8):
     assert O.max_rel_err(out.cpu(), ref) < TOL
 
 
+@pytest.mark.parametrize("counts,dt,fuse,gather", [
+    ([300, 0, 129, 257], torch.float16, False, False), ([97, 260, 100, 511, 16], torch.bfloat16, False, True),
+    ([400, 33, 290], torch.bfloat16, True, True), ([256, 256, 256, 256], torch.float16, True, False),
+    ([1, 0, 700], torch.float16, False, False)])
+def test_moe_gemm_prefill_tiled(v, dev, counts, dt, fuse, gather):
+    # experts averaging 96 rows or more (w8a16): the grouped launch of the tiled matrix-core GEMM, with
+    # empty experts, partial last tiles, a row gather and the fused SiLU * up epilogue
+    E, N, K = len(counts), 384, 512
+    g = torch.Generator().manual_seed(sum(counts) + fuse)
+    total = sum(counts)
+    st = torch.zeros(E + 1, dtype=torch.int32)
+    st[1:] = torch.tensor(counts).cumsum(0)
+    nsrc = total // 2 if gather else total
+    src = (torch.randn(nsrc, K, generator=g) * 0.5).to(dt)
+    row_map = torch.randint(0, nsrc, (total,), generator=g).to(torch.int32) if gather else None
+    x = src[row_map.long()] if gather else src
+    w8, ws = O.fp8_quantize_block(torch.randn(E, N, K, generator=g) * 0.05)
+    dw = O.fp8_dequant_block(w8, ws, out_dtype=dt)     # the block scale is folded into 16-bit weights on this path
+    n_out = N // 2 if fuse else N
+    out = torch.full((total, n_out), float("nan"), dtype=dt, device=dev)
+    v.moe_gemm_fp8_block(src.to(dev), None, None if row_map is None else row_map.to(dev), w8.to(dev), ws.to(dev),
+                         st.to(dev), out, N, K, E, fuse)
+    ref = _grouped_ref(x, dw, counts)
+    if fuse:
+        ref = torch.nn.functional.silu(ref[:, :N // 2]) * ref[:, N // 2:]
+    o = out.cpu()
+    assert torch.isfinite(o.float()).all()
+    assert O.max_rel_err(o, ref) < TOL
+
+
+def test_moe_gemm_prefill_tiled_matches_streaming_kernel(v, dev):
+    # the same problem through both grouped kernels (the streaming one keeps fp32 output): agreement
+    # to the rounding of the 16-bit output and of the folded block scale
+    counts = [200, 150, 333]
+    E, N, K = len(counts), 256, 768
+    g = torch.Generator().manual_seed(5)
+    total = sum(counts)
+    st = torch.zeros(E + 1, dtype=torch.int32)
+    st[1:] = torch.tensor(counts).cumsum(0)
+    x = (torch.randn(total, K, generator=g) * 0.5).half().to(dev)
+    w8, ws = O.fp8_quantize_block(torch.randn(E, N, K, generator=g) * 0.05)
+    a = torch.empty(total, N, dtype=torch.float16, device=dev)
+    b = torch.empty(total, N, dtype=torch.float32, device=dev)
+    v.moe_gemm_fp8_block(x, None, None, w8.to(dev), ws.to(dev), st.to(dev), a, N, K, E, False)
+    v.moe_gemm_fp8_block(x, None, None, w8.to(dev), ws.to(dev), st.to(dev), b, N, K, E, False)
+    assert O.max_rel_err(a.cpu(), b.cpu()) < 5e-3
+
+
 # ------------------------------------------------------------------ full forward
 def _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq):
     """The fused op's own pipeline, run stage by stage through the same ops, so that the
@@ -370,6 +418,20 @@ def _check_forward(v, dev, T, E, K, H, I, aq, seed):
                                           (12, 16, 4, 256, 128, False), (1, 16, 4, 256, 128, True)])
 def test_moe_forward_small(v, dev, T, E, K, H, I, aq):
     _check_forward(v, dev, T, E, K, H, I, aq, seed=T + E)
+
+
+@pytest.mark.parametrize("T,E,K,H,I,dt", [(800, 8, 2, 256, 128, torch.bfloat16), (1100, 4, 2, 384, 256, torch.float16)])
+def test_moe_forward_w8a16_prefill(v, dev, T, E, K, H, I, dt):
+    """16-bit activations with >= 96 rows per expert on average: both grouped GEMMs take the tiled
+    matrix-core route and the expert outputs are kept in the activation type before the combine."""
+    x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I, seed=T, act_dtype=dt)
+    out = torch.empty(T, H, dtype=dt, device=dev)
+    v.moe_forward_fp8_block(x.to(dev), logits.to(dev), w13q.view(torch.float8_e4m3fn).to(dev), w13s.to(dev),
+                            w2q.view(torch.float8_e4m3fn).to(dev), w2s.to(dev), out, K, False)
+    rtw, rti = O.moe_topk(logits, K)
+    ref = O.moe_forward_grouped(x, rtw, rti, w13q, w13s, w2q, w2s, E, act_quant=False)
+    assert O.max_rel_err(out.cpu(), ref) < TOL
+    assert O.max_rel_err_abs_floor(out.cpu(), ref) < 3e-2
 
 
 def test_cfg3_moe_forward(v, dev):
