@@ -29,6 +29,7 @@
 // chunk as a sequence of small pieces, and an optional factor on the finished sums.
 #pragma once
 #include "qlinear_common.hpp"
+#include <type_traits>
 
 namespace qlin {
 
@@ -414,6 +415,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   const uint32_t xtiles = GROUPED ? (uint32_t)p.x_blocks : (uint32_t)(Mp >> 4);
   const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x, xtiles * 16u * (uint32_t)K * 2u);
   const typename Fmt::Res res = Fmt::make(p, expert);
+  // 16-row activation tile b of this wavefront inside the BM-row tile.  GROUPED: the two wavefront
+  // rows take the tiles alternately and a wavefront multiplies only the first TM, TM / 2 or TM / 4 of
+  // its tiles, whichever covers the `live` ones with rows of the expert in them (the K loop exists
+  // in these three lengths; a branch per MFMA costs more than it saves), so a short last tile of an
+  // expert costs a fraction of the matrix-core time.
+  const int wr = wave >> 1;
+  auto mtile = [&](int b) { return GROUPED ? 2 * b + wr : wr * TM + b; };
+  int live = TM;
+  if constexpr (GROUPED) live = __builtin_amdgcn_readfirstlane((((M + 15) >> 4) - wr + 1) >> 1);
   // weight row of row r of the LDS tile
   auto tile_row = [&](int r) { return FUSE ? n0 + (r >> 5) * 16 + (r & 15) + ((r >> 4) & 1) * p.n_half : n0 + r; };
 
@@ -426,12 +436,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   // ---- activations: register ring.  Block (16-row tile t, 32-wide step q) of the
   // re-tiled x sits at (t * Q + q) * 1024; tile and step enter as a scalar offset.
   const uint32_t xlane = (uint32_t)lane * 16u;
-  const uint32_t xtile0 = (uint32_t)xblk0 + (uint32_t)((m0 + wm0) >> 4);
+  const uint32_t xtile0 = (uint32_t)xblk0 + (uint32_t)(m0 >> 4);
   u32x4 xring[4][TM];
   uint32_t xtoff[TM];                                 // scalar: byte offset of tile b's block row
 #pragma unroll
   for (int b = 0; b < TM; ++b) {
-    const uint32_t t = xtile0 + b < xtiles ? xtile0 + b : xtiles - 1;     // tiles past M: any valid block
+    const uint32_t t = xtile0 + mtile(b) < xtiles ? xtile0 + mtile(b) : xtiles - 1;   // tiles past M: any valid block
     xtoff[b] = __builtin_amdgcn_readfirstlane(t * (uint32_t)Q * 1024u);
   }
   auto load_x1 = [&](int slot, int b, int q) {        // a step beyond the last re-reads the last (never used)
@@ -485,10 +495,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   // ring slots slot0 and slot0 + 1) while the next step's weights (`cur`, loaded one
   // step earlier) are dequantized into the other buffer and the weights two steps
   // ahead are fetched into `nxt`.
-  constexpr int kMfmas = 2 * TN * TM;
   // pieces are spread evenly over the MFMAs of the step: piece I goes behind the
   // first MFMA slot with (slot + 1) * kPieces / kMfmas > I
-  auto step64 = [&](int kt, int buf, int slot0, StageB& cur, StageB& nxt) {
+  auto step64 = [&](auto live_c, int kt, int buf, int slot0, StageB& cur, StageB& nxt) __attribute__((always_inline)) {
+    constexpr int L = decltype(live_c)::value;        // activation tiles multiplied (<= TM)
+    constexpr int kMfmas = 2 * TN * L;
     const Elem* Bb = Bs + buf * BNP * kPitch;
     DqState q;
     Fmt::begin(res, cur, q);
@@ -497,8 +508,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
     };
     // the weight operand of row a + 1 is fetched from LDS while row a is multiplied
     u32x4 wnext = rd_w(0, 0);
-    constexpr int kHalf = TN * TM;                    // MFMAs per 32-wide step
-    constexpr int kXEvery = kHalf / TM;               // one activation load per kXEvery MFMAs
+    constexpr int kHalf = TN * L;                     // MFMAs per 32-wide step
+    constexpr int kXEvery = kHalf / L;                // one activation load per kXEvery MFMAs
     constexpr int kBEvery = kHalf / kLoads > 0 ? kHalf / kLoads : 1;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -508,9 +519,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
         if (a + 1 < TN) wnext = rd_w(a + 1, s);
         else if (s == 0) wnext = rd_w(0, 1);
 #pragma unroll
-        for (int b = 0; b < TM; ++b) {
+        for (int b = 0; b < L; ++b) {
           mfma_agpr<Act>(acc[a][b], wcur, xring[slot0 + s][b]);
-          const int m = a * TM + b;                   // MFMA index inside this 32-wide step
+          const int m = a * L + b;                    // MFMA index inside this 32-wide step
           const int slot = s * kHalf + m;
           const int p0 = slot * kPieces / kMfmas, p1 = (slot + 1) * kPieces / kMfmas;
 #pragma unroll
@@ -518,7 +529,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
           // global loads, one at a time: the ring slot multiplied in the previous
           // 32-wide step is refilled 3 steps ahead, and in the first half the weight
           // chunks two 64-wide steps ahead are fetched
-          if (m % kXEvery == kXEvery / 2 && m / kXEvery < TM)
+          if (m % kXEvery == kXEvery / 2 && m / kXEvery < L)
             load_x1((slot0 + s + 3) & 3, m / kXEvery, 2 * kt + s + 3);
           if (s == 0 && m % kBEvery == 0 && m / kBEvery < kLoads) load_b1(nxt, kt + 2, m / kBEvery);
           // keep MFMAs, vector-ALU pieces and memory accesses in this order
@@ -545,9 +556,18 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
     for (int I = 0; I < kPieces; ++I) dq_piece(s0, 0, I, q);
   }
   __syncthreads();
-  for (int kt = 0; kt < KT; kt += 2) {
-    step64(kt, 0, 0, s1, s0);
-    step64(kt + 1, 1, 2, s0, s1);
+  auto k_loop = [&](auto live_c) __attribute__((always_inline)) {
+    for (int kt = 0; kt < KT; kt += 2) {
+      step64(live_c, kt, 0, 0, s1, s0);
+      step64(live_c, kt + 1, 1, 2, s0, s1);
+    }
+  };
+  if constexpr (!GROUPED) {
+    k_loop(std::integral_constant<int, TM>{});
+  } else {
+    if (live > TM / 2) k_loop(std::integral_constant<int, TM>{});
+    else if (live > TM / 4) k_loop(std::integral_constant<int, TM / 2>{});
+    else k_loop(std::integral_constant<int, (TM / 4 > 0 ? TM / 4 : 1)>{});
   }
 
   // the last MFMAs are still in the matrix pipe: wait before reading their results
@@ -560,7 +580,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   float rw[TM];
 #pragma unroll
   for (int b = 0; b < TM; ++b) {
-    const int m = m0 + wm0 + b * 16 + j;
+    const int m = m0 + mtile(b) * 16 + j;
     orow[b] = m < M ? m : -1;
     rw[b] = 1.0f;
     if constexpr (GROUPED) {

@@ -149,17 +149,28 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* wave_t
   return v + (wave ? wave_tot[wave - 1] : 0u);
 }
 
+struct SortSmem {
+  uint32_t bitmap[kSortWords];
+  uint32_t wordpre[kSortWords + 4];
+  int32_t count[1024];
+  int32_t start[1025];
+  int32_t base[1024];
+  int32_t own[1024];
+  uint32_t wave_tot[16];
+  int32_t mx;
+};
+
 __device__ __forceinline__ void moe_sort_body(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
-    int32_t* __restrict__ max_count, int T, int K, int E) {
-  __shared__ uint32_t bitmap[kSortWords];
-  __shared__ uint32_t wordpre[kSortWords + 4];
-  __shared__ int32_t count[1024];
-  __shared__ int32_t start[1025];
-  __shared__ int32_t base[1024];
-  __shared__ uint32_t wave_tot[16];
-  __shared__ int32_t mx;
+    int32_t* __restrict__ max_count, int T, int K, int E, SortSmem& sm) {
+  uint32_t (&bitmap)[kSortWords] = sm.bitmap;
+  uint32_t (&wordpre)[kSortWords + 4] = sm.wordpre;
+  int32_t (&count)[1024] = sm.count;
+  int32_t (&start)[1025] = sm.start;
+  int32_t (&base)[1024] = sm.base;
+  uint32_t (&wave_tot)[16] = sm.wave_tot;
+  int32_t& mx = sm.mx;
   const int tid = threadIdx.x;
   const int P = T * K;
   const int wpe = kSortWords / E;                     // words per expert in one chunk
@@ -298,11 +309,97 @@ __device__ __forceinline__ void moe_sort_body(
   }
 }
 
+// The same sort spread over several workgroups, for thousands of tokens: workgroup c owns the S
+// tokens from c * S on (S * E <= 32 * kSortWords, so that its pairs fit one bitmap).  Every
+// workgroup counts all pairs per expert (total, and those of earlier tokens than its own) — ids
+// are 4 bytes a pair and come out of L2 — derives the experts' first positions and its own first
+// position inside each expert from that, and places its own pairs by their rank in the bitmap.
+// Nothing passes between the workgroups.  Ids a top-k never produces: as in moe_sort_body (a
+// position that no pair claims lies at the end of the owning workgroup's part of an expert's range
+// and is filled by that workgroup).
+__device__ __forceinline__ void moe_sort_wide_body(
+    const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
+    int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
+    int32_t* __restrict__ max_count, int T, int K, int E, int S, int c, SortSmem& sm) {
+  const int tid = threadIdx.x;
+  const int P = T * K;
+  const int wpe = kSortWords / E;
+  const int lo = c * S, hi = min(T, lo + S);
+  const int p_lo = lo * K, p_hi = hi * K;
+  constexpr int WPT = kSortWords / kSortThreads;
+#pragma unroll
+  for (int i = 0; i < WPT; ++i) sm.bitmap[tid + i * kSortThreads] = 0;
+  sm.count[tid] = 0;                                  // pairs per expert, all tokens
+  sm.base[tid] = 0;                                   // ... of tokens before lo
+  sm.own[tid] = 0;                                    // ... of this workgroup's tokens
+  if (tid == 0) sm.mx = 0;
+  __syncthreads();
+  for (int p = tid; p < P; p += kSortThreads) {
+    const int e = sort_expert(top_ids, p, E);
+    atomicAdd(&sm.count[e], 1);
+    if (p < p_lo) {
+      atomicAdd(&sm.base[e], 1);
+    } else if (p < p_hi) {
+      const int tl = p / K - lo;
+      atomicAdd(&sm.own[e], 1);
+      atomicOr(&sm.bitmap[e * wpe + (tl >> 5)], 1u << (tl & 31));
+    }
+  }
+  __syncthreads();
+  const uint32_t mine = tid < E ? (uint32_t)sm.count[tid] : 0u;
+  const uint32_t incl = block_scan_1024(mine, sm.wave_tot, tid);
+  if (tid < E) sm.start[tid + 1] = (int32_t)incl;
+  if (tid == 0) sm.start[0] = 0;
+  int claimed = 0;
+  if (tid < E) {
+    for (int w = 0; w < wpe; ++w) {
+      sm.wordpre[tid * wpe + w] = (uint32_t)claimed;
+      claimed += __popc(sm.bitmap[tid * wpe + w]);
+    }
+    if (c == 0 && max_count) atomicMax(&sm.mx, (int)mine);
+  }
+  __syncthreads();
+  if (c == 0) {
+    for (int e = tid; e <= E; e += kSortThreads) expert_start[e] = sm.start[e];
+    if (max_count && tid == 0) max_count[0] = sm.mx;
+  }
+  for (int q = p_lo + tid; q < p_hi; q += kSortThreads) {
+    const int e = sort_expert(top_ids, q, E);
+    const int t = q / K, tl = t - lo;
+    const int wi = e * wpe + (tl >> 5);
+    const int pos = sm.start[e] + sm.base[e] + (int)sm.wordpre[wi] + __popc(sm.bitmap[wi] & ((1u << (tl & 31)) - 1u));
+    sorted_pairs[pos] = q;
+    inv[q] = pos;
+    if (sorted_token) sorted_token[pos] = t;
+  }
+  if (tid < E) {
+    const int first = sm.start[tid] + sm.base[tid];
+    for (int pos = first + claimed; pos < first + sm.own[tid]; ++pos) {
+      sorted_pairs[pos] = 0;
+      if (sorted_token) sorted_token[pos] = 0;
+    }
+  }
+}
+
+// Tokens per workgroup of the spread-out sort, or 0 where one workgroup does it all (few tokens, or
+// more than 256 workgroups' worth).
+static inline int sort_wide_span(int T, int E) {
+  const int cap = (kSortWords / E) * 32;              // tokens whose pairs fit one bitmap
+  if (T <= cap && T < 2048) return 0;
+  int S = (T + 63) / 64;
+  S = (S + 31) & ~31;
+  if (S < 128) S = 128;
+  if (S > cap) S = cap;
+  return (T + S - 1) / S <= 256 ? S : 0;
+}
+
 __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
-    int32_t* __restrict__ max_count, int T, int K, int E) {
-  moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+    int32_t* __restrict__ max_count, int T, int K, int E, int S) {
+  __shared__ SortSmem sm;
+  if (S) moe_sort_wide_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, S, blockIdx.x, sm);
+  else moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, sm);
 }
 
 // ---------------------------------------------------------------- activation quant
@@ -352,19 +449,22 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* 
   act_quant_body<Act>(x, q, s, groups16, (size_t)blockIdx.x * 256 + threadIdx.x);
 }
 
-// The expert sort (one workgroup, latency-bound) and the quantisation of the token
-// activations (independent of the routing) in one launch: workgroup 0 sorts, the others
-// quantise 1024 lanes' worth each.
+// The expert sort (latency-bound) and the quantisation of the token activations (independent of
+// the routing) in one launch: the first workgroup(s) sort, the others quantise 1024 lanes' worth
+// each.
 template <class Act>
 __global__ __launch_bounds__(kSortThreads) void moe_sort_quant_kernel(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
     int32_t* __restrict__ max_count, int T, int K, int E, const typename Act::v8* __restrict__ x,
-    u32x2* __restrict__ q, float* __restrict__ s, size_t groups16) {
-  if (blockIdx.x == 0)
-    moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+    u32x2* __restrict__ q, float* __restrict__ s, size_t groups16, int S, int nsort) {
+  __shared__ SortSmem sm;
+  if ((int)blockIdx.x >= nsort)
+    act_quant_body<Act>(x, q, s, groups16, (size_t)(blockIdx.x - nsort) * kSortThreads + threadIdx.x);
+  else if (S)
+    moe_sort_wide_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, S, blockIdx.x, sm);
   else
-    act_quant_body<Act>(x, q, s, groups16, (size_t)(blockIdx.x - 1) * kSortThreads + threadIdx.x);
+    moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, sm);
 }
 
 // ---------------------------------------------------------------- elementwise
@@ -600,8 +700,9 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
   if (!expert_start) return MI_ERR_ARG;
   if (T < 0 || K < 1 || E < 1 || E > 1024) return MI_ERR_SHAPE;
   if (T > 0 && (!top_ids || !sorted_pairs || !inv)) return MI_ERR_ARG;   // T == 0 only fills expert_start
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(kSortThreads), 0, (hipStream_t)stream, top_ids,
-                     sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E);
+  const int S = sort_wide_span(T, E);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(S ? (unsigned)((T + S - 1) / S) : 1u), dim3(kSortThreads), 0,
+                     (hipStream_t)stream, top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, S);
   return launch_status();
 }
 
@@ -614,16 +715,18 @@ int mi_moe_sort_quant(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* ex
   if (rows < 0 || H <= 0 || (H % 128)) return MI_ERR_SHAPE;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
   const size_t groups16 = (size_t)rows * (H / 128);
-  const unsigned grid = 1u + (unsigned)((groups16 * 16 + kSortThreads - 1) / kSortThreads);
+  const int S = sort_wide_span(T, E);
+  const int nsort = S ? (T + S - 1) / S : 1;
+  const unsigned grid = (unsigned)nsort + (unsigned)((groups16 * 16 + kSortThreads - 1) / kSortThreads);
   hipStream_t st = (hipStream_t)stream;
   if (act_dtype == DT_F16)
     hipLaunchKernelGGL(moe_sort_quant_kernel<ActF16>, dim3(grid), dim3(kSortThreads), 0, st, top_ids, sorted_pairs,
                        expert_start, inv, sorted_token, max_count, T, K, E, (const f16x8*)x, (u32x2*)q, scale,
-                       groups16);
+                       groups16, S, nsort);
   else
     hipLaunchKernelGGL(moe_sort_quant_kernel<ActBF16>, dim3(grid), dim3(kSortThreads), 0, st, top_ids, sorted_pairs,
                        expert_start, inv, sorted_token, max_count, T, K, E, (const bf16x8*)x, (u32x2*)q, scale,
-                       groups16);
+                       groups16, S, nsort);
   return launch_status();
 }
 

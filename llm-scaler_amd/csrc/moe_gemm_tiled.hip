@@ -105,44 +105,36 @@ static inline TiledMoeLayout tiled_moe_layout(int total_rows, int E, int K, int 
   L.total = L.cnt_off + 256;
   return L;
 }
-// rows per M-tile: 256 once the experts average enough rows to fill such tiles
-static inline int tiled_moe_bm(int total_rows, int E) { return (long)total_rows >= 160L * E ? 256 : 128; }
+// Rows per M-tile.  A wavefront skips the 16-row tiles past an expert's last row, so the large tile
+// (each weight dequantized once per 256 rows) also serves experts with fewer rows.
+constexpr int kMoeBM = 256;
 
 template <class Act, template <class, int> class FMT, bool FUSE>
-static int launch_grouped(GemmArgs p, int bm, int max_tiles, hipStream_t st) {
+static int launch_grouped(GemmArgs p, int max_tiles, hipStream_t st) {
+  constexpr int BN = 256;
   p.tiles_m = max_tiles;
-  if (bm == 256) {
-    constexpr int BN = 256;
-    p.tiles_n = FUSE ? (p.n_half + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
-    using F = FMT<Act, BN>;
-    auto kern = gemm_tiled_kernel<Act, F, 256, BN, true, FUSE>;
-    const size_t lds = (size_t)2 * (F::B_CH * 256 / F::CPR) * kPitch * 2;
-    static bool raised = false;
-    if (lds > 64 * 1024 && !raised) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-          hipSuccess)
-        return MI_ERR_LAUNCH;
-      raised = true;
-    }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), lds, st, p);
-  } else {
-    constexpr int BN = 128;
-    p.tiles_n = FUSE ? (p.n_half + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
-    using F = FMT<Act, BN>;
-    const size_t lds = (size_t)2 * (F::B_CH * 256 / F::CPR) * kPitch * 2;
-    hipLaunchKernelGGL((gemm_tiled_kernel<Act, F, 128, BN, true, FUSE>), dim3((unsigned)(p.tiles_m * p.tiles_n)),
-                       dim3(256), lds, st, p);
+  p.tiles_n = FUSE ? (p.n_half + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
+  using F = FMT<Act, BN>;
+  auto kern = gemm_tiled_kernel<Act, F, kMoeBM, BN, true, FUSE>;
+  const size_t lds = (size_t)2 * (F::B_CH * 256 / F::CPR) * kPitch * 2;
+  static bool raised = false;
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess)
+      return MI_ERR_LAUNCH;
+    raised = true;
   }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), lds, st, p);
   return launch_status();
 }
 
 template <class Act>
-static int run_grouped(const GemmArgs& p, bool per_expert, int fuse, int bm, int max_tiles, hipStream_t st) {
+static int run_grouped(const GemmArgs& p, bool per_expert, int fuse, int max_tiles, hipStream_t st) {
   if (per_expert)
-    return fuse ? launch_grouped<Act, WFp8PlainG, true>(p, bm, max_tiles, st)
-                : launch_grouped<Act, WFp8PlainG, false>(p, bm, max_tiles, st);
-  return fuse ? launch_grouped<Act, WFp8BlockG, true>(p, bm, max_tiles, st)
-              : launch_grouped<Act, WFp8BlockG, false>(p, bm, max_tiles, st);
+    return fuse ? launch_grouped<Act, WFp8PlainG, true>(p, max_tiles, st)
+                : launch_grouped<Act, WFp8PlainG, false>(p, max_tiles, st);
+  return fuse ? launch_grouped<Act, WFp8BlockG, true>(p, max_tiles, st)
+              : launch_grouped<Act, WFp8BlockG, false>(p, max_tiles, st);
 }
 
 }  // namespace qlin
@@ -154,7 +146,7 @@ extern "C" {
 int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes) {
   if (!bytes) return MI_ERR_ARG;
   if (total_rows < 0 || E < 0 || E > kMapThreads || K <= 0) return MI_ERR_SHAPE;
-  *bytes = tiled_moe_layout(total_rows, E, K, 128).total;      // the larger of the two tile tables
+  *bytes = tiled_moe_layout(total_rows, E, K, kMoeBM).total;
   return MI_OK;
 }
 
@@ -169,10 +161,10 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* 
   if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31)) return MI_ERR_SHAPE;
   if (!E || !total_rows) return MI_OK;
-  const int bm = tiled_moe_bm(total_rows, E);
+  const int bm = kMoeBM;
   const TiledMoeLayout L = tiled_moe_layout(total_rows, E, K, bm);
   if ((uint64_t)L.x_bytes >= (1ull << 31)) return MI_ERR_SHAPE;
-  if (!workspace || workspace_bytes < tiled_moe_layout(total_rows, E, K, 128).total) return MI_ERR_ARG;
+  if (!workspace || workspace_bytes < L.total) return MI_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   int32_t* g_tile = (int32_t*)(ws + L.tile_off);
@@ -192,8 +184,8 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* 
   p.x_blocks = L.max_blocks;
   p.n_half = N / 2; p.gelu = fuse_act == 2;
   p.out_rows = total_rows;
-  return act_dtype == DT_F16 ? run_grouped<ActF16>(p, scale_per_expert != 0, fuse_act, bm, L.max_tiles, st)
-                             : run_grouped<ActBF16>(p, scale_per_expert != 0, fuse_act, bm, L.max_tiles, st);
+  return act_dtype == DT_F16 ? run_grouped<ActF16>(p, scale_per_expert != 0, fuse_act, L.max_tiles, st)
+                             : run_grouped<ActBF16>(p, scale_per_expert != 0, fuse_act, L.max_tiles, st);
 }
 
 }  // extern "C"

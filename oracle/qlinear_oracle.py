@@ -429,7 +429,8 @@ def moe_forward(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, *, act_quant: bool,
 
 
 def moe_forward_grouped(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, num_experts, *,
-                        act_quant: bool, act_dtype=torch.bfloat16, inter_q=None, return_parts=False):
+                        act_quant: bool, act_dtype=torch.bfloat16, inter_q=None, return_parts=False,
+                        weight_dtype=None):
     """Same result as moe_forward, computed expert by expert on the sorted rows
     (V/tests/test_fp8_blockscale_moe_prefill.py:113-118).  Fast enough for cfg3.
 
@@ -439,6 +440,7 @@ def moe_forward_grouped(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, num_experts
     group's grid), so a check of the down GEMM and of the combine has to start
     from the very codes the kernel under test produced.
     return_parts -> (out, inter [T*k, I] in act_dtype, y [T*k, H] fp32), sorted order.
+    weight_dtype: round the block-scaled weights to this type first (see fp8_dequant_block).
     """
     T, H = x.shape
     k = top_ids.shape[1]
@@ -459,8 +461,8 @@ def moe_forward_grouped(x, top_w, top_ids, w13_q, w13_s, w2_q, w2_s, num_experts
         if hi == lo:
             continue
         rows = tok[lo:hi]
-        dw13 = fp8_dequant_block(w13_q[e], w13_s[e])
-        dw2 = fp8_dequant_block(w2_q[e], w2_s[e])
+        dw13 = fp8_dequant_block(w13_q[e], w13_s[e], out_dtype=weight_dtype)
+        dw2 = fp8_dequant_block(w2_q[e], w2_s[e], out_dtype=weight_dtype)
         inter = silu_mul(x32[rows] @ dw13.t()).to(act_dtype)
         inter_all[lo:hi] = inter
         if inter_q is not None:

@@ -429,9 +429,21 @@ def test_moe_forward_w8a16_prefill(v, dev, T, E, K, H, I, dt):
     v.moe_forward_fp8_block(x.to(dev), logits.to(dev), w13q.view(torch.float8_e4m3fn).to(dev), w13s.to(dev),
                             w2q.view(torch.float8_e4m3fn).to(dev), w2s.to(dev), out, K, False)
     rtw, rti = O.moe_topk(logits, K)
-    ref = O.moe_forward_grouped(x, rtw, rti, w13q, w13s, w2q, w2s, E, act_quant=False)
-    assert O.max_rel_err(out.cpu(), ref) < TOL
-    assert O.max_rel_err_abs_floor(out.cpu(), ref) < 3e-2
+    free = O.moe_forward_grouped(x, rtw, rti, w13q, w13s, w2q, w2s, E, act_quant=False, act_dtype=dt)
+    o = out.cpu().float()
+    mean_rel = ((o - free).abs().mean() / free.abs().mean()).item()
+    cos = torch.nn.functional.cosine_similarity(o.flatten(), free.flatten(), dim=0).item()
+    assert mean_rel < (3e-3 if dt == torch.float16 else 1e-2) and cos > 0.9999, (mean_rel, cos)
+    # element-wise, against the same arithmetic: block scales folded into weights of the activation type (as the
+    # tiled kernel feeds the matrix core), plus one rounding of each expert output to that type (the reference's
+    # grouped GEMM writes it too), which cancellation between a token's experts can make visible
+    ref, _, y = O.moe_forward_grouped(x, rtw, rti, w13q, w13s, w2q, w2s, E, act_quant=False, act_dtype=dt,
+                                      return_parts=True, weight_dtype=dt)
+    order, _, _ = O.moe_sort(rti, E)
+    mag = torch.zeros(T, H).index_add_(0, (order // K).long(), y.abs() * rtw.reshape(-1).float()[order.long()][:, None])
+    ulp = 2.0 ** -8 if dt == torch.bfloat16 else 2.0 ** -11
+    bound = TOL * ref.abs().clamp(min=ref.abs().mean()) + ulp * mag
+    assert bool(((o - ref).abs() <= bound).all()), ((o - ref).abs() / bound).max()
 
 
 def test_cfg3_moe_forward(v, dev):
