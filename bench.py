@@ -507,6 +507,76 @@ def wl_gemv_fp16(dev):
                 name=f"next: 16-bit weight GEMV (router) M={M} K={K} N={N} fp16", kernel="gemv_w16_kernel", cpu=cpu)
 
 
+def wl_int4_fused2(dev):
+    """The two GDN input projections of a Qwen3-Next decode step in one launch, as the reference's caller
+    issues them (vllm/patches/vllm_for_multi_arc.patch:4490-4524): in_proj_qkvz [12288, 2048] and
+    in_proj_ba [64, 2048], W4A16 group 128, one token."""
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    K, N0, N1 = 2048, 12288, 64
+    x, p0, s0, _ = O.make_int4_case(1, K, N0, seed=31)
+    _, p1, s1, _ = O.make_int4_case(1, K, N1, seed=32)
+    per = (N0 + N1) * (K // 2 + (K // 128) * 2)
+    R = _copies(per)
+    g = torch.Generator().manual_seed(97)
+    W = []
+    for _ in range(R):
+        a, b = torch.randperm(N0, generator=g), torch.randperm(N1, generator=g)
+        W.append((p0[a].to(dev), s0[a].to(dev), p1[b].to(dev), s1[b].to(dev)))
+    xd = x.to(dev)
+    o0 = torch.empty(1, N0, dtype=torch.float16, device=dev)
+    o1 = torch.empty(1, N1, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        a, b, c, d = W[i % R]
+        v.esimd_gemv_int4_fused2(xd, a, b, o0, c, d, o1)
+
+    def cpu():
+        return O.matmul_ref(x, O.int4_dequant(p0, s0)).half(), O.matmul_ref(x, O.int4_dequant(p1, s1)).half()
+
+    return dict(launch=launch, R=R, bytes=per + 2 * K + 2 * (N0 + N1), flops=2 * (N0 + N1) * K, bound="hbm", dtype="f16",
+                name=f"next: W4A16 fused2 GEMV (GDN in_proj_qkvz + in_proj_ba) M=1 K={K} N={N0}+{N1} fp16",
+                kernel="gemv_rows_kernel", cpu=cpu)
+
+
+def wl_fp8_pert_fused(dev, three: bool):
+    """Per-tensor FP8 projections sharing one activation row in one launch: fused2 = the GDN in_proj_qkvz +
+    in_proj_ba pair the reference's caller issues (vllm/patches/vllm_for_multi_arc.patch:4340-4355,
+    10521-10529); fused3 = the q / k / v projections of a Qwen3-Next full-attention layer (gated q:
+    16 heads x 256 x 2; 2 kv heads x 256)."""
+    import custom_esimd_kernels_vllm as v
+    from oracle import qlinear_oracle as O
+    K = 2048
+    Ns = [8192, 512, 512] if three else [12288, 64]
+    g = torch.Generator().manual_seed(96)
+    x = torch.randn(1, K, generator=g).half()
+    w8 = [O.e4m3_quantize(torch.randn(n, K, generator=g).clamp(-3, 3) * (448.0 / 3)) for n in Ns]
+    sc = [torch.tensor([0.02 / 448 * (i + 1)], dtype=torch.float32) for i in range(len(Ns))]
+    per = sum(Ns) * K
+    R = _copies(per)
+    W = []
+    for _ in range(R):
+        W.append([w[torch.randperm(w.shape[0], generator=g)].to(dev).view(torch.float8_e4m3fn) for w in w8])
+    xd = x.to(dev)
+    sd = [t.to(dev) for t in sc]
+    outs = [torch.empty(1, n, dtype=torch.float16, device=dev) for n in Ns]
+
+    def launch(i):
+        w = W[i % R]
+        if three:
+            v.esimd_gemv_fp8_pert_fused3(xd, w[0], sd[0], outs[0], w[1], sd[1], outs[1], w[2], sd[2], outs[2])
+        else:
+            v.esimd_gemv_fp8_pert_fused2(xd, w[0], sd[0], outs[0], w[1], sd[1], outs[1])
+
+    def cpu():
+        return [O.matmul_ref(x, O.fp8_dequant_per_tensor(w, t)).half() for w, t in zip(w8, sc)]
+
+    n = "+".join(str(t) for t in Ns)
+    return dict(launch=launch, R=R, bytes=per + 2 * K + 2 * sum(Ns) + 4 * len(Ns), flops=2 * sum(Ns) * K, bound="hbm",
+                dtype="f16", name=f"next: FP8 per-tensor fused{len(Ns)} GEMV M=1 K={K} N={n} fp16",
+                kernel="gemv_rows_kernel", cpu=cpu)
+
+
 WORKLOADS = {
     "cfg1_m1": lambda dev: wl_fp8_pern(1, dev),
     "cfg1_m8": lambda dev: wl_fp8_pern(8, dev),
@@ -521,6 +591,9 @@ WORKLOADS = {
     "next_fp8_prefill_m2048": wl_fp8_prefill,
     "next_fp8_block_prefill_m2048": lambda dev: wl_fp8_prefill(dev, "block"),
     "next_q4k_prefill_m2048": wl_q4k_prefill,
+    "next_int4_fused2": wl_int4_fused2,
+    "next_fp8_pert_fused2": lambda dev: wl_fp8_pert_fused(dev, False),
+    "next_fp8_pert_fused3": lambda dev: wl_fp8_pert_fused(dev, True),
     "next_q4k_m8": lambda dev: wl_q4k(8, dev),
     "next_q4k_m32": lambda dev: wl_q4k(32, dev),
     "next_q4_0_m1": lambda dev: wl_gguf("q4_0", 1, dev),
@@ -580,6 +653,31 @@ def run_gpu(wl, steps: int, warmup: int):
         torch.cuda.synchronize()
         t1 = time.perf_counter()
     return t1 - t0, e0.elapsed_time(e1)
+
+
+def floor_us(nbytes: int, dev, steps: int = CASE_MIN_STEPS):
+    """Microseconds a pure streaming read of `nbytes` takes on this device (the library's read yardstick over
+    cold memory: consecutive launches walk a buffer of at least 1 GiB), timed like a workload."""
+    from mi355x_qlinear import capi
+    import ctypes
+    nbytes = (int(nbytes) + 15) // 16 * 16
+    slices = max(2, -(-CACHE_BUST_BYTES // nbytes))
+    buf = torch.empty(slices * nbytes, dtype=torch.uint8, device=dev).fill_(3)
+    words = ctypes.c_longlong(0)
+    if capi.lib().mi_stream_read_sink_words(ctypes.byref(words)) != 0:
+        return None
+    sink = torch.zeros(words.value, dtype=torch.int32, device=dev)
+    base = buf.data_ptr()
+
+    best = None
+    for variant in range(capi.lib().mi_stream_read_variants()):     # launch shapes; which is fastest depends on the size
+        def launch(i, variant=variant):
+            capi.call("mi_stream_read", buf, base + (i % slices) * nbytes, nbytes, capi.ptr(sink), variant)
+
+        _, ev = run_gpu(dict(launch=launch, R=slices), steps, 3)
+        best = ev if best is None else min(best, ev)
+    del buf
+    return best * 1e3 / steps
 
 
 def measured_traffic(workload_id):
@@ -652,6 +750,13 @@ def run_case(wid, dev, steps, warmup, with_cpu, cpu_budget_s):
     wl = WORKLOADS[wid](dev)
     wall, ev = run_gpu(wl, steps, warmup)
     c = summarize(wl, wid, steps, warmup, wall, ev)
+    if wl["bound"] == "hbm":
+        # the same number of bytes through a pure streaming read: what is left of the gap to the HBM peak once
+        # the device's own read ceiling and the fixed cost of a launch are taken out
+        f = floor_us(wl["bytes"], dev)
+        if f:
+            c["roofline"]["floor_us"] = f
+            c["roofline"]["frac_of_floor"] = f / c["us_per_launch_events"]
     c["cpu_baseline"] = cpu_baseline(wl, cpu_budget_s) if with_cpu else None
     del wl
     torch.cuda.empty_cache()

@@ -457,6 +457,18 @@ int mi_moe_kmajor_finalize(const float* partial, int splits, const float* down_s
 int mi_gemv_w16(const void* x, const void* w, void* out, int M, int N, int K, int gelu_mul, int act_dtype,
                 void* stream);
 
+/* ---- measurement yardstick -------------------------------------------------------------
+ * No counterpart in the reference.  mi_stream_read fetches `bytes` (a multiple of 16, src 16-byte
+ * aligned) from HBM with non-temporal 16-byte loads and keeps nothing: the time a kernel that
+ * must read that many bytes cannot beat on this device, which the benchmark reports beside each
+ * memory-bound configuration.  The fastest launch shape depends on the size, so the shapes are
+ * numbered `variant`s in [0, mi_stream_read_variants()); the floor is the minimum over them.
+ * `sink` must hold the number of 32-bit words mi_stream_read_sink_words returns (it is written
+ * only if a lane's XOR hits one magic value). */
+int mi_stream_read_variants(void);
+int mi_stream_read_sink_words(long long* words);
+int mi_stream_read(const void* src, long long bytes, unsigned int* sink, int variant, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
