@@ -345,16 +345,17 @@ int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const v
 /* ---- MoE prefill: grouped FP8 GEMM on the tiled matrix-core kernel ---------------
  * mi_moe_gemm_fp8_grouped in w8a16 mode (no a_scale, output in the activation type) for experts
  * with hundreds of rows: a device-built table of M-tiles per expert, activations gathered and
- * re-tiled per 16-row block, then the 256 x 256 (128 x 128) tiled GEMM with one weight matrix per
- * expert, so that an expert's weights are read once per 256 of its rows.  Same arguments and
+ * re-tiled per 16-row block, then the 256 x 256 tiled GEMM with one weight matrix per expert, so
+ * that an expert's weights are read once per 256 of its rows (a wavefront skips the 16-row tiles
+ * past an expert's last row).  Same arguments and
  * results; K % 128 == 0, E <= 1024.  workspace: mi_moe_gemm_fp8_tiled_workspace bytes.
  * mi_moe_gemm_fp8_grouped takes this route itself (per-stream scratch) when the experts average
  * 96 rows or more.  Reference: the 64-row expert tiles with a device-built tile map of
  * V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:83-120, 187-302 and the per-expert M-tiled
  * GEMMs of S/csrc/moe_prefill/moe_prefill_fp8.sycl:167-410. */
 int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes);
-int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* w, const float* w_scale,
-                             int scale_per_expert, const int32_t* expert_start, void* out,
+int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_div, const void* w,
+                             const float* w_scale, int scale_per_expert, const int32_t* expert_start, void* out,
                              const int32_t* out_map, const void* row_weight, int a_rows, int total_rows,
                              int E, int N, int K, int fuse_act, int act_dtype, void* workspace,
                              long long workspace_bytes, void* stream);
@@ -398,7 +399,12 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
  * kernels and their epilogues:
  *   scale_per_expert = 1: w_scale is [E] fp32 (one factor per expert); K may then be
  *     any multiple of 16 (the chunks of the last 128-granule past K read as zeros).
+ *     scale_per_expert = 2: w_scale is [E, 2] fp32, the first factor for weight rows [0, N/2)
+ *     and the second for rows [N/2, N) (the gate / up scales of the sglang prefill kernels,
+ *     S/csrc/moe_prefill/moe_prefill_fp8.sycl:480-530); without fuse_act N/2 must be a multiple of 16.
  *     scale_per_expert = 0: block scales [E, ceil(N/128), ceil(K/128)] as above.
+ *   row_map_div (>= 1): the source row of sorted position r is row_map[r] / row_map_div, so that a
+ *     map of pair indices (token * top_k + slot) gathers token rows with row_map_div = top_k.
  *   fuse_act: 0 none, 1 silu(gate) * up, 2 gelu_tanh(gate) * up (exp argument held in
  *     [-30, 30]); gate = weight rows [0, N/2), up = rows [N/2, N); N/2 need not be a
  *     multiple of 128.
@@ -411,8 +417,8 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
  * / moe_down_routed_e4m3_vllm_layout_kernel (V/csrc/moe_batch/moe.sycl:458-558, :870-924)
  * and the scatter at the end of the sglang prefill kernels
  * (S/csrc/moe_prefill/moe_prefill_fp8.sycl:280-300, :385-411). */
-int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
-                            const float* w_scale, int scale_per_expert, const int32_t* expert_start, void* out,
+int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* row_map, int row_map_div,
+                            const void* w, const float* w_scale, int scale_per_expert, const int32_t* expert_start, void* out,
                             const int32_t* out_map, const void* row_weight, int a_rows, int total_rows, int E,
                             int N, int K, int fuse_act, int act_dtype, int out_f32, void* stream);
 

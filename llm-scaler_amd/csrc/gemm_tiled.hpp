@@ -41,7 +41,8 @@ struct GemmArgs {
   void* out;
   int M, N, K;
   int tiles_m, tiles_n;
-  int scale_mode;             // fp8: 0 = per output channel, 1 = per tensor
+  int scale_mode;             // fp8: 0 = per output channel, 1 = per tensor / expert, 2 = 128x128 blocks,
+                              // 3 = two per expert: weight rows below n_half, rows from n_half on
   int scale_f16;              // fp8 per channel: the scales are fp16 instead of fp32
   // Grouped launch (GROUPED kernels): M-tile i of the grid belongs to expert g_tile[4 i] and covers
   // the rows [g_tile[4 i + 1], + g_tile[4 i + 2]) of the expert-sorted order; its activations
@@ -362,6 +363,7 @@ struct WFp8 {
   }
   static __device__ __forceinline__ float out_scale(const Res& r, const GemmArgs& p, int n) {
     if (p.scale_mode == 1) return ((const float*)r.se)[0];
+    if (p.scale_mode == 3) return ((const float*)r.se)[n >= p.n_half ? 1 : 0];
     return p.scale_f16 ? (float)((const _Float16*)r.se)[n] : ((const float*)r.se)[n];
   }
 };
@@ -599,6 +601,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
     // first of this lane's 4 output columns; FUSE: gate tile a pairs with up tile a + 1
     const int n = FUSE ? n0 + (wn0 >> 1) + ao * 16 + g * 4 : n0 + wn0 + a * 16 + g * 4;
     float os[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    [[maybe_unused]] float os_up = 1.0f;
+    if constexpr (Fmt::kOutScale && FUSE) os_up = Fmt::out_scale(res, p, p.n_half);
     if constexpr (Fmt::kOutScale) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) os[v] = Fmt::out_scale(res, p, n + v < N ? n + v : N - 1);
@@ -611,8 +615,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
         for (int v = 0; v < 4; ++v) {
           float r;
           if constexpr (FUSE) {
-            // per-tensor / per-expert scale only: one factor for gate and up
-            const float gate = acc[a][b][v] * os[v], up = acc[a + 1][b][v] * os[v];
+            // one factor per tensor / expert, or one for the gate rows and one for the up rows
+            const float gate = acc[a][b][v] * os[v], up = acc[a + 1][b][v] * (p.scale_mode == 3 ? os_up : os[v]);
             if (p.gelu) {
               float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
               two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);

@@ -32,7 +32,8 @@ namespace qlin {
 struct MoeGemmArgs {
   const void* a;              // activations: fp8 [rows, K] (A8) or 16-bit [rows, K]
   const float* a_scale;       // A8: [rows, K/128]
-  const int32_t* row_map;     // optional: sorted position -> source row of `a` / `a_scale`
+  const int32_t* row_map;     // optional: sorted position -> source row of `a` / `a_scale`, times row_div
+  int row_div;                // the source row is row_map[position] / row_div (pair index -> token)
   const void* w;              // [E, N, K] e4m3
   const float* w_scale;       // [E, ceil(N/128), ceil(K/128)], or [E]
   const int32_t* start;       // [E+1]
@@ -41,7 +42,7 @@ struct MoeGemmArgs {
   const void* row_weight;     // optional, activation dtype: factor per row of `out`
   int out_f32;
   int gelu;                   // fused epilogue: tanh-GELU instead of SiLU
-  int scale_per_expert;       // w_scale is [E] instead of block scales
+  int scale_per_expert;       // 1: w_scale is [E] instead of block scales; 2: [E, 2], first / second half of the N rows
   int E, N, K;                // N = weight rows per expert
   int n_out;                  // output columns (N, or N/2 with the fused SiLU*mul)
   int tiles_per_expert;       // workgroups per expert
@@ -138,9 +139,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   const int Nb = (N + 127) >> 7;
   // read through a restrict kernel argument so the (uniform) scale loads stay on the
   // scalar unit and do not queue behind the vector prefetch
-  // PE: one scale per expert, read once; otherwise the block scales of this expert
-  const float* __restrict__ wsc = PE ? w_scale + e : w_scale + (size_t)e * Nb * Kb;
+  // PE: one scale per expert (or one per half of its rows: gate / up), read once; otherwise the
+  // block scales of this expert
+  const bool pe_pair = PE && p.scale_per_expert == 2;
+  const float* __restrict__ wsc = PE ? w_scale + (pe_pair ? 2 * e : e) : w_scale + (size_t)e * Nb * Kb;
   const float ws_expert = PE ? wsc[0] : 1.0f;
+  const float ws_second = pe_pair ? wsc[1] : ws_expert;
   const uint32_t tg_stride = (uint32_t)kCols * (uint32_t)K;   // weight bytes between tile groups
 
   struct Regs {                                       // one granule in flight
@@ -160,7 +164,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       const int m = mc + wrow0 + mt * 16 + j;
       const bool ok = m < cnt;
       const int pos = r0 + (ok ? m : 0);
-      const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
+      const uint32_t src = p.row_map ? (uint32_t)p.row_map[pos] / (uint32_t)p.row_div : (uint32_t)pos;
       xsoff[mt] = (src * (uint32_t)Kb * 4u) | ((uint32_t)(!ok) << 31);
     }
     uint32_t aoff[MT][NAI];
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
         const int m = mc + wrow0 + mt * 16 + row;
         const bool ok = m < cnt;
         const int pos = r0 + (ok ? m : 0);
-        const uint32_t src = (uint32_t)(p.row_map ? p.row_map[pos] : pos);
+        const uint32_t src = p.row_map ? (uint32_t)p.row_map[pos] / (uint32_t)p.row_div : (uint32_t)pos;
         aoff[mt][i] = (src * (uint32_t)K * a_esz + (uint32_t)ch * 16u) | ((uint32_t)(!ok) << 31);
         alds[mt][i] = al + (mt * 16 + row) * APitch + ch * 16;
         ach[i] = A8 ? ch * 16 : ch * 8;               // first k of the chunk inside the granule
@@ -251,7 +255,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
           }
           float wsv[RT];
 #pragma unroll
-          for (int t = 0; t < RT; ++t) wsv[t] = PE ? ws_expert : wsc[(size_t)nb[t] * Kb + gi];
+          for (int t = 0; t < RT; ++t)
+            wsv[t] = PE ? (tile_hi(t) + col0 + tg * kCols + tile_col(t) >= half ? ws_second : ws_expert)
+                        : wsc[(size_t)nb[t] * Kb + gi];
           // prefetch D granules ahead, across the tile-group boundary
           {
             int ngi = gi + D, ntgi = tg;
@@ -408,9 +414,6 @@ static int dispatch_moe2(const MoeGemmArgs& p, hipStream_t st) {
   // short K: walk two tile groups per workgroup so the prefetch pipeline stays filled
   const int tpw = (G < 16 && wgs_with(rt) >= 2048) ? 2 : 1;
   const bool d2 = (G % 2) == 0;                       // two granules in flight need an even count
-  // hundreds of rows per expert (prefill): 256 rows per pass over the weights instead of 64
-  if (rt == 8 && (long)p.total_rows > 96L * p.E)
-    return d2 ? launch_moe<Act, A8, SILU, 8, 2, 4>(p, 1, st) : launch_moe<Act, A8, SILU, 8, 1, 4>(p, 1, st);
   if (rt == 8) return d2 ? launch_moe<Act, A8, SILU, 8, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 8, 1>(p, tpw, st);
   if (rt == 4) return d2 ? launch_moe<Act, A8, SILU, 4, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 4, 1>(p, tpw, st);
   return d2 ? launch_moe<Act, A8, SILU, 2, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 2, 1>(p, tpw, st);
@@ -427,7 +430,7 @@ using namespace qlin;
 
 extern "C" {
 
-int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
+int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* row_map, int row_map_div, const void* w,
                             const float* w_scale, int scale_per_expert, const int32_t* expert_start, void* out,
                             const int32_t* out_map, const void* row_weight, int a_rows, int total_rows, int E,
                             int N, int K, int fuse_act, int act_dtype, int out_f32, void* stream) {
@@ -437,6 +440,8 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
   if (E < 0 || N <= 0 || K <= 0 || (K % 16) || a_rows < 0 || total_rows < 0) return MI_ERR_SHAPE;
   if (a_scale && (K % 128)) return MI_ERR_SHAPE;      // quantised activations carry whole 128-groups
   if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
+  if (scale_per_expert < 0 || scale_per_expert > 2 || row_map_div < 1) return MI_ERR_ARG;
+  if (scale_per_expert == 2 && (N % 2 || (!fuse_act && (N / 2) % 16))) return MI_ERR_SHAPE;   // halves of whole 16-row tiles
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || (uint64_t)a_rows * (uint64_t)K * 2 >= (1ull << 31))
     return MI_ERR_SHAPE;
   if (!E || !total_rows) return MI_OK;
@@ -446,18 +451,18 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
     if (mi_moe_gemm_fp8_tiled_workspace(total_rows, E, K, &bytes) != MI_OK) return MI_ERR_SHAPE;
     void* ws = scratch_get((hipStream_t)stream, (size_t)bytes);
     if (!ws) return MI_ERR_LAUNCH;
-    return mi_moe_gemm_fp8_tiled_ws(a, row_map, w, w_scale, scale_per_expert, expert_start, out, out_map, row_weight,
+    return mi_moe_gemm_fp8_tiled_ws(a, row_map, row_map_div, w, w_scale, scale_per_expert, expert_start, out, out_map, row_weight,
                                     a_rows, total_rows, E, N, K, fuse_act, act_dtype, ws, bytes, stream);
   }
   MoeGemmArgs p{};
-  p.a = a; p.a_scale = a_scale; p.row_map = row_map; p.w = w; p.w_scale = w_scale;
+  p.a = a; p.a_scale = a_scale; p.row_map = row_map; p.row_div = row_map_div; p.w = w; p.w_scale = w_scale;
   p.start = expert_start; p.out = out; p.E = E; p.N = N; p.K = K; p.a_rows = a_rows;
   p.total_rows = total_rows;
   p.out_map = out_map; p.row_weight = row_weight;
   p.out_f32 = out_f32;
   p.gelu = fuse_act == 2;
   if (a_scale && scale_per_expert) return MI_ERR_ARG;
-  p.scale_per_expert = scale_per_expert ? 1 : 0;
+  p.scale_per_expert = scale_per_expert;
   hipStream_t st = (hipStream_t)stream;
   if (a_scale) {
     return act_dtype == DT_F16 ? dispatch_moe<ActF16, true>(p, fuse_act, st)
@@ -471,7 +476,7 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
                           const float* w_scale, const int32_t* expert_start, void* out, int a_rows,
                           int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,
                           int out_f32, void* stream) {
-  return mi_moe_gemm_fp8_grouped(a, a_scale, row_map, w, w_scale, 0, expert_start, out, nullptr, nullptr, a_rows,
+  return mi_moe_gemm_fp8_grouped(a, a_scale, row_map, 1, w, w_scale, 0, expert_start, out, nullptr, nullptr, a_rows,
                                  total_rows, E, N, K, fuse_silu_mul ? 1 : 0, act_dtype, out_f32, stream);
 }
 

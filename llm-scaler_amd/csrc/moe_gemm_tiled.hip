@@ -73,7 +73,8 @@ __global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __r
                                                              const int32_t* __restrict__ row_map,
                                                              const int32_t* __restrict__ blk,
                                                              const int32_t* __restrict__ counts,
-                                                             u32x4* __restrict__ xp, int a_rows, int K, int Q) {
+                                                             u32x4* __restrict__ xp, int a_rows, int K, int Q,
+                                                             int row_div) {
   const int b = blockIdx.y;
   if (b >= counts[1]) return;
   const int l = threadIdx.x & 63;
@@ -83,8 +84,8 @@ __global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __r
   u32x4 v = {0u, 0u, 0u, 0u};
   if (r < blk[2 * b + 1]) {
     const int pos = blk[2 * b] + r;
-    const int src = row_map ? row_map[pos] : pos;
-    if ((unsigned)src < (unsigned)a_rows)
+    const unsigned src = row_map ? (unsigned)row_map[pos] / (unsigned)row_div : (unsigned)pos;
+    if (src < (unsigned)a_rows)
       v = *reinterpret_cast<const u32x4*>(x + (size_t)src * K + q * 32 + (l >> 4) * 8);
   }
   xp[((size_t)b * Q + q) * 64 + l] = v;
@@ -150,13 +151,14 @@ int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* byt
   return MI_OK;
 }
 
-int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* w, const float* w_scale,
+int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_div, const void* w, const float* w_scale,
                              int scale_per_expert, const int32_t* expert_start, void* out, const int32_t* out_map,
                              const void* row_weight, int a_rows, int total_rows, int E, int N, int K, int fuse_act,
                              int act_dtype, void* workspace, long long workspace_bytes, void* stream) {
   if (!a || !w || !w_scale || !expert_start || !out) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (fuse_act < 0 || fuse_act > 2) return MI_ERR_ARG;
+  if (fuse_act < 0 || fuse_act > 2 || scale_per_expert < 0 || scale_per_expert > 2 || row_map_div < 1) return MI_ERR_ARG;
+  if (scale_per_expert == 2 && (N % 2)) return MI_ERR_SHAPE;
   if (E < 0 || E > kMapThreads || N <= 0 || K <= 0 || (K % 128) || a_rows < 0 || total_rows < 0) return MI_ERR_SHAPE;
   if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31)) return MI_ERR_SHAPE;
@@ -173,13 +175,13 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, const void* 
   hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(kMapThreads), 0, st, expert_start, E, bm, g_tile, blk, counts);
   const int Q = K / 32;
   hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((Q + 3) / 4, L.max_blocks), dim3(256), 0, st, (const uint16_t*)a,
-                     row_map, blk, counts, (u32x4*)ws, a_rows, K, Q);
+                     row_map, blk, counts, (u32x4*)ws, a_rows, K, Q, row_map_div);
   GemmArgs p{};
   p.x = ws; p.w = w; p.scale = w_scale; p.out = out; p.M = total_rows; p.N = N; p.K = K;
-  p.scale_mode = scale_per_expert ? 1 : 2;
+  p.scale_mode = scale_per_expert == 2 ? 3 : (scale_per_expert ? 1 : 2);
   p.g_tile = g_tile; p.g_count = counts;
   p.g_w_stride = (long long)N * K;
-  p.g_s_stride = scale_per_expert ? 4 : (long long)((N + 127) / 128) * (K / 128) * 4;
+  p.g_s_stride = scale_per_expert ? 4 * scale_per_expert : (long long)((N + 127) / 128) * (K / 128) * 4;
   p.out_map = out_map; p.row_weight = row_weight;
   p.x_blocks = L.max_blocks;
   p.n_half = N / 2; p.gelu = fuse_act == 2;

@@ -936,18 +936,22 @@ _ACT_NONE, _ACT_SILU, _ACT_GELU_TANH = 0, 1, 2
 
 
 def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse, who, *, per_expert=False,
-              out_map=None, row_weight=None):
+              out_map=None, row_weight=None, row_map_div=1):
     """Grouped GEMM over expert-sorted rows.  fuse: False / True (SiLU) or one of _ACT_*.
-    per_expert: w_scale holds one fp32 per expert instead of 128x128 block scales.
+    per_expert: w_scale holds one fp32 per expert (True / 1), or two — rows [0, N/2) and [N/2, N) —
+    (2), instead of 128x128 block scales.
     out_map (int32): sorted position -> row of `out`; row_weight (activation dtype): factor
-    per row of `out`."""
+    per row of `out`; the source row of a position is row_map[position] // row_map_div."""
     _chk_fp8(w, who)
     _chk(w.numel() == E * N * K, f"{who}: weight must be [num_experts, N, K]")
     fuse = int(fuse)
+    per_expert = int(per_expert)
     if per_expert:
         _chk(K % 16 == 0, f"{who}: K={K} must be a multiple of 16")
-        _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() >= E,
-             f"{who}: weight_scale must be contiguous fp32 [E]")
+        _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and w_scale.numel() >= E * per_expert,
+             f"{who}: weight_scale must be contiguous fp32 [E]" + (" x 2" if per_expert == 2 else ""))
+        _chk(per_expert == 1 or (N % 2 == 0 and (fuse or (N // 2) % 16 == 0)),
+             f"{who}: with gate / up scales N/2 must be a multiple of 16")
     else:
         _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
         _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and
@@ -977,12 +981,12 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
         if rc != 0:
             raise RuntimeError(f"{who}: {capi.MI_ERRORS.get(rc, rc)}")
         buf = torch.empty(need.value, dtype=torch.uint8, device=out.device)
-        capi.call("mi_moe_gemm_fp8_tiled_ws", out, capi.ptr(a), capi.ptr(row_map), capi.ptr(w), capi.ptr(w_scale),
-                  1 if per_expert else 0, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map), capi.ptr(row_weight),
+        capi.call("mi_moe_gemm_fp8_tiled_ws", out, capi.ptr(a), capi.ptr(row_map), int(row_map_div), capi.ptr(w),
+                  capi.ptr(w_scale), per_expert, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map), capi.ptr(row_weight),
                   a_rows, total, E, N, K, fuse, adt, capi.ptr(buf), need.value)
         return out
-    capi.call("mi_moe_gemm_fp8_grouped", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), capi.ptr(w),
-              capi.ptr(w_scale), 1 if per_expert else 0, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map),
+    capi.call("mi_moe_gemm_fp8_grouped", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), int(row_map_div),
+              capi.ptr(w), capi.ptr(w_scale), per_expert, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map),
               capi.ptr(row_weight), a_rows, total, E, N, K, fuse, adt, 1 if out.dtype == torch.float32 else 0)
     return out
 
@@ -1413,15 +1417,6 @@ def esimd_norm_gemv_fp8_blockscale(x, z, norm_weight, gemv_weight, gemv_scale, o
 # --------------------------------------------------------------------------
 # sglang FP8 MoE prefill ops (per-expert scalar scales), moe_fp8_prefill_ops
 # --------------------------------------------------------------------------
-def _expert_block_scales(scale, E, parts, rows_per_part, K, who):
-    """[E, parts] per-expert scalars -> [E, parts * rows_per_part / 128, K / 128] block scales
-    (every block of part p of expert e carries scale[e, p])."""
-    _chk(rows_per_part % 128 == 0 and K % 128 == 0,
-         f"{who}: intermediate and hidden sizes must be multiples of 128")
-    s = scale.to(torch.float32).reshape(-1)[:E * parts].reshape(E, parts, 1, 1)
-    return s.expand(E, parts, rows_per_part // 128, K // 128).reshape(E, parts * rows_per_part // 128, K // 128).contiguous()
-
-
 def _prefill_starts(expert_offsets, total):
     """[E] exclusive offsets -> [E + 1] with the total appended."""
     tail = torch.full((1,), total, dtype=torch.int32, device=expert_offsets.device)
@@ -1452,12 +1447,13 @@ def moe_prefill_up_forward_fp8(x, gate_up_weight, gate_up_scale, expert_offsets,
     P = expert_tokens.numel()
     k = int(top_k)
     dev = x.device
-    bs = _expert_block_scales(gate_up_scale, E, 2, I, H, who)
+    _chk(H % 16 == 0 and two_i % 2 == 0, f"{who}: H must be a multiple of 16")
     start = _prefill_starts(expert_offsets, P)
     tokens = expert_tokens.contiguous()
-    row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
     out = torch.empty(P, I, dtype=x.dtype, device=dev)
-    return _moe_gemm(x, None, row_map, gate_up_weight, bs, start, out, E, two_i, H, _ACT_SILU, who, out_map=tokens)
+    # the gate / up scalars of an expert go to the kernel as they are; the pair index -> token division too
+    return _moe_gemm(x, None, tokens, gate_up_weight, gate_up_scale.contiguous(), start, out, E, two_i, H, _ACT_SILU, who,
+                     per_expert=2, out_map=tokens, row_map_div=k)
 
 
 def moe_prefill_down_forward_fp8(intermediate, down_weight, down_scale, expert_offsets, expert_tokens):
@@ -1474,11 +1470,12 @@ def moe_prefill_down_forward_fp8(intermediate, down_weight, down_scale, expert_o
     _chk(intermediate.shape[1] == I, f"{who}: intermediate dim must equal w2 last dim")
     _chk(down_scale.numel() >= E, f"{who}: down_scale must have >= E entries")
     P = expert_tokens.numel()
-    bs = _expert_block_scales(down_scale, E, 1, H, I, who)
+    _chk(I % 16 == 0, f"{who}: I must be a multiple of 16")
     start = _prefill_starts(expert_offsets, P)
     tokens = expert_tokens.contiguous()
     out = torch.empty(P, H, dtype=intermediate.dtype, device=intermediate.device)
-    return _moe_gemm(intermediate, None, tokens, down_weight, bs, start, out, E, H, I, _ACT_NONE, who, out_map=tokens)
+    return _moe_gemm(intermediate, None, tokens, down_weight, down_scale.contiguous(), start, out, E, H, I, _ACT_NONE, who,
+                     per_expert=1, out_map=tokens)
 
 
 def moe_prefill_accumulate_forward_fp8(output, routing_weights):
@@ -1499,8 +1496,8 @@ def moe_prefill_accumulate_forward_fp8(output, routing_weights):
 def moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, w2, w2_scale, top_k, num_experts):
     """Prefill MoE with per-expert scalar scales: stable expert sort -> grouped gate_up GEMM with
     SiLU*mul -> grouped down GEMM -> weighted combine (S/csrc/moe_prefill/moe_prefill_fp8.sycl:616-649).
-    The intermediate stays in expert-sorted order and the down output in fp32, so the two
-    pair-order round trips of the separate ops are not made here."""
+    The intermediate stays in expert-sorted order, so the two pair-order round trips of the
+    separate ops are not made here; H and I may be any multiples of 16."""
     who = "moe_prefill_full_fp8"
     _chk(hidden_states.dtype in (torch.float16, torch.bfloat16), f"{who}: hidden_states must be fp16 (bf16 accepted)")
     _chk(topk_weights.dtype == hidden_states.dtype, f"{who}: topk_weights must be fp16 (the activation dtype)")
@@ -1525,10 +1522,13 @@ def moe_prefill_full_fp8(hidden_states, topk_weights, topk_ids, w13, w13_scale, 
     sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
     moe_sort(ids, E, sorted_pairs, start, inv, sorted_token, None)
     inter = torch.empty(P, I, dtype=x.dtype, device=dev)
-    y = torch.empty(P, H, dtype=torch.float32, device=dev)
-    moe_gemm_fp8_block(x, None, sorted_token, w13, _expert_block_scales(w13_scale, E, 2, I, H, who), start, inter,
-                       2 * I, H, E, True)
-    moe_gemm_fp8_block(inter, None, None, w2, _expert_block_scales(w2_scale, E, 1, H, I, who), start, y, H, I, E, False)
+    # fp32 expert outputs; with hundreds of rows per expert the tiled grouped GEMM takes over, which writes
+    # the activation type (as the reference's kernels do)
+    prefill = P >= 96 * E and H % 128 == 0 and I % 128 == 0
+    y = torch.empty(P, H, dtype=x.dtype if prefill else torch.float32, device=dev)
+    _chk(H % 16 == 0 and I % 16 == 0, f"{who}: H and I must be multiples of 16")
+    _moe_gemm(x, None, sorted_token, w13, w13_scale.contiguous(), start, inter, E, 2 * I, H, _ACT_SILU, who, per_expert=2)
+    _moe_gemm(inter, None, None, w2, w2_scale.contiguous(), start, y, E, H, I, _ACT_NONE, who, per_expert=1)
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     moe_combine(y, inv, topk_weights.contiguous(), out, k)
     return out

@@ -525,7 +525,11 @@ def _prefill_case(T, E, H, I, k, seed, dtype):
 
 
 @pytest.mark.parametrize("T,E,H,I,k,dtype", [(64, 8, 256, 128, 2, torch.float16), (200, 16, 512, 256, 4, torch.bfloat16),
-                                             (1, 4, 128, 128, 1, torch.float16)])
+                                             (1, 4, 128, 128, 1, torch.float16),
+                                             # sizes that are multiples of 16 / 32 only, as the reference accepts
+                                             (50, 8, 144, 80, 2, torch.float16), (33, 4, 2816 // 8, 704 // 4, 2, torch.float16),
+                                             # hundreds of rows per expert: both GEMMs on the tiled matrix-core route
+                                             (700, 4, 256, 128, 2, torch.float16)])
 def test_moe_prefill_full_fp8(s, dev, T, E, H, I, k, dtype):
     x, tw, ti, w13, s13, w2, s2 = _prefill_case(T, E, H, I, k, 300 + T, dtype)
     want, inter_ref, y_ref = O.moe_prefill_scalar(x, tw, ti, w13, s13, w2, s2, return_parts=True)
@@ -725,12 +729,16 @@ def test_moe_gemm_grouped_argument_errors(v, dev):
     sc = torch.ones(E, device=dev)
     start = torch.tensor([0, 2, 4], dtype=torch.int32, device=dev)
     out = torch.zeros(R, N, dtype=torch.float16, device=dev)
-    args = lambda k, act: (capi.ptr(a), None, None, capi.ptr(w), capi.ptr(sc), 1, capi.ptr(start), capi.ptr(out), None, None,
-                           R, R, E, N, k, act, capi.DT_F16, 0)
+    args = lambda k, act, se=1, div=1: (capi.ptr(a), None, None, div, capi.ptr(w), capi.ptr(sc), se, capi.ptr(start),
+                                        capi.ptr(out), None, None, R, R, E, N, k, act, capi.DT_F16, 0)
     with pytest.raises(RuntimeError):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(K, 0))
     with pytest.raises(RuntimeError):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 3))
+    with pytest.raises(RuntimeError):
+        capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 0, 3))          # no such scale form
+    with pytest.raises(RuntimeError):
+        capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 0, 1, 0))       # row-map divisor below 1
 
 
 # ----------------------------------------------------------------- per-tensor decode op on K-major routed weights
