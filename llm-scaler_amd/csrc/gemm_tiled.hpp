@@ -686,6 +686,11 @@ static int launch_gemm_tiled(GemmArgs p, hipStream_t st) {
   return launch_status();
 }
 
+// Per K step a workgroup pays for its tile's columns (MFMAs) plus a part that does not shrink with
+// the tile (activation loads, barrier, pipeline fill): measured on 5120 x 5120 and 14336 x 4096
+// weights, 160- and 192-column tiles cost about (BN + 48) / (256 + 48) of a 256-column tile.
+constexpr long kTileFixedCols = 48;
+
 static inline long device_cu_count_gemm() {
   static int cus = 0;
   if (!cus) {
@@ -699,8 +704,10 @@ static inline long device_cu_count_gemm() {
 }
 
 // Re-tiles x into `workspace` and runs the tile shape that fits the problem: 128 x 128 tiles
-// while 256-row tiles would leave more than half of the chip idle, else 256 x 256 or 256 x 224,
-// whichever leaves the last round of workgroups fuller.  FMT is a template taking (Act, BN).
+// while 256-row tiles would leave more than half of the chip idle, else 256 rows x 256 / 224 /
+// 192 / 160 columns, whichever needs the least time over its rounds of resident workgroups (a
+// 5120-column weight is 32 tiles of 160: with 8 row tiles exactly one round of 256 workgroups,
+// where 256-column tiles fill 160 of the 256 CUs).  FMT is a template taking (Act, BN).
 template <class Act, template <class, int> class FMT>
 static int run_gemm_tiled(GemmArgs p, const void* x, void* workspace, hipStream_t st) {
   const int Mp = (p.M + 15) & ~15;
@@ -714,8 +721,14 @@ static int run_gemm_tiled(GemmArgs p, const void* x, void* workspace, hipStream_
   const long tiles_m = (p.M + 255) / 256;
   const bool big = p.M > 128 && tiles_m * ((p.N + 255) / 256) * 2 > cus;
   if (!big) return launch_gemm_tiled<Act, FMT<Act, 128>, 128, 128>(p, st);
-  auto cost = [&](long bn) { return ((tiles_m * ((p.N + bn - 1) / bn) + cus - 1) / cus) * bn; };
-  if (cost(224) < cost(256)) return launch_gemm_tiled<Act, FMT<Act, 224>, 256, 224>(p, st);
+  // time ~ rounds of resident workgroups x (columns of a tile + a fixed part per K step)
+  auto cost = [&](long bn) { return ((tiles_m * ((p.N + bn - 1) / bn) + cus - 1) / cus) * (bn + kTileFixedCols); };
+  long best = 256;
+  for (long bn : {224L, 192L, 160L})
+    if (cost(bn) < cost(best)) best = bn;
+  if (best == 160) return launch_gemm_tiled<Act, FMT<Act, 160>, 256, 160>(p, st);
+  if (best == 192) return launch_gemm_tiled<Act, FMT<Act, 192>, 256, 192>(p, st);
+  if (best == 224) return launch_gemm_tiled<Act, FMT<Act, 224>, 256, 224>(p, st);
   return launch_gemm_tiled<Act, FMT<Act, 256>, 256, 256>(p, st);
 }
 

@@ -250,7 +250,9 @@ def test_fp8_register_resident_activations(ops, dev, M, K, N, dt, mode):
 @pytest.mark.parametrize("M,K,N,dt,mode", [
     (65, 1024, 520, torch.float16, "pern"), (200, 2048, 1000, torch.bfloat16, "pern"), (2048, 4096, 14336, torch.bfloat16, "pern"),
     (130, 512, 64, torch.float16, "pern16"), (300, 1024, 777, torch.float16, "pert"), (65, 5120, 5120, torch.float16, "block"),
-    (200, 1024, 4160, torch.bfloat16, "block"), (2048, 5120, 5120, torch.bfloat16, "block"), (513, 768, 200, torch.bfloat16, "block")])
+    (200, 1024, 4160, torch.bfloat16, "block"), (2048, 5120, 5120, torch.bfloat16, "block"), (513, 768, 200, torch.bfloat16, "block"),
+    # 192- and 160-column tiles
+    (1900, 256, 6144, torch.float16, "pern"), (2047, 384, 5100, torch.float16, "pert"), (2040, 256, 6100, torch.bfloat16, "block")])
 def test_fp8_prefill_tiled_gemm(ops, dev, M, K, N, dt, mode):
     # more than 64 rows: the tiled matrix-core GEMM (the weight is read once per 256 rows); the same
     # bar as the small-M path, on a strided sample of rows and columns where the problem is large
@@ -403,7 +405,7 @@ def test_cfg4_q4k(ops, dev, M):
     assert b < (0.6 if M == 1 else 0.1)
 
 
-@pytest.mark.parametrize("M,K,N", [(65, 512, 130), (200, 2048, 1000), (2048, 5120, 5120)])
+@pytest.mark.parametrize("M,K,N", [(65, 512, 130), (200, 2048, 1000), (2048, 5120, 5120), (1800, 256, 6144)])
 def test_q4k_prefill_tiled_gemm(ops, dev, M, K, N):
     # M > 64: the tiled matrix-core GEMM with the two-rounding Q4_K dequantization staged through LDS
     # (the reference dequantizes densely and calls a matmul, sglang_for_multi_arc.patch:3211-3213)
@@ -466,7 +468,9 @@ def _run_gemm_int4(v, dev, M, K, N, dt, asym, seed):
     (65, 256, 64, torch.float16, False), (128, 512, 128, torch.bfloat16, True),
     (200, 1024, 272, torch.bfloat16, True), (257, 384, 520, torch.float16, True),
     (300, 128, 16, torch.bfloat16, False), (1000, 2048, 1000, torch.bfloat16, True),
-    (4096, 512, 4096, torch.bfloat16, True), (4100, 256, 4100, torch.float16, False)])
+    (4096, 512, 4096, torch.bfloat16, True), (4100, 256, 4100, torch.float16, False),
+    # 160- and 192-column tiles (32 of them per row tile: one round of workgroups)
+    (2048, 256, 5120, torch.float16, True), (2000, 384, 6144, torch.bfloat16, False)])
 def test_gemm_int4_shapes(ops, dev, M, K, N, dt, asym):
     v, _ = ops
     assert _run_gemm_int4(v, dev, M, K, N, dt, asym, seed=M + N) < TOL
