@@ -41,6 +41,7 @@ struct GemmArgs {
   void* out;
   int M, N, K;
   int tiles_m, tiles_n;
+  int xcd_m;                  // dense launches: the 8 XCDs form an xcd_m x (8 / xcd_m) grid over the tiles (0: none)
   int scale_mode;             // fp8: 0 = per output channel, 1 = per tensor / expert, 2 = 128x128 blocks,
                               // 3 = two per expert: weight rows below n_half, rows from n_half on
   int scale_f16;              // fp8 per channel: the scales are fp16 instead of fp32
@@ -90,6 +91,7 @@ constexpr int kPitch = kBK + 8;                      // elements per LDS row (14
 template <class Act, int BN>
 struct WInt4 {
   static constexpr int CPR = 2;                       // chunks per row and 64-wide step
+  static constexpr double kWeightBytesPerK = 0.5;
   static constexpr int B_CH = (BN * CPR + 255) / 256; // chunks per thread
   static constexpr int LPC = 3;                       // load instructions per chunk
   static constexpr int kPieces = B_CH * 4 * 8;        // 8 pieces per packed dword of 8 nibbles
@@ -193,6 +195,7 @@ template <class Act, int BN>
 struct WQ4K {
   static_assert(Act::dt == DT_F16, "Q4_K runs in fp16");
   static constexpr int CPR = 2;
+  static constexpr double kWeightBytesPerK = 0.5;
   static constexpr int B_CH = (BN * CPR + 255) / 256;
   static constexpr int LPC = 3;
   static constexpr int PPD = 12;                      // pieces per dword of 8 nibbles
@@ -282,6 +285,7 @@ struct WQ4K {
 template <class Act, int BN, bool BLOCK>
 struct WFp8 {
   static constexpr int CPR = 4;
+  static constexpr double kWeightBytesPerK = 1.0;
   static constexpr int B_CH = (BN * CPR + 255) / 256;
   static constexpr int LPC = BLOCK ? 2 : 1;
   static constexpr int kPPC = BLOCK ? 10 : 4;         // pieces per chunk
@@ -393,10 +397,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   const int j = lane & 15, g = lane >> 4;
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
 
-  // tile order: consecutive workgroups share the weight tile (same n-tile) so that
-  // the 8 XCDs, which take workgroups round-robin, each keep re-using one slab of x
-  const int tn = blockIdx.x / p.tiles_m;
-  const int tm = blockIdx.x - tn * p.tiles_m;
+  // Tile order.  The 8 XCDs take workgroups round-robin and each has its own L2, so the tile of a
+  // workgroup is derived from (XCD = id % 8, slot on that XCD = id / 8):
+  //   dense: the XCDs form an xcd_m x (8 / xcd_m) grid over the tile matrix and each walks its
+  //     block of it M-tile first, so that the workgroups resident on an XCD share a few weight
+  //     tiles and a few slabs of x and every operand byte is fetched by as few L2s as possible
+  //     (xcd_m = 0: plain order, consecutive workgroups share the weight tile);
+  //   grouped: XCD x owns one M-tile of every 8 and walks the N-tiles of one M-tile
+  //     back to back, so an M-tile's activations are fetched into one L2 once (its N-tiles read
+  //     different weight rows: there is nothing else to share).
+  int tm, tn;
+  if constexpr (GROUPED) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int round = slot / p.tiles_n;               // rotate, so that no XCD gets all the experts' short last tiles
+    tm = round * 8 + ((xcd + round) & 7);
+    tn = slot - round * p.tiles_n;
+  } else if (p.xcd_m) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int per_m = p.tiles_m / p.xcd_m, per_n = p.tiles_n / (8 / p.xcd_m);
+    tm = (xcd % p.xcd_m) * per_m + slot % per_m;
+    tn = (xcd / p.xcd_m) * per_n + slot / per_m;
+  } else {
+    tn = blockIdx.x / p.tiles_m;
+    tm = blockIdx.x - tn * p.tiles_m;
+  }
   int m0 = tm * BM;
   const int n0 = FUSE ? tn * (BN / 2) : tn * BN;      // FUSE: first gate row of the tile
   int M = p.M;
@@ -671,6 +695,18 @@ template <class Act, class Fmt, int BM, int BN>
 static int launch_gemm_tiled(GemmArgs p, hipStream_t st) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
+  // XCD grid: among the splits that divide both tile counts, the one with the least operand
+  // traffic (a weight tile is fetched by xcd_m L2s, a slab of x by 8 / xcd_m)
+  p.xcd_m = 0;
+  {
+    const double wbytes = (double)p.N * p.K * Fmt::kWeightBytesPerK, xbytes = (double)p.M * p.K * 2.0;
+    double best = 0.0;
+    for (int a = 1; a <= 8; a *= 2) {
+      if (p.tiles_m % a || p.tiles_n % (8 / a)) continue;
+      const double cost = a * wbytes + (8 / a) * xbytes;
+      if (!p.xcd_m || cost < best) { best = cost; p.xcd_m = a; }
+    }
+  }
   const size_t lds = (size_t)2 * (Fmt::B_CH * 256 / Fmt::CPR) * kPitch * 2;
   auto kern = gemm_tiled_kernel<Act, Fmt, BM, BN>;
   if (lds > 64 * 1024) {

@@ -113,7 +113,7 @@ constexpr int kMoeBM = 256;
 template <class Act, template <class, int> class FMT, bool FUSE>
 static int launch_grouped(GemmArgs p, int max_tiles, hipStream_t st) {
   constexpr int BN = 256;
-  p.tiles_m = max_tiles;
+  p.tiles_m = (max_tiles + 7) / 8 * 8;                // whole rounds of the 8 XCDs (surplus workgroups exit)
   p.tiles_n = FUSE ? (p.n_half + BN / 2 - 1) / (BN / 2) : (p.N + BN - 1) / BN;
   using F = FMT<Act, BN>;
   auto kern = gemm_tiled_kernel<Act, F, kMoeBM, BN, true, FUSE>;
