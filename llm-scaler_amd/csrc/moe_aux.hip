@@ -52,7 +52,8 @@ template <class Act, int SLOTS>
 __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,
                                                        typename Act::elem* __restrict__ top_w,
                                                        int32_t* __restrict__ top_ids, int T, int E,
-                                                       int K, int renorm) {
+                                                       int K, int renorm,
+                                                       const float* __restrict__ expert_scale) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
@@ -94,7 +95,10 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
   }
   if (lane < K) {
     const float w = renorm ? my_w / sel_sum : my_w;
-    top_w[(size_t)t * K + lane] = Act::from_f32(w);
+    typename Act::elem w16 = Act::from_f32(w);
+    // optional factor per selected expert, applied to the rounded weight and rounded again
+    if (expert_scale) w16 = Act::from_f32(Act::to_f32(w16) * expert_scale[my_id]);
+    top_w[(size_t)t * K + lane] = w16;
     top_ids[(size_t)t * K + lane] = my_id;
   }
 }
@@ -671,7 +675,7 @@ using namespace qlin;
 extern "C" {
 
 int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
-                int act_dtype, void* stream) {
+                const float* expert_scale, int act_dtype, void* stream) {
   if (!logits || !top_w || !top_ids) return MI_ERR_ARG;
   if (T < 0 || E < 1 || E > 64 * kTopkSlots || K < 1 || K > 64 || K > E) return MI_ERR_SHAPE;
   if (!T) return MI_OK;
@@ -682,10 +686,10 @@ int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E,
   do {                                                                                              \
     if (act_dtype == DT_F16)                                                                        \
       hipLaunchKernelGGL((moe_topk_kernel<ActF16, SLOTS>), grid, block, 0, st, (const _Float16*)logits, \
-                         (_Float16*)top_w, top_ids, T, E, K, renorm);                               \
+                         (_Float16*)top_w, top_ids, T, E, K, renorm, expert_scale);                               \
     else                                                                                            \
       hipLaunchKernelGGL((moe_topk_kernel<ActBF16, SLOTS>), grid, block, 0, st, (const __bf16*)logits,  \
-                         (__bf16*)top_w, top_ids, T, E, K, renorm);                                 \
+                         (__bf16*)top_w, top_ids, T, E, K, renorm, expert_scale);                                 \
   } while (0)
   if (E <= 128) QLIN_TOPK(2);
   else if (E <= 256) QLIN_TOPK(4);

@@ -92,8 +92,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   constexpr int kCols = SILU ? (RT / 2) * 16 : RT * 16;   // output columns per tile group
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // 2 * kWBuf + 4 * MT * 16 * APitch
 
-  const int e = blockIdx.x / p.tiles_per_expert;
-  const int wg = blockIdx.x - e * p.tiles_per_expert;
+  // The 8 XCDs take workgroups round-robin and each has its own L2: all workgroups of an expert
+  // go to XCD (expert % 8), so that the expert's activation rows are fetched into one L2 only.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int e = (slot / p.tiles_per_expert) * 8 + xcd;
+  const int wg = slot % p.tiles_per_expert;
+  if (e >= p.E) return;
   const int r0 = expert_start[e];
   const int cnt = expert_start[e + 1] - r0;
   if (cnt <= 0) return;
@@ -389,7 +393,7 @@ static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
   p.tpw = tpw;
   p.tiles_per_expert = (groups + tpw - 1) / tpw;
   p.n_out = cols;
-  const long wgs = (long)p.E * p.tiles_per_expert;
+  const long wgs = (long)((p.E + 7) / 8) * 8 * p.tiles_per_expert;   // whole rounds of the 8 XCDs
   if (wgs <= 0) return MI_OK;
   const size_t lds = (size_t)2 * RT * 16 * kWPitch + (size_t)4 * MT * 16 * (A8 ? kWPitch : kA16Pitch);
   static bool raised_pe = false, raised_block = false; // per instantiation of this function = per kernel

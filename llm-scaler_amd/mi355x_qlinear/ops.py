@@ -781,19 +781,20 @@ def esimd_moe_topk(router_logits, top_values, top_indices, T):
          f"{who}: top_indices must be contiguous int32 [T, K]")
     _chk(E <= 1024 and 1 <= K <= min(64, E), f"{who}: needs E <= 1024 and 1 <= K <= min(64, E)")
     capi.call("mi_moe_topk", router_logits, capi.ptr(router_logits), capi.ptr(top_values),
-              capi.ptr(top_indices), T, E, K, 1, capi.act_dtype(router_logits))
+              capi.ptr(top_indices), T, E, K, 1, None, capi.act_dtype(router_logits))
     return top_values
 
 
-def moe_topk(logits, top_k, norm):
-    """moe_ops::moe_topk(logits, top_k, norm) -> (weights, ids); outputs are allocated here."""
+def moe_topk(logits, top_k, norm, expert_scale=None):
+    """moe_ops::moe_topk(logits, top_k, norm) -> (weights, ids); outputs are allocated here.
+    expert_scale (fp32 [E], not part of the op's schema): factor on the rounded weight of each selected expert."""
     _chk(logits.dim() == 2 and logits.is_contiguous(), "moe_topk: logits must be contiguous [T, E]")
     T, E = logits.shape
     w = torch.empty(T, int(top_k), dtype=logits.dtype, device=logits.device)
     ids = torch.empty(T, int(top_k), dtype=torch.int32, device=logits.device)
     _chk(E <= 1024 and 1 <= int(top_k) <= min(64, E), "moe_topk: needs E <= 1024 and 1 <= top_k <= min(64, E)")
     capi.call("mi_moe_topk", logits, capi.ptr(logits), capi.ptr(w), capi.ptr(ids), T, E, int(top_k),
-              1 if norm else 0, capi.act_dtype(logits))
+              1 if norm else 0, capi.ptr(expert_scale), capi.act_dtype(logits))
     return w, ids
 
 
@@ -1566,10 +1567,9 @@ def moe_up_fp8_grouped(x, gate_up_weight, gate_up_scale, expert_offsets, expert_
     P = x.shape[0] * k
     _chk(expert_tokens.numel() == P and expert_offsets.numel() >= E, f"{who}: expert_tokens must hold T*top_k pairs")
     tokens = expert_tokens.contiguous()
-    row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
     out = torch.empty(P, two_i // 2, dtype=x.dtype, device=x.device)
-    return _moe_gemm(x, None, row_map, gate_up_weight, gate_up_scale.contiguous(), _prefill_starts(expert_offsets[:E], P),
-                     out, E, two_i, H, _ACT_GELU_TANH, who, per_expert=True, out_map=tokens)
+    return _moe_gemm(x, None, tokens, gate_up_weight, gate_up_scale.contiguous(), _prefill_starts(expert_offsets[:E], P),
+                     out, E, two_i, H, _ACT_GELU_TANH, who, per_expert=True, out_map=tokens, row_map_div=k)
 
 
 def moe_down_fp8_grouped(intermediate, down_weight, down_scale, routing_weights, expert_offsets, expert_tokens,
@@ -1610,10 +1610,9 @@ def moe_forward_full_fp8_grouped(x, gate_up_weight, gate_up_scale, down_weight, 
          f"{who}: routing_weights and expert_tokens must hold one entry per pair, weights in the activation dtype")
     tokens = expert_tokens.contiguous()
     start = _prefill_starts(expert_offsets[:E], P)
-    row_map = torch.div(tokens, k, rounding_mode="floor").to(torch.int32)
     inter = torch.empty(P, I, dtype=x.dtype, device=x.device)
-    _moe_gemm(x, None, row_map, gate_up_weight, gate_up_scale.contiguous(), start, inter, E, two_i, H, _ACT_GELU_TANH, who,
-              per_expert=True)
+    _moe_gemm(x, None, tokens, gate_up_weight, gate_up_scale.contiguous(), start, inter, E, two_i, H, _ACT_GELU_TANH, who,
+              per_expert=True, row_map_div=k)
     y = torch.empty(P, H, dtype=torch.float32, device=x.device)
     _moe_gemm(inter, None, None, down_weight, down_scale.contiguous(), start, y, E, H, I, _ACT_NONE, who, per_expert=True,
               out_map=tokens)
@@ -1761,8 +1760,7 @@ def moe_forward_full_gelu_tanh_decode(x, logits, gate_up_weight, gate_up_scale, 
          f"{who}: logits must be [1, n_routed_experts] in the activation dtype")
     _chk(per_expert_scale.dtype == torch.float32 and per_expert_scale.numel() >= int(n_routed_experts),
          f"{who}: per_expert_scale must be float32 [n_routed_experts]")
-    top_w, top_ids = moe_topk(logits, int(top_k), True)
-    top_w = (top_w.float() * per_expert_scale.reshape(-1)[top_ids.long()]).to(x.dtype)
+    top_w, top_ids = moe_topk(logits, int(top_k), True, per_expert_scale.contiguous())
     return _moe_pert_routed(x, top_w, top_ids, gate_up_weight, gate_up_scale, down_weight, down_scale, top_k,
                             _ACT_GELU_TANH, True, who)
 
