@@ -404,7 +404,8 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
  *     scale_per_expert = 2: w_scale is [E, 2] fp32, the first factor for weight rows [0, N/2)
  *     and the second for rows [N/2, N) (the gate / up scales of the sglang prefill kernels,
  *     S/csrc/moe_prefill/moe_prefill_fp8.sycl:480-530); without fuse_act N/2 must be a multiple of 16.
- *     scale_per_expert = 0: block scales [E, ceil(N/128), ceil(K/128)] as above.
+ *     scale_per_expert = 0: block scales [E, ceil(N/128), ceil(K/128)] as above; with fuse_act
+ *     N/2 must then be a multiple of 16 (a 16-row tile of the up half stays inside one block).
  *   row_map_div (>= 1): the source row of sorted position r is row_map[r] / row_map_div, so that a
  *     map of pair indices (token * top_k + slot) gathers token rows with row_map_div = top_k.
  *   fuse_act: 0 none, 1 silu(gate) * up, 2 gelu_tanh(gate) * up (exp argument held in

@@ -446,6 +446,8 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
   if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
   if (scale_per_expert < 0 || scale_per_expert > 2 || row_map_div < 1) return MI_ERR_ARG;
   if (scale_per_expert == 2 && (N % 2 || (!fuse_act && (N / 2) % 16))) return MI_ERR_SHAPE;   // halves of whole 16-row tiles
+  // block scales with the fused epilogue: a 16-row tile of the up half must not straddle two 128-row blocks
+  if (!scale_per_expert && fuse_act && (N / 2) % 16) return MI_ERR_SHAPE;
   if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || (uint64_t)a_rows * (uint64_t)K * 2 >= (1ull << 31))
     return MI_ERR_SHAPE;
   if (!E || !total_rows) return MI_OK;

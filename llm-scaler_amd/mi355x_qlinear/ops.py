@@ -955,6 +955,7 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
              f"{who}: with gate / up scales N/2 must be a multiple of 16")
     else:
         _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+        _chk(not fuse or (N // 2) % 16 == 0, f"{who}: with block scales and the fused gate * up epilogue N/2 must be a multiple of 16")
         _chk(w_scale.dtype == torch.float32 and w_scale.is_contiguous() and
              w_scale.numel() == E * ((N + 127) // 128) * (K // 128),
              f"{who}: weight_scale must be contiguous fp32 [E, ceil(N/128), K/128]")

@@ -737,6 +737,12 @@ def test_moe_gemm_grouped_argument_errors(v, dev):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 3))
     with pytest.raises(RuntimeError):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 0, 3))          # no such scale form
+    # block scales with the fused epilogue: N/2 = 500 would put 16-row tiles of the up half across two scale blocks
+    with pytest.raises(RuntimeError):
+        v.moe_gemm_fp8_block(torch.zeros(4, 128, dtype=torch.float16, device=dev), None, None,
+                             torch.zeros(2, 1000, 128, dtype=torch.uint8, device=dev),
+                             torch.ones(2, 8, 1, device=dev), start, torch.zeros(4, 500, dtype=torch.float16, device=dev),
+                             1000, 128, 2, True)
     with pytest.raises(RuntimeError):
         capi.call("mi_moe_gemm_fp8_grouped", a, *args(64, 0, 1, 0))       # row-map divisor below 1
 
