@@ -75,9 +75,9 @@ constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of
 // The weights are the MFMA A operand and the activations the B operand, so a lane
 // ends up holding ONE activation row (16 w + j) and four consecutive weight rows
 // (4 g + v): the per-row activation scale is a single value per lane and granule.
-// MT = 16-row activation tiles per wavefront and pass (1: up to 64 rows per pass, the decode /
-// small-prefill case; 4: up to 256 rows per pass for experts with hundreds of rows, so that a
-// weight granule fetched once serves four times as many rows).
+// MT = 16-row activation tiles per wavefront and pass.  Only MT = 1 (up to 64 rows per pass) is
+// launched: with 4 the kernel is bound by its LDS traffic and gained nothing for experts with
+// hundreds of rows, which run on the tiled matrix-core GEMM instead (moe_gemm_tiled.hip).
 template <class Act, bool A8, bool SILU, int RT, int D, bool PE, int MT = 1>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, const float* __restrict__ w_scale,
                                                         const int32_t* __restrict__ expert_start) {
