@@ -619,49 +619,55 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
     }
   }
   constexpr int TNO = FUSE ? TN / 2 : TN;             // output column tiles of this wavefront
+  // first of this lane's 4 output columns in column tile ao; FUSE: gate tile 2 ao pairs with up tile 2 ao + 1
+  auto col_of = [&](int ao) { return FUSE ? n0 + (wn0 >> 1) + ao * 16 + g * 4 : n0 + wn0 + ao * 16 + g * 4; };
+  [[maybe_unused]] float os_all[Fmt::kOutScale ? TNO : 1][4];
+  [[maybe_unused]] float os_up = 1.0f;
+  if constexpr (Fmt::kOutScale) {
+    if constexpr (FUSE) os_up = Fmt::out_scale(res, p, p.n_half);
 #pragma unroll
-  for (int ao = 0; ao < TNO; ++ao) {
-    const int a = FUSE ? 2 * ao : ao;
-    // first of this lane's 4 output columns; FUSE: gate tile a pairs with up tile a + 1
-    const int n = FUSE ? n0 + (wn0 >> 1) + ao * 16 + g * 4 : n0 + wn0 + a * 16 + g * 4;
-    float os[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    [[maybe_unused]] float os_up = 1.0f;
-    if constexpr (Fmt::kOutScale && FUSE) os_up = Fmt::out_scale(res, p, p.n_half);
-    if constexpr (Fmt::kOutScale) {
+    for (int ao = 0; ao < TNO; ++ao)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) os[v] = Fmt::out_scale(res, p, n + v < N ? n + v : N - 1);
-    }
+      for (int v = 0; v < 4; ++v) os_all[ao][v] = Fmt::out_scale(res, p, col_of(ao) + v < N ? col_of(ao) + v : N - 1);
+  }
+  // Row tile outermost: the stores that follow each other fill one output row's columns from left to
+  // right (32 bytes each), so a row's 128-byte lines are completed by consecutive instructions and can be
+  // merged on their way to memory.
 #pragma unroll
-    for (int b = 0; b < TM; ++b) {
-      if (orow[b] >= 0) {
-        Elem v4[4];
+  for (int b = 0; b < TM; ++b) {
+    if (orow[b] < 0) continue;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          float r;
-          if constexpr (FUSE) {
-            // one factor per tensor / expert, or one for the gate rows and one for the up rows
-            const float gate = acc[a][b][v] * os[v], up = acc[a + 1][b][v] * (p.scale_mode == 3 ? os_up : os[v]);
-            if (p.gelu) {
-              float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
-              two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
-              const float ex = __expf(two_z);
-              r = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up;
-            } else {
-              r = gate / (1.0f + __expf(-gate)) * up;
-            }
+    for (int ao = 0; ao < TNO; ++ao) {
+      const int a = FUSE ? 2 * ao : ao;
+      const int n = col_of(ao);
+      Elem v4[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float r;
+        if constexpr (FUSE) {
+          // one factor per tensor / expert, or one for the gate rows and one for the up rows
+          const float osv = Fmt::kOutScale ? os_all[Fmt::kOutScale ? ao : 0][v] : 1.0f;
+          const float gate = acc[a][b][v] * osv, up = acc[a + 1][b][v] * (p.scale_mode == 3 ? os_up : osv);
+          if (p.gelu) {
+            float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
+            two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
+            const float ex = __expf(two_z);
+            r = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up;
           } else {
-            r = Fmt::kOutScale ? acc[a][b][v] * os[v] : acc[a][b][v];
+            r = gate / (1.0f + __expf(-gate)) * up;
           }
-          v4[v] = Act::from_f32(GROUPED ? r * rw[b] : r);
-        }
-        Elem* dst = out + (size_t)orow[b] * n_out + n;
-        if (n + 3 < n_out && (n_out & 3) == 0) {
-          *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(v4);
         } else {
-#pragma unroll
-          for (int v = 0; v < 4; ++v)
-            if (n + v < n_out) dst[v] = v4[v];
+          r = Fmt::kOutScale ? acc[a][b][v] * os_all[Fmt::kOutScale ? ao : 0][v] : acc[a][b][v];
         }
+        v4[v] = Act::from_f32(GROUPED ? r * rw[b] : r);
+      }
+      Elem* dst = out + (size_t)orow[b] * n_out + n;
+      if (n + 3 < n_out && (n_out & 3) == 0) {
+        *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(v4);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (n + v < n_out) dst[v] = v4[v];
       }
     }
   }
