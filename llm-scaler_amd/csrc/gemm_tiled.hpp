@@ -682,8 +682,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
 static __global__ __launch_bounds__(256) void pack_x_kernel(const uint16_t* __restrict__ x, u32x4* __restrict__ xp,
                                                             int M, int K, int Q, int perm_k) {
   const int l = threadIdx.x & 63;
-  const int q = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int t = blockIdx.y;
+  const int nq4 = (Q + 3) >> 2;                       // flat grid: 4 steps of one row tile per workgroup
+  const int t = blockIdx.x / nq4;
+  const int q = (blockIdx.x - t * nq4) * 4 + (threadIdx.x >> 6);
   if (q >= Q) return;
   const int m = t * 16 + (l & 15);
   u32x4 v = {0u, 0u, 0u, 0u};
@@ -754,7 +755,7 @@ template <class Act, template <class, int> class FMT>
 static int run_gemm_tiled(GemmArgs p, const void* x, void* workspace, hipStream_t st) {
   const int Mp = (p.M + 15) & ~15;
   const int Q = p.K / 32;
-  hipLaunchKernelGGL(pack_x_kernel, dim3((Q + 3) / 4, Mp / 16), dim3(256), 0, st, (const uint16_t*)x,
+  hipLaunchKernelGGL(pack_x_kernel, dim3((unsigned)(((Q + 3) / 4) * (Mp / 16))), dim3(256), 0, st, (const uint16_t*)x,
                      (u32x4*)workspace, p.M, p.K, Q, FMT<Act, 128>::kPermK ? 1 : 0);
   p.x = workspace;
   // 256-row tiles once they occupy more than half of the CUs (a 128 x 128 tile does a quarter of the

@@ -75,10 +75,11 @@ __global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __r
                                                              const int32_t* __restrict__ counts,
                                                              u32x4* __restrict__ xp, int a_rows, int K, int Q,
                                                              int row_div) {
-  const int b = blockIdx.y;
+  const int nq4 = (Q + 3) >> 2;                       // flat grid: 4 steps of one block per workgroup
+  const int b = blockIdx.x / nq4;
   if (b >= counts[1]) return;
   const int l = threadIdx.x & 63;
-  const int q = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int q = (blockIdx.x - b * nq4) * 4 + (threadIdx.x >> 6);
   if (q >= Q) return;
   const int r = l & 15;
   u32x4 v = {0u, 0u, 0u, 0u};
@@ -174,7 +175,7 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_
   int32_t* counts = (int32_t*)(ws + L.cnt_off);
   hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(kMapThreads), 0, st, expert_start, E, bm, g_tile, blk, counts);
   const int Q = K / 32;
-  hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((Q + 3) / 4, L.max_blocks), dim3(256), 0, st, (const uint16_t*)a,
+  hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((unsigned)(((Q + 3) / 4) * L.max_blocks)), dim3(256), 0, st, (const uint16_t*)a,
                      row_map, blk, counts, (u32x4*)ws, a_rows, K, Q, row_map_div);
   GemmArgs p{};
   p.x = ws; p.w = w; p.scale = w_scale; p.out = out; p.M = total_rows; p.N = N; p.K = K;

@@ -252,7 +252,9 @@ def test_fp8_register_resident_activations(ops, dev, M, K, N, dt, mode):
     (130, 512, 64, torch.float16, "pern16"), (300, 1024, 777, torch.float16, "pert"), (65, 5120, 5120, torch.float16, "block"),
     (200, 1024, 4160, torch.bfloat16, "block"), (2048, 5120, 5120, torch.bfloat16, "block"), (513, 768, 200, torch.bfloat16, "block"),
     # 192- and 160-column tiles
-    (1900, 256, 6144, torch.float16, "pern"), (2047, 384, 5100, torch.float16, "pert"), (2040, 256, 6100, torch.bfloat16, "block")])
+    (1900, 256, 6144, torch.float16, "pern"), (2047, 384, 5100, torch.float16, "pert"), (2040, 256, 6100, torch.bfloat16, "block"),
+    # more than 65535 16-row tiles of activations
+    (1_050_001, 128, 16, torch.bfloat16, "pern")])
 def test_fp8_prefill_tiled_gemm(ops, dev, M, K, N, dt, mode):
     # more than 64 rows: the tiled matrix-core GEMM (the weight is read once per 256 rows); the same
     # bar as the small-M path, on a strided sample of rows and columns where the problem is large
