@@ -904,3 +904,28 @@ def test_short_rows_fp8_and_int4(ops, dev, N, K, M):
         v.esimd_gemv_int4(xb.to(dev), packed.to(dev), scale.to(dev), outb)
         ref = O.matmul_ref(xb, O.int4_dequant(packed, scale, out_dtype=torch.float32))
         assert O.max_rel_err(outb.cpu(), ref) < TOL
+
+
+def test_stream_read_yardstick(dev):
+    """The read yardstick the benchmark reports as floor_us: every launch shape runs on sizes from one 16-byte
+    word to tens of MB, leaves the sink alone on ordinary data, and bad arguments are refused."""
+    import ctypes
+    from mi355x_qlinear import capi
+    lib = capi.lib()
+    words = ctypes.c_longlong(0)
+    assert lib.mi_stream_read_sink_words(ctypes.byref(words)) == 0 and words.value > 0
+    sink = torch.zeros(words.value, dtype=torch.int32, device=dev)
+    buf = torch.arange(0, 48 << 20, dtype=torch.int64, device=dev).view(torch.uint8)[: 40 << 20]
+    nvar = lib.mi_stream_read_variants()
+    assert nvar >= 1
+    for variant in range(nvar):
+        for nbytes in (16, 4096, 1 << 20, (40 << 20) - 16):
+            capi.call("mi_stream_read", buf, capi.ptr(buf), nbytes, capi.ptr(sink), variant)
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0
+    with pytest.raises(RuntimeError):
+        capi.call("mi_stream_read", buf, capi.ptr(buf), 24, capi.ptr(sink), 0)          # not a multiple of 16
+    with pytest.raises(RuntimeError):
+        capi.call("mi_stream_read", buf, capi.ptr(buf), 1024, capi.ptr(sink), nvar)     # no such shape
+    with pytest.raises(RuntimeError):
+        capi.call("mi_stream_read", buf, buf.data_ptr() + 8, 1024, capi.ptr(sink), 0)   # misaligned source
