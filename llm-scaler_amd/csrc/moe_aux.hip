@@ -11,43 +11,34 @@ namespace qlin {
 // One wavefront per token.  Expert e lives in lane e % 64, slot e / 64.  The
 // selection runs on the logits (softmax is monotone): K rounds of wave-wide
 // argmax where the LOWEST index wins ties, then the selected probabilities are
-// renormalised.  A round is one 64-bit wave maximum over keys
-// (order-preserving logit bits, ~index), reduced with DPP inside rows of 16
-// lanes and v_readlane across the four rows.
+// renormalised.  The logits are 16-bit values, so a round is one 32-bit wave
+// maximum over keys (order-preserving 16 logit bits << 16 | 0xFFFF - index),
+// reduced with DPP inside rows of 16 lanes and v_readlane across the four rows;
+// the winner's logit is recovered from the key itself.
 constexpr int kTopkSlots = 16;                       // up to 1024 experts
 
 template <int CTRL>
-__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {
-  const int lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, 0xF, 0xF, true);
-  const int hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, 0xF, 0xF, true);
-  const uint64_t o = ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo;
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
   return o > v ? o : v;
 }
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-  v = dpp_max_u64<0xB1>(v);
-  v = dpp_max_u64<0x4E>(v);
-  v = dpp_max_u64<0x141>(v);
-  v = dpp_max_u64<0x140>(v);
-  uint64_t r = 0;
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = dpp_max_u32<0xB1>(v);
+  v = dpp_max_u32<0x4E>(v);
+  v = dpp_max_u32<0x141>(v);
+  v = dpp_max_u32<0x140>(v);
+  uint32_t r = 0;
 #pragma unroll
   for (int row = 0; row < 4; ++row) {
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, row * 16);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), row * 16);
-    const uint64_t o = ((uint64_t)hi << 32) | lo;
+    const uint32_t o = (uint32_t)__builtin_amdgcn_readlane((int)v, row * 16);
     r = o > r ? o : r;
   }
   return r;
 }
-// float -> unsigned, monotone (NaN-free inputs; -inf maps below every finite value)
-__device__ __forceinline__ uint32_t f32_order(float f) {
-  const uint32_t b = __builtin_bit_cast(uint32_t, f);
-  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-}
-__device__ __forceinline__ float f32_unorder(uint32_t u) {
-  const uint32_t b = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
-  return __builtin_bit_cast(float, b);
-}
-
+// 16-bit float pattern (fp16 or bf16) -> unsigned, monotone, and back; the smallest key, 0, is kept for
+// "no value" (it would be the pattern of the negative NaN with every bit set)
+__device__ __forceinline__ uint32_t f16_order(uint32_t b) { return (b & 0x8000u) ? (~b & 0xFFFFu) : (b | 0x8000u); }
+__device__ __forceinline__ uint32_t f16_unorder(uint32_t u) { return (u & 0x8000u) ? (u & 0x7FFFu) : (~u & 0xFFFFu); }
 template <class Act, int SLOTS>
 __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,
                                                        typename Act::elem* __restrict__ top_w,
@@ -59,11 +50,14 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
   if (t >= T) return;
   const typename Act::elem* row = logits + (size_t)t * E;
   float v[SLOTS];
+  uint32_t key[SLOTS];                               // selection keys; 0 = taken or past E
   float mx = -INFINITY;
 #pragma unroll
   for (int s = 0; s < SLOTS; ++s) {
     const int e = s * 64 + lane;
-    v[s] = e < E ? Act::to_f32(row[e]) : -INFINITY;
+    const typename Act::elem raw = e < E ? row[e] : Act::from_f32(0.f);
+    v[s] = e < E ? Act::to_f32(raw) : -INFINITY;
+    key[s] = e < E ? (f16_order((uint32_t)__builtin_bit_cast(uint16_t, raw)) << 16) | (0xFFFFu - (uint32_t)e) : 0u;
     mx = fmaxf(mx, v[s]);
   }
   mx = wave_max(mx);
@@ -76,19 +70,16 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
   int my_id = 0;
   float sel_sum = 0.f;
   for (int r = 0; r < K; ++r) {
-    uint64_t key = 0;
+    uint32_t best = 0;
 #pragma unroll
-    for (int s = 0; s < SLOTS; ++s) {
-      const uint64_t k = ((uint64_t)f32_order(v[s]) << 32) | (uint32_t)~(uint32_t)(s * 64 + lane);
-      key = k > key ? k : key;
-    }
-    key = wave_max_u64(key);
-    const int cand = (int)~(uint32_t)key;
-    const float wbest = f32_unorder((uint32_t)(key >> 32));
+    for (int s = 0; s < SLOTS; ++s) best = key[s] > best ? key[s] : best;
+    best = wave_max_u32(best);
+    const int cand = (int)(0xFFFFu - (best & 0xFFFFu));
+    const float wbest = Act::to_f32(__builtin_bit_cast(typename Act::elem, (uint16_t)f16_unorder(best >> 16)));
     // remove the winner from its owner lane
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
-      if (s * 64 + lane == cand) v[s] = -INFINITY;
+      if (s * 64 + lane == cand) key[s] = 0u;
     const float p = __expf(wbest - mx) / sum;
     sel_sum += p;
     if (lane == r) { my_w = p; my_id = cand; }
