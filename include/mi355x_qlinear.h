@@ -207,7 +207,10 @@ int mi_q4_0_quantize(const void* x, void* qweight, void* scale, int rows, int K,
  *   descending probability) -> optional renormalisation; top_w in the activation
  *   dtype, top_ids int32.  E <= 1024, K <= 64.  expert_scale (optional, fp32 [E]): the rounded
  *   weight of a selected expert is multiplied by its entry and rounded again (MoeFoldExpertScale,
- *   V/csrc/moe_batch/moe_decode_gemv.h:146-158).  Replaces esimd_moe_topk /
+ *   V/csrc/moe_batch/moe_decode_gemv.h:146-158).  gate_out (optional, fp32 [T], with gate_x [T, H]
+ *   and gate_weight [H] in the activation type, H % 8 == 0): the same launch also writes
+ *   sigmoid(gate_x[t] . gate_weight), the shared expert's gate of the fused decode ops (what
+ *   mi_moe_shared_gate computes on its own).  Replaces esimd_moe_topk /
  *   moe_ops::moe_topk (V/csrc/xpu/esimd_kernels/moe_ops.h:106-231,
  *   V/csrc/xpu/esimd_kernel_moe.sycl:71-84).
  * mi_moe_sort: stable counting sort of the T*K (token, route) pairs by expert:
@@ -220,7 +223,8 @@ int mi_q4_0_quantize(const void* x, void* qweight, void* scale, int rows, int K,
  *   (S/csrc/moe_prefill/moe_prefill_fp8.sycl:105-161), whose in-expert order is
  *   atomic-arrival order. */
 int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
-                const float* expert_scale, int act_dtype, void* stream);
+                const float* expert_scale, const void* gate_x, const void* gate_weight, float* gate_out, int H,
+                int act_dtype, void* stream);
 int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
                 int32_t* sorted_token, int32_t* max_count, int T, int K, int E, void* stream);
 

@@ -44,10 +44,23 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
                                                        typename Act::elem* __restrict__ top_w,
                                                        int32_t* __restrict__ top_ids, int T, int E,
                                                        int K, int renorm,
-                                                       const float* __restrict__ expert_scale) {
+                                                       const float* __restrict__ expert_scale,
+                                                       const typename Act::v8* __restrict__ gate_x,
+                                                       const typename Act::v8* __restrict__ gate_w,
+                                                       float* __restrict__ gate_out, int H8) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
+  // optional second result of the same wavefront: gate_out[t] = sigmoid(gate_x[t, :] . gate_w[:]) (the
+  // shared expert's gate of the fused decode ops); its loads are in flight while the selection runs
+  float gate_acc = 0.f;
+  if (gate_out) {
+    for (int c = lane; c < H8; c += 64) {
+      const typename Act::v8 a = gate_x[(size_t)t * H8 + c], b = gate_w[c];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) gate_acc += Act::to_f32(a[e]) * Act::to_f32(b[e]);
+    }
+  }
   const typename Act::elem* row = logits + (size_t)t * E;
   float v[SLOTS];
   uint32_t key[SLOTS];                               // selection keys; 0 = taken or past E
@@ -91,6 +104,10 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
     if (expert_scale) w16 = Act::from_f32(Act::to_f32(w16) * expert_scale[my_id]);
     top_w[(size_t)t * K + lane] = w16;
     top_ids[(size_t)t * K + lane] = my_id;
+  }
+  if (gate_out) {
+    gate_acc = wave_sum(gate_acc);
+    if (lane == 0) gate_out[t] = 1.0f / (1.0f + __expf(-gate_acc));
   }
 }
 
@@ -666,8 +683,12 @@ using namespace qlin;
 extern "C" {
 
 int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
-                const float* expert_scale, int act_dtype, void* stream) {
+                const float* expert_scale, const void* gate_x, const void* gate_weight, float* gate_out, int H,
+                int act_dtype, void* stream) {
   if (!logits || !top_w || !top_ids) return MI_ERR_ARG;
+  if (gate_out && (!gate_x || !gate_weight)) return MI_ERR_ARG;
+  if (gate_out && (H <= 0 || (H % 8))) return MI_ERR_SHAPE;
+  const int H8 = gate_out ? H / 8 : 0;
   if (T < 0 || E < 1 || E > 64 * kTopkSlots || K < 1 || K > 64 || K > E) return MI_ERR_SHAPE;
   if (!T) return MI_OK;
   hipStream_t st = (hipStream_t)stream;
@@ -677,10 +698,12 @@ int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E,
   do {                                                                                              \
     if (act_dtype == DT_F16)                                                                        \
       hipLaunchKernelGGL((moe_topk_kernel<ActF16, SLOTS>), grid, block, 0, st, (const _Float16*)logits, \
-                         (_Float16*)top_w, top_ids, T, E, K, renorm, expert_scale);                               \
+                         (_Float16*)top_w, top_ids, T, E, K, renorm, expert_scale, (const f16x8*)gate_x,        \
+                         (const f16x8*)gate_weight, gate_out, H8);                               \
     else                                                                                            \
       hipLaunchKernelGGL((moe_topk_kernel<ActBF16, SLOTS>), grid, block, 0, st, (const __bf16*)logits,  \
-                         (__bf16*)top_w, top_ids, T, E, K, renorm, expert_scale);                                 \
+                         (__bf16*)top_w, top_ids, T, E, K, renorm, expert_scale, (const bf16x8*)gate_x,         \
+                         (const bf16x8*)gate_weight, gate_out, H8);                                 \
   } while (0)
   if (E <= 128) QLIN_TOPK(2);
   else if (E <= 256) QLIN_TOPK(4);

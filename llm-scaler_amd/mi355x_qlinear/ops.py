@@ -768,7 +768,9 @@ def e4m3_decode(codes, output):
 # --------------------------------------------------------------------------
 # MoE: routing, permutation, grouped GEMM, combine
 # --------------------------------------------------------------------------
-def esimd_moe_topk(router_logits, top_values, top_indices, T):
+def esimd_moe_topk(router_logits, top_values, top_indices, T, gate=None):
+    """gate (not part of the op's schema) = (x [T, H], gate_weight [H], out fp32 [T]): the same launch also
+    writes out[t] = sigmoid(x[t] . gate_weight)."""
     who = "esimd_moe_topk"
     _chk(router_logits.dim() == 2 and router_logits.is_contiguous(), f"{who}: router_logits must be contiguous [T, E]")
     T = int(T)
@@ -781,20 +783,26 @@ def esimd_moe_topk(router_logits, top_values, top_indices, T):
          f"{who}: top_indices must be contiguous int32 [T, K]")
     _chk(E <= 1024 and 1 <= K <= min(64, E), f"{who}: needs E <= 1024 and 1 <= K <= min(64, E)")
     capi.call("mi_moe_topk", router_logits, capi.ptr(router_logits), capi.ptr(top_values),
-              capi.ptr(top_indices), T, E, K, 1, None, capi.act_dtype(router_logits))
+              capi.ptr(top_indices), T, E, K, 1, None, capi.ptr(gate[0]) if gate else None,
+              capi.ptr(gate[1]) if gate else None, capi.ptr(gate[2]) if gate else None,
+              gate[0].shape[1] if gate else 0, capi.act_dtype(router_logits))
     return top_values
 
 
-def moe_topk(logits, top_k, norm, expert_scale=None):
+def moe_topk(logits, top_k, norm, expert_scale=None, gate=None):
     """moe_ops::moe_topk(logits, top_k, norm) -> (weights, ids); outputs are allocated here.
-    expert_scale (fp32 [E], not part of the op's schema): factor on the rounded weight of each selected expert."""
+    Not part of the op's schema: expert_scale (fp32 [E]), a factor on the rounded weight of each selected
+    expert; gate = (x [T, H], gate_weight [H], out fp32 [T]): the same launch also writes
+    out[t] = sigmoid(x[t] . gate_weight)."""
     _chk(logits.dim() == 2 and logits.is_contiguous(), "moe_topk: logits must be contiguous [T, E]")
     T, E = logits.shape
     w = torch.empty(T, int(top_k), dtype=logits.dtype, device=logits.device)
     ids = torch.empty(T, int(top_k), dtype=torch.int32, device=logits.device)
     _chk(E <= 1024 and 1 <= int(top_k) <= min(64, E), "moe_topk: needs E <= 1024 and 1 <= top_k <= min(64, E)")
+    gx, gw, go = gate if gate is not None else (None, None, None)
     capi.call("mi_moe_topk", logits, capi.ptr(logits), capi.ptr(w), capi.ptr(ids), T, E, int(top_k),
-              1 if norm else 0, capi.ptr(expert_scale), capi.act_dtype(logits))
+              1 if norm else 0, capi.ptr(expert_scale), capi.ptr(gx), capi.ptr(gw), capi.ptr(go),
+              gx.shape[1] if gx is not None else 0, capi.act_dtype(logits))
     return w, ids
 
 
@@ -1132,7 +1140,9 @@ def moe_forward_full_fp8_block(x, logits, output, gate_up_weight, gate_up_scale,
     # routing and routed experts (w8a16 grouped GEMMs on the expert-sorted pairs)
     top_w = torch.empty(T, k, dtype=x.dtype, device=dev)
     top_ids = torch.empty(T, k, dtype=torch.int32, device=dev)
-    esimd_moe_topk(logits, top_w, top_ids, T)
+    gate = torch.empty(T, dtype=torch.float32, device=dev)
+    # routing and the shared expert's gate sigmoid(x . w) in one launch
+    esimd_moe_topk(logits, top_w, top_ids, T, gate=(x, shared_expert_gate_weight, gate))
     sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
     start = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(P, dtype=torch.int32, device=dev)
@@ -1149,9 +1159,6 @@ def moe_forward_full_fp8_block(x, logits, output, gate_up_weight, gate_up_scale,
     esimd_moe_silu_mul(sh_gu, sh_inter, 2 * I, I, T)
     sh_out = torch.empty(T, H, dtype=x.dtype, device=dev)
     esimd_gemm_fp8_blockscale(sh_inter, shared_down_weight, shared_down_scale, sh_out, 128, 128)
-    gate = torch.empty(T, dtype=torch.float32, device=dev)
-    capi.call("mi_moe_shared_gate", x, capi.ptr(x), capi.ptr(shared_expert_gate_weight), capi.ptr(gate), T, H,
-              capi.act_dtype(x))
     capi.call("mi_moe_combine_shared", y, capi.ptr(y), capi.ptr(inv), capi.ptr(top_w), capi.ptr(output),
               capi.ptr(sh_out), capi.ptr(gate), H, k, T, 0, capi.act_dtype(output), 1)
     return output
@@ -1803,7 +1810,13 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
          down_scale.numel() >= E, f"{who}: routed scales must be float32 [E]")
     dev = x.device
     P = T * k
-    top_w, top_ids = moe_topk(logits, k, True)
+    gate = gate_args = None
+    if S > 0:
+        _chk(shared_expert_gate_weight.dtype == x.dtype and shared_expert_gate_weight.numel() == H,
+             f"{who}: shared_expert_gate_weight must be [1, H] in x's dtype")
+        gate = torch.empty(T, dtype=torch.float32, device=dev)
+        gate_args = (x, shared_expert_gate_weight.contiguous(), gate)
+    top_w, top_ids = moe_topk(logits, k, True, gate=gate_args)     # routing + the shared expert's gate, one launch
     route_expert = top_ids.reshape(-1)
     adt = capi.act_dtype(x)
     s_up = _km_splits(P, H, 2 * I, dev)
@@ -1814,7 +1827,7 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
     dn_part = torch.empty(P, s_dn, H, dtype=torch.float32, device=dev)
     capi.call("mi_moe_kmajor_down", x, capi.ptr(up_part), s_up, capi.ptr(gate_up_scale.contiguous()), capi.ptr(down_weight),
               capi.ptr(route_expert), capi.ptr(dn_part), P, E, I, H, s_dn, 0, adt)
-    shared = gate = None
+    shared = None
     if S > 0:
         _chk(S == 1, f"{who}: one shared expert is supported")
         _chk_fp8(shared_gate_up_weight, who)
@@ -1823,16 +1836,12 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
              f"{who}: shared weights must be [1, 2*I, H] and [1, H, I]")
         _chk(shared_gate_up_scale.dtype == torch.float32 and shared_down_scale.dtype == torch.float32,
              f"{who}: shared scales must be float32")
-        _chk(shared_expert_gate_weight.dtype == x.dtype and shared_expert_gate_weight.numel() == H,
-             f"{who}: shared_expert_gate_weight must be [1, H] in x's dtype")
         sh_gu = torch.empty(T, 2 * I, dtype=x.dtype, device=dev)
         esimd_gemm_fp8_pert(x, shared_gate_up_weight.reshape(2 * I, H), shared_gate_up_scale.reshape(-1)[:1], sh_gu)
         sh_inter = torch.empty(T, I, dtype=x.dtype, device=dev)
         esimd_moe_silu_mul(sh_gu, sh_inter, 2 * I, I, T)
         shared = torch.empty(T, H, dtype=x.dtype, device=dev)
         esimd_gemm_fp8_pert(sh_inter, shared_down_weight.reshape(H, I), shared_down_scale.reshape(-1)[:1], shared)
-        gate = torch.empty(T, dtype=torch.float32, device=dev)
-        capi.call("mi_moe_shared_gate", x, capi.ptr(x), capi.ptr(shared_expert_gate_weight.contiguous()), capi.ptr(gate), T, H, adt)
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     capi.call("mi_moe_kmajor_finalize", x, capi.ptr(dn_part), s_dn, capi.ptr(down_scale.contiguous()), capi.ptr(route_expert),
               capi.ptr(top_w), capi.ptr(shared), capi.ptr(gate), capi.ptr(out), T, k, E, H, adt)
