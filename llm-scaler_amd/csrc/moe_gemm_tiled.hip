@@ -68,28 +68,36 @@ __global__ __launch_bounds__(kMapThreads) void moe_tile_map_kernel(const int32_t
 }
 
 // Gather + re-tile: block b of the table -> MFMA operand order (see pack_x_kernel); rows past the
-// block's count are zero.  One workgroup writes four 32-wide steps of one block.
+// block's count are zero.  One workgroup writes 16 consecutive 32-wide steps of one block (4 per
+// wavefront, their loads in flight together).
+constexpr int kPackQ = 16;
 __global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __restrict__ x,
                                                              const int32_t* __restrict__ row_map,
                                                              const int32_t* __restrict__ blk,
                                                              const int32_t* __restrict__ counts,
                                                              u32x4* __restrict__ xp, int a_rows, int K, int Q,
                                                              int row_div) {
-  const int nq4 = (Q + 3) >> 2;                       // flat grid: 4 steps of one block per workgroup
-  const int b = blockIdx.x / nq4;
+  const int nq = (Q + kPackQ - 1) / kPackQ;           // flat grid: kPackQ steps of one block per workgroup
+  const int b = blockIdx.x / nq;
   if (b >= counts[1]) return;
   const int l = threadIdx.x & 63;
-  const int q = (blockIdx.x - b * nq4) * 4 + (threadIdx.x >> 6);
-  if (q >= Q) return;
+  const int q0 = (blockIdx.x - b * nq) * kPackQ + (threadIdx.x >> 6) * 4;
   const int r = l & 15;
-  u32x4 v = {0u, 0u, 0u, 0u};
+  const uint16_t* src = nullptr;
   if (r < blk[2 * b + 1]) {
     const int pos = blk[2 * b] + r;
-    const unsigned src = row_map ? (unsigned)row_map[pos] / (unsigned)row_div : (unsigned)pos;
-    if (src < (unsigned)a_rows)
-      v = *reinterpret_cast<const u32x4*>(x + (size_t)src * K + q * 32 + (l >> 4) * 8);
+    const unsigned row = row_map ? (unsigned)row_map[pos] / (unsigned)row_div : (unsigned)pos;
+    if (row < (unsigned)a_rows) src = x + (size_t)row * K + (l >> 4) * 8;
   }
-  xp[((size_t)b * Q + q) * 64 + l] = v;
+  u32x4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[i] = u32x4{0u, 0u, 0u, 0u};
+    if (src && q0 + i < Q) v[i] = *reinterpret_cast<const u32x4*>(src + (q0 + i) * 32);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (q0 + i < Q) xp[((size_t)b * Q + q0 + i) * 64 + l] = v[i];
 }
 
 struct TiledMoeLayout {
@@ -175,7 +183,7 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_
   int32_t* counts = (int32_t*)(ws + L.cnt_off);
   hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(kMapThreads), 0, st, expert_start, E, bm, g_tile, blk, counts);
   const int Q = K / 32;
-  hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((unsigned)(((Q + 3) / 4) * L.max_blocks)), dim3(256), 0, st, (const uint16_t*)a,
+  hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((unsigned)(((Q + kPackQ - 1) / kPackQ) * L.max_blocks)), dim3(256), 0, st, (const uint16_t*)a,
                      row_map, blk, counts, (u32x4*)ws, a_rows, K, Q, row_map_div);
   GemmArgs p{};
   p.x = ws; p.w = w; p.scale = w_scale; p.out = out; p.M = total_rows; p.N = N; p.K = K;
