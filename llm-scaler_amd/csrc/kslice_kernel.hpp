@@ -4,9 +4,9 @@
 // workgroup can hold all of x in its register file (x is the matrix-core operand that never
 // changes while the weight streams past).  One workgroup owns up to 64 weight rows; its 8
 // wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
-//   - a wavefront loads its slice of x ONCE, straight into operand layout, before any weight
-//     load is issued (x comes from L2; the vector-memory counter retires in order, so these
-//     loads never queue behind the weight stream),
+//   - a wavefront loads its slice of x ONCE, before any weight load is issued (x comes from L2;
+//     the vector-memory counter retires in order, so these loads never queue behind the weight
+//     stream),
 //   - the loop is weight loads -> wave-private LDS transpose -> E4M3 decode -> MFMA, with the
 //     next 16-row tile in flight while the current one is consumed: no barrier, no x traffic,
 //   - the 8 partial tiles meet once, at the end, in LDS.
@@ -67,27 +67,58 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
   const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * (uint32_t)K);
   const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
 
-  // ---- x: the wavefront's slice of every row, once ----
-  u32x4 xq[MT][NQ][2];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int q = 0; q < NQ; ++q)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int m = mt * 16 + j;
-        const int k = kbase + 64 * q + 16 * g + 8 * h;
-        xq[mt][q][h] = buf_load16(xr, (m < M && k < K) ? ((uint32_t)m * (uint32_t)K + (uint32_t)k) * 2u : kOOB);
-      }
-
-  // ---- weights: two 16-row tiles in flight in registers ----
-  // The 64 NQ chunks of a tile's slice (16 rows x kCPR chunks) are walked row-major: load i takes
-  // chunks 64 i .. 64 i + 63, i.e. 1 KiB of consecutive slice bytes, row after row.
+  // The 64 NQ 16-byte chunks of a 16-row tile (16 rows x kCPR chunks) are walked row-major: load i
+  // takes chunks 64 i .. 64 i + 63, i.e. 1 KiB of consecutive bytes, row after row.
   auto chunk_of = [&](int i, int& r, int& c) {
     const int f = i * 64 + lane;
     r = f / kCPR;
     c = f - r * kCPR;
   };
+  unsigned char* stage = smem + wave * kStage;
+
+  // ---- x: the wavefront's slice of every row, once ----
+  // Loaded like the weights, row-contiguous: x is read by every workgroup, and an instruction
+  // whose lanes gather 16-byte operand pieces from 16 rows takes the L1 four times as long as
+  // one that reads 1 KiB in a row (measured: 256 workgroups x 32 rows x 4096, 6.5 against 1.6 us).
+  // A 16-row tile of the slice is two LDS tiles wide (16-bit elements), so it is staged in two
+  // halves; slot [mt][hx NQ/2 + i / 2][i % 2] holds load i of half hx until the transposition.
+  u32x4 xq[MT][NQ][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int hx = 0; hx < 2; ++hx)
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) {
+        int r, c;
+        chunk_of(i, r, c);
+        const int m = mt * 16 + r;
+        const int k = kbase + hx * (kSliceB / 2) + 8 * c;
+        xq[mt][hx * (NQ / 2) + i / 2][i & 1] =
+            buf_load16(xr, (m < M && k < K) ? ((uint32_t)m * (uint32_t)K + (uint32_t)k) * 2u : kOOB);
+      }
+  // registers (row-contiguous) -> LDS tile -> registers (operand layout: lane (j, g) of slot
+  // [mt][q][h] holds x[16 mt + j][slice + 64 q + 16 g + 8 h .. + 7])
+  auto transpose_x = [&]() {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int hx = 0; hx < 2; ++hx) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+          int r, c;
+          chunk_of(i, r, c);
+          *reinterpret_cast<u32x4*>(stage + r * kPitch + c * 16) = xq[mt][hx * (NQ / 2) + i / 2][i & 1];
+        }
+#pragma unroll
+        for (int q = 0; q < NQ / 2; ++q)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            xq[mt][hx * (NQ / 2) + q][h] =
+                *reinterpret_cast<const u32x4*>(stage + j * kPitch + 128 * q + 32 * g + 16 * h);
+      }
+  };
+
+  // ---- weights: two 16-row tiles in flight in registers ----
   auto load_tile = [&](u32x4 (&w)[NQ], int t) {
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
@@ -99,7 +130,6 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
       w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, ok ? (uint32_t)n * (uint32_t)K + (uint32_t)k : kOOB, 0, 2 /* nt */);
     }
   };
-  unsigned char* stage = smem + wave * kStage;
   // registers (row-contiguous) -> this wavefront's LDS tile -> registers (operand layout)
   auto transpose_tile = [&](u32x4 (&w)[NQ]) {
 #pragma unroll
@@ -159,6 +189,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
   load_tile(w0, 0);
   load_tile(w1, 1);
   __builtin_amdgcn_sched_barrier(0);
+  transpose_x();
   // Tiles 0 .. 3 with static register slots.  Every load is issued unconditionally (a tile past
   // the workgroup's range loads nothing), so the wait counts stay exact on every path; only the
   // arithmetic of a missing tile is skipped.
