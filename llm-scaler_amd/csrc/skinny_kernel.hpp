@@ -422,39 +422,30 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     }
   }
 
-  // ---- reduce the NW partial tiles through LDS ----
+  // ---- the NW partial tiles meet in LDS; the wavefronts share the output tiles ----
   __syncthreads();                                    // the buffer overlays the staging tiles
-  if (wave > 0) {
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) red[wave - 1][t][mt][lane] = acc[t][mt];
-  }
+    for (int mt = 0; mt < MT; ++mt) red[wave][t][mt][lane] = acc[t][mt];
   __syncthreads();
-  if (wave != 0) return;
-#pragma unroll
-  for (int w = 0; w < NW - 1; ++w)
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[t][mt] += red[w][t][mt][lane];
-
   // D layout: lane holds output column n0 + 16 t + j, rows mt*16 + 4 g + v.
   Elem* out = (Elem*)a.out[mat];
-#pragma unroll
-  for (int t = 0; t < RT; ++t) {
+  for (int o = wave; o < RT * MT; o += NW) {
+    const int t = o / MT, mt = o - t * MT;
     const int n = n0 + t * 16 + j;
+    f32x4 sum = red[0][t][mt][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[w][t][mt][lane];
     if (n < nend) {
       float os = 1.0f;
       if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[n] : s32[n];
       if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int m = mt * 16 + g * 4 + v;
-          if (m < M) out[(size_t)m * N + n] = Act::from_f32(acc[t][mt][v] * os);
-        }
+      for (int v = 0; v < 4; ++v) {
+        const int m = mt * 16 + g * 4 + v;
+        if (m < M) out[(size_t)m * N + n] = Act::from_f32(sum[v] * os);
+      }
     }
   }
 }
@@ -478,7 +469,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
   }
   if (tiles == 0) return;
   constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
-  constexpr int kRed = (NW - 1) * RT * MT * 1024;
+  constexpr int kRed = NW * RT * MT * 1024;
   static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
   const int with_tables = kStage + (SL ? skinny_table_bytes<FMT, RT>(a.K) : 0);
   const int lds = with_tables > kRed ? with_tables : kRed;
