@@ -14,9 +14,10 @@
 // bytes of a granule (loading MFMA operand layout directly makes every lane touch
 // a different 16-byte piece, and the texture addresser, not HBM, becomes the
 // limit), and a wave-private LDS tile turns them into operand layout.  The
-// weights always take this path (non-temporal loads); the activations only when
-// there are many rows (M > 32) — for few rows their direct loads are cheaper than
-// the extra LDS traffic.
+// weights always take this path (non-temporal loads); the activations from 17 rows
+// on — up to 16 rows their direct loads are cheaper than the extra LDS traffic
+// (INT4, N = 14336, K = 4096: 12.7 against 13.5 us at M = 8; 17.7 against 16.6 us at
+// M = 32, 11.9 against 9.8 us for N = 4096).
 //
 // Lane mapping inside one granule (128 k): lane = (j = lane % 16, g = lane / 16)
 // holds the 32 consecutive k  [128 gi + 32 g, +32)  of weight row n0 + j and of
@@ -28,6 +29,7 @@
 namespace qlin {
 
 constexpr int kMaxMat = 3;
+constexpr int kSkinnyXLdsFrom = 2;                  // 16-row activation tiles from which x is staged through LDS
 
 struct SkinnyArgs {
   const void* x;
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr int kWRowB = kByteW ? 128 : 64;           // weight bytes per row per granule
   constexpr int kWP = kWRowB + 16;                    // LDS pitch: operand reads hit distinct banks
   constexpr int kXP = 256 + 16;                       // activation tile pitch
-  constexpr bool kXLds = MT >= 4;                     // stage the activations through LDS too
+  constexpr bool kXLds = MT >= kSkinnyXLdsFrom;                    // stage the activations through LDS too
   constexpr int kWStage = NW * RT * 16 * kWP;         // activation tiles follow the weight tiles
   constexpr int kTiles = kWStage + (kXLds ? NW * MT * 16 * kXP : 0);   // SL: the scale tables follow
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -468,7 +470,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
     tiles += a.tiles[i];
   }
   if (tiles == 0) return;
-  constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
+  constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * MT * 16 * (256 + 16) : 0);
   constexpr int kRed = NW * RT * MT * 1024;
   static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
   const int with_tables = kStage + (SL ? skinny_table_bytes<FMT, RT>(a.K) : 0);
@@ -489,7 +491,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
 template <int FMT, int MT, int RT, int NW>
 static inline bool skinny_tables_fit(int K) {
   if constexpr (FMT == 1 || FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
-    constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= 4 ? NW * MT * 16 * (256 + 16) : 0);
+    constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * MT * 16 * (256 + 16) : 0);
     return (FMT == 1 || K % 256 == 0) && kStage + skinny_table_bytes<FMT, RT>(K) <= 160 * 1024;
   }
   return false;

@@ -435,6 +435,76 @@ def test_q4k_shapes(ops, dev, M, K, N):
     assert O.max_rel_err(out.cpu(), O.matmul_ref(x, w)) < TOL
 
 
+@pytest.mark.parametrize("fmt,M,K,N,dt", [
+    ("q4k", 64, 5120, 5120, torch.float16), ("q4k", 33, 1024, 1024, torch.float16), ("q4k", 50, 3328, 9000, torch.float16),
+    ("q4k", 64, 2048, 2060, torch.float16),
+    ("int4", 64, 4096, 4096, torch.bfloat16), ("int4", 40, 1664, 5000, torch.float16), ("int4", 64, 1024, 10240, torch.float16),
+    ("pern", 64, 4096, 5120, torch.bfloat16), ("pern", 48, 1664, 1500, torch.float16), ("pert", 35, 2048, 8192, torch.bfloat16),
+    ("block", 64, 5120, 5120, torch.float16), ("block", 34, 1536, 2304, torch.bfloat16), ("block", 64, 640, 4100, torch.bfloat16)])
+def test_mid_m_k_split(ops, dev, fmt, M, K, N, dt):
+    # 33 .. 64 rows against at most 40 weight rows per CU: workgroups split K, exchange fp32 partial
+    # tiles and the last one to arrive adds them in slice order.  Granule counts that do not divide
+    # by the split (13, 26, 5), a last 16-row tile that is partly empty, every scale form; each
+    # case runs three times into fresh outputs, which must agree bit for bit (the arrival
+    # counters are back at zero, the sum does not depend on who arrives last).
+    v, sg = ops
+    if fmt == "q4k":
+        x, raw = O.make_q4k_case(M, K, N, seed=M + N)
+        ql, sc, mn = O.q4k_repack(raw)
+        args = [torch.from_numpy(t).to(dev) for t in (ql, sc, mn)]
+        run = lambda out: sg.esimd_gemv_q4_k(xd, args[0], args[1], args[2], out)
+        ref = O.matmul_ref(x, torch.from_numpy(O.q4k_dequant(ql, sc, mn)))
+    elif fmt == "int4":
+        x, packed, scale, _ = O.make_int4_case(M, K, N, seed=M + N, act_dtype=dt)
+        pd, sd = packed.to(dev), scale.to(dev)
+        run = lambda out: v.esimd_gemv_int4(xd, pd, sd, out)
+        ref = O.matmul_ref(x, O.int4_dequant(packed, scale, out_dtype=dt))
+    elif fmt == "block":
+        x, w8, s = O.make_fp8_block_case(M, K, (N + 127) // 128 * 128, seed=M + K, act_dtype=dt, std=0.3)
+        w8 = w8[:N].contiguous()
+        wd, sd = w8.to(dev), s.to(dev)
+        run = lambda out: v.esimd_gemm_fp8_blockscale(xd, wd, sd, out)
+        ref = O.matmul_ref(x, O.fp8_dequant_block(w8, s))
+    else:
+        x, w8, s = O.make_fp8_pern_case(M, K, N, seed=M + K, act_dtype=dt)
+        if fmt == "pert":
+            s = torch.tensor([3.0e-4])
+            ref = O.matmul_ref(x, O.fp8_dequant_per_tensor(w8, s))
+        else:
+            ref = O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))
+        wd, sd = w8.to(dev), s.to(dev)
+        run = (lambda out: v.esimd_gemm_fp8_pert(xd, wd, sd, out)) if fmt == "pert" else \
+              (lambda out: v.esimd_gemv_fp8_pern(xd, wd, sd, out, N, K))
+    xd = x.to(dev)
+    outs = [torch.full((M, N), float("nan"), dtype=dt, device=dev) for _ in range(3)]
+    for out in outs:
+        run(out)
+    assert O.max_rel_err(outs[0].cpu(), ref) < TOL
+    assert _same_bits(outs[0], outs[1]) and _same_bits(outs[0], outs[2])
+
+
+def test_mid_m_k_split_fused(ops, dev):
+    # fused launches share the row blocks' counters: two INT4 matrices, three per-tensor FP8 ones
+    v, _ = ops
+    M, K = 64, 2048
+    x, p1, s1, _ = O.make_int4_case(M, K, 2048, seed=5, act_dtype=torch.float16)
+    _, p2, s2, _ = O.make_int4_case(M, K, 1000, seed=6, act_dtype=torch.float16)
+    o1 = torch.empty(M, 2048, dtype=torch.float16, device=dev)
+    o2 = torch.empty(M, 1000, dtype=torch.float16, device=dev)
+    v.esimd_gemv_int4_fused2(x.to(dev), p1.to(dev), s1.to(dev), o1, p2.to(dev), s2.to(dev), o2)
+    assert O.max_rel_err(o1.cpu(), O.matmul_ref(x, O.int4_dequant(p1, s1, out_dtype=torch.float16))) < TOL
+    assert O.max_rel_err(o2.cpu(), O.matmul_ref(x, O.int4_dequant(p2, s2, out_dtype=torch.float16))) < TOL
+    xb, w1, _ = O.make_fp8_pern_case(48, 4096, 2048, seed=7, act_dtype=torch.bfloat16)
+    _, w2, _ = O.make_fp8_pern_case(48, 4096, 512, seed=8, act_dtype=torch.bfloat16)
+    _, w3, _ = O.make_fp8_pern_case(48, 4096, 520, seed=9, act_dtype=torch.bfloat16)
+    sc = [torch.tensor([2.0e-4]), torch.tensor([5.0e-4]), torch.tensor([1.0e-3])]
+    outs = [torch.empty(48, n, dtype=torch.bfloat16, device=dev) for n in (2048, 512, 520)]
+    v.esimd_gemv_fp8_pert_fused3(xb.to(dev), w1.to(dev), sc[0].to(dev), outs[0], w2.to(dev), sc[1].to(dev), outs[1],
+                                 w3.to(dev), sc[2].to(dev), outs[2])
+    for o, w, s_ in zip(outs, (w1, w2, w3), sc):
+        assert O.max_rel_err(o.cpu(), O.matmul_ref(xb, O.fp8_dequant_per_tensor(w, s_))) < TOL
+
+
 # ----------------------------------------------------------------- error behaviour
 def test_argument_errors_raise(ops, dev):
     v, _ = ops
