@@ -441,12 +441,11 @@ def test_q4k_shapes(ops, dev, M, K, N):
     ("int4", 64, 4096, 4096, torch.bfloat16), ("int4", 40, 1664, 5000, torch.float16), ("int4", 64, 1024, 10240, torch.float16),
     ("pern", 64, 4096, 5120, torch.bfloat16), ("pern", 48, 1664, 1500, torch.float16), ("pert", 35, 2048, 8192, torch.bfloat16),
     ("block", 64, 5120, 5120, torch.float16), ("block", 34, 1536, 2304, torch.bfloat16), ("block", 64, 640, 4100, torch.bfloat16)])
-def test_mid_m_k_split(ops, dev, fmt, M, K, N, dt):
-    # 33 .. 64 rows against at most 40 weight rows per CU: workgroups split K, exchange fp32 partial
-    # tiles and the last one to arrive adds them in slice order.  Granule counts that do not divide
-    # by the split (13, 26, 5), a last 16-row tile that is partly empty, every scale form; each
-    # case runs three times into fresh outputs, which must agree bit for bit (the arrival
-    # counters are back at zero, the sum does not depend on who arrives last).
+def test_mid_m_few_weight_rows_per_cu(ops, dev, fmt, M, K, N, dt):
+    # 33 .. 64 rows of x against weights with few rows per CU (N up to 10240): every workgroup stages
+    # all of x through LDS for 16 .. 48 weight rows.  Granule counts that the wavefronts do not split
+    # evenly (13, 26, 5), a last 16-row tile that is partly empty, every scale form; each case runs
+    # three times into fresh outputs, which must agree bit for bit.
     v, sg = ops
     if fmt == "q4k":
         x, raw = O.make_q4k_case(M, K, N, seed=M + N)
@@ -483,8 +482,8 @@ def test_mid_m_k_split(ops, dev, fmt, M, K, N, dt):
     assert _same_bits(outs[0], outs[1]) and _same_bits(outs[0], outs[2])
 
 
-def test_mid_m_k_split_fused(ops, dev):
-    # fused launches share the row blocks' counters: two INT4 matrices, three per-tensor FP8 ones
+def test_mid_m_fused(ops, dev):
+    # fused launches at 48 and 64 rows: two INT4 matrices, three per-tensor FP8 ones
     v, _ = ops
     M, K = 64, 2048
     x, p1, s1, _ = O.make_int4_case(M, K, 2048, seed=5, act_dtype=torch.float16)
