@@ -44,6 +44,9 @@ struct SkinnyArgs {
   int M, K;
   int rpw;                    // weight rows owned by one workgroup (<= 16 RT)
   int scale_f16;              // fp8 per-channel: scale is fp16 instead of fp32
+  // msplit > 1: the rows of x are split over msplit workgroups per weight row block (16 MT rows
+  // each); tiles_total = row blocks of all matrices.
+  int msplit, tiles_total;
 };
 
 enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
@@ -87,13 +90,22 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
 
   int tile = blockIdx.x;
+  int m0 = 0;                                         // first row of x of this workgroup
+  if (a.msplit > 1) {
+    // The workgroups of a row block sit 8 apart: workgroups are dealt to the 8 XCDs in turn, so
+    // the block's weights come from HBM once and from that XCD's L2 afterwards.
+    const int grp = blockIdx.x / (8 * a.msplit), rem = blockIdx.x - grp * 8 * a.msplit;
+    m0 = (rem >> 3) * (MT * 16);
+    tile = grp * 8 + (rem & 7);
+    if (tile >= a.tiles_total || m0 >= a.M) return;
+  }
   int mat = 0;
 #pragma unroll
   for (int i = 0; i + 1 < kMaxMat; ++i) {
     if (mat == i && i + 1 < a.nmat && tile >= a.tiles[i]) { tile -= a.tiles[i]; mat = i + 1; }
   }
   const int N = a.N[mat];
-  const int K = a.K, M = a.M;
+  const int K = a.K, M = min(a.M - m0, MT * 16);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = lane & 15, g = lane >> 4;
@@ -105,7 +117,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   const uint32_t hrow = kIsQ5K ? ((uint32_t)K >> 3) : ((uint32_t)K >> 2);   // high-bit bytes per row
   const __amdgpu_buffer_rsrc_t hr = make_rsrc(a.h[mat], kHigh ? (uint32_t)N * hrow : 0u);
   const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
-  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc((const char*)a.x + (size_t)m0 * K * 2, (uint32_t)M * (uint32_t)K * 2u);
 
   const _Float16* s16 = (const _Float16*)a.s[mat];
   const float* s32 = (const float*)a.s[mat];
@@ -432,7 +444,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     for (int mt = 0; mt < MT; ++mt) red[wave][t][mt][lane] = acc[t][mt];
   __syncthreads();
   // D layout: lane holds output column n0 + 16 t + j, rows mt*16 + 4 g + v.
-  Elem* out = (Elem*)a.out[mat];
+  Elem* out = (Elem*)a.out[mat] + (size_t)m0 * N;
   for (int o = wave; o < RT * MT; o += NW) {
     const int t = o / MT, mt = o - t * MT;
     const int n = n0 + t * 16 + j;
@@ -470,6 +482,8 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
     tiles += a.tiles[i];
   }
   if (tiles == 0) return;
+  a.tiles_total = tiles;
+  const int wgs = a.msplit > 1 ? ((tiles + 7) / 8) * 8 * a.msplit : tiles;
   constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * MT * 16 * (256 + 16) : 0);
   constexpr int kRed = NW * RT * MT * 1024;
   static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
@@ -483,7 +497,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
       raised = lds;
     }
   }
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(NW * 64), lds, st, a);
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(NW * 64), lds, st, a);
 }
 
 // The SL instantiation when the format has per-32 scales, K allows whole 16-byte chunks per row
@@ -522,6 +536,22 @@ static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
     // block scales: tiles must not straddle a 128-row scale block
     rpw = (FMT == 0 && SC == SC_BLOCK) ? ((rpw + 15) & ~15) : ((rpw + 7) & ~7);
     if (rpw > 64) rpw = 64;
+    // 33 .. 64 rows against at most 32 weight rows per CU: every workgroup would stage all of x
+    // through its LDS for one or two weight tiles.  Two workgroups per (twice as tall) row block
+    // take 32 rows of x each instead: half the x traffic and LDS work per weight row; the second
+    // reads the block's weights from L2.  FP8 and INT4 only (K = 4096, M = 64: FP8 N = 5120 17.3 ->
+    // 12.4 us, INT4 N = 4096 13.5 -> 11.9 us); the formats with per-32 scale tables lose, since both
+    // workgroups stage the block's tables (Q4_K K = N = 5120: 17.8 -> 19.7 us).
+    if ((FMT == 0 || FMT == 1) && a.M > 32 && rounds == 1 && rpw <= 32 && ntot >= 16L * cus) {
+      SkinnyArgs h = a;
+      h.msplit = 2;
+      int r2 = (int)((2 * ntot + cus - 1) / cus);
+      r2 = (FMT == 0 && SC == SC_BLOCK) ? ((r2 + 15) & ~15) : ((r2 + 7) & ~7);
+      if (r2 <= 32) launch_pick<Act, FMT, SC, 2, 2, 8, 2>(h, r2, st);
+      else if (r2 <= 48) launch_pick<Act, FMT, SC, 2, 3, 8, 2>(h, r2, st);
+      else launch_pick<Act, FMT, SC, 2, 4, 8, 1>(h, r2 > 64 ? 64 : r2, st);
+      return launch_status();
+    }
     if (rpw <= 16) {
       if (a.M <= 16) launch_pick<Act, FMT, SC, 1, 1, 8, 4>(a, rpw, st);
       else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 1, 8, 2>(a, rpw, st);
