@@ -1,13 +1,13 @@
-// Small-M FP8 weight-only GEMM with the activations resident in registers.
+// Small-M weight-only GEMM (FP8 E4M3 or INT4 group 128) with the activations resident in registers.
 //
-// Regime: 5 <= M <= 32 rows against an [N, K] FP8 weight, M * K small enough that a
+// Regime: 5 <= M <= 32 rows against an [N, K] quantized weight, M * K small enough that a
 // workgroup can hold all of x in its register file (x is the matrix-core operand that never
 // changes while the weight streams past).  One workgroup owns up to 64 weight rows; its 8
 // wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
 //   - a wavefront loads its slice of x ONCE, before any weight load is issued (x comes from L2;
 //     the vector-memory counter retires in order, so these loads never queue behind the weight
 //     stream),
-//   - the loop is weight loads -> wave-private LDS transpose -> E4M3 decode -> MFMA, with the
+//   - the loop is weight loads -> wave-private LDS transpose -> decode -> MFMA, with the
 //     next 16-row tile in flight while the current one is consumed: no barrier, no x traffic,
 //   - the 8 partial tiles meet once, at the end, in LDS.
 // Weight loads are row-contiguous (one instruction reads 1 KiB of consecutive slice bytes, row
@@ -15,9 +15,12 @@
 // about 3 us slower on a 56 MB weight); the wavefront's own LDS tile (pitch + 16 bytes) turns
 // them into operand layout.
 //
-// k assignment inside a slice: read q (0 .. NQ-1) of lane (j = lane % 16, g = lane / 16) holds
-// bytes [64 q + 16 g, +16) of weight row n0 + 16 t + j; MFMA 2 q + h consumes bytes 8 h .. 8 h + 7
-// of it against x[j][slice + 64 q + 16 g + 8 h .. + 7].
+// k assignment inside a slice: step q (0 .. NQ-1) of lane (j = lane % 16, g = lane / 16) covers
+// k = 64 q + 16 g .. + 15 of weight row n0 + 16 t + j (16 bytes of FP8, 8 bytes of INT4); MFMA
+// 2 q + h consumes its k = 8 h .. 8 h + 7 against x[j][slice + 64 q + 16 g + 8 h .. + 7].
+// INT4: the fp16 scales and zero-point bytes of the row's NQ / 2 groups inside the slice travel
+// with the tile (one or two small loads per lane), and the nibbles are decoded with the scale
+// folded in (the routines of the dequantization kernels), so the sums need no factor.
 #pragma once
 #include "skinny_kernel.hpp"
 
@@ -31,19 +34,27 @@ constexpr int kslice_lds_bytes() {
   return kKsliceWaves * 16 * (64 * NQ + 16) + kKsliceWaves * kKsliceMaxTiles * MT * 1024;
 }
 
-// MT = 16-row activation tiles (M <= 16 MT), NQ = 16-byte loads per lane, row tile and slice
-// (slice = 64 NQ k), BLOCK = 128x128 block scales (otherwise one scale per output channel or
-// per tensor, applied to the finished sum).
-template <class Act, bool BLOCK, int MT, int NQ>
-__global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const SkinnyArgs a, const int scale_mode) {
+// FMT = 0: FP8 E4M3, 1: INT4 group 128.  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
+// k steps per slice (slice = 64 NQ k; FP8: NQ 16-byte loads per lane and tile, INT4: NQ / 2),
+// BLOCK = 128x128 block scales (FP8; otherwise one scale per output channel or per tensor,
+// applied to the finished sum).
+template <class Act, int FMT, bool BLOCK, int MT, int NQ>
+__global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyArgs a, const int scale_mode) {
   using V8 = typename Act::v8;
   using Elem = typename Act::elem;
+  constexpr bool kInt4 = FMT == 1;
+  static_assert(!kInt4 || (NQ % 4 == 0 && !BLOCK), "INT4: whole pairs of groups per slice");
   constexpr int NW = kKsliceWaves;
   constexpr int kMaxTiles = kKsliceMaxTiles;
-  constexpr int kSliceB = 64 * NQ;                    // bytes of one weight row inside a slice
+  constexpr int kSliceB = 64 * NQ;                    // k of a slice = bytes of half a slice row of x
   constexpr int kPitch = kSliceB + 16;                // LDS row pitch: operand reads hit distinct banks
   constexpr int kStage = 16 * kPitch;                 // one wavefront's staging tile
-  constexpr int kCPR = kSliceB / 16;                  // 16-byte chunks per row of the slice
+  constexpr int kCPR = kSliceB / 16;                  // 16-byte chunks per row of the tile (x halves, FP8 weights)
+  constexpr int kWRowB = kInt4 ? kSliceB / 2 : kSliceB;   // bytes of one weight row inside a slice
+  constexpr int kWPitch = kWRowB + 16;
+  constexpr int kWCPR = kWRowB / 16;
+  constexpr int NL = kInt4 ? NQ / 2 : NQ;             // 16-byte weight loads per lane and tile
+  constexpr int NS = kInt4 ? NQ / 4 : 1;              // INT4: 32-bit words of scales (two groups each)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // the partial tiles live beside the staging tiles
   f32x4 (*red)[kMaxTiles][MT][64] = reinterpret_cast<f32x4 (*)[kMaxTiles][MT][64]>(smem + NW * kStage);
@@ -64,7 +75,13 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
   const int ntiles = (nend - n0 + 15) >> 4;           // <= kMaxTiles
   const int kbase = wave * kSliceB;                   // first k of this wavefront's slice
 
-  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * (uint32_t)K);
+  const uint32_t wrow = kInt4 ? (uint32_t)K >> 1 : (uint32_t)K;   // weight bytes per row
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
+  // INT4 side data: fp16 scales and (optional) zero-point bytes per 128-wide group
+  const int Kg = K >> 7;
+  const bool has_zp = kInt4 && a.z[mat] != nullptr;
+  const __amdgpu_buffer_rsrc_t sr = make_rsrc(a.s[mat], kInt4 ? (uint32_t)N * (uint32_t)Kg * 2u : 0u);
+  const __amdgpu_buffer_rsrc_t zr = make_rsrc(has_zp ? a.z[mat] : a.s[mat], has_zp ? (uint32_t)N * (uint32_t)Kg : 0u);
   const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
 
   // The 64 NQ 16-byte chunks of a 16-row tile (16 rows x kCPR chunks) are walked row-major: load i
@@ -119,31 +136,78 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
   };
 
   // ---- weights: two 16-row tiles in flight in registers ----
-  auto load_tile = [&](u32x4 (&w)[NQ], int t) {
+  // A tile in registers: NL 16-byte loads per lane (row-contiguous until the transposition, then
+  // step q's bytes: FP8 w[q], INT4 dwords 2 (q % 2) and 2 (q % 2) + 1 of w[q / 2]); INT4 also the
+  // lane's row's scales (two fp16 per word) and zero-points (two bytes per word) of the slice.
+  struct Tile {
+    u32x4 w[NL];
+    uint32_t s[NS], z[NS];
+  };
+  auto wchunk_of = [&](int i, int& r, int& c) {
+    const int f = i * 64 + lane;
+    r = f / kWCPR;
+    c = f - r * kWCPR;
+  };
+  auto load_tile = [&](Tile& tl, int t) {
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
+    for (int i = 0; i < NL; ++i) {
       int r, c;
-      chunk_of(i, r, c);
+      wchunk_of(i, r, c);
       const int n = n0 + t * 16 + r;
-      const int k = kbase + 16 * c;
+      const int k = kbase + (kInt4 ? 32 : 16) * c;    // first k of the chunk
       const bool ok = t < ntiles && n < nend && k < K;
-      w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, ok ? (uint32_t)n * (uint32_t)K + (uint32_t)k : kOOB, 0, 2 /* nt */);
+      tl.w[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          wr, ok ? (uint32_t)n * wrow + (uint32_t)(kInt4 ? k >> 1 : k) : kOOB, 0, 2 /* nt */);
+    }
+    if constexpr (kInt4) {
+      const int n = n0 + t * 16 + j;
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        const int grp = (kbase >> 7) + 2 * i;         // K % 256 == 0: a pair of groups never straddles the row end
+        const bool ok = t < ntiles && n < nend && grp < Kg;
+        const uint32_t e = (uint32_t)n * (uint32_t)Kg + (uint32_t)grp;
+        tl.s[i] = __builtin_amdgcn_raw_buffer_load_b32(sr, ok ? e * 2u : kOOB, 0, 0);
+        tl.z[i] = has_zp ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(zr, ok ? e : kOOB, 0, 0) : 0x0808u;
+      }
     }
   };
   // registers (row-contiguous) -> this wavefront's LDS tile -> registers (operand layout)
-  auto transpose_tile = [&](u32x4 (&w)[NQ]) {
+  auto transpose_tile = [&](Tile& tl) {
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
+    for (int i = 0; i < NL; ++i) {
       int r, c;
-      chunk_of(i, r, c);
-      *reinterpret_cast<u32x4*>(stage + r * kPitch + c * 16) = w[i];
+      wchunk_of(i, r, c);
+      *reinterpret_cast<u32x4*>(stage + r * kWPitch + c * 16) = tl.w[i];
     }
+    if constexpr (kInt4) {
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) w[q] = *reinterpret_cast<const u32x4*>(stage + j * kPitch + 64 * q + 16 * g);
+      for (int q = 0; q < NQ; ++q) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(stage + j * kWPitch + 32 * q + 8 * g);
+        tl.w[q >> 1][(q & 1) * 2] = v[0];
+        tl.w[q >> 1][(q & 1) * 2 + 1] = v[1];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) tl.w[q] = *reinterpret_cast<const u32x4*>(stage + j * kWPitch + 64 * q + 16 * g);
+    }
+  };
+  // the 8 k of MFMA 2 q + h as the activation type
+  auto operand = [&](const Tile& tl, int q, int h) -> V8 {
+    if constexpr (kInt4) {
+      const uint32_t dw = tl.w[q >> 1][(q & 1) * 2 + h];
+      const int gq = q >> 1;                          // group inside the slice
+      const uint32_t sbits = (tl.s[gq >> 1] >> (16 * (gq & 1))) & 0xFFFFu;
+      const float zf = (float)((tl.z[gq >> 1] >> (8 * (gq & 1))) & 0xFFu);
+      const float sf = (float)__builtin_bit_cast(_Float16, (uint16_t)sbits);
+      if constexpr (Act::dt == DT_F16) return int4x8_to_f16(dw, (_Float16)sf, (_Float16)(1024.0f + zf));
+      else return int4x8_to_bf16(dw, sf, zf);
+    } else {
+      return fp8x8_to_act<Act>(tl.w[q][2 * h], tl.w[q][2 * h + 1]);
+    }
   };
   const float* s32 = (const float*)a.s[mat];
   const int Kb = (K + 127) >> 7;
-  auto compute_tile = [&](u32x4 (&w)[NQ], int t) {
+  auto compute_tile = [&](Tile& w, int t) {
     transpose_tile(w);
     f32x4 acc[MT];
 #pragma unroll
@@ -163,7 +227,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
           const int q = q2 * 2 + qq;
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
-            const V8 b = fp8x8_to_act<Act>(w[q][2 * h], w[q][2 * h + 1]);
+            const V8 b = operand(w, q, h);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) part[mt] = Act::mfma(as_v8<V8>(xq[mt][q][h]), b, part[mt]);
           }
@@ -176,7 +240,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
       for (int q = 0; q < NQ; ++q)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const V8 b = fp8x8_to_act<Act>(w[q][2 * h], w[q][2 * h + 1]);
+          const V8 b = operand(w, q, h);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) acc[mt] = Act::mfma(as_v8<V8>(xq[mt][q][h]), b, acc[mt]);
         }
@@ -185,7 +249,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
     for (int mt = 0; mt < MT; ++mt) red[wave][t][mt][lane] = acc[mt];
   };
 
-  u32x4 w0[NQ], w1[NQ];
+  Tile w0, w1;
   load_tile(w0, 0);
   load_tile(w1, 1);
   __builtin_amdgcn_sched_barrier(0);
@@ -213,7 +277,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
     const int n = n0 + t * 16 + j;
     if (n < nend) {
       float os = 1.0f;
-      if constexpr (!BLOCK) {
+      if constexpr (!BLOCK && !kInt4) {
         if (scale_mode == SC_PERT) os = s32[0];
         else os = a.scale_f16 ? (float)((const _Float16*)a.s[mat])[n] : s32[n];
       }
@@ -227,27 +291,29 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_fp8_kernel(const Ski
   }
 }
 
-// Whether the register-resident path covers a problem: FP8, 5 .. 32 rows, the slice of x within
-// 128 registers per lane, 16-byte aligned rows.
-static inline int kslice_loads(int M, int K) {
-  if (M < 5 || M > 32 || (K % 16)) return 0;
+// Whether the register-resident path covers a problem (0: no; else the steps per slice): 5 .. 32
+// rows, the slice of x within 128 registers per lane; FP8: 16-byte aligned rows; INT4 (int4 =
+// true): K a multiple of 512, so that a slice holds whole pairs of groups and the side loads
+// are aligned.
+static inline int kslice_loads(int M, int K, bool int4 = false) {
+  if (M < 5 || M > 32 || (K % 16) || (int4 && (K % 512))) return 0;
   const int mt = M <= 16 ? 1 : 2;
-  int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // loads per lane to cover K with 8 slices
-  nq = (nq + 1) & ~1;                                            // even: whole 128-wide scale blocks
-  const int choices[] = {2, 4, 6, 8, 10, 12};          // 16 loads spill
+  int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // steps to cover K with 8 slices
+  nq = int4 ? ((nq + 3) & ~3) : ((nq + 1) & ~1);                // FP8: whole 128-wide scale blocks
+  const int choices[] = {2, 4, 6, 8, 10, 12};          // 16 steps spill
   for (int c : choices)
     if (c >= nq) return (mt * c <= 16) ? c : 0;                 // x registers: mt * c * 8 <= 128
   return 0;
 }
 
-template <class Act, bool BLOCK, int MT>
+template <class Act, int FMT, bool BLOCK, int MT>
 static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_mode, hipStream_t st) {
   const dim3 grid(tiles), block(kKsliceWaves * 64);
 #define QLIN_KSLICE(NQ_)                                                                                       \
   case NQ_:                                                                                                    \
-    if constexpr (MT * NQ_ <= 16)                                                                              \
+    if constexpr (MT * NQ_ <= 16 && (FMT == 0 || NQ_ % 4 == 0))                                                \
     {                                                                                                          \
-      auto kern = kslice_fp8_kernel<Act, BLOCK, MT, NQ_>;                                                      \
+      auto kern = kslice_kernel<Act, FMT, BLOCK, MT, NQ_>;                                                     \
       constexpr int lds = kslice_lds_bytes<MT, NQ_>();                                                         \
       static_assert(lds <= 160 * 1024, "staging tiles exceed the LDS");                                        \
       static bool raised = false;                                                                              \
@@ -265,9 +331,9 @@ static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_m
 #undef QLIN_KSLICE
 }
 
-// scale_mode: SC_PERN / SC_PERT / SC_BLOCK.  Rows per workgroup as in the skinny kernel: one
+// scale_mode (FP8): SC_PERN / SC_PERT / SC_BLOCK.  Rows per workgroup as in the skinny kernel: one
 // workgroup per CU and round, a multiple of 16 rows, at most 64.
-template <class Act>
+template <class Act, int FMT = 0>
 static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
   long ntot = 0;
   for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
@@ -285,13 +351,18 @@ static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
     tiles += a.tiles[i];
   }
   if (!tiles) return MI_OK;
-  const bool block = scale_mode == SC_BLOCK;
-  if (a.M <= 16) {
-    if (block) kslice_launch_nq<Act, true, 1>(a, nq, tiles, scale_mode, st);
-    else kslice_launch_nq<Act, false, 1>(a, nq, tiles, scale_mode, st);
+  if constexpr (FMT == 1) {
+    if (a.M <= 16) kslice_launch_nq<Act, 1, false, 1>(a, nq, tiles, scale_mode, st);
+    else kslice_launch_nq<Act, 1, false, 2>(a, nq, tiles, scale_mode, st);
   } else {
-    if (block) kslice_launch_nq<Act, true, 2>(a, nq, tiles, scale_mode, st);
-    else kslice_launch_nq<Act, false, 2>(a, nq, tiles, scale_mode, st);
+    const bool block = scale_mode == SC_BLOCK;
+    if (a.M <= 16) {
+      if (block) kslice_launch_nq<Act, 0, true, 1>(a, nq, tiles, scale_mode, st);
+      else kslice_launch_nq<Act, 0, false, 1>(a, nq, tiles, scale_mode, st);
+    } else {
+      if (block) kslice_launch_nq<Act, 0, true, 2>(a, nq, tiles, scale_mode, st);
+      else kslice_launch_nq<Act, 0, false, 2>(a, nq, tiles, scale_mode, st);
+    }
   }
   return launch_status();
 }

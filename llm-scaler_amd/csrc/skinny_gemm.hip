@@ -60,6 +60,13 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     if (const int nq = pays ? kslice_loads(a.M, a.K) : 0)
       return act_dtype == DT_F16 ? kslice_launch<ActF16>(a, SC, nq, st) : kslice_launch<ActBF16>(a, SC, nq, st);
   }
+  if constexpr (FMT == 1) {
+    // INT4: the same kernel, nibbles decoded with their group's scale; ahead of the granule-interleaved
+    // kernel at every N measured (K = 4096, fp16: N = 14336 M=8 13.2 -> 11.6 us, M=32 16.8 -> 14.6 us;
+    // N = 4096 7.2 -> 6.5 and 9.7 -> 8.7 us; N = 2048 M=16 8.2 -> 6.3 us)
+    if (const int nq = kslice_loads(a.M, a.K, true))
+      return act_dtype == DT_F16 ? kslice_launch<ActF16, 1>(a, 0, nq, st) : kslice_launch<ActBF16, 1>(a, 0, nq, st);
+  }
   // prefill: the tiled matrix-core GEMM reads the weight once per 256 rows instead of once per 64
   if constexpr (FMT == 0 || FMT == 2) {
     if (a.M > 64 && a.K % 128 == 0) {

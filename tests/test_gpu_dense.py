@@ -547,6 +547,39 @@ def test_gemm_int4_shapes(ops, dev, M, K, N, dt, asym):
     assert _run_gemm_int4(v, dev, M, K, N, dt, asym, seed=M + N) < TOL
 
 
+@pytest.mark.parametrize("M,K,N,dt,asym", [
+    (5, 4096, 8200, torch.bfloat16, False), (8, 4096, 14336, torch.float16, True), (16, 2048, 333, torch.float16, False),
+    (17, 4096, 9000, torch.float16, True), (32, 4096, 4096, torch.bfloat16, True), (9, 5120, 5120, torch.float16, False),
+    (12, 6144, 2000, torch.bfloat16, True), (24, 1536, 4160, torch.bfloat16, False), (31, 3584, 1024, torch.float16, True),
+    (32, 512, 40, torch.float16, False), (7, 1024, 16, torch.bfloat16, True)])
+def test_int4_register_resident_activations(ops, dev, M, K, N, dt, asym):
+    # 5 .. 32 rows, K a multiple of 512: x held in registers, K split over the wavefronts in slices,
+    # the nibbles decoded with their group's scale and zero-point.  Slices that end inside K (1536,
+    # 3584, 5120), row counts off the 16-row tiles, with and without zero-points.
+    v, _ = ops
+    assert _run_gemm_int4(v, dev, M, K, N, dt, asym, seed=M + K) < TOL
+
+
+def test_int4_register_resident_zero_points_exact(ops, dev):
+    # x = one-hot rows, scales = powers of two: every output is one weight, exactly (nib - zp) * scale,
+    # for every nibble, every zero-point and both halves of a byte
+    v, _ = ops
+    M, K, N = 16, 512, 256
+    g = torch.Generator().manual_seed(3)
+    packed = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g)
+    zp = torch.randint(0, 16, (N, K // 128), dtype=torch.uint8, generator=g)
+    scale = (2.0 ** torch.randint(-6, 3, (N, K // 128), generator=g).float()).to(torch.float16)
+    ks = torch.randint(0, K, (M,), generator=g)
+    x = torch.zeros(M, K, dtype=torch.float16)
+    x[torch.arange(M), ks] = 1.0
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    v.esimd_gemm_int4_pgrp_zp(x.to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out)
+    byte = packed[:, ks // 2].long()                      # [N, M]
+    nib = torch.where((ks % 2 == 0)[None, :], byte & 15, byte >> 4).float()
+    want = ((nib - zp[:, ks // 128].float()) * scale[:, ks // 128].float()).t().to(torch.float16)
+    assert _same_bits(out, want)
+
+
 def test_gemm_int4_c_abi_without_workspace(ops, dev):
     """mi_gemm_int4 (no workspace argument) takes its scratch from the stream-ordered allocator
     and must agree bit for bit with the workspace entry point the torch op uses."""
