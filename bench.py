@@ -76,7 +76,7 @@ def wl_fp8_pern(M: int, dev):
     alg_bytes = N * K + 4 * N + 2 * M * K + 2 * M * N
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="bf16",
                 name=f"cfg1 FP8 e4m3 per-channel weight-only GEMV M={M} K={K} N={N} bf16",
-                kernel="gemv_rows_kernel" if M <= 4 else "skinny_kernel", cpu=cpu)
+                kernel="gemv_rows_kernel" if M <= 4 else "kslice_kernel", cpu=cpu)
 
 
 def wl_int4_gemv(dev):
@@ -286,7 +286,7 @@ def wl_gemm_w4a16(dev):
     alg_bytes = N * K // 2 + N * (K // 128) * 3 + 2 * M * K + 2 * M * N
     return dict(launch=launch, R=1, bytes=alg_bytes, flops=2 * M * N * K, bound="mfma", dtype="bf16",
                 name=f"cfg2 W4A16 asymmetric group-128 prefill GEMM M={M} K={K} N={N} bf16",
-                kernel="gemm_w4a16_kernel", cpu=cpu)
+                kernel="gemm_tiled_kernel", cpu=cpu)
 
 
 def wl_fp8_prefill(dev, mode="pern"):
