@@ -79,10 +79,10 @@ def wl_fp8_pern(M: int, dev):
                 kernel="gemv_rows_kernel" if M <= 4 else "kslice_kernel", cpu=cpu)
 
 
-def wl_int4_gemv(dev):
+def wl_int4_gemv(dev, M=1, N=4096):
     import custom_esimd_kernels_vllm as v
     from oracle import qlinear_oracle as O
-    M, K, N = 1, 4096, 4096
+    K = 4096
     x, packed, scale, _ = O.make_int4_case(M, K, N)
     R = _copies(N * K // 2)
     g = torch.Generator().manual_seed(98)
@@ -100,9 +100,11 @@ def wl_int4_gemv(dev):
     def cpu():
         return O.matmul_ref(x, O.int4_dequant(packed, scale)).to(torch.float16)
 
-    alg_bytes = N * K // 2 + N * (K // 128) * 2 + K * 2 + N * 2
+    alg_bytes = N * K // 2 + N * (K // 128) * 2 + M * K * 2 + M * N * 2
+    cfg0 = M == 1 and N == 4096
     return dict(launch=launch, R=R, bytes=alg_bytes, flops=2 * M * N * K, bound="hbm", dtype="f16",
-                name=f"cfg0 W4A16 group-128 GEMV M={M} K={K} N={N} fp16", kernel="gemv_rows_kernel", cpu=cpu)
+                name=("cfg0" if cfg0 else "next:") + f" W4A16 group-128 GEMV M={M} K={K} N={N} fp16",
+                kernel="gemv_rows_kernel" if M <= 2 else "kslice_kernel", cpu=cpu)
 
 
 def wl_q4k(M: int, dev):
@@ -594,6 +596,8 @@ WORKLOADS = {
     "next_int4_fused2": wl_int4_fused2,
     "next_fp8_pert_fused2": lambda dev: wl_fp8_pert_fused(dev, False),
     "next_fp8_pert_fused3": lambda dev: wl_fp8_pert_fused(dev, True),
+    "next_int4_m8": lambda dev: wl_int4_gemv(dev, 8, 14336),
+    "next_int4_m32": lambda dev: wl_int4_gemv(dev, 32, 14336),
     "next_q4k_m8": lambda dev: wl_q4k(8, dev),
     "next_q4k_m32": lambda dev: wl_q4k(32, dev),
     "next_q4_0_m1": lambda dev: wl_gguf("q4_0", 1, dev),
