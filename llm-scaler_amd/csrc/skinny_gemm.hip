@@ -1,107 +1,8 @@
 // Entry points of the weight-streaming GEMV / small-M GEMM for FP8 (per-channel, per-tensor,
-// 128x128 block), INT4 group 128 and GGUF Q4_K: M <= 4 takes the one-wavefront-per-row
-// kernel (gemv_rows.hpp), larger M the MFMA kernel (skinny_kernel.hpp).
-#include "skinny_kernel.hpp"
-#include "kslice_kernel.hpp"
-#include "scratch.hpp"
-#include "../../include/mi355x_qlinear.h"
-
-namespace qlin {
-
-// Runs M in chunks of 64 rows (the skinny kernel's limit); each chunk streams
-// the weight once, so this is meant for decode-sized M.
-template <int FMT, int SC>
-static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
-  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (FMT == 2 && act_dtype != DT_F16) return MI_ERR_ARG;
-  if (a.M < 0 || a.K <= 0) return MI_ERR_SHAPE;
-  if (FMT == 0 && (a.K % 32)) return MI_ERR_SHAPE;
-  if (FMT == 1 && (a.K % 128)) return MI_ERR_SHAPE;
-  if (FMT == 2 && (a.K % 32)) return MI_ERR_SHAPE;
-  for (int i = 0; i < a.nmat; ++i) {
-    if (a.N[i] < 0 || !a.w[i] || !a.out[i]) return MI_ERR_ARG;
-    if (FMT == 1 && (a.z[i] != nullptr) != (a.z[0] != nullptr)) return MI_ERR_ARG;   // zero-points for all or none
-    if ((uint64_t)a.N[i] * (uint64_t)a.K >= (1ull << 31)) return MI_ERR_SHAPE;
-    a.tiles[i] = (a.N[i] + 15) / 16;
-  }
-  if (!a.x) return MI_ERR_ARG;
-  if (a.M == 0) return MI_OK;
-  // decode regime: one wavefront per weight row, activations staged in LDS
-  // INT4 with 3 or 4 rows: the MFMA kernel is as fast (bf16) or faster (fp16: 13.3 against 15.8 us at
-  // N=14336, K=4096) than the row kernel's LDS-staged activations
-  constexpr int rows_max_m = FMT == 1 ? 2 : 4;
-  if (a.M <= rows_max_m && rows_lds_bytes(FMT, a.M == 3 ? 4 : a.M, a.K) <= 64 * 1024 && (FMT != 0 || a.K % 16 == 0)) {
-    RowsArgs r{};
-    r.x = a.x; r.nmat = a.nmat; r.M = a.M; r.K = a.K; r.scale_f16 = a.scale_f16;
-    for (int i = 0; i < a.nmat; ++i) {
-      r.w[i] = a.w[i]; r.s[i] = a.s[i]; r.z[i] = a.z[i]; r.out[i] = a.out[i]; r.N[i] = a.N[i];
-    }
-    if constexpr (FMT == 1) {                          // int4: the zero-point load is a template choice
-      if (a.z[0]) {
-        if (act_dtype == DT_F16) launch_rows_m<ActF16, RF_INT4, RS_ZP>(r, st);
-        else launch_rows_m<ActBF16, RF_INT4, RS_ZP>(r, st);
-      } else {
-        if (act_dtype == DT_F16) launch_rows_m<ActF16, RF_INT4, RS_PERN>(r, st);
-        else launch_rows_m<ActBF16, RF_INT4, RS_PERN>(r, st);
-      }
-    } else if (FMT == 2 || act_dtype == DT_F16)
-      launch_rows_m<ActF16, FMT, SC>(r, st);
-    else
-      launch_rows_m<ActBF16, FMT, SC>(r, st);
-    return launch_status();
-  }
-  // few rows whose slice of x fits the register file: activations resident, weights streamed
-  if constexpr (FMT == 0) {
-    long ntot = 0;
-    for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
-    // measured against the granule-interleaved kernel (M = 5 .. 32): ahead by 5-35 % when a workgroup
-    // owns at least two 16-row tiles or rows are short, behind by 10-25 % for one tile of long rows
-    const bool pays = ntot > 16L * device_cu_count() || a.K <= 2048;
-    if (const int nq = pays ? kslice_loads(a.M, a.K) : 0)
-      return act_dtype == DT_F16 ? kslice_launch<ActF16>(a, SC, nq, st) : kslice_launch<ActBF16>(a, SC, nq, st);
-  }
-  if constexpr (FMT == 1) {
-    // INT4: the same kernel, nibbles decoded with their group's scale; ahead of the granule-interleaved
-    // kernel at every N measured (K = 4096, fp16: N = 14336 M=8 13.2 -> 11.6 us, M=32 16.8 -> 14.6 us;
-    // N = 4096 7.2 -> 6.5 and 9.7 -> 8.7 us; N = 2048 M=16 8.2 -> 6.3 us)
-    if (const int nq = kslice_loads(a.M, a.K, true))
-      return act_dtype == DT_F16 ? kslice_launch<ActF16, 1>(a, 0, nq, st) : kslice_launch<ActBF16, 1>(a, 0, nq, st);
-  }
-  // prefill: the tiled matrix-core GEMM reads the weight once per 256 rows instead of once per 64
-  if constexpr (FMT == 0 || FMT == 2) {
-    if (a.M > 64 && a.K % 128 == 0) {
-      long long bytes = 0;
-      if (mi_gemm_tiled_workspace(a.M, a.K, &bytes) != MI_OK) return MI_ERR_SHAPE;
-      void* ws = scratch_get(st, (size_t)bytes);
-      if (!ws) return MI_ERR_LAUNCH;
-      for (int i = 0; i < a.nmat; ++i) {
-        const int rc = FMT == 0 ? mi_gemm_fp8_tiled_ws(a.x, a.w[i], a.s[i], SC, a.scale_f16, a.out[i], ws, bytes, a.M,
-                                                       a.N[i], a.K, act_dtype, st)
-                                : mi_gemm_q4k_tiled_ws(a.x, a.w[i], a.s[i], a.z[i], a.out[i], ws, bytes, a.M, a.N[i],
-                                                       a.K, st);
-        if (rc != MI_OK) return rc;
-      }
-      return MI_OK;
-    }
-  }
-  const int M = a.M;
-  const size_t esz = 2;
-  for (int m0 = 0; m0 < M; m0 += 64) {
-    SkinnyArgs c = a;
-    c.M = (M - m0) < 64 ? (M - m0) : 64;
-    c.x = (const char*)a.x + (size_t)m0 * a.K * esz;
-    for (int i = 0; i < a.nmat; ++i) c.out[i] = (char*)a.out[i] + (size_t)m0 * a.N[i] * esz;
-    int rc;
-    if (FMT == 2)
-      rc = launch_mt<ActF16, FMT, SC>(c, st);
-    else
-      rc = act_dtype == DT_F16 ? launch_mt<ActF16, FMT, SC>(c, st) : launch_mt<ActBF16, FMT, SC>(c, st);
-    if (rc != MI_OK) return rc;
-  }
-  return MI_OK;
-}
-
-}  // namespace qlin
+// 128x128 block): M <= 4 takes the one-wavefront-per-row kernel (gemv_rows.hpp), larger M the
+// MFMA kernels (kslice_kernel.hpp, skinny_kernel.hpp), M > 64 the tiled GEMM.  The INT4 and
+// Q4_K entry points are in skinny_gemm_w4.hip.
+#include "skinny_run.hpp"
 
 using namespace qlin;
 
@@ -159,34 +60,6 @@ int mi_gemm_fp8_blockscale_multi(const void* x, int nmat, const void* const* w,
 int mi_gemm_fp8_blockscale(const void* x, const void* w, const float* scale, void* out, int M, int N,
                            int K, int act_dtype, void* stream) {
   return mi_gemm_fp8_blockscale_multi(x, 1, &w, &scale, &out, &N, M, K, act_dtype, stream);
-}
-
-int mi_gemv_int4_multi(const void* x, int nmat, const void* const* w, const void* const* scale,
-                       const void* const* zp, void* const* out, const int* N, int M, int K,
-                       int act_dtype, void* stream) {
-  if (nmat < 1 || nmat > kMaxMat || !w || !scale || !out || !N) return MI_ERR_ARG;
-  SkinnyArgs a{};
-  a.x = x; a.nmat = nmat; a.M = M; a.K = K;
-  for (int i = 0; i < nmat; ++i) {
-    if (!scale[i]) return MI_ERR_ARG;
-    a.w[i] = w[i]; a.s[i] = scale[i]; a.z[i] = zp ? zp[i] : nullptr; a.out[i] = out[i]; a.N[i] = N[i];
-  }
-  return run<1, 0>(a, act_dtype, (hipStream_t)stream);
-}
-
-int mi_gemv_int4(const void* x, const void* w, const void* scale, const void* zp, void* out, int M,
-                 int N, int K, int act_dtype, void* stream) {
-  const void* zps[1] = {zp};
-  return mi_gemv_int4_multi(x, 1, &w, &scale, zp ? zps : nullptr, &out, &N, M, K, act_dtype, stream);
-}
-
-int mi_gemv_q4k(const void* x, const void* ql, const void* scale, const void* qmin, void* out, int M,
-                int N, int K, void* stream) {
-  if (!scale || !qmin) return MI_ERR_ARG;
-  SkinnyArgs a{};
-  a.x = x; a.nmat = 1; a.M = M; a.K = K;
-  a.w[0] = ql; a.s[0] = scale; a.z[0] = qmin; a.out[0] = out; a.N[0] = N;
-  return run<2, 0>(a, DT_F16, (hipStream_t)stream);
 }
 
 }  // extern "C"
