@@ -34,7 +34,7 @@ constexpr int kslice_lds_bytes() {
   return kKsliceWaves * 16 * (64 * NQ + 16) + kKsliceWaves * kKsliceMaxTiles * MT * 1024;
 }
 
-// FMT = 0: FP8 E4M3, 1: INT4 group 128.  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
+// FMT = 0: FP8 E4M3, 1: INT4 group 128, 2: GGUF Q4_K (repacked; fp16 scale and min per 32 k).  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
 // k steps per slice (slice = 64 NQ k; FP8: NQ 16-byte loads per lane and tile, INT4: NQ / 2),
 // BLOCK = 128x128 block scales (FP8; otherwise one scale per output channel or per tensor,
 // applied to the finished sum).
@@ -43,18 +43,23 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   using V8 = typename Act::v8;
   using Elem = typename Act::elem;
   constexpr bool kInt4 = FMT == 1;
+  constexpr bool kQ4K = FMT == 2;
+  constexpr bool kNib = kInt4 || kQ4K;                // two weights per byte
   static_assert(!kInt4 || (NQ % 4 == 0 && !BLOCK), "INT4: whole pairs of groups per slice");
+  static_assert(!kQ4K || (NQ % 2 == 0 && !BLOCK && Act::dt == DT_F16), "Q4_K runs in fp16");
   constexpr int NW = kKsliceWaves;
   constexpr int kMaxTiles = kKsliceMaxTiles;
   constexpr int kSliceB = 64 * NQ;                    // k of a slice = bytes of half a slice row of x
   constexpr int kPitch = kSliceB + 16;                // LDS row pitch: operand reads hit distinct banks
   constexpr int kStage = 16 * kPitch;                 // one wavefront's staging tile
   constexpr int kCPR = kSliceB / 16;                  // 16-byte chunks per row of the tile (x halves, FP8 weights)
-  constexpr int kWRowB = kInt4 ? kSliceB / 2 : kSliceB;   // bytes of one weight row inside a slice
+  constexpr int kWRowB = kNib ? kSliceB / 2 : kSliceB;   // bytes of one weight row inside a slice
   constexpr int kWPitch = kWRowB + 16;
   constexpr int kWCPR = kWRowB / 16;
-  constexpr int NL = kInt4 ? NQ / 2 : NQ;             // 16-byte weight loads per lane and tile
-  constexpr int NS = kInt4 ? NQ / 4 : 1;              // INT4: 32-bit words of scales (two groups each)
+  constexpr int NL = kNib ? NQ / 2 : NQ;              // 16-byte weight loads per lane and tile
+  // side words per lane and tile: INT4 one per pair of groups (two fp16 scales / two zero-point
+  // bytes), Q4_K one per step (the fp16 scales / mins of its two 32-wide sub-blocks)
+  constexpr int NS = kInt4 ? NQ / 4 : (kQ4K ? NQ : 1);
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // the partial tiles live beside the staging tiles
   f32x4 (*red)[kMaxTiles][MT][64] = reinterpret_cast<f32x4 (*)[kMaxTiles][MT][64]>(smem + NW * kStage);
@@ -75,13 +80,17 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   const int ntiles = (nend - n0 + 15) >> 4;           // <= kMaxTiles
   const int kbase = wave * kSliceB;                   // first k of this wavefront's slice
 
-  const uint32_t wrow = kInt4 ? (uint32_t)K >> 1 : (uint32_t)K;   // weight bytes per row
+  const uint32_t wrow = kNib ? (uint32_t)K >> 1 : (uint32_t)K;   // weight bytes per row
   const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
   // INT4 side data: fp16 scales and (optional) zero-point bytes per 128-wide group
   const int Kg = K >> 7;
   const bool has_zp = kInt4 && a.z[mat] != nullptr;
-  const __amdgpu_buffer_rsrc_t sr = make_rsrc(a.s[mat], kInt4 ? (uint32_t)N * (uint32_t)Kg * 2u : 0u);
-  const __amdgpu_buffer_rsrc_t zr = make_rsrc(has_zp ? a.z[mat] : a.s[mat], has_zp ? (uint32_t)N * (uint32_t)Kg : 0u);
+  const int Kc = K >> 5;                              // Q4_K: fp16 scale and min per 32-wide sub-block
+  const __amdgpu_buffer_rsrc_t sr =
+      make_rsrc(a.s[mat], kInt4 ? (uint32_t)N * (uint32_t)Kg * 2u : (kQ4K ? (uint32_t)N * (uint32_t)Kc * 2u : 0u));
+  const __amdgpu_buffer_rsrc_t zr =
+      make_rsrc((has_zp || kQ4K) ? a.z[mat] : a.s[mat],
+                has_zp ? (uint32_t)N * (uint32_t)Kg : (kQ4K ? (uint32_t)N * (uint32_t)Kc * 2u : 0u));
   const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
 
   // The 64 NQ 16-byte chunks of a 16-row tile (16 rows x kCPR chunks) are walked row-major: load i
@@ -154,10 +163,10 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
       int r, c;
       wchunk_of(i, r, c);
       const int n = n0 + t * 16 + r;
-      const int k = kbase + (kInt4 ? 32 : 16) * c;    // first k of the chunk
+      const int k = kbase + (kNib ? 32 : 16) * c;     // first k of the chunk
       const bool ok = t < ntiles && n < nend && k < K;
       tl.w[i] = __builtin_amdgcn_raw_buffer_load_b128(
-          wr, ok ? (uint32_t)n * wrow + (uint32_t)(kInt4 ? k >> 1 : k) : kOOB, 0, 2 /* nt */);
+          wr, ok ? (uint32_t)n * wrow + (uint32_t)(kNib ? k >> 1 : k) : kOOB, 0, 2 /* nt */);
     }
     if constexpr (kInt4) {
       const int n = n0 + t * 16 + j;
@@ -170,6 +179,20 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
         tl.z[i] = has_zp ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(zr, ok ? e : kOOB, 0, 0) : 0x0808u;
       }
     }
+    if constexpr (kQ4K) {
+      // the row's 2 NQ sub-blocks inside the slice, four entries (one step pair) per 64-bit load
+      const int n = n0 + t * 16 + j;
+#pragma unroll
+      for (int i = 0; i < NQ / 2; ++i) {
+        const int sb = (kbase >> 5) + 4 * i;          // K % 256 == 0: four entries never straddle the row end
+        const bool ok = t < ntiles && n < nend && sb < Kc;
+        const uint32_t off = ok ? ((uint32_t)n * (uint32_t)Kc + (uint32_t)sb) * 2u : kOOB;
+        const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(sr, off, 0, 0);
+        const u32x2 mv = __builtin_amdgcn_raw_buffer_load_b64(zr, off, 0, 0);
+        tl.s[2 * i] = sv[0]; tl.s[2 * i + 1] = sv[1];
+        tl.z[2 * i] = mv[0]; tl.z[2 * i + 1] = mv[1];
+      }
+    }
   };
   // registers (row-contiguous) -> this wavefront's LDS tile -> registers (operand layout)
   auto transpose_tile = [&](Tile& tl) {
@@ -179,7 +202,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
       wchunk_of(i, r, c);
       *reinterpret_cast<u32x4*>(stage + r * kWPitch + c * 16) = tl.w[i];
     }
-    if constexpr (kInt4) {
+    if constexpr (kNib) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const u32x2 v = *reinterpret_cast<const u32x2*>(stage + j * kWPitch + 32 * q + 8 * g);
@@ -201,6 +224,14 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
       const float sf = (float)__builtin_bit_cast(_Float16, (uint16_t)sbits);
       if constexpr (Act::dt == DT_F16) return int4x8_to_f16(dw, (_Float16)sf, (_Float16)(1024.0f + zf));
       else return int4x8_to_bf16(dw, sf, zf);
+    } else if constexpr (kQ4K) {
+      // step q covers sub-blocks 2 q (lanes g = 0, 1) and 2 q + 1 (g = 2, 3) of the slice
+      const uint32_t dw = tl.w[q >> 1][(q & 1) * 2 + h];
+      const uint32_t sh = (uint32_t)(g >> 1) * 16u;
+      const _Float16 sc = __builtin_bit_cast(_Float16, (uint16_t)(tl.s[q] >> sh));
+      const _Float16 mn = __builtin_bit_cast(_Float16, (uint16_t)(tl.z[q] >> sh));
+      if constexpr (Act::dt == DT_F16) return q4kx8_to_f16(dw, sc, mn);
+      else return V8{};
     } else {
       return fp8x8_to_act<Act>(tl.w[q][2 * h], tl.w[q][2 * h + 1]);
     }
@@ -277,7 +308,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
     const int n = n0 + t * 16 + j;
     if (n < nend) {
       float os = 1.0f;
-      if constexpr (!BLOCK && !kInt4) {
+      if constexpr (!BLOCK && !kNib) {
         if (scale_mode == SC_PERT) os = s32[0];
         else os = a.scale_f16 ? (float)((const _Float16*)a.s[mat])[n] : s32[n];
       }
@@ -295,14 +326,17 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
 // rows, the slice of x within 128 registers per lane; FP8: 16-byte aligned rows; INT4 (int4 =
 // true): K a multiple of 512, so that a slice holds whole pairs of groups and the side loads
 // are aligned.
-static inline int kslice_loads(int M, int K, bool int4 = false) {
-  if (M < 5 || M > 32 || (K % 16) || (int4 && (K % 512))) return 0;
+static inline int kslice_loads(int M, int K, int fmt = 0) {
+  if (M < 5 || M > 32 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
   const int mt = M <= 16 ? 1 : 2;
   int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // steps to cover K with 8 slices
-  nq = int4 ? ((nq + 3) & ~3) : ((nq + 1) & ~1);                // FP8: whole 128-wide scale blocks
+  nq = fmt == 1 ? ((nq + 3) & ~3) : ((nq + 1) & ~1);            // FP8: whole 128-wide scale blocks
   const int choices[] = {2, 4, 6, 8, 10, 12};          // 16 steps spill
   for (int c : choices)
-    if (c >= nq) return (mt * c <= 16) ? c : 0;                 // x registers: mt * c * 8 <= 128
+    if (c >= nq) {
+      if (fmt == 2) return (mt * c + c <= 20) ? c : 0;          // Q4_K: a scale and a min word per step and tile on top
+      return (mt * c <= 16) ? c : 0;                            // x registers: mt * c * 8 <= 128
+    }
   return 0;
 }
 
@@ -311,7 +345,7 @@ static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_m
   const dim3 grid(tiles), block(kKsliceWaves * 64);
 #define QLIN_KSLICE(NQ_)                                                                                       \
   case NQ_:                                                                                                    \
-    if constexpr (MT * NQ_ <= 16 && (FMT == 0 || NQ_ % 4 == 0))                                                \
+    if constexpr (MT * NQ_ <= 16 && (FMT != 1 || NQ_ % 4 == 0) && (FMT != 2 || MT * NQ_ + NQ_ <= 20))          \
     {                                                                                                          \
       auto kern = kslice_kernel<Act, FMT, BLOCK, MT, NQ_>;                                                     \
       constexpr int lds = kslice_lds_bytes<MT, NQ_>();                                                         \
@@ -351,9 +385,9 @@ static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
     tiles += a.tiles[i];
   }
   if (!tiles) return MI_OK;
-  if constexpr (FMT == 1) {
-    if (a.M <= 16) kslice_launch_nq<Act, 1, false, 1>(a, nq, tiles, scale_mode, st);
-    else kslice_launch_nq<Act, 1, false, 2>(a, nq, tiles, scale_mode, st);
+  if constexpr (FMT != 0) {
+    if (a.M <= 16) kslice_launch_nq<Act, FMT, false, 1>(a, nq, tiles, scale_mode, st);
+    else kslice_launch_nq<Act, FMT, false, 2>(a, nq, tiles, scale_mode, st);
   } else {
     const bool block = scale_mode == SC_BLOCK;
     if (a.M <= 16) {

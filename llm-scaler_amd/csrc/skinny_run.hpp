@@ -65,8 +65,13 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     // INT4: the same kernel, nibbles decoded with their group's scale; ahead of the granule-interleaved
     // kernel at every N measured (K = 4096, fp16: N = 14336 M=8 13.2 -> 11.6 us, M=32 16.8 -> 14.6 us;
     // N = 4096 7.2 -> 6.5 and 9.7 -> 8.7 us; N = 2048 M=16 8.2 -> 6.3 us)
-    if (const int nq = kslice_loads(a.M, a.K, true))
+    if (const int nq = kslice_loads(a.M, a.K, 1))
       return act_dtype == DT_F16 ? kslice_launch<ActF16, 1>(a, 0, nq, st) : kslice_launch<ActBF16, 1>(a, 0, nq, st);
+  }
+  if constexpr (FMT == 2) {
+    // Q4_K on the same kernel (fp16; up to 16 rows for K <= 5120, up to 32 for K <= 3072): K = N = 5120
+    // M=8 12.6 -> 11.2 us, M=16 14.0 -> 11.5 us; K=2048 N=8192 M=32 8.6 -> 7.6 us
+    if (const int nq = kslice_loads(a.M, a.K, 2)) return kslice_launch<ActF16, 2>(a, 0, nq, st);
   }
   // prefill: the tiled matrix-core GEMM reads the weight once per 256 rows instead of once per 64
   if constexpr (FMT == 0 || FMT == 2) {

@@ -423,7 +423,10 @@ def test_q4k_prefill_tiled_gemm(ops, dev, M, K, N):
     assert O.max_rel_err(out.cpu()[rows][:, cols], O.matmul_ref(x[rows], w[cols])) < TOL
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 256, 3), (5, 768, 100), (40, 512, 33)])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 3), (5, 768, 100), (40, 512, 33),
+                                   # 5 .. 32 rows with x held in registers and K split over the wavefronts
+                                   (8, 5120, 5120), (16, 2048, 333), (32, 1536, 1000), (12, 256, 40), (31, 3072, 4100),
+                                   (17, 4096, 520), (9, 6144, 300)])
 def test_q4k_shapes(ops, dev, M, K, N):
     _, s = ops
     x, raw = O.make_q4k_case(M, K, N, seed=M + N)
