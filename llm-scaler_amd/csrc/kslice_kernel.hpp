@@ -1,6 +1,6 @@
 // Small-M weight-only GEMM (FP8 E4M3 or INT4 group 128) with the activations resident in registers.
 //
-// Regime: 5 <= M <= 32 rows against an [N, K] quantized weight, M * K small enough that a
+// Regime: 5 <= M <= 32 rows (up to 64 for K <= 2048) against an [N, K] quantized weight, M * K small enough that a
 // workgroup can hold all of x in its register file (x is the matrix-core operand that never
 // changes while the weight streams past).  One workgroup owns up to 64 weight rows; its 8
 // wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
@@ -27,11 +27,13 @@
 namespace qlin {
 
 constexpr int kKsliceWaves = 8;
-constexpr int kKsliceMaxTiles = 4;                    // 16-row weight tiles per workgroup
+// 16-row weight tiles per workgroup: four, or what the partial tiles of four activation tiles
+// leave of the LDS
+constexpr int kslice_max_tiles(int MT) { return MT <= 3 ? 4 : 3; }
 
 template <int MT, int NQ>
 constexpr int kslice_lds_bytes() {
-  return kKsliceWaves * 16 * (64 * NQ + 16) + kKsliceWaves * kKsliceMaxTiles * MT * 1024;
+  return kKsliceWaves * 16 * (64 * NQ + 16) + kKsliceWaves * kslice_max_tiles(MT) * MT * 1024;
 }
 
 // FMT = 0: FP8 E4M3, 1: INT4 group 128, 2: GGUF Q4_K (repacked; fp16 scale and min per 32 k).  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   static_assert(!kInt4 || (NQ % 4 == 0 && !BLOCK), "INT4: whole pairs of groups per slice");
   static_assert(!kQ4K || (NQ % 2 == 0 && !BLOCK && Act::dt == DT_F16), "Q4_K runs in fp16");
   constexpr int NW = kKsliceWaves;
-  constexpr int kMaxTiles = kKsliceMaxTiles;
+  constexpr int kMaxTiles = kslice_max_tiles(MT);
   constexpr int kSliceB = 64 * NQ;                    // k of a slice = bytes of half a slice row of x
   constexpr int kPitch = kSliceB + 16;                // LDS row pitch: operand reads hit distinct banks
   constexpr int kStage = 16 * kPitch;                 // one wavefront's staging tile
@@ -295,7 +297,9 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   load_tile(w1, 3);
   __builtin_amdgcn_sched_barrier(0);
   if (ntiles > 2) compute_tile(w0, 2);
-  if (ntiles > 3) compute_tile(w1, 3);
+  if constexpr (kMaxTiles > 3) {
+    if (ntiles > 3) compute_tile(w1, 3);
+  }
 
   // ---- the 8 slices meet: wavefront w finishes output tile (t, mt) = w ----
   __syncthreads();
@@ -327,8 +331,8 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
 // true): K a multiple of 512, so that a slice holds whole pairs of groups and the side loads
 // are aligned.
 static inline int kslice_loads(int M, int K, int fmt = 0) {
-  if (M < 5 || M > 32 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
-  const int mt = M <= 16 ? 1 : 2;
+  if (M < 5 || M > 64 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
+  const int mt = (M + 15) / 16;
   int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // steps to cover K with 8 slices
   nq = fmt == 1 ? ((nq + 3) & ~3) : ((nq + 1) & ~1);            // FP8: whole 128-wide scale blocks
   const int choices[] = {2, 4, 6, 8, 10, 12};          // 16 steps spill
@@ -372,11 +376,12 @@ static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
   long ntot = 0;
   for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
   const int cus = device_cu_count();
-  int rounds = (int)((ntot + (long)cus * 64 - 1) / ((long)cus * 64));
+  const int max_rows = 16 * kslice_max_tiles((a.M + 15) / 16);
+  int rounds = (int)((ntot + (long)cus * max_rows - 1) / ((long)cus * max_rows));
   if (rounds < 1) rounds = 1;
   int rpw = (int)((ntot + (long)cus * rounds - 1) / ((long)cus * rounds));
   rpw = scale_mode == SC_BLOCK ? ((rpw + 15) & ~15) : ((rpw + 7) & ~7);
-  if (rpw > 64) rpw = 64;
+  if (rpw > max_rows) rpw = max_rows;
   if (rpw < 8) rpw = 8;
   a.rpw = rpw;
   int tiles = 0;
@@ -385,19 +390,18 @@ static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
     tiles += a.tiles[i];
   }
   if (!tiles) return MI_OK;
-  if constexpr (FMT != 0) {
-    if (a.M <= 16) kslice_launch_nq<Act, FMT, false, 1>(a, nq, tiles, scale_mode, st);
-    else kslice_launch_nq<Act, FMT, false, 2>(a, nq, tiles, scale_mode, st);
-  } else {
-    const bool block = scale_mode == SC_BLOCK;
-    if (a.M <= 16) {
-      if (block) kslice_launch_nq<Act, 0, true, 1>(a, nq, tiles, scale_mode, st);
-      else kslice_launch_nq<Act, 0, false, 1>(a, nq, tiles, scale_mode, st);
-    } else {
-      if (block) kslice_launch_nq<Act, 0, true, 2>(a, nq, tiles, scale_mode, st);
-      else kslice_launch_nq<Act, 0, false, 2>(a, nq, tiles, scale_mode, st);
-    }
+  const bool block = FMT == 0 && scale_mode == SC_BLOCK;
+#define QLIN_KSLICE_MT(MT_)                                                              \
+  case MT_:                                                                              \
+    if constexpr (FMT != 0) kslice_launch_nq<Act, FMT, false, MT_>(a, nq, tiles, scale_mode, st);   \
+    else if (block) kslice_launch_nq<Act, 0, true, MT_>(a, nq, tiles, scale_mode, st);   \
+    else kslice_launch_nq<Act, 0, false, MT_>(a, nq, tiles, scale_mode, st);             \
+    break;
+  switch ((a.M + 15) / 16) {
+    QLIN_KSLICE_MT(1) QLIN_KSLICE_MT(2) QLIN_KSLICE_MT(3) QLIN_KSLICE_MT(4)
+    default: return MI_ERR_SHAPE;
   }
+#undef QLIN_KSLICE_MT
   return launch_status();
 }
 

@@ -57,20 +57,25 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
     for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
     // measured against the granule-interleaved kernel (M = 5 .. 32): ahead by 5-35 % when a workgroup
     // owns at least two 16-row tiles or rows are short, behind by 10-25 % for one tile of long rows
-    const bool pays = ntot > 16L * device_cu_count() || a.K <= 2048;
+    const long cus = device_cu_count();
+    // 33 .. 64 rows (K <= 2048): between 16 and 32 weight rows per CU the row-split launch of the
+    // granule-interleaved kernel is ahead (M=64 K=2048: N=4096 7.4 against 8.5 us, block-scaled
+    // N=8192 8.8 against 9.7 us; N=12288 14.1 against 11.8 us, N=2048 8.7 against 8.2 us)
+    const bool pays = a.M > 32 ? (ntot > 32 * cus || ntot < 16 * cus) : (ntot > 16 * cus || a.K <= 2048);
     if (const int nq = pays ? kslice_loads(a.M, a.K) : 0)
       return act_dtype == DT_F16 ? kslice_launch<ActF16>(a, SC, nq, st) : kslice_launch<ActBF16>(a, SC, nq, st);
   }
   if constexpr (FMT == 1) {
     // INT4: the same kernel, nibbles decoded with their group's scale; ahead of the granule-interleaved
     // kernel at every N measured (K = 4096, fp16: N = 14336 M=8 13.2 -> 11.6 us, M=32 16.8 -> 14.6 us;
-    // N = 4096 7.2 -> 6.5 and 9.7 -> 8.7 us; N = 2048 M=16 8.2 -> 6.3 us)
+    // N = 4096 7.2 -> 6.5 and 9.7 -> 8.7 us; N = 2048 M=16 8.2 -> 6.3 us; K = 2048 M=64 N = 12288
+    // 15.1 -> 11.0 us)
     if (const int nq = kslice_loads(a.M, a.K, 1))
       return act_dtype == DT_F16 ? kslice_launch<ActF16, 1>(a, 0, nq, st) : kslice_launch<ActBF16, 1>(a, 0, nq, st);
   }
   if constexpr (FMT == 2) {
-    // Q4_K on the same kernel (fp16; up to 16 rows for K <= 5120, up to 32 for K <= 3072): K = N = 5120
-    // M=8 12.6 -> 11.2 us, M=16 14.0 -> 11.5 us; K=2048 N=8192 M=32 8.6 -> 7.6 us
+    // Q4_K on the same kernel (fp16; up to 16 rows for K <= 5120, 32 for K <= 3072, 64 for K <= 2048):
+    // K = N = 5120 M=8 12.6 -> 11.2 us, M=16 14.0 -> 11.5 us; K=2048 N=8192 M=32 8.6 -> 7.6 us
     if (const int nq = kslice_loads(a.M, a.K, 2)) return kslice_launch<ActF16, 2>(a, 0, nq, st);
   }
   // prefill: the tiled matrix-core GEMM reads the weight once per 256 rows instead of once per 64

@@ -443,7 +443,12 @@ def test_q4k_shapes(ops, dev, M, K, N):
     ("q4k", 64, 2048, 2060, torch.float16),
     ("int4", 64, 4096, 4096, torch.bfloat16), ("int4", 40, 1664, 5000, torch.float16), ("int4", 64, 1024, 10240, torch.float16),
     ("pern", 64, 4096, 5120, torch.bfloat16), ("pern", 48, 1664, 1500, torch.float16), ("pert", 35, 2048, 8192, torch.bfloat16),
-    ("block", 64, 5120, 5120, torch.float16), ("block", 34, 1536, 2304, torch.bfloat16), ("block", 64, 640, 4100, torch.bfloat16)])
+    ("block", 64, 5120, 5120, torch.float16), ("block", 34, 1536, 2304, torch.bfloat16), ("block", 64, 640, 4100, torch.bfloat16),
+    # K <= 2048: three or four 16-row tiles of x held in registers, K split over the wavefronts
+    ("pern", 64, 2048, 12288, torch.bfloat16), ("pern", 33, 1024, 300, torch.float16), ("pert", 48, 2048, 9000, torch.float16),
+    ("block", 64, 2048, 12288, torch.bfloat16), ("block", 40, 1024, 1024, torch.float16),
+    ("int4", 64, 2048, 12288, torch.float16), ("int4", 47, 1024, 520, torch.bfloat16), ("int4", 64, 512, 4096, torch.bfloat16),
+    ("q4k", 64, 2048, 8192, torch.float16), ("q4k", 40, 1024, 4096, torch.float16), ("q4k", 63, 256, 100, torch.float16)])
 def test_mid_m_few_weight_rows_per_cu(ops, dev, fmt, M, K, N, dt):
     # 33 .. 64 rows of x against weights with few rows per CU (N up to 10240): every workgroup stages
     # all of x through LDS for 16 .. 48 weight rows.  Granule counts that the wavefronts do not split
