@@ -559,9 +559,10 @@ def test_gemm_int4_shapes(ops, dev, M, K, N, dt, asym):
     (5, 4096, 8200, torch.bfloat16, False), (8, 4096, 14336, torch.float16, True), (16, 2048, 333, torch.float16, False),
     (17, 4096, 9000, torch.float16, True), (32, 4096, 4096, torch.bfloat16, True), (9, 5120, 5120, torch.float16, False),
     (12, 6144, 2000, torch.bfloat16, True), (24, 1536, 4160, torch.bfloat16, False), (31, 3584, 1024, torch.float16, True),
-    (32, 512, 40, torch.float16, False), (7, 1024, 16, torch.bfloat16, True)])
+    (32, 512, 40, torch.float16, False), (7, 1024, 16, torch.bfloat16, True),
+    (3, 4096, 520, torch.float16, True), (4, 1024, 4100, torch.bfloat16, False)])
 def test_int4_register_resident_activations(ops, dev, M, K, N, dt, asym):
-    # 5 .. 32 rows, K a multiple of 512: x held in registers, K split over the wavefronts in slices,
+    # 3 .. 32 rows, K a multiple of 512: x held in registers, K split over the wavefronts in slices,
     # the nibbles decoded with their group's scale and zero-point.  Slices that end inside K (1536,
     # 3584, 5120), row counts off the 16-row tiles, with and without zero-points.
     v, _ = ops
