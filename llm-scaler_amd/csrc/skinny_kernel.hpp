@@ -85,7 +85,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr int kXP = 256 + 16;                       // activation tile pitch
   constexpr bool kXLds = MT >= kSkinnyXLdsFrom;                    // stage the activations through LDS too
   constexpr int kWStage = NW * RT * 16 * kWP;         // activation tiles follow the weight tiles
-  constexpr int kTiles = kWStage + (kXLds ? NW * MT * 16 * kXP : 0);   // SL: the scale tables follow
+  constexpr int kTiles = kWStage + (kXLds ? NW * 16 * kXP : 0);   // one tile per wavefront, reused by its MT tiles; SL: the scale tables follow
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
 
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
       // lane (j, g) ends up with row j, k = 32 g + 8 i .. + 7 of the granule
 #pragma unroll
       for (int mt = 0; mt < (kXLds ? MT : 0); ++mt) {
-        unsigned char* xl = smem + kWStage + (wave * MT + mt) * 16 * kXP;
+        unsigned char* xl = smem + kWStage + wave * 16 * kXP;   // the wavefront's LDS operations retire in order
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           *reinterpret_cast<u32x4*>(xl + ((lane >> 4) + 4 * i) * kXP + (lane & 15) * 16) = st.xa[u][mt][i];
@@ -484,7 +484,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
   if (tiles == 0) return;
   a.tiles_total = tiles;
   const int wgs = a.msplit > 1 ? ((tiles + 7) / 8) * 8 * a.msplit : tiles;
-  constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * MT * 16 * (256 + 16) : 0);
+  constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * 16 * (256 + 16) : 0);
   constexpr int kRed = NW * RT * MT * 1024;
   static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
   const int with_tables = kStage + (SL ? skinny_table_bytes<FMT, RT>(a.K) : 0);
@@ -505,7 +505,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
 template <int FMT, int MT, int RT, int NW>
 static inline bool skinny_tables_fit(int K) {
   if constexpr (FMT == 1 || FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
-    constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * MT * 16 * (256 + 16) : 0);
+    constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * 16 * (256 + 16) : 0);
     return (FMT == 1 || K % 256 == 0) && kStage + skinny_table_bytes<FMT, RT>(K) <= 160 * 1024;
   }
   return false;
@@ -563,14 +563,17 @@ static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
         if (a.K > 4096 && a.K <= 6144) launch_pick<Act, FMT, SC, 1, 2, 8, 6>(a, rpw, st);
         else launch_pick<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
       } else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
-      else if constexpr (FMT == 0 || FMT == 4) launch_pick<Act, FMT, SC, 4, 2, 4, 1>(a, rpw, st);
+      else if constexpr (FMT == 0 || FMT == 4) launch_pick<Act, FMT, SC, 4, 2, 8, 1>(a, rpw, st);
       else if (skinny_tables_fit<FMT, 4, 2, 6>(a.K)) launch_pick<Act, FMT, SC, 4, 2, 6, 1>(a, rpw, st);
       else launch_one<Act, FMT, SC, 4, 2, 8, 1>(a, rpw, st);   // nibble formats: eight waves' tiles fit the LDS
       // (cfg4 M=64, Q4_K: 24.1 us with four waves, 21.9 with eight, 18.6 with six + the LDS tables)
     } else {
       if (a.M <= 16) launch_pick<Act, FMT, SC, 1, 4, 8, 2>(a, rpw, st);
       else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 4, 8, 1>(a, rpw, st);
-      else launch_pick<Act, FMT, SC, 4, 4, 4, 1>(a, rpw, st);
+      // eight wavefronts since the activations pass through one LDS tile per wavefront (four would
+      // leave one per SIMD and nothing to overlap its load -> LDS -> MFMA chain with): K=4096 N=14336
+      // M=64 FP8 24.2 -> 21.9 us, INT4 25.7 -> 21.1 us
+      else launch_pick<Act, FMT, SC, 4, 4, 8, 1>(a, rpw, st);
     }
   }
   return launch_status();
