@@ -68,36 +68,44 @@ __global__ __launch_bounds__(kMapThreads) void moe_tile_map_kernel(const int32_t
 }
 
 // Gather + re-tile: block b of the table -> MFMA operand order (see pack_x_kernel); rows past the
-// block's count are zero.  One workgroup writes 16 consecutive 32-wide steps of one block (4 per
-// wavefront, their loads in flight together).
-constexpr int kPackQ = 16;
+// block's count are zero.  One workgroup re-tiles 16 consecutive 32-wide steps of one block: each
+// wavefront reads 1 KiB of each of four (gathered) rows, the rows meet in an LDS tile and leave
+// as 16 contiguous blocks.
 __global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __restrict__ x,
                                                              const int32_t* __restrict__ row_map,
                                                              const int32_t* __restrict__ blk,
                                                              const int32_t* __restrict__ counts,
                                                              u32x4* __restrict__ xp, int a_rows, int K, int Q,
                                                              int row_div) {
+  __shared__ __attribute__((aligned(16))) unsigned char tile[16 * kPackPitch];
   const int nq = (Q + kPackQ - 1) / kPackQ;           // flat grid: kPackQ steps of one block per workgroup
   const int b = blockIdx.x / nq;
   if (b >= counts[1]) return;
-  const int l = threadIdx.x & 63;
-  const int q0 = (blockIdx.x - b * nq) * kPackQ + (threadIdx.x >> 6) * 4;
-  const int r = l & 15;
-  const uint16_t* src = nullptr;
-  if (r < blk[2 * b + 1]) {
-    const int pos = blk[2 * b] + r;
-    const unsigned row = row_map ? (unsigned)row_map[pos] / (unsigned)row_div : (unsigned)pos;
-    if (row < (unsigned)a_rows) src = x + (size_t)row * K + (l >> 4) * 8;
-  }
+  const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q0 = (blockIdx.x - b * nq) * kPackQ;
+  const int live = blk[2 * b + 1], first = blk[2 * b];
   u32x4 v[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
+    const int r = wave * 4 + i;
+    const int k = q0 * 32 + l * 8;
     v[i] = u32x4{0u, 0u, 0u, 0u};
-    if (src && q0 + i < Q) v[i] = *reinterpret_cast<const u32x4*>(src + (q0 + i) * 32);
+    if (r < live && k < K) {
+      const int pos = first + r;
+      const unsigned row = row_map ? (unsigned)row_map[pos] / (unsigned)row_div : (unsigned)pos;
+      if (row < (unsigned)a_rows) v[i] = *reinterpret_cast<const u32x4*>(x + (size_t)row * K + k);
+    }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    if (q0 + i < Q) xp[((size_t)b * Q + q0 + i) * 64 + l] = v[i];
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(tile + (wave * 4 + i) * kPackPitch + l * 16) = v[i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int q = q0 + wave * 4 + i;
+    if (q < Q)
+      xp[((size_t)b * Q + q) * 64 + l] =
+          *reinterpret_cast<const u32x4*>(tile + (l & 15) * kPackPitch + (wave * 4 + i) * 64 + (l >> 4) * 16);
+  }
 }
 
 struct TiledMoeLayout {
