@@ -328,11 +328,11 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
 
 // Whether the register-resident path covers a problem (0: no; else the steps per slice): 5 .. 64
 // rows (INT4 from 3: the row kernel takes it up to 2 rows only), the slice of x within 128
-// registers per lane; fmt 0 (FP8): 16-byte aligned rows; fmt 1 (INT4): K a multiple of 512, so
+// registers per lane (3 and 4 rows too: the row kernel is slower there); fmt 0 (FP8): 16-byte aligned rows; fmt 1 (INT4): K a multiple of 512, so
 // that a slice holds whole pairs of groups and the side loads are aligned; fmt 2 (Q4_K): K a
 // multiple of 256.
 static inline int kslice_loads(int M, int K, int fmt = 0) {
-  if (M < (fmt == 1 ? 3 : 5) || M > 64 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
+  if (M < 3 || M > 64 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
   const int mt = (M + 15) / 16;
   int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // steps to cover K with 8 slices
   nq = fmt == 1 ? ((nq + 3) & ~3) : ((nq + 1) & ~1);            // FP8: whole 128-wide scale blocks

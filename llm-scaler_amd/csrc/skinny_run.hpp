@@ -28,9 +28,16 @@ static int run(SkinnyArgs a, int act_dtype, hipStream_t st) {
   if (!a.x) return MI_ERR_ARG;
   if (a.M == 0) return MI_OK;
   // decode regime: one wavefront per weight row, activations staged in LDS
-  // INT4 with 3 or 4 rows: the MFMA kernel is as fast (bf16) or faster (fp16: 13.3 against 15.8 us at
-  // N=14336, K=4096) than the row kernel's LDS-staged activations
-  constexpr int rows_max_m = FMT == 1 ? 2 : 4;
+  // 3 or 4 rows: the MFMA kernels are ahead of the row kernel's LDS-staged activations (N=14336,
+  // K=4096: INT4 fp16 11.0 against 15.8 us, FP8 13.5 against 15.8 us, block-scaled 12.9 against
+  // 16.3 us; Q4_K K=N=5120 11.1 against 11.7 us), except FP8 with at most 16 weight rows per CU and
+  // long rows (N=4096, K=4096: 7.1 against 6.7 us)
+  int rows_max_m = 2;
+  if constexpr (FMT == 0) {
+    long ntot = 0;
+    for (int i = 0; i < a.nmat; ++i) ntot += a.N[i];
+    if (!(ntot > 16L * device_cu_count() || a.K <= 2048)) rows_max_m = 4;
+  }
   if (a.M <= rows_max_m && rows_lds_bytes(FMT, a.M == 3 ? 4 : a.M, a.K) <= 64 * 1024 && (FMT != 0 || a.K % 16 == 0)) {
     RowsArgs r{};
     r.x = a.x; r.nmat = a.nmat; r.M = a.M; r.K = a.K; r.scale_f16 = a.scale_f16;
