@@ -1,6 +1,6 @@
 // Small-M weight-only GEMM (FP8 E4M3 or INT4 group 128) with the activations resident in registers.
 //
-// Regime: 5 <= M <= 32 rows (up to 64 for K <= 2048) against an [N, K] quantized weight, M * K small enough that a
+// Regime: 3 <= M <= 32 rows (up to 64 for K <= 2048) against an [N, K] quantized weight, M * K small enough that a
 // workgroup can hold all of x in its register file (x is the matrix-core operand that never
 // changes while the weight streams past).  One workgroup owns up to 64 weight rows; its 8
 // wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
@@ -326,11 +326,10 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   }
 }
 
-// Whether the register-resident path covers a problem (0: no; else the steps per slice): 5 .. 64
-// rows (INT4 from 3: the row kernel takes it up to 2 rows only), the slice of x within 128
-// registers per lane (3 and 4 rows too: the row kernel is slower there); fmt 0 (FP8): 16-byte aligned rows; fmt 1 (INT4): K a multiple of 512, so
-// that a slice holds whole pairs of groups and the side loads are aligned; fmt 2 (Q4_K): K a
-// multiple of 256.
+// Whether the register-resident path covers a problem (0: no; else the steps per slice): 3 .. 64
+// rows, the slice of x within 128 registers per lane; fmt 0 (FP8): 16-byte aligned rows; fmt 1
+// (INT4): K a multiple of 512, so that a slice holds whole pairs of groups and the side loads are
+// aligned; fmt 2 (Q4_K): K a multiple of 256, and a scale and a min word per step on top of x.
 static inline int kslice_loads(int M, int K, int fmt = 0) {
   if (M < 3 || M > 64 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
   const int mt = (M + 15) / 16;
