@@ -561,8 +561,12 @@ static int launch_mt(const SkinnyArgs& a, hipStream_t st) {
         // more than 32 granules: six per wavefront in flight cover K in one turn of the ring
         // (Q4_K K = N = 5120: M=8 13.5 -> 12.7 us, M=16 15.5 -> 13.9 us)
         // (not for Q5_K / Q6_K: with their high-bit registers six granules spill)
-        if (FMT != 5 && FMT != 6 && a.K > 4096 && a.K <= 6144) launch_pick<Act, FMT, SC, 1, 2, 8, 6>(a, rpw, st);
-        else launch_pick<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
+        bool six = false;
+        if constexpr (FMT != 5 && FMT != 6) {
+          six = a.K > 4096 && a.K <= 6144;
+          if (six) launch_pick<Act, FMT, SC, 1, 2, 8, 6>(a, rpw, st);
+        }
+        if (!six) launch_pick<Act, FMT, SC, 1, 2, 8, 4>(a, rpw, st);
       } else if (a.M <= 32) launch_pick<Act, FMT, SC, 2, 2, 8, 2>(a, rpw, st);
       else if constexpr (FMT == 0 || FMT == 4) launch_pick<Act, FMT, SC, 4, 2, 8, 1>(a, rpw, st);
       else if (skinny_tables_fit<FMT, 4, 2, 6>(a.K)) launch_pick<Act, FMT, SC, 4, 2, 6, 1>(a, rpw, st);
