@@ -1,5 +1,6 @@
 #include "gguf_skinny.hpp"
 #include "skinny_kernel.hpp"
+#include "kslice_kernel.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -12,7 +13,11 @@ static int gguf_skinny_fmt(SkinnyArgs a, hipStream_t st) {
     c.M = (M - m0) < 64 ? (M - m0) : 64;
     c.x = (const char*)a.x + (size_t)m0 * a.K * 2;
     c.out[0] = (char*)a.out[0] + (size_t)m0 * a.N[0] * 2;
-    const int rc = launch_mt<ActF16, FMT, 0>(c, st);
+    int rc;
+    int nq = 0;
+    if constexpr (FMT == 3 || FMT == 4) nq = kslice_loads(c.M, c.K, FMT);   // few rows: x resident in registers
+    if constexpr (FMT == 3 || FMT == 4) rc = nq ? kslice_launch<ActF16, FMT>(c, 0, nq, st) : launch_mt<ActF16, FMT, 0>(c, st);
+    else rc = launch_mt<ActF16, FMT, 0>(c, st);
     if (rc != MI_OK) return rc;
   }
   return MI_OK;

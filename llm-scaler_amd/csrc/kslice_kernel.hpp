@@ -36,7 +36,8 @@ constexpr int kslice_lds_bytes() {
   return kKsliceWaves * 16 * (64 * NQ + 16) + kKsliceWaves * kslice_max_tiles(MT) * MT * 1024;
 }
 
-// FMT = 0: FP8 E4M3, 1: INT4 group 128, 2: GGUF Q4_K (repacked; fp16 scale and min per 32 k).  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
+// FMT = 0: FP8 E4M3, 1: INT4 group 128, 2: GGUF Q4_K (repacked; fp16 scale and min per 32 k),
+// 3: Q4_0, 4: Q8_0 (repacked; fp16 scale per 32 k).  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
 // k steps per slice (slice = 64 NQ k; FP8: NQ 16-byte loads per lane and tile, INT4: NQ / 2),
 // BLOCK = 128x128 block scales (FP8; otherwise one scale per output channel or per tensor,
 // applied to the finished sum).
@@ -46,9 +47,12 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   using Elem = typename Act::elem;
   constexpr bool kInt4 = FMT == 1;
   constexpr bool kQ4K = FMT == 2;
-  constexpr bool kNib = kInt4 || kQ4K;                // two weights per byte
+  constexpr bool kQ40 = FMT == 3;
+  constexpr bool kQ80 = FMT == 4;
+  constexpr bool kSide32 = kQ4K || kQ40 || kQ80;      // one fp16 scale (Q4_K: and min) per 32 k
+  constexpr bool kNib = kInt4 || kQ4K || kQ40;        // two weights per byte
   static_assert(!kInt4 || (NQ % 4 == 0 && !BLOCK), "INT4: whole pairs of groups per slice");
-  static_assert(!kQ4K || (NQ % 2 == 0 && !BLOCK && Act::dt == DT_F16), "Q4_K runs in fp16");
+  static_assert(!kSide32 || (NQ % 2 == 0 && !BLOCK && Act::dt == DT_F16), "the GGUF formats run in fp16");
   constexpr int NW = kKsliceWaves;
   constexpr int kMaxTiles = kslice_max_tiles(MT);
   constexpr int kSliceB = 64 * NQ;                    // k of a slice = bytes of half a slice row of x
@@ -61,7 +65,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   constexpr int NL = kNib ? NQ / 2 : NQ;              // 16-byte weight loads per lane and tile
   // side words per lane and tile: INT4 one per pair of groups (two fp16 scales / two zero-point
   // bytes), Q4_K one per step (the fp16 scales / mins of its two 32-wide sub-blocks)
-  constexpr int NS = kInt4 ? NQ / 4 : (kQ4K ? NQ : 1);
+  constexpr int NS = kInt4 ? NQ / 4 : (kSide32 ? NQ : 1);
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // the partial tiles live beside the staging tiles
   f32x4 (*red)[kMaxTiles][MT][64] = reinterpret_cast<f32x4 (*)[kMaxTiles][MT][64]>(smem + NW * kStage);
@@ -89,7 +93,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   const bool has_zp = kInt4 && a.z[mat] != nullptr;
   const int Kc = K >> 5;                              // Q4_K: fp16 scale and min per 32-wide sub-block
   const __amdgpu_buffer_rsrc_t sr =
-      make_rsrc(a.s[mat], kInt4 ? (uint32_t)N * (uint32_t)Kg * 2u : (kQ4K ? (uint32_t)N * (uint32_t)Kc * 2u : 0u));
+      make_rsrc(a.s[mat], kInt4 ? (uint32_t)N * (uint32_t)Kg * 2u : (kSide32 ? (uint32_t)N * (uint32_t)Kc * 2u : 0u));
   const __amdgpu_buffer_rsrc_t zr =
       make_rsrc((has_zp || kQ4K) ? a.z[mat] : a.s[mat],
                 has_zp ? (uint32_t)N * (uint32_t)Kg : (kQ4K ? (uint32_t)N * (uint32_t)Kc * 2u : 0u));
@@ -181,7 +185,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
         tl.z[i] = has_zp ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(zr, ok ? e : kOOB, 0, 0) : 0x0808u;
       }
     }
-    if constexpr (kQ4K) {
+    if constexpr (kSide32) {
       // the row's 2 NQ sub-blocks inside the slice, four entries (one step pair) per 64-bit load
       const int n = n0 + t * 16 + j;
 #pragma unroll
@@ -190,9 +194,11 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
         const bool ok = t < ntiles && n < nend && sb < Kc;
         const uint32_t off = ok ? ((uint32_t)n * (uint32_t)Kc + (uint32_t)sb) * 2u : kOOB;
         const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(sr, off, 0, 0);
-        const u32x2 mv = __builtin_amdgcn_raw_buffer_load_b64(zr, off, 0, 0);
         tl.s[2 * i] = sv[0]; tl.s[2 * i + 1] = sv[1];
-        tl.z[2 * i] = mv[0]; tl.z[2 * i + 1] = mv[1];
+        if constexpr (kQ4K) {
+          const u32x2 mv = __builtin_amdgcn_raw_buffer_load_b64(zr, off, 0, 0);
+          tl.z[2 * i] = mv[0]; tl.z[2 * i + 1] = mv[1];
+        }
       }
     }
   };
@@ -233,6 +239,15 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
       const _Float16 sc = __builtin_bit_cast(_Float16, (uint16_t)(tl.s[q] >> sh));
       const _Float16 mn = __builtin_bit_cast(_Float16, (uint16_t)(tl.z[q] >> sh));
       if constexpr (Act::dt == DT_F16) return q4kx8_to_f16(dw, sc, mn);
+      else return V8{};
+    } else if constexpr (kQ40) {
+      const uint32_t dw = tl.w[q >> 1][(q & 1) * 2 + h];
+      const _Float16 sc = __builtin_bit_cast(_Float16, (uint16_t)(tl.s[q] >> ((uint32_t)(g >> 1) * 16u)));
+      if constexpr (Act::dt == DT_F16) return int4x8_to_f16(dw, sc, (_Float16)1032.0f);   // (nib - 8) * d
+      else return V8{};
+    } else if constexpr (kQ80) {
+      const _Float16 sc = __builtin_bit_cast(_Float16, (uint16_t)(tl.s[q] >> ((uint32_t)(g >> 1) * 16u)));
+      if constexpr (Act::dt == DT_F16) return i8x8_to_f16(tl.w[q][2 * h], tl.w[q][2 * h + 1], sc);
       else return V8{};
     } else {
       return fp8x8_to_act<Act>(tl.w[q][2 * h], tl.w[q][2 * h + 1]);
@@ -312,7 +327,7 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
     const int n = n0 + t * 16 + j;
     if (n < nend) {
       float os = 1.0f;
-      if constexpr (!BLOCK && !kNib) {
+      if constexpr (FMT == 0 && !BLOCK) {
         if (scale_mode == SC_PERT) os = s32[0];
         else os = a.scale_f16 ? (float)((const _Float16*)a.s[mat])[n] : s32[n];
       }
@@ -329,16 +344,19 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
 // Whether the register-resident path covers a problem (0: no; else the steps per slice): 3 .. 64
 // rows, the slice of x within 128 registers per lane; fmt 0 (FP8): 16-byte aligned rows; fmt 1
 // (INT4): K a multiple of 512, so that a slice holds whole pairs of groups and the side loads are
-// aligned; fmt 2 (Q4_K): K a multiple of 256, and a scale and a min word per step on top of x.
+// aligned; fmt 2 (Q4_K): K a multiple of 256, and a scale and a min word per step on top of x;
+// fmt 3, 4 (Q4_0, Q8_0): K a multiple of 128.
 static inline int kslice_loads(int M, int K, int fmt = 0) {
-  if (M < 3 || M > 64 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256))) return 0;
+  if (M < 3 || M > 64 || (K % 16) || (fmt == 1 && (K % 512)) || (fmt == 2 && (K % 256)) ||
+      ((fmt == 3 || fmt == 4) && (K % 128)))
+    return 0;
   const int mt = (M + 15) / 16;
   int nq = (K + 64 * kKsliceWaves - 1) / (64 * kKsliceWaves);   // steps to cover K with 8 slices
   nq = fmt == 1 ? ((nq + 3) & ~3) : ((nq + 1) & ~1);            // FP8: whole 128-wide scale blocks
   const int choices[] = {2, 4, 6, 8, 10, 12};          // 16 steps spill
   for (int c : choices)
     if (c >= nq) {
-      if (fmt == 2) return (mt * c + c <= 20) ? c : 0;          // Q4_K: a scale and a min word per step and tile on top
+      if (fmt >= 2) return (mt * c + c <= 20) ? c : 0;          // GGUF: scale (and min) words per step and tile on top
       return (mt * c <= 16) ? c : 0;                            // x registers: mt * c * 8 <= 128
     }
   return 0;
@@ -349,7 +367,7 @@ static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_m
   const dim3 grid(tiles), block(kKsliceWaves * 64);
 #define QLIN_KSLICE(NQ_)                                                                                       \
   case NQ_:                                                                                                    \
-    if constexpr (MT * NQ_ <= 16 && (FMT != 1 || NQ_ % 4 == 0) && (FMT != 2 || MT * NQ_ + NQ_ <= 20))          \
+    if constexpr (MT * NQ_ <= 16 && (FMT != 1 || NQ_ % 4 == 0) && (FMT < 2 || MT * NQ_ + NQ_ <= 20))           \
     {                                                                                                          \
       auto kern = kslice_kernel<Act, FMT, BLOCK, MT, NQ_>;                                                     \
       constexpr int lds = kslice_lds_bytes<MT, NQ_>();                                                         \
