@@ -133,7 +133,7 @@ def _gemv(s, kind, x, rep, out, name=None):
                                    (4, 256, 8192), (1, 40, 14336), (7, 48, 1536), (16, 130, 2048), (33, 72, 1024),
                                    (64, 520, 5120), (100, 40, 512),
                                    # Q4_0 / Q8_0 with few rows and K % 128 == 0: x resident in registers, K sliced over wavefronts
-                                   (12, 300, 5120), (40, 96, 2048), (5, 64, 768), (16, 1000, 4096)])
+                                   (12, 300, 5120), (40, 96, 2048), (5, 64, 1024), (16, 1000, 4096)])
 def test_gemv(ops, dev, kind, M, N, K):
     _, s = ops
     raw = _raw_case(kind, N, K, seed=7 * M + N + K)
