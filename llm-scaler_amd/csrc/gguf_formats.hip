@@ -366,8 +366,9 @@ static int run_gguf_gemv(RowsArgs r, int M, hipStream_t st) {
   if (M < 0 || r.N[0] < 0 || r.K <= 0) return MI_ERR_SHAPE;
   if ((uint64_t)r.N[0] * (uint64_t)r.K >= (1ull << 31)) return MI_ERR_SHAPE;
   if (M == 0 || r.N[0] == 0) return MI_OK;
-  // more than four rows: the MFMA kernel (64 rows per pass)
-  if (M > 4)
+  // more than four rows: the MFMA kernels (64 rows per pass); Q4_0 from three rows when x fits the
+  // registers (K=N=5120: 10.0 against 11.6-11.9 us on the row kernel)
+  if (M > 4 || (FMT == 3 && M > 2 && gguf_skinny_resident(FMT, M, r.K)))
     return gguf_skinny(FMT, r.x, r.w[0], r.h[0], r.s[0], r.z[0], r.out[0], M, r.N[0], r.K, st);
   // rows per launch: as many (4, 2, 1) as the staged activations allow in 64 KiB of LDS
   int step = 4;

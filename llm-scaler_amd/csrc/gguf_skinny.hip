@@ -23,6 +23,8 @@ static int gguf_skinny_fmt(SkinnyArgs a, hipStream_t st) {
   return MI_OK;
 }
 
+bool gguf_skinny_resident(int fmt, int M, int K) { return (fmt == 3 || fmt == 4) && kslice_loads(M, K, fmt) != 0; }
+
 int gguf_skinny(int fmt, const void* x, const void* w, const void* h, const void* s, const void* z, void* out,
                 int M, int N, int K, hipStream_t st) {
   SkinnyArgs a{};

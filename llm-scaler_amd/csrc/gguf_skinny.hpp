@@ -11,4 +11,8 @@ namespace qlin {
 int gguf_skinny(int fmt, const void* x, const void* w, const void* h, const void* s, const void* z, void* out,
                 int M, int N, int K, hipStream_t st);
 
+// Whether gguf_skinny would run the register-resident K-sliced kernel (Q4_0 / Q8_0, few rows,
+// K % 128 == 0): with 3 or 4 rows that kernel is ahead of the row kernel for Q4_0.
+bool gguf_skinny_resident(int fmt, int M, int K);
+
 }  // namespace qlin
