@@ -1,9 +1,10 @@
-// Small-M weight-only GEMM (FP8 E4M3 or INT4 group 128) with the activations resident in registers.
+// Small-M weight-only GEMM (FP8 E4M3, INT4 group 128, GGUF Q4_K / Q4_0 / Q8_0) with the
+// activations resident in registers.
 //
-// Regime: 3 <= M <= 32 rows (up to 64 for K <= 2048) against an [N, K] quantized weight, M * K small enough that a
-// workgroup can hold all of x in its register file (x is the matrix-core operand that never
-// changes while the weight streams past).  One workgroup owns up to 64 weight rows; its 8
-// wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
+// Regime: 3 <= M <= 32 rows (up to 64 for K <= 2048) against an [N, K] quantized weight, M * K
+// small enough that a workgroup can hold all of x in its register file (x is the matrix-core
+// operand that never changes while the weight streams past).  One workgroup owns up to 64 weight
+// rows; its 8 wavefronts split K into 8 contiguous slices instead of interleaving granules, so that
 //   - a wavefront loads its slice of x ONCE, before any weight load is issued (x comes from L2;
 //     the vector-memory counter retires in order, so these loads never queue behind the weight
 //     stream),
@@ -13,14 +14,17 @@
 // Weight loads are row-contiguous (one instruction reads 1 KiB of consecutive slice bytes, row
 // after row: operand-layout loads whose lanes read 64-byte pieces of 16 rows were measured
 // about 3 us slower on a 56 MB weight); the wavefront's own LDS tile (pitch + 16 bytes) turns
-// them into operand layout.
+// them into operand layout.  The slice of x is loaded the same way.
 //
 // k assignment inside a slice: step q (0 .. NQ-1) of lane (j = lane % 16, g = lane / 16) covers
-// k = 64 q + 16 g .. + 15 of weight row n0 + 16 t + j (16 bytes of FP8, 8 bytes of INT4); MFMA
-// 2 q + h consumes its k = 8 h .. 8 h + 7 against x[j][slice + 64 q + 16 g + 8 h .. + 7].
-// INT4: the fp16 scales and zero-point bytes of the row's NQ / 2 groups inside the slice travel
-// with the tile (one or two small loads per lane), and the nibbles are decoded with the scale
-// folded in (the routines of the dequantization kernels), so the sums need no factor.
+// k = 64 q + 16 g .. + 15 of weight row n0 + 16 t + j (16 bytes of a byte format, 8 bytes of a
+// nibble format); MFMA 2 q + h consumes its k = 8 h .. 8 h + 7 against
+// x[j][slice + 64 q + 16 g + 8 h .. + 7].
+// Side data travels with the tile as a few small loads per lane: INT4 the fp16 scales and
+// zero-point bytes of the row's NQ / 2 groups inside the slice, the GGUF formats the fp16 scales
+// (Q4_K: and mins) of its 2 NQ sub-blocks.  The weights are decoded with the scale folded in
+// (the routines of the dequantization kernels), so the sums need no factor; FP8 per-channel /
+// per-tensor scales multiply the finished sums, block scales each 128-wide partial.
 #pragma once
 #include "skinny_kernel.hpp"
 
@@ -37,8 +41,9 @@ constexpr int kslice_lds_bytes() {
 }
 
 // FMT = 0: FP8 E4M3, 1: INT4 group 128, 2: GGUF Q4_K (repacked; fp16 scale and min per 32 k),
-// 3: Q4_0, 4: Q8_0 (repacked; fp16 scale per 32 k).  MT = 16-row activation tiles (M <= 16 MT), NQ = 64-wide
-// k steps per slice (slice = 64 NQ k; FP8: NQ 16-byte loads per lane and tile, INT4: NQ / 2),
+// 3: Q4_0, 4: Q8_0 (repacked; fp16 scale per 32 k).  MT = 16-row activation tiles (M <= 16 MT),
+// NQ = 64-wide k steps per slice (slice = 64 NQ k; byte formats: NQ 16-byte loads per lane and
+// tile, nibble formats: NQ / 2),
 // BLOCK = 128x128 block scales (FP8; otherwise one scale per output channel or per tensor,
 // applied to the finished sum).
 template <class Act, int FMT, bool BLOCK, int MT, int NQ>
