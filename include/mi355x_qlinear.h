@@ -149,8 +149,8 @@ int mi_q4k_repack(const void* raw, void* ql, void* scale, void* qmin, int N, int
  *   3047-3054, 2952-2970, 3011-3026), the reference's route for M > 1.
  * mi_gemv_*: out [M,N] fp16 = x [M,K] fp16 @ w^T, fp32 accumulation.  Replace
  *   esimd_gemv_q4_0, esimd_gemm_q4_0, esimd_gemv_q8_0(_m), esimd_gemv_q5_k,
- *   esimd_gemv_q6_k(_m) (S/csrc/xpu/torch_extension.cc:48-106), for any M (M <= 4: one
- *   wavefront per row; larger M: the MFMA kernel, 64 rows per pass).
+ *   esimd_gemv_q6_k(_m) (S/csrc/xpu/torch_extension.cc:48-106), for any M (up to 4 rows: one
+ *   wavefront per weight row; more rows: the MFMA kernels, 64 rows per pass).
  * mi_q4_0_quantize: x [rows,K] fp16/bf16 -> qweight [rows,K/8] int32 (nibble i of
  *   word w = element 8w+i, value + 8) + scale [rows,K/128] fp16 = max/-8, the
  *   layout mi_gemv_int4 reads.  GGML's quantize_row_q4_0 rule on 128-wide blocks;
