@@ -220,7 +220,10 @@ def test_fp8_pern_shapes(ops, dev, M, K, N, dt, s16):
     (5, 4096, 8200, torch.bfloat16, "pern"), (16, 2048, 333, torch.float16, "pern"), (17, 4096, 9000, torch.float16, "pern"),
     (32, 4096, 8192, torch.bfloat16, "pert"), (9, 5120, 5120, torch.float16, "block"), (24, 1024, 4160, torch.bfloat16, "block"),
     (31, 3584, 9216, torch.float16, "block"), (8, 6144, 8448, torch.bfloat16, "pern"), (12, 1056, 520, torch.float16, "pern"),
-    (6, 6112, 8300, torch.float16, "pert")])
+    (6, 6112, 8300, torch.float16, "pert"),
+    # 3 and 4 rows take this kernel too (the row kernel stops at 2 unless the weight has few, long rows)
+    (3, 4096, 8200, torch.bfloat16, "pern"), (4, 2048, 333, torch.float16, "block"), (4, 4096, 14336, torch.bfloat16, "pert"),
+    (3, 5120, 5120, torch.float16, "block"), (4, 4096, 4096, torch.float16, "pern")])
 def test_fp8_register_resident_activations(ops, dev, M, K, N, dt, mode):
     # 5 .. 32 rows with x held in registers and K split over the wavefronts in slices: slices that
     # end inside K (3584, 1056, 6112), row counts off the 16-row tiles, every scale mode
@@ -426,7 +429,7 @@ def test_q4k_prefill_tiled_gemm(ops, dev, M, K, N):
 @pytest.mark.parametrize("M,K,N", [(1, 256, 3), (5, 768, 100), (40, 512, 33),
                                    # 5 .. 32 rows with x held in registers and K split over the wavefronts
                                    (8, 5120, 5120), (16, 2048, 333), (32, 1536, 1000), (12, 256, 40), (31, 3072, 4100),
-                                   (17, 4096, 520), (9, 6144, 300)])
+                                   (17, 4096, 520), (9, 6144, 300), (3, 5120, 520), (4, 1024, 4100)])
 def test_q4k_shapes(ops, dev, M, K, N):
     _, s = ops
     x, raw = O.make_q4k_case(M, K, N, seed=M + N)
