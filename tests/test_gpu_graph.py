@@ -67,6 +67,21 @@ def test_graph_fp8_pern_m8(ops, dev):
     _check_graph(dev, lambda: v.esimd_gemv_fp8_pern(xd, wd, sd, out, N, K), [out])
 
 
+def test_graph_int4_m16_and_fp8_m64(ops, dev):
+    # the K-sliced kernel on INT4 (16 rows) and the row-split launch of the skinny kernel (64 rows of x
+    # against 16 weight rows per CU)
+    v, _ = ops
+    x, packed, scale, _ = O.make_int4_case(16, 2048, 1024, seed=31)
+    xd, wd, sd = x.to(dev), packed.to(dev), scale.to(dev)
+    out = torch.empty(16, 1024, dtype=torch.float16, device=dev)
+    _check_graph(dev, lambda: v.esimd_gemm_int4_pgrp(xd, wd, sd, out), [out])
+    M, K, N = 64, 4096, 4096
+    x, w8, s = O.make_fp8_pern_case(M, K, N, seed=32)
+    xf, wf, sf = x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), s.to(dev)
+    out2 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    _check_graph(dev, lambda: v.esimd_gemv_fp8_pern(xf, wf, sf, out2, N, K), [out2])
+
+
 def test_graph_int4_gemm(ops, dev):
     v, _ = ops
     M, K, N = 200, 1024, 512
