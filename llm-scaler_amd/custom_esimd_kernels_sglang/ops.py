@@ -140,3 +140,11 @@ def esimd_moe_down_q5k(inter, ql, qh, sc, mn, sel, topk_w, out_partial, n_tokens
 
 def esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k):
     return _ops.esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k)
+
+
+# Imported at module level by the patched SGLang's XPU attention backend
+# (sglang/patches/sglang_for_multi_arc.patch:684); paged attention is outside the quantized-linear path:
+# the name exists so that module imports, and raises when called.
+from mi355x_qlinear.not_provided import NotProvided as _NotProvided  # noqa: E402
+
+eagle_page_attn_decode = _NotProvided("eagle_page_attn_decode", "an attention backend other than xpu")

@@ -6,3 +6,4 @@ import mi355x_qlinear  # noqa: F401  (registers torch.ops.* for ROCm tensors)
 from .ops import *  # noqa: F401,F403
 from . import moe_ops  # noqa: F401,E402
 from . import moe_int4_prefill_ops  # noqa: F401,E402
+from . import eagle_ops  # noqa: F401,E402

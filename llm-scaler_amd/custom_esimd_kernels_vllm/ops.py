@@ -315,3 +315,17 @@ def q4_0_quantize(input, out_qweight, out_scale):
     """torch.ops.custom_esimd_kernels_vllm.q4_0_quantize (the reference registers it from its
     q4_0_quant_ops module): [M, K] fp16/bf16 -> int32 [M, K/8] + fp16 scale [M, K/128]."""
     return _ops.q4_0_quantize(input, out_qweight, out_scale)
+
+
+# Read unguarded by the patched callers but outside the quantized-linear path (attention, GDN, RoPE and
+# INT4-MoE fusions): the names exist so the callers import, and raise when called
+# (vllm/patches/vllm_for_multi_arc.patch:3149, :3159-3160, :8518-8520, :10011-10014).
+from mi355x_qlinear.not_provided import NotProvided as _NotProvided  # noqa: E402
+
+esimd_qkv_split_norm_rope = _NotProvided("esimd_qkv_split_norm_rope", "DISABLE_ESIMD_QKV=1")
+esimd_qkv_split_norm_rope_v = _NotProvided("esimd_qkv_split_norm_rope_v", "DISABLE_ESIMD_QKV_FUSED=1")
+esimd_gdn_conv_fused = _NotProvided("esimd_gdn_conv_fused", "DISABLE_ESIMD_GDN_CONV=1")
+esimd_gdn_conv_fused_seq = _NotProvided("esimd_gdn_conv_fused_seq", "DISABLE_ESIMD_GDN_CONV=1")
+moe_forward_full_cutlass_nmajor_int4 = _NotProvided("moe_forward_full_cutlass_nmajor_int4", "DISABLE_ESIMD_INT4=1 (sym_int4 MoE models)")
+moe_forward_tiny_cutlass_nmajor_int4_full_fp16_shared_from_logits = _NotProvided(
+    "moe_forward_tiny_cutlass_nmajor_int4_full_fp16_shared_from_logits", "DISABLE_ESIMD_INT4=1 (sym_int4 MoE models)")
