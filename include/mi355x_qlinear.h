@@ -9,14 +9,21 @@
  *   - every pointer is device memory; outputs are pre-allocated by the caller;
  *   - the call enqueues on `stream` (a hipStream_t, 0 = the null stream) and
  *     returns without synchronising; nothing is allocated or freed, except by the
- *     entries that say so (mi_gemm_int4: a grow-only scratch buffer; mi_norm_gemv: a
- *     2 KiB counter block per device and stream, on first use);
+ *     entries that say so: a grow-only scratch buffer per (device, stream), allocated with
+ *     hipMalloc on first use or growth (not possible under stream capture), is used by
+ *     mi_gemm_int4, by mi_gemm_fp8_{pern,pert,blockscale}[_multi] and mi_gemv_q4k for M > 64,
+ *     and by mi_moe_gemm_fp8_grouped / _block when the experts average 96 rows or more;
+ *     mi_norm_gemv[_scaled] takes a 2 KiB counter block per device and stream on first use.
+ *     Callers that capture or must not allocate use the *_ws variants with
+ *     mi_gemm_tiled_workspace / mi_moe_gemm_fp8_tiled_workspace bytes of their own memory
+ *     (what the torch ops do), and mi_norm_gemv_static;
  *   - tensors are dense row-major;
  *   - act_dtype: 0 = fp16, 1 = bf16 (inputs and outputs share it);
  *   - return value: 0 on success, MI_ERR_ARG (-1) for a null pointer or bad
  *     enum, MI_ERR_SHAPE (-2) for a shape the kernels do not cover,
  *     MI_ERR_LAUNCH (-3) if the launch itself failed, MI_ERR_LIMIT (-4) for a size
- *     beyond the fixed capacity of an entry point that allocates nothing.
+ *     beyond the fixed capacity of an entry point that allocates nothing,
+ *     MI_ERR_BUSY (-5) when that entry point's static scratch belongs to another stream.
  */
 #ifndef MI355X_QLINEAR_H_
 #define MI355X_QLINEAR_H_
@@ -98,6 +105,26 @@ int mi_gemm_int4_workspace(int M, int N, int K, long long* bytes);
 int mi_gemm_int4_ws(const void* x, const void* w, const void* scale, const void* zp, void* out,
                     void* workspace, long long workspace_bytes, int M, int N, int K, int act_dtype,
                     void* stream);
+
+/* ---- GPTQ / AWQ style operands of the reference's asymmetric W4A16 linear -----------
+ * The reference calls a third-party op for these weights,
+ * int4_gemm_w4a16(x, qweight[K/8, N] int32, bias, scales[K/g, N], qzeros, g, g_idx)
+ * (vllm/patches/vllm_for_multi_arc.patch:5492-5500, AWQ :5002-5010, GPTQ :5080-5088; the op's
+ * source is not part of the reference tree, so its zero-point packing is restated here from
+ * the published GPTQ layout).  mi_w4a16_kmajor_prepare turns those operands into the ones
+ * mi_gemm_int4 / mi_gemv_int4 read, bit for bit, on the device:
+ *   w_out [N, K/8] int32  = qweight transposed (nibble z of a word = element 8i + z on both
+ *                           sides); pass qweight = w_out = NULL when the caller's [K/8, N]
+ *                           tensor already has strides (1, K/8), i.e. the same bytes;
+ *   s_out [N, K/128] fp16 = scales [K/128, N] transposed;
+ *   zp_out[N, K/128] u8   = zero_scalar ? qzeros[0]
+ *                         : ((qzeros[g][n / 8] >> 4 (n % 8)) & 15) + zero_bias, qzeros [K/128, N/8]
+ *                           int32 (zero_bias 1 for checkpoints that store zero - 1); NULL for none.
+ * Group size 128 only; N % 8 == 0 with packed zero-points.  mi_add_bias adds bias[N] to every
+ * row of out[M, N] in place (fp32 sum, one rounding), the op's optional bias argument. */
+int mi_w4a16_kmajor_prepare(const int32_t* qweight, const void* scales, const int32_t* qzeros, int zero_scalar,
+                            int zero_bias, void* w_out, void* s_out, uint8_t* zp_out, int N, int K, void* stream);
+int mi_add_bias(void* out, const void* bias, int M, int N, int act_dtype, void* stream);
 
 /* ---- GGUF Q4_K on the repacked representation, fp16 -------------------------
  * ql [N, K/2] uint8 interleaved nibbles, scale/qmin [N, K/32] fp16;
@@ -339,9 +366,14 @@ int mi_norm_gemv_scaled(const void* x, void* residual, const void* gate, const v
  * beyond its limit (K > 16384, or K whose staged row exceeds 64 KiB of LDS) return
  * MI_ERR_LIMIT (-4) instead of taking the two-kernel route.  All calls on one GPU share the
  * counters: the kernel leaves them at zero when it ends, so back-to-back calls on one stream
- * are fine, while calls that overlap on one GPU (different streams) race.
+ * are fine, while calls that overlap on one GPU (different streams) would race.  Therefore the
+ * first call after a set-up claims the array for its stream, and a call on any other stream of
+ * that GPU returns MI_ERR_BUSY (-5) without launching.
  * mi_static_scratch_setup resolves the array's address on the current device (the first call
- * of mi_norm_gemv_static on a device does the same); call it once per device before capturing. */
+ * of mi_norm_gemv_static on a device does the same), clears the counters with a blocking
+ * hipMemset and releases the claim: call it once per device before capturing; call it again,
+ * with no mi_norm_gemv_static work in flight on that GPU, to hand the array to another stream
+ * or to recover after a kernel that ended abnormally and left counters non-zero. */
 int mi_static_scratch_setup(void);
 int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const void* norm_weight,
                         void* normed_out, int norm_len, float eps, float residual_scale, int fmt, int nmat,
@@ -354,9 +386,11 @@ int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const v
  * re-tiled per 16-row block, then the 256 x 256 tiled GEMM with one weight matrix per expert, so
  * that an expert's weights are read once per 256 of its rows (a wavefront skips the 16-row tiles
  * past an expert's last row).  Same arguments and
- * results; K % 128 == 0, E <= 1024.  workspace: mi_moe_gemm_fp8_tiled_workspace bytes.
- * mi_moe_gemm_fp8_grouped takes this route itself (per-stream scratch) when the experts average
- * 96 rows or more.  Reference: the 64-row expert tiles with a device-built tile map of
+ * results; K % 128 == 0, E <= 1024.  workspace: mi_moe_gemm_fp8_tiled_workspace bytes; that call
+ * returns MI_ERR_SHAPE (with *bytes still set) when the re-tiled activations,
+ * (total_rows / 16 + E) * 16 * K * 2 bytes, would reach 2 GiB: such a launch belongs to the
+ * streaming kernel.  mi_moe_gemm_fp8_grouped takes this route itself (per-stream scratch) when the
+ * experts average 96 rows or more and the workspace call succeeds, and streams otherwise.  Reference: the 64-row expert tiles with a device-built tile map of
  * V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:83-120, 187-302 and the per-expert M-tiled
  * GEMMs of S/csrc/moe_prefill/moe_prefill_fp8.sycl:167-410. */
 int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes);

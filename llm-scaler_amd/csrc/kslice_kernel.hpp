@@ -367,8 +367,10 @@ static inline int kslice_loads(int M, int K, int fmt = 0) {
   return 0;
 }
 
+// true when a kernel was launched; false when no instantiation covers (MT, nq, FMT), in which case
+// the caller reports MI_ERR_SHAPE and leaves the output untouched
 template <class Act, int FMT, bool BLOCK, int MT>
-static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_mode, hipStream_t st) {
+static bool kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_mode, hipStream_t st) {
   const dim3 grid(tiles), block(kKsliceWaves * 64);
 #define QLIN_KSLICE(NQ_)                                                                                       \
   case NQ_:                                                                                                    \
@@ -383,13 +385,15 @@ static void kslice_launch_nq(const SkinnyArgs& a, int nq, int tiles, int scale_m
         raised = true;                                                                                         \
       }                                                                                                        \
       hipLaunchKernelGGL(kern, grid, block, lds, st, a, scale_mode);                                           \
-    }         \
+      return true;                                                                                             \
+    }                                                                                                          \
     break;
   switch (nq) {
     QLIN_KSLICE(2) QLIN_KSLICE(4) QLIN_KSLICE(6) QLIN_KSLICE(8) QLIN_KSLICE(10) QLIN_KSLICE(12)
     default: break;
   }
 #undef QLIN_KSLICE
+  return false;
 }
 
 // scale_mode (FP8): SC_PERN / SC_PERT / SC_BLOCK.  Rows per workgroup as in the skinny kernel: one
@@ -416,15 +420,17 @@ static int kslice_launch(SkinnyArgs a, int scale_mode, int nq, hipStream_t st) {
   const bool block = FMT == 0 && scale_mode == SC_BLOCK;
 #define QLIN_KSLICE_MT(MT_)                                                              \
   case MT_:                                                                              \
-    if constexpr (FMT != 0) kslice_launch_nq<Act, FMT, false, MT_>(a, nq, tiles, scale_mode, st);   \
-    else if (block) kslice_launch_nq<Act, 0, true, MT_>(a, nq, tiles, scale_mode, st);   \
-    else kslice_launch_nq<Act, 0, false, MT_>(a, nq, tiles, scale_mode, st);             \
+    if constexpr (FMT != 0) launched = kslice_launch_nq<Act, FMT, false, MT_>(a, nq, tiles, scale_mode, st);   \
+    else if (block) launched = kslice_launch_nq<Act, 0, true, MT_>(a, nq, tiles, scale_mode, st);   \
+    else launched = kslice_launch_nq<Act, 0, false, MT_>(a, nq, tiles, scale_mode, st);             \
     break;
+  bool launched = false;
   switch ((a.M + 15) / 16) {
     QLIN_KSLICE_MT(1) QLIN_KSLICE_MT(2) QLIN_KSLICE_MT(3) QLIN_KSLICE_MT(4)
     default: return MI_ERR_SHAPE;
   }
 #undef QLIN_KSLICE_MT
+  if (!launched) return MI_ERR_SHAPE;      // kslice_loads() and the instantiation guards disagree
   return launch_status();
 }
 

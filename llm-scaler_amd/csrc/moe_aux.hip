@@ -37,7 +37,11 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 }
 // 16-bit float pattern (fp16 or bf16) -> unsigned, monotone, and back; the smallest key, 0, is kept for
 // "no value" (it would be the pattern of the negative NaN with every bit set)
-__device__ __forceinline__ uint32_t f16_order(uint32_t b) { return (b & 0x8000u) ? (~b & 0xFFFFu) : (b | 0x8000u); }
+// -0 is ordered as +0: a float compare calls them equal, and then the lowest index wins the tie
+__device__ __forceinline__ uint32_t f16_order(uint32_t b) {
+  b = b == 0x8000u ? 0u : b;
+  return (b & 0x8000u) ? (~b & 0xFFFFu) : (b | 0x8000u);
+}
 __device__ __forceinline__ uint32_t f16_unorder(uint32_t u) { return (u & 0x8000u) ? (u & 0x7FFFu) : (~u & 0xFFFFu); }
 template <class Act, int SLOTS>
 __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,

@@ -454,11 +454,14 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
   // prefill (experts averaging 96 rows or more, 16-bit activations and output): the tiled matrix-core GEMM
   if (!a_scale && !out_f32 && (K % 128) == 0 && E <= 1024 && (long)total_rows >= 96L * E) {
     long long bytes = 0;
-    if (mi_moe_gemm_fp8_tiled_workspace(total_rows, E, K, &bytes) != MI_OK) return MI_ERR_SHAPE;
-    void* ws = scratch_get((hipStream_t)stream, (size_t)bytes);
-    if (!ws) return MI_ERR_LAUNCH;
-    return mi_moe_gemm_fp8_tiled_ws(a, row_map, row_map_div, w, w_scale, scale_per_expert, expert_start, out, out_map, row_weight,
-                                    a_rows, total_rows, E, N, K, fuse_act, act_dtype, ws, bytes, stream);
+    // MI_ERR_SHAPE here means the re-tiled activations would pass 2 GiB: the streaming kernel below,
+    // which only bounds a_rows * K, takes such a launch
+    if (mi_moe_gemm_fp8_tiled_workspace(total_rows, E, K, &bytes) == MI_OK) {
+      void* ws = scratch_get((hipStream_t)stream, (size_t)bytes);
+      if (!ws) return MI_ERR_LAUNCH;
+      return mi_moe_gemm_fp8_tiled_ws(a, row_map, row_map_div, w, w_scale, scale_per_expert, expert_start, out, out_map, row_weight,
+                                      a_rows, total_rows, E, N, K, fuse_act, act_dtype, ws, bytes, stream);
+    }
   }
   MoeGemmArgs p{};
   p.a = a; p.a_scale = a_scale; p.row_map = row_map; p.row_div = row_map_div; p.w = w; p.w_scale = w_scale;

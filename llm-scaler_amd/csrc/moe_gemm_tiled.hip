@@ -164,7 +164,11 @@ extern "C" {
 int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes) {
   if (!bytes) return MI_ERR_ARG;
   if (total_rows < 0 || E < 0 || E > kMapThreads || K <= 0) return MI_ERR_SHAPE;
-  *bytes = tiled_moe_layout(total_rows, E, K, kMoeBM).total;
+  const TiledMoeLayout L = tiled_moe_layout(total_rows, E, K, kMoeBM);
+  *bytes = L.total;
+  // the re-tiled activations are addressed through a 32-bit buffer resource: beyond 2 GiB the tiled
+  // route does not apply and the caller stays on the streaming grouped kernel
+  if ((uint64_t)L.x_bytes >= (1ull << 31)) return MI_ERR_SHAPE;
   return MI_OK;
 }
 

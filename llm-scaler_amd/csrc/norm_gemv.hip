@@ -22,7 +22,9 @@ using namespace qlin;
 // pointer that hipGetSymbolAddress returns.  The loader zero-fills it and the kernel
 // leaves every counter at zero when it ends, so one call finds what the previous one
 // left: zeros.  Calls that overlap on one GPU (two streams) would share the counters
-// and race; calls on one stream are ordered by the stream.
+// and race; calls on one stream are ordered by the stream.  So one stream per GPU owns the
+// array: the first call after a set-up claims it for its stream, and a call on another
+// stream is refused with MI_ERR_BUSY until mi_static_scratch_setup releases the claim.
 constexpr int kStaticCounterWords = 512;                       // 2 KiB, the size the kernel indexes into
 static __device__ __align__(256) unsigned int scratch[kStaticCounterWords];
 
@@ -30,18 +32,20 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_static_mu;
 unsigned int* g_static_ptr[kMaxDevices];                       // per device, resolved once
+hipStream_t g_static_owner[kMaxDevices];                       // the stream that claimed the array
+bool g_static_owned[kMaxDevices];
 
-// MI_OK and *out = the current device's copy of `scratch`
-int static_counters(unsigned int** out) {
+// MI_OK and *out = the current device's copy of `scratch`; *dev_out = the device
+int static_counters_locked(unsigned int** out, int* dev_out) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
-  std::lock_guard<std::mutex> lock(g_static_mu);
   if (!g_static_ptr[dev]) {
     void* p = nullptr;
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
     g_static_ptr[dev] = static_cast<unsigned int*>(p);
   }
   *out = g_static_ptr[dev];
+  *dev_out = dev;
   return MI_OK;
 }
 
@@ -58,7 +62,15 @@ extern "C" {
 
 int mi_static_scratch_setup(void) {
   unsigned int* p = nullptr;
-  return static_counters(&p);
+  int dev = -1;
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  const int rc = static_counters_locked(&p, &dev);
+  if (rc != MI_OK) return rc;
+  // back to the state the loader left: all counters zero (a kernel that ended abnormally may have
+  // left some non-zero), nobody owns the array.  A blocking clear: not for use under capture.
+  if (hipMemset(p, 0, sizeof(unsigned int) * kStaticCounterWords) != hipSuccess) { (void)hipGetLastError(); return MI_ERR_LAUNCH; }
+  g_static_owned[dev] = false;
+  return MI_OK;
 }
 
 int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const void* norm_weight, void* normed_out,
@@ -66,8 +78,18 @@ int mi_norm_gemv_static(const void* x, void* residual, const void* gate, const v
                         const void* const* scale, void* const* out, const int* N, int K, int act_dtype,
                         void* stream) {
   unsigned int* counters = nullptr;
-  const int rc = static_counters(&counters);
-  if (rc != MI_OK) return rc;
+  {
+    int dev = -1;
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    const int rc = static_counters_locked(&counters, &dev);
+    if (rc != MI_OK) return rc;
+    if (!g_static_owned[dev]) {
+      g_static_owned[dev] = true;
+      g_static_owner[dev] = (hipStream_t)stream;
+    } else if (g_static_owner[dev] != (hipStream_t)stream) {
+      return MI_ERR_BUSY;                  // another stream's calls could overlap with this one
+    }
+  }
   return norm_gemv_run(x, residual, gate, norm_weight, normed_out, norm_len, eps, residual_scale, fmt, nmat, w, scale,
                        out, N, K, act_dtype, stream, counters);
 }

@@ -27,6 +27,7 @@ enum : int {
   MI_ERR_SHAPE = -2,      // shape or divisibility the kernels do not cover
   MI_ERR_LAUNCH = -3,     // hipGetLastError() after the launch
   MI_ERR_LIMIT = -4,      // size beyond the fixed capacity of a no-allocation entry point
+  MI_ERR_BUSY = -5,       // the static scratch is claimed by another stream
 };
 
 // ---- raw buffer loads -------------------------------------------------------

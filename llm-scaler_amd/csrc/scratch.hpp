@@ -6,8 +6,10 @@
 // that addresses baked into a captured graph stay valid
 // (V/csrc/xpu/esimd_kernel_moe.sycl:45-67, V/csrc/moe_batch/moe.sycl:1460-1498);
 // this is the same convention.  A buffer that has become too small is replaced by
-// a larger one and kept allocated until the process ends (work already queued on
-// the stream may still read it).  Growing calls hipMalloc, which is not allowed
+// a larger one and kept allocated until the process ends: work already queued on
+// the stream may still read it, and a graph captured earlier has its address baked
+// in, so no later point is safe for freeing it.  Sizes grow in powers of two, so
+// the replaced buffers of a stream add up to less than the one in use.  Growing calls hipMalloc, which is not allowed
 // while the stream is being captured: run a call of the same size once before
 // capturing, as graph users do anyway.  Calls on different streams never share a
 // buffer; calls on one stream are ordered by the stream.

@@ -85,6 +85,19 @@ def esimd_gemm_int4_pgrp_zp(input, weight, weight_scale, weight_zp, output):
     return _ops.esimd_gemm_int4_pgrp_zp(input, weight, weight_scale, weight_zp, output)
 
 
+def int4_gemm_w4a16(x, qweight, bias, scales, qzeros, group_size, g_idx=None):
+    """The GPTQ / AWQ / sym_int4 linear call of the patched vLLM
+    (vllm/patches/vllm_for_multi_arc.patch:5492-5500): qweight logical [K/8, N] int32, scales [K/128, N]
+    fp16, qzeros [K/128, N/8] int32 or one value; returns a new [M, N] tensor."""
+    return _ops.int4_gemm_w4a16(x, qweight, bias, scales, qzeros, group_size, g_idx)
+
+
+def w4a16_prepare(qweight, scales, qzeros, group_size, zero_bias=0):
+    """Load-time conversion of those operands into (weight [N, K/8], scale [N, K/128], zp [N, K/128]) for
+    esimd_gemm_int4_pgrp_zp / esimd_gemv_int4."""
+    return _ops.w4a16_prepare(qweight, scales, qzeros, group_size, zero_bias)
+
+
 def int4_dequant(weight, weight_scale, weight_zp, output):
     return _ops.int4_dequant(weight, weight_scale, weight_zp, output)
 

@@ -20,7 +20,8 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libmi355x_qlinear.so")
 MI_ERRORS = {-1: "invalid argument (null pointer or bad enum)",
              -2: "unsupported shape or divisibility",
              -3: "kernel launch failed",
-             -4: "size beyond the fixed capacity of this no-allocation entry point"}
+             -4: "size beyond the fixed capacity of this no-allocation entry point",
+             -5: "the static scratch is claimed by another stream on this GPU"}
 
 DT_F16, DT_BF16 = 0, 1
 _ACT_DT = {torch.float16: DT_F16, torch.bfloat16: DT_BF16}

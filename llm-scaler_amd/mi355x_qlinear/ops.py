@@ -944,6 +944,19 @@ def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, t
 _ACT_NONE, _ACT_SILU, _ACT_GELU_TANH = 0, 1, 2
 
 
+def _moe_tiled_workspace(w8a16, out16, total, E, K):
+    """Workspace bytes of the tiled (prefill) grouped GEMM when that route takes the launch, else None:
+    16-bit activations and output, whole 128-granules, at most 1024 experts averaging 96 rows or more,
+    and re-tiled activations below 2 GiB (the library's own limits, asked of the library so the two
+    cannot drift; past them the streaming grouped kernel runs)."""
+    if not (w8a16 and out16 and K % 128 == 0 and E <= 1024 and total >= 96 * E):
+        return None
+    need = ctypes.c_longlong(0)
+    if capi.lib().mi_moe_gemm_fp8_tiled_workspace(int(total), int(E), int(K), ctypes.byref(need)) != 0:
+        return None
+    return need.value
+
+
 def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse, who, *, per_expert=False,
               out_map=None, row_weight=None, row_map_div=1):
     """Grouped GEMM over expert-sorted rows.  fuse: False / True (SiLU) or one of _ACT_*.
@@ -984,16 +997,13 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
     if row_weight is not None:
         _chk(out.dtype != torch.float32 and row_weight.dtype == out.dtype and row_weight.is_contiguous() and
              row_weight.numel() >= total, f"{who}: row weights must share the output dtype, one per output row")
-    if a_scale is None and out.dtype != torch.float32 and K % 128 == 0 and E <= 1024 and total >= 96 * E:
+    need = _moe_tiled_workspace(a_scale is None, out.dtype != torch.float32, total, E, K)
+    if need is not None:
         # prefill: the tiled matrix-core GEMM, workspace from the caching allocator (graph-capturable)
-        need = ctypes.c_longlong(0)
-        rc = capi.lib().mi_moe_gemm_fp8_tiled_workspace(total, E, K, ctypes.byref(need))
-        if rc != 0:
-            raise RuntimeError(f"{who}: {capi.MI_ERRORS.get(rc, rc)}")
-        buf = torch.empty(need.value, dtype=torch.uint8, device=out.device)
+        buf = torch.empty(need, dtype=torch.uint8, device=out.device)
         capi.call("mi_moe_gemm_fp8_tiled_ws", out, capi.ptr(a), capi.ptr(row_map), int(row_map_div), capi.ptr(w),
                   capi.ptr(w_scale), per_expert, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map), capi.ptr(row_weight),
-                  a_rows, total, E, N, K, fuse, adt, capi.ptr(buf), need.value)
+                  a_rows, total, E, N, K, fuse, adt, capi.ptr(buf), need)
         return out
     capi.call("mi_moe_gemm_fp8_grouped", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), int(row_map_div),
               capi.ptr(w), capi.ptr(w_scale), per_expert, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map),
@@ -1848,6 +1858,77 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
     return out
 
 
+def w4a16_prepare(qweight, scales, qzeros, group_size, zero_bias=0):
+    """GPTQ / AWQ style operands -> (weight [N, K/8] int32, scale [N, K/128] fp16, zp [N, K/128] uint8),
+    the resident layout of esimd_gemm_int4_pgrp_zp / esimd_gemv_int4, converted on the device.
+    qweight: logical [K/8, N] int32, either contiguous or with strides (1, K/8) (then its bytes are
+    used as they are); scales [K/128, N] fp16; qzeros: [K/128, N/8] int32 packed along N, or a
+    one-element tensor holding the zero-point of every group (the symmetric case: 8)."""
+    who = "w4a16_prepare"
+    _chk(int(group_size) == 128, f"{who}: only group_size 128 is supported, got {group_size}")
+    _chk(qweight.dim() == 2 and qweight.dtype == torch.int32, f"{who}: qweight must be int32 [K/8, N]")
+    K8, N = qweight.shape
+    K = K8 * 8
+    _chk(K % 128 == 0, f"{who}: K={K} must be a multiple of 128")
+    G = K // 128
+    _chk(scales.dtype == torch.float16 and scales.is_contiguous() and tuple(scales.shape) == (G, N),
+         f"{who}: scales must be contiguous fp16 [K/128, N]")
+    scalar = qzeros.numel() == 1
+    _chk(qzeros.dtype == torch.int32 and qzeros.is_contiguous(), f"{who}: qzeros must be contiguous int32")
+    _chk(scalar or (N % 8 == 0 and tuple(qzeros.shape) == (G, N // 8)),
+         f"{who}: qzeros must be [K/128, N/8] int32 (N a multiple of 8) or hold one value")
+    dev = qweight.device
+    n_major = qweight.stride() == (1, K8) or N == 1
+    _chk(n_major or qweight.is_contiguous(), f"{who}: qweight must be contiguous or have strides (1, K/8)")
+    w_out = qweight.t() if n_major else torch.empty(N, K8, dtype=torch.int32, device=dev)
+    s_out = torch.empty(N, G, dtype=torch.float16, device=dev)
+    zp_out = torch.empty(N, G, dtype=torch.uint8, device=dev)
+    capi.call("mi_w4a16_kmajor_prepare", scales, None if n_major else capi.ptr(qweight), capi.ptr(scales), capi.ptr(qzeros),
+              1 if scalar else 0, int(zero_bias), None if n_major else capi.ptr(w_out), capi.ptr(s_out), capi.ptr(zp_out), N, K)
+    return w_out, s_out, zp_out
+
+
+def _w4a16_prepare_meta(qweight, scales, qzeros, group_size, zero_bias=0):
+    K8, N = qweight.shape
+    G = K8 * 8 // 128
+    return (qweight.new_empty(N, K8), scales.new_empty(N, G), scales.new_empty(N, G, dtype=torch.uint8))
+
+
+def int4_gemm_w4a16(x, qweight, bias, scales, qzeros, group_size, g_idx):
+    """The call the reference's GPTQ / AWQ / sym_int4 linears make
+    (vllm/patches/vllm_for_multi_arc.patch:5492-5500): out[M, N] = x @ ((q - z) * s) + bias, output
+    allocated here.  The operands are converted per call (the weight only when it is not already
+    N-major in memory); a loader that calls w4a16_prepare once and esimd_gemm_int4_pgrp_zp per
+    step skips that."""
+    who = "int4_gemm_w4a16"
+    _chk(g_idx is None, f"{who}: activation reordering (g_idx) is not supported")
+    _chk(x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous(),
+         f"{who}: x must be contiguous fp16 / bf16 [M, K]")
+    w, s, zp = w4a16_prepare(qweight, scales, qzeros, group_size)
+    M, N = x.shape[0], w.shape[0]
+    _chk(x.shape[1] == w.shape[1] * 8, f"{who}: x has K={x.shape[1]}, the weight K={w.shape[1] * 8}")
+    out = torch.empty(M, N, dtype=x.dtype, device=x.device)
+    _gemm_int4(x, w.contiguous() if not w.is_contiguous() else w, s, zp, out, who)
+    if bias is not None:
+        _chk(bias.dtype == x.dtype and bias.is_contiguous() and bias.numel() == N, f"{who}: bias must be [N] in x's dtype")
+        capi.call("mi_add_bias", out, capi.ptr(out), capi.ptr(bias), M, N, capi.act_dtype(x))
+    return out
+
+
+def _int4_gemm_w4a16_meta(x, qweight, bias, scales, qzeros, group_size, g_idx):
+    return x.new_empty(x.shape[0], qweight.shape[1])
+
+
+def register_xpu_c_alias():
+    """Also registers int4_gemm_w4a16 as torch.ops._xpu_C.int4_gemm_w4a16, the name the reference's
+    GPTQ / AWQ / sym_int4 linears call (vllm/patches/vllm_for_multi_arc.patch:5492).  Opt-in, because
+    `_xpu_C` is another package's namespace: call it only where that package is not installed."""
+    if "_xpu_C" in _DEFINED and "int4_gemm_w4a16" in _DEFINED["_xpu_C"]:
+        return
+    _define("_xpu_C", "int4_gemm_w4a16(Tensor x, Tensor qweight, Tensor? bias, Tensor scales, Tensor qzeros, "
+                      "int group_size, Tensor? g_idx) -> Tensor", int4_gemm_w4a16, _int4_gemm_w4a16_meta)
+
+
 def moe_forward_full_v2(*args):
     """The reference's variant for more than one token (V/csrc/moe_batch/moe.sycl:2337-2430): same
     arguments and result as moe_forward_full; one implementation serves both here."""
@@ -1901,6 +1982,10 @@ def register():
                     "Tensor output) -> Tensor", esimd_gemm_int4_pgrp, _ret(3))
         _define(ns, "esimd_gemm_int4_pgrp_zp(Tensor input, Tensor weight, Tensor weight_scale, Tensor weight_zp, "
                     "Tensor(a!) output) -> Tensor(a!)", esimd_gemm_int4_pgrp_zp, _ret(4))
+        _define(ns, "int4_gemm_w4a16(Tensor x, Tensor qweight, Tensor? bias, Tensor scales, Tensor qzeros, "
+                    "int group_size, Tensor? g_idx) -> Tensor", int4_gemm_w4a16, _int4_gemm_w4a16_meta)
+        _define(ns, "w4a16_prepare(Tensor qweight, Tensor scales, Tensor qzeros, int group_size, int zero_bias=0) "
+                    "-> (Tensor, Tensor, Tensor)", w4a16_prepare, _w4a16_prepare_meta)
         _define(ns, "esimd_gemm_fp8_pert(Tensor input, Tensor weight, Tensor weight_scale, "
                     "Tensor output) -> Tensor", esimd_gemm_fp8_pert, _ret(3))
         _define(ns, "esimd_gemm_fp8_blockscale(Tensor input, Tensor weight, Tensor weight_scale, "

@@ -23,6 +23,14 @@ Pinning status (see tests/test_oracle_*.py):
   * per-token-per-128 activation quantisation (cfg3) and the asymmetric int4
     zero-point layout have NO counterpart in the reference: parity unpinned in
     the reference, pinned here only by their closed forms.
+  * w4a16_kmajor_* (the operand layout of the third-party int4_gemm_w4a16 the
+    reference calls for GPTQ / AWQ weights, VP:5492-5500): PARITY UNPINNED in the
+    reference -- that op's source is not in the reference tree and no reference
+    test exercises it.  Restated from the published GPTQ packing (eight nibbles
+    per int32, lowest nibble first, along K for weights and along N for
+    zero-points) and pinned by the reference's statement that its [K/8, N]
+    tensor with strides (1, K/8) holds the same bytes as the ESIMD [N, K/2]
+    weight (VP:5516-5523), hand-placed nibbles and a round trip.
 """
 from __future__ import annotations
 
@@ -129,6 +137,54 @@ def int4_dequant(packed: torch.Tensor, scale: torch.Tensor, out_dtype=torch.floa
     z = z.repeat_interleave(group, dim=-1)
     s = scale.to(torch.float32).repeat_interleave(group, dim=-1)
     return _round_to((u - z) * s, out_dtype)
+
+
+def w4a16_kmajor_pack(u4: torch.Tensor, scale: torch.Tensor, zp: torch.Tensor):
+    """Stored nibbles u4 [N, K] (0..15), scale [N, K/128] fp16, zp [N, K/128] (0..15) -> the operands
+    of int4_gemm_w4a16 (VP:5492-5500): qweight [K/8, N] int32 with nibble z of word (i, n) = element
+    k = 8 i + z of column n; scales [K/128, N] fp16; qzeros [K/128, N/8] int32 with nibble c of word
+    (g, j) = zero-point of column n = 8 j + c in group g.  Parity unpinned in the reference (see the
+    module header)."""
+    N, K = u4.shape
+    a = u4.to(torch.int64).numpy().reshape(N, K // 8, 8)
+    words = np.zeros((N, K // 8), dtype=np.int64)
+    for z in range(8):
+        words |= a[:, :, z] << (4 * z)
+    qweight = torch.from_numpy(words.astype(np.uint32).view(np.int32).T.copy())
+    zz = zp.to(torch.int64).numpy().T.reshape(K // INT4_GROUP, N // 8, 8)
+    zw = np.zeros((K // INT4_GROUP, N // 8), dtype=np.int64)
+    for c in range(8):
+        zw |= zz[:, :, c] << (4 * c)
+    qzeros = torch.from_numpy(zw.astype(np.uint32).view(np.int32).copy())
+    return qweight, scale.t().contiguous(), qzeros
+
+
+def w4a16_kmajor_unpack(qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor, zero_bias: int = 0):
+    """Inverse of w4a16_kmajor_pack, element by element: (u4 [N, K] int32, scale [N, G] fp16,
+    zp [N, G] uint8).  A one-element qzeros is the zero-point of every group (the symmetric case)."""
+    K8, N = qweight.shape
+    G = scales.shape[0]
+    w = qweight.numpy().astype(np.int64) & 0xFFFFFFFF
+    u4 = np.zeros((N, K8 * 8), dtype=np.int32)
+    for i in range(K8):
+        for z in range(8):
+            u4[:, 8 * i + z] = (w[i, :] >> (4 * z)) & 0xF
+    if qzeros.numel() == 1:
+        zp = np.full((N, G), int(qzeros.reshape(-1)[0]), dtype=np.uint8)
+    else:
+        q = qzeros.numpy().astype(np.int64) & 0xFFFFFFFF
+        zp = np.zeros((N, G), dtype=np.uint8)
+        for n in range(N):
+            zp[n, :] = ((q[:, n // 8] >> (4 * (n % 8))) & 0xF) + zero_bias
+    return torch.from_numpy(u4), scales.t().contiguous(), torch.from_numpy(zp)
+
+
+def w4a16_kmajor_dequant(qweight, scales, qzeros, out_dtype=torch.float16, zero_bias: int = 0) -> torch.Tensor:
+    """Dense [N, K] weight of those operands: rne(f32(q - z) * f32(s)), the asymmetric form of int4_dequant."""
+    u4, s, zp = w4a16_kmajor_unpack(qweight, scales, qzeros, zero_bias)
+    z = zp.to(torch.float32).repeat_interleave(INT4_GROUP, dim=-1)
+    sf = s.to(torch.float32).repeat_interleave(INT4_GROUP, dim=-1)
+    return _round_to((u4.to(torch.float32) - z) * sf, out_dtype)
 
 
 # ----------------------------------------------------------------------------

@@ -48,6 +48,30 @@ def test_topk_ids_exact_weights_close(v, dev, T, E, K, dt):
     assert torch.equal(i2.cpu(), ri) and torch.equal(w2, tw)
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_topk_signed_zero_ties(v, dev, dt):
+    """+0 and -0 logits are equal to a float compare, so the lowest index wins among them
+    (V/csrc/xpu/esimd_kernels/moe_ops.h:77-104): a -0 at a lower index must beat a +0 further on."""
+    T, E, K = 4, 64, 4
+    logits = torch.full((T, E), -1.0).to(dt)
+    logits[0, 3], logits[0, 9], logits[0, 20], logits[0, 40], logits[0, 50] = -0.0, 0.0, -0.0, 0.0, 0.0
+    logits[1, :] = -0.0
+    logits[1, 7], logits[1, 30] = 0.0, 0.0
+    logits[2, 10], logits[2, 11] = 2.0, 2.0
+    logits[2, 60], logits[2, 61], logits[2, 62] = 0.0, -0.0, 0.0
+    logits[2, 5] = -0.0
+    logits[3, :] = 0.0
+    logits[3, 0] = -0.0
+    tw = torch.empty(T, K, dtype=dt, device=dev)
+    ti = torch.empty(T, K, dtype=torch.int32, device=dev)
+    v.esimd_moe_topk(logits.to(dev), tw, ti, T)
+    rw, ri = O.moe_topk(logits, K, out_dtype=dt)
+    assert ri.tolist() == [[3, 9, 20, 40], [0, 1, 2, 3], [10, 11, 5, 60], [0, 1, 2, 3]]
+    assert torch.equal(ti.cpu(), ri)
+    ulp = 2.0 ** -8 if dt == torch.bfloat16 else 2.0 ** -11
+    assert ((tw.cpu().float() - rw.float()).abs() <= 2 * ulp * rw.float().abs() + 1e-7).all()
+
+
 def test_topk_v2_matches_topk(v, dev):
     T, E, K = 9, 128, 8
     logits = torch.randn(T, E, generator=torch.Generator().manual_seed(5)).half().to(dev)
@@ -371,7 +395,7 @@ def _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq):
     return dict(tw=tw, ti=ti, inter=inter, iq=iq, isc=isc, y=y, out=out)
 
 
-def _check_forward(v, dev, T, E, K, H, I, aq, seed):
+def _check_forward(v, dev, T, E, K, H, I, aq, seed, free_bar=None):
     x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I, seed=seed)
     g = _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq)
     rtw, rti = O.moe_topk(logits, K)
@@ -410,6 +434,11 @@ def _check_forward(v, dev, T, E, K, H, I, aq, seed):
           f"(1e-3 floor) {O.max_rel_err_abs_floor(g['out'].cpu(), ref):.3e}; free-running max-rel (mean floor) "
           f"{O.max_rel_err(out.cpu(), free):.3e}, (1e-3 floor) {O.max_rel_err_abs_floor(out.cpu(), free):.3e}, "
           f"mean-rel {mean_rel:.3e}, cos {cos:.6f}", flush=True)
+    if free_bar is not None:
+        # the free-running maximum is discontinuous in the intermediate's quantisation grid, so it cannot
+        # meet the staged bar; it is held to twice the recorded figure instead, which still fails on a
+        # regression of the forward as a whole
+        assert O.max_rel_err(out.cpu(), free) < free_bar
     return out
 
 
@@ -449,7 +478,8 @@ def test_moe_forward_w8a16_prefill(v, dev, T, E, K, H, I, dt):
 def test_cfg3_moe_forward(v, dev):
     # the stage-wise 1e-2 bars (mean floor) are inside _check_forward; it also prints the staged and the
     # free-running maxima under both denominators (free-running, this shape: 4e-2 with the mean floor)
-    out = _check_forward(v, dev, 512, 128, 8, 2048, 768, True, seed=1237)
+    # and asserts the free-running maximum at twice the recorded 4.1e-2
+    out = _check_forward(v, dev, 512, 128, 8, 2048, 768, True, seed=1237, free_bar=8e-2)
     assert torch.isfinite(out.float()).all()
 
 

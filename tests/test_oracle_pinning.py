@@ -458,3 +458,40 @@ def test_moe_forward_full_kmajor_against_block_oracle():
                               ss13.expand(2 * I // 128, H // 128).contiguous(), w2.transpose(1, 2).contiguous(),
                               blk(s2, H, I), sw2, ss2.expand(H // 128, I // 128).contiguous(), gate, k)
     assert torch.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+# ---- K-major W4A16 operands (the reference's int4_gemm_w4a16 call) ----
+def test_w4a16_kmajor_matches_the_esimd_bytes():
+    """vllm/patches/vllm_for_multi_arc.patch:5516-5523: the [K/8, N] tensor with strides (1, K/8)
+    is the N-major ESIMD weight, byte for byte; so the transposed K-major words must equal the
+    int32 view of int4_pack's bytes."""
+    g = torch.Generator().manual_seed(3)
+    N, K = 24, 256
+    q = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int32)
+    packed = O.int4_pack(q)
+    scale = (torch.rand(N, K // 128, generator=g) * 0.01 + 0.005).half()
+    zp = torch.randint(0, 16, (N, K // 128), generator=g, dtype=torch.int32).to(torch.uint8)
+    qw, sc, qz = O.w4a16_kmajor_pack(q + 8, scale, zp)
+    assert qw.shape == (K // 8, N) and sc.shape == (K // 128, N) and qz.shape == (K // 128, N // 8)
+    assert torch.equal(qw.t().contiguous(), packed.view(torch.int32))
+    u4, s2, z2 = O.w4a16_kmajor_unpack(qw, sc, qz)
+    assert torch.equal(u4, q + 8) and torch.equal(s2, scale) and torch.equal(z2, zp)
+    assert torch.equal(O.w4a16_kmajor_dequant(qw, sc, qz), O.int4_dequant(packed, scale, zp=zp))
+    # symmetric form: one value for every group
+    assert torch.equal(O.w4a16_kmajor_dequant(qw, sc, torch.tensor([8], dtype=torch.int32)), O.int4_dequant(packed, scale))
+
+
+def test_w4a16_kmajor_hand_placed_nibbles():
+    N, K = 16, 128
+    u4 = torch.zeros(N, K, dtype=torch.int32)
+    u4[5, 13] = 0xF                              # k = 13 = 8 * 1 + 5: word (1, 5), nibble 5
+    u4[0, 7] = 0x9                               # the top nibble of word (0, 0): sign bit set
+    zp = torch.zeros(N, 1, dtype=torch.uint8)
+    zp[11, 0] = 9                                # column 11 = 8 * 1 + 3: word (0, 1), nibble 3
+    qw, sc, qz = O.w4a16_kmajor_pack(u4, torch.ones(N, 1).half(), zp)
+    assert qw[1, 5].item() == 0x00F00000 and qw[0, 0].item() == 0x90000000 - (1 << 32)
+    assert int((qw != 0).sum()) == 2
+    assert qz[0, 1].item() == 9 << 12 and int((qz != 0).sum()) == 1
+    w = O.w4a16_kmajor_dequant(qw, sc, qz, out_dtype=torch.float32)
+    assert w[5, 13].item() == 15.0 and w[0, 7].item() == 9.0 and w[11, 0].item() == -9.0 and w[11, 127].item() == -9.0
+    assert O.w4a16_kmajor_unpack(qw, sc, qz, zero_bias=1)[2][11, 0].item() == 10

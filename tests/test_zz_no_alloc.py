@@ -77,3 +77,29 @@ def test_static_entry_refuses_rows_beyond_its_limit(dev):
     assert torch.isfinite(want[0][0].float()).all()
     with pytest.raises(RuntimeError, match="fixed capacity"):
         _run("mi_norm_gemv_static", dev, *case)
+
+
+def test_static_entry_refuses_a_second_stream(dev):
+    """All calls on one GPU share the static counters, so calls that overlap on two streams would
+    race.  The first call after a set-up claims the array for its stream; a call on another stream
+    is refused (nothing launched, outputs untouched) until the set-up releases the claim."""
+    from mi355x_qlinear import capi
+    assert capi.lib().mi_static_scratch_setup() == 0
+    case = _case(1024, [136], 5, dev)
+    want = _run("mi_norm_gemv_scaled", dev, *case)
+    side = torch.cuda.Stream()
+    got = _run("mi_norm_gemv_static", dev, *case)              # claims the array for the current stream
+    assert torch.equal(_bits(got[0][0]), _bits(want[0][0]))
+    with torch.cuda.stream(side):
+        with pytest.raises(RuntimeError, match="claimed by another stream"):
+            _run("mi_norm_gemv_static", dev, *case)
+    again = _run("mi_norm_gemv_static", dev, *case)            # the owner keeps working
+    assert torch.equal(_bits(again[0][0]), _bits(want[0][0]))
+    torch.cuda.synchronize()
+    assert capi.lib().mi_static_scratch_setup() == 0           # hand-over: nothing in flight
+    with torch.cuda.stream(side):
+        moved = _run("mi_norm_gemv_static", dev, *case)
+    assert torch.equal(_bits(moved[0][0]), _bits(want[0][0]))
+    assert torch.equal(_bits(moved[1]), _bits(want[1])) and torch.equal(_bits(moved[2]), _bits(want[2]))
+    torch.cuda.synchronize()
+    assert capi.lib().mi_static_scratch_setup() == 0           # leave it unclaimed for whoever comes next
