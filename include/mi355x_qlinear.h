@@ -288,6 +288,13 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
 int mi_moe_sort_quant(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
                       int32_t* sorted_token, int32_t* max_count, int T, int K, int E, const void* x,
                       void* q, float* scale, long long rows, int H, int act_dtype, void* stream);
+/* mi_moe_topk (without the expert factors and the shared gate) and mi_act_quant_fp8 of the token
+ * activations x [T, H] in one launch: the routing reads the logits, the quantisation reads x, and
+ * neither waits for the other, while the expert sort needs every token's selection and follows
+ * alone (mi_moe_sort).  Same results as the two separate calls, bit for bit.  No counterpart in the
+ * reference: its MoE path keeps 16-bit activations. */
+int mi_moe_topk_quant(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
+                      const void* x, void* q, float* scale, int H, int act_dtype, void* stream);
 int mi_act_quant_fp8(const void* x, void* q, float* scale, long long rows, int K, int act_dtype,
                      void* stream);
 int mi_moe_silu_mul(const void* in, void* out, int n_gate_up, int n_half, int rows, int act_dtype,

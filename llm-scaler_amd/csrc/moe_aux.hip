@@ -44,16 +44,16 @@ __device__ __forceinline__ uint32_t f16_order(uint32_t b) {
 }
 __device__ __forceinline__ uint32_t f16_unorder(uint32_t u) { return (u & 0x8000u) ? (u & 0x7FFFu) : (~u & 0xFFFFu); }
 template <class Act, int SLOTS>
-__global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,
-                                                       typename Act::elem* __restrict__ top_w,
-                                                       int32_t* __restrict__ top_ids, int T, int E,
-                                                       int K, int renorm,
-                                                       const float* __restrict__ expert_scale,
-                                                       const typename Act::v8* __restrict__ gate_x,
-                                                       const typename Act::v8* __restrict__ gate_w,
-                                                       float* __restrict__ gate_out, int H8) {
+__device__ __forceinline__ void moe_topk_body(const typename Act::elem* __restrict__ logits,
+                                              typename Act::elem* __restrict__ top_w,
+                                              int32_t* __restrict__ top_ids, int T, int E,
+                                              int K, int renorm,
+                                              const float* __restrict__ expert_scale,
+                                              const typename Act::v8* __restrict__ gate_x,
+                                              const typename Act::v8* __restrict__ gate_w,
+                                              float* __restrict__ gate_out, int H8, int block) {
   const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int t = block * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   // optional second result of the same wavefront: gate_out[t] = sigmoid(gate_x[t, :] . gate_w[:]) (the
   // shared expert's gate of the fused decode ops); its loads are in flight while the selection runs
@@ -113,6 +113,19 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem*
     gate_acc = wave_sum(gate_acc);
     if (lane == 0) gate_out[t] = 1.0f / (1.0f + __expf(-gate_acc));
   }
+}
+
+template <class Act, int SLOTS>
+__global__ __launch_bounds__(256) void moe_topk_kernel(const typename Act::elem* __restrict__ logits,
+                                                       typename Act::elem* __restrict__ top_w,
+                                                       int32_t* __restrict__ top_ids, int T, int E,
+                                                       int K, int renorm,
+                                                       const float* __restrict__ expert_scale,
+                                                       const typename Act::v8* __restrict__ gate_x,
+                                                       const typename Act::v8* __restrict__ gate_w,
+                                                       float* __restrict__ gate_out, int H8) {
+  moe_topk_body<Act, SLOTS>(logits, top_w, top_ids, T, E, K, renorm, expert_scale, gate_x, gate_w, gate_out, H8,
+                            (int)blockIdx.x);
 }
 
 // ---------------------------------------------------------------- sort
@@ -418,6 +431,66 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
   else moe_sort_body(top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, sm);
 }
 
+// The same stable sort with one workgroup per EXPERT, for the serving sizes (a few thousand pairs):
+// workgroup e reads all P ids itself (P * 4 bytes from L2) and needs nothing from the others -- the
+// number of pairs of lower experts is its first position, and a pair's rank among the expert's own is
+// the number of earlier pairs with the same id.  Thread t owns the contiguous pairs
+// [t * chunk, (t + 1) * chunk), chunk <= 32, so ranks follow from an exclusive scan over the threads
+// plus a popcount inside the thread's own mask.  One dependent round trip to memory instead of the
+// single workgroup's clear / mark / scan / place sequence.  Ids outside [0, E) are held into the
+// range like in the other paths; every pair gets a position of its own.
+constexpr int kSortExpertThreads = 256;
+constexpr int kSortExpertMaxPairs = 32 * kSortExpertThreads;
+
+__global__ __launch_bounds__(kSortExpertThreads) void moe_sort_expert_kernel(
+    const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
+    int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
+    int P, int K, int E, int chunk) {
+  __shared__ int32_t wave_lt[4], wave_eq[4];
+  const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int q0 = tid * chunk;
+  uint32_t mask = 0;
+  int lt = 0;
+  for (int b = 0; b < chunk; ++b) {
+    const int q = q0 + b;
+    if (q < P) {
+      const int id = sort_expert(top_ids, q, E);
+      lt += id < e;
+      mask |= (uint32_t)(id == e) << b;
+    }
+  }
+  const int eq = __popc(mask);
+  // wave-inclusive scan of eq, wave sum of lt
+  int incl = eq, lsum = lt;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += o;
+    lsum += __shfl_xor(lsum, off, 64);
+  }
+  if (lane == 63) { wave_eq[wave] = incl; wave_lt[wave] = lsum; }
+  __syncthreads();
+  int start = 0, before = incl - eq;                  // pairs of this expert in earlier threads
+  for (int w = 0; w < 4; ++w) {
+    start += wave_lt[w];
+    if (w < wave) before += wave_eq[w];
+  }
+  if (tid == 0) {
+    expert_start[e] = start;
+    if (e == E - 1) expert_start[E] = start + wave_eq[0] + wave_eq[1] + wave_eq[2] + wave_eq[3];
+  }
+  int pos = start + before;
+  while (mask) {
+    const int b = __ffs(mask) - 1;
+    mask &= mask - 1;
+    const int q = q0 + b;
+    sorted_pairs[pos] = q;
+    inv[q] = pos;
+    if (sorted_token) sorted_token[pos] = q / K;
+    ++pos;
+  }
+}
+
 // ---------------------------------------------------------------- activation quant
 // Per row, per 128-wide group: s = max|x| / 448 (clamped at 1e-12), q = e4m3(x / s).
 // 16 lanes own one group (8 elements each); the group maximum is a DPP butterfly
@@ -463,6 +536,23 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const typename Act::v8* 
                                                         u32x2* __restrict__ q, float* __restrict__ s,
                                                         size_t groups16) {   // 16-lane groups in total
   act_quant_body<Act>(x, q, s, groups16, (size_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+// The routing (top-k) and the quantisation of the token activations read different inputs and
+// neither waits for the other: one launch, the first `ntopk` workgroups select, the others quantise
+// 256 lanes' worth each.  The expert sort, which needs every token's selection, follows alone.
+template <class Act, int SLOTS>
+__global__ __launch_bounds__(256) void moe_topk_quant_kernel(const typename Act::elem* __restrict__ logits,
+                                                             typename Act::elem* __restrict__ top_w,
+                                                             int32_t* __restrict__ top_ids, int T, int E, int K,
+                                                             int renorm, const typename Act::v8* __restrict__ x,
+                                                             u32x2* __restrict__ q, float* __restrict__ s,
+                                                             size_t groups16, int ntopk) {
+  if ((int)blockIdx.x < ntopk)
+    moe_topk_body<Act, SLOTS>(logits, top_w, top_ids, T, E, K, renorm, nullptr, nullptr, nullptr, nullptr, 0,
+                              (int)blockIdx.x);
+  else
+    act_quant_body<Act>(x, q, s, groups16, (size_t)(blockIdx.x - ntopk) * 256 + threadIdx.x);
 }
 
 // The expert sort (latency-bound) and the quantisation of the token activations (independent of
@@ -538,42 +628,73 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const u32x4* __restri
 // final[t] = sum_j w_j * y[pos(t, j)]; weights either per sorted position
 // (by_pos = 1, the reference's scattered_weights) or per pair (top_w).
 // With a shared expert: + gate[t] * shared[t], added in fp32 before the one rounding.
+// A thread owns 4 columns of fp32 rows (one 16-byte load per row, so a wavefront reads 1 KiB in a
+// row) or 8 columns of 16-bit rows.  The positions, weights and row pieces of up to 8 routes are
+// requested before any is used: walked one route at a time, every route is a dependent pair of
+// round trips (position, then row), and eight of those in sequence were the whole run time.
 template <class Act, bool Y32>
 __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ yv,
                                                       const int32_t* __restrict__ inv,
                                                       const typename Act::elem* __restrict__ w,
-                                                      typename Act::v8* __restrict__ out, int H8, int topk,
+                                                      void* __restrict__ outv, int HC, int topk,
                                                       int T, int by_pos,
-                                                      const typename Act::v8* __restrict__ shared,
+                                                      const void* __restrict__ sharedv,
                                                       const float* __restrict__ gate) {
+  using Elem = typename Act::elem;
+  constexpr int CW = Y32 ? 4 : 8;                     // columns per thread
+  constexpr int kBatch = 8;                           // routes in flight
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (size_t)T * H8) return;
-  const int t = (int)(i / H8), c = (int)(i % H8);
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int j = 0; j < topk; ++j) {
-    const int pos = inv ? inv[(size_t)t * topk + j] : t * topk + j;   // no map: y is in pair order
-    const float wj = w ? Act::to_f32(w[by_pos ? pos : t * topk + j]) : 1.0f;   // no weights: plain sum
+  if (i >= (size_t)T * HC) return;
+  const int t = (int)(i / HC), c = (int)(i % HC);
+  float acc[CW];
+#pragma unroll
+  for (int e = 0; e < CW; ++e) acc[e] = 0.f;
+  for (int j0 = 0; j0 < topk; j0 += kBatch) {
+    int pos[kBatch];
+    float wj[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int j = j0 + b < topk ? j0 + b : topk - 1;
+      pos[b] = inv ? inv[(size_t)t * topk + j] : t * topk + j;       // no map: y is in pair order
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int j = j0 + b < topk ? j0 + b : topk - 1;
+      wj[b] = w ? Act::to_f32(w[by_pos ? pos[b] : t * topk + j]) : 1.0f;   // no weights: plain sum
+    }
     if constexpr (Y32) {
-      const f32x4* y = (const f32x4*)yv;
-      const f32x4 a = y[((size_t)pos * H8 + c) * 2], b = y[((size_t)pos * H8 + c) * 2 + 1];
+      f32x4 v[kBatch];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { acc[e] += wj * a[e]; acc[4 + e] += wj * b[e]; }
+      for (int b = 0; b < kBatch; ++b) v[b] = ((const f32x4*)yv)[(size_t)pos[b] * HC + c];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+        if (j0 + b < topk) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] += wj[b] * v[b][e];
+        }
     } else {
-      const typename Act::v8 v = ((const typename Act::v8*)yv)[(size_t)pos * H8 + c];
+      typename Act::v8 v[kBatch];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += wj * Act::to_f32(v[e]);
+      for (int b = 0; b < kBatch; ++b) v[b] = ((const typename Act::v8*)yv)[(size_t)pos[b] * HC + c];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+        if (j0 + b < topk) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] += wj[b] * Act::to_f32(v[b][e]);
+        }
     }
   }
-  if (shared) {
-    const typename Act::v8 sv = shared[i];
+  if (sharedv) {
     const float gt = gate ? gate[t] : 1.0f;
+    const Elem* sv = (const Elem*)sharedv + i * CW;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += gt * Act::to_f32(sv[e]);
+    for (int e = 0; e < CW; ++e) acc[e] += gt * Act::to_f32(sv[e]);
   }
-  typename Act::v8 o;
+  Elem o[CW];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = Act::from_f32(acc[e]);
-  out[i] = o;
+  for (int e = 0; e < CW; ++e) o[e] = Act::from_f32(acc[e]);
+  if constexpr (Y32) *reinterpret_cast<uint64_t*>((Elem*)outv + i * CW) = *reinterpret_cast<const uint64_t*>(o);
+  else *reinterpret_cast<u32x4*>((Elem*)outv + i * CW) = *reinterpret_cast<const u32x4*>(o);
 }
 
 // gate[t] = sigmoid(x[t, :] . gw[:]) in fp32, one wavefront per token.
@@ -717,11 +838,47 @@ int mi_moe_topk(const void* logits, void* top_w, int32_t* top_ids, int T, int E,
   return launch_status();
 }
 
+int mi_moe_topk_quant(const void* logits, void* top_w, int32_t* top_ids, int T, int E, int K, int renorm,
+                      const void* x, void* q, float* scale, int H, int act_dtype, void* stream) {
+  if (!logits || !top_w || !top_ids || !x || !q || !scale) return MI_ERR_ARG;
+  if (T < 0 || E < 1 || E > 64 * kTopkSlots || K < 1 || K > 64 || K > E) return MI_ERR_SHAPE;
+  if (H <= 0 || (H % 128)) return MI_ERR_SHAPE;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (!T) return MI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t groups16 = (size_t)T * (H / 128);
+  const int ntopk = (T + 3) / 4;
+  const dim3 grid((unsigned)ntopk + (unsigned)((groups16 * 16 + 255) / 256)), block(256);
+#define QLIN_TOPKQ(SLOTS)                                                                                   \
+  do {                                                                                                      \
+    if (act_dtype == DT_F16)                                                                                \
+      hipLaunchKernelGGL((moe_topk_quant_kernel<ActF16, SLOTS>), grid, block, 0, st, (const _Float16*)logits, \
+                         (_Float16*)top_w, top_ids, T, E, K, renorm, (const f16x8*)x, (u32x2*)q, scale, groups16, ntopk); \
+    else                                                                                                    \
+      hipLaunchKernelGGL((moe_topk_quant_kernel<ActBF16, SLOTS>), grid, block, 0, st, (const __bf16*)logits,  \
+                         (__bf16*)top_w, top_ids, T, E, K, renorm, (const bf16x8*)x, (u32x2*)q, scale, groups16, ntopk); \
+  } while (0)
+  if (E <= 128) QLIN_TOPKQ(2);
+  else if (E <= 256) QLIN_TOPKQ(4);
+  else if (E <= 512) QLIN_TOPKQ(8);
+  else QLIN_TOPKQ(16);
+#undef QLIN_TOPKQ
+  return launch_status();
+}
+
 int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_start, int32_t* inv,
                 int32_t* sorted_token, int32_t* max_count, int T, int K, int E, void* stream) {
   if (!expert_start) return MI_ERR_ARG;
   if (T < 0 || K < 1 || E < 1 || E > 1024) return MI_ERR_SHAPE;
   if (T > 0 && (!top_ids || !sorted_pairs || !inv)) return MI_ERR_ARG;   // T == 0 only fills expert_start
+  const long P = (long)T * K;
+  if (!max_count && P > 0 && P <= kSortExpertMaxPairs && (long)P * E <= (4l << 20)) {
+    // one workgroup per expert; each reads all ids (at most 16 MiB from L2 over the whole launch)
+    const int chunk = (int)((P + kSortExpertThreads - 1) / kSortExpertThreads);
+    hipLaunchKernelGGL(moe_sort_expert_kernel, dim3((unsigned)E), dim3(kSortExpertThreads), 0, (hipStream_t)stream,
+                       top_ids, sorted_pairs, expert_start, inv, sorted_token, (int)P, K, E, chunk);
+    return launch_status();
+  }
   const int S = sort_wide_span(T, E);
   hipLaunchKernelGGL(moe_sort_kernel, dim3(S ? (unsigned)((T + S - 1) / S) : 1u), dim3(kSortThreads), 0,
                      (hipStream_t)stream, top_ids, sorted_pairs, expert_start, inv, sorted_token, max_count, T, K, E, S);
@@ -818,14 +975,15 @@ int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
   if (!T) return MI_OK;
   hipStream_t st = (hipStream_t)stream;
-  const dim3 grid = grid1d((size_t)T * (H / 8));
-#define QLIN_COMBINE(ACT, Y32, WT, OT)                                                                   \
-  hipLaunchKernelGGL((combine_kernel<ACT, Y32>), grid, dim3(256), 0, st, y, inv, (const WT*)w, (OT*)out, \
-                     H / 8, topk, T, weights_by_position, (const OT*)shared, gate)
+  const int HC = y_f32 ? H / 4 : H / 8;               // column groups per row: 4 columns of fp32, 8 of 16 bit
+  const dim3 grid = grid1d((size_t)T * HC);
+#define QLIN_COMBINE(ACT, Y32, WT)                                                                         \
+  hipLaunchKernelGGL((combine_kernel<ACT, Y32>), grid, dim3(256), 0, st, y, inv, (const WT*)w, out, HC, topk, T, \
+                     weights_by_position, shared, gate)
   if (act_dtype == DT_F16) {
-    if (y_f32) QLIN_COMBINE(ActF16, true, _Float16, f16x8); else QLIN_COMBINE(ActF16, false, _Float16, f16x8);
+    if (y_f32) QLIN_COMBINE(ActF16, true, _Float16); else QLIN_COMBINE(ActF16, false, _Float16);
   } else {
-    if (y_f32) QLIN_COMBINE(ActBF16, true, __bf16, bf16x8); else QLIN_COMBINE(ActBF16, false, __bf16, bf16x8);
+    if (y_f32) QLIN_COMBINE(ActBF16, true, __bf16); else QLIN_COMBINE(ActBF16, false, __bf16);
   }
 #undef QLIN_COMBINE
   return launch_status();

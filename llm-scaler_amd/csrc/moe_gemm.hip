@@ -79,7 +79,7 @@ constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of
 // launched: with 4 the kernel is bound by its LDS traffic and gained nothing for experts with
 // hundreds of rows, which run on the tiled matrix-core GEMM instead (moe_gemm_tiled.hip).
 template <class Act, bool A8, bool SILU, int RT, int D, bool PE, int MT = 1>
-__global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, const float* __restrict__ w_scale,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2))) void moe_gemm_kernel(const MoeGemmArgs p, const float* __restrict__ w_scale,
                                                         const int32_t* __restrict__ expert_start) {
   static_assert(RT == 2 || RT == 4 || RT == 8, "two, four or eight weight tiles");
   using Elem = typename Act::elem;
@@ -120,19 +120,19 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
   auto tile_col = [&](int t) { return SILU ? (t >> 1) * 16 : t * 16; };
   auto tile_hi = [&](int t) { return SILU ? (t & 1) * half : 0; };
 
-  // cooperative weight staging slots of this thread
-  uint32_t wvoff[WL];
-  int wcol[WL], wch[WL];
-  unsigned char* wlds[WL];
-#pragma unroll
-  for (int i = 0; i < WL; ++i) {
-    const int c = tid + 256 * i;
-    const int row = c >> 3, t = row >> 4, r = row & 15, ch = c & 7;
-    wcol[i] = col0 + tile_col(t) + r;
-    wch[i] = ch * 16;
-    wvoff[i] = (uint32_t)(tile_hi(t) + wcol[i]) * (uint32_t)K + (uint32_t)ch * 16u;
-    wlds[i] = smem + row * kWPitch + ch * 16;
-  }
+  // Cooperative weight staging: thread `tid` fetches chunk (tid & 7) of row (tid >> 3) + 32 i of the
+  // tile group's RT * 16 rows, i < WL.  32 rows further on is two weight tiles further on, which is
+  // the same step in memory for every i (32 rows of the matrix, or 16 rows of the gate and of the up
+  // half alike), so one offset register serves all of a thread's chunks and the rest is uniform.
+  // Columns at or past `limit` are masked per load (the uniform part of the address travels in the
+  // scalar offset, which the buffer bound does not see).
+  const int wrow = tid >> 3, wt = wrow >> 4;
+  const int wcol = col0 + tile_col(wt) + (wrow & 15);  // output column of chunk 0 in tile group 0
+  const int wch = (tid & 7) * 16;                     // first k of the chunk inside the granule
+  const uint32_t wvoff = (uint32_t)(tile_hi(wt) + col0 + tile_col(wt) + (wrow & 15)) * (uint32_t)K + (uint32_t)wch;
+  const uint32_t wistep = (SILU ? 16u : 32u) * (uint32_t)K;
+  unsigned char* const wlds = smem + wrow * kWPitch + wch;
+  constexpr int kWldsStep = 32 * kWPitch;
   unsigned char* al = smem + 2 * kWBuf + wave * MT * 16 * APitch;
 
   const uint8_t* wexp = (const uint8_t*)p.w + (size_t)e * N * K;
@@ -195,11 +195,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       const uint32_t wso = (uint32_t)tg * tg_stride + (uint32_t)gi * 128u;
       // quantised activations come in whole 128-groups: no partial granule there
       const int kext = (!A8 && gi == G - 1) ? ktail : 128;   // uniform
+      const uint32_t wv = wvoff | dead | ((uint32_t)(wch >= kext) << 31);
+      const int wc = wcol + tg * kCols;
 #pragma unroll
-      for (int i = 0; i < WL; ++i) {
-        const bool ok = wcol[i] + tg * kCols < limit && wch[i] < kext;
-        r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i] | dead | ((uint32_t)(!ok) << 31), wso, 2);
-      }
+      for (int i = 0; i < WL; ++i)
+        r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wv | ((uint32_t)(wc + i * 16 * (SILU ? 1 : 2) >= limit) << 31),
+                                                       wso + (uint32_t)i * wistep, 2);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -212,131 +213,165 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
       }
     };
 
-    Regs r[D];
+    // destination row and routing weight of this lane's activation row: fetched once per pass, ahead
+    // of the weight stream (a load issued inside the loop would wait for every prefetch before it:
+    // the counter of outstanding loads retires in order)
+    int dst_row[MT];
+    float dst_w[MT];
 #pragma unroll
-    for (int s = 0; s < D; ++s) {                     // G is a multiple of D
-      load_granule(r[s], 0, s);
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mc + wrow0 + mt * 16 + j;
+      int dst = m < cnt ? (p.out_map ? p.out_map[r0 + m] : r0 + m) : -1;
+      if ((unsigned)dst >= (unsigned)p.total_rows) dst = -1;    // a mapped row outside the output is dropped
+      dst_row[mt] = dst;
+      dst_w[mt] = (p.row_weight && dst >= 0) ? Act::to_f32(((const Elem*)p.row_weight)[dst]) : 1.0f;
+    }
+    // the same for the row-contiguous store layout of the epilogue: lane l stores 16 bytes of rows
+    // (l >> 3) and (l >> 3) + 8 of the wavefront's tile
+    int dst_line[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int m = mc + wrow0 + mt * 16 + (lane >> 3) + 8 * h;
+        int dst = m < cnt ? (p.out_map ? p.out_map[r0 + m] : r0 + m) : -1;
+        if ((unsigned)dst >= (unsigned)p.total_rows) dst = -1;
+        dst_line[mt][h] = dst;
+      }
+
+    // The (tile group, granule) steps of this workgroup form one linear sequence; D of them are in
+    // flight in a register ring.  Steps past the end (the sequence is walked in multiples of D) load
+    // nothing and compute nothing.
+    const int total = ntg * G;
+    Regs r[D];
+    int ptg = 0, pgi = 0;                             // position of the next step to fetch
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+      load_granule(r[s], ptg, pgi);
+      if (++pgi == G) { pgi = 0; ++ptg; }
       // keep the stages' loads in issue order: the counter of outstanding loads
       // retires in order, and the loop waits for "all but the younger stages"
       __builtin_amdgcn_sched_barrier(0);
     }
 
     f32x4 acc[MT][RT];
-    int odd_par = 0;
-    for (int tg = 0; tg < ntg; ++tg) {
+    int tg = 0, gi = 0, par = 0;
+    for (int q0 = 0; q0 < total; q0 += D) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int s = 0; s < D; ++s) {
+        const bool live = q0 + s < total;             // uniform
+        if (gi == 0) {
 #pragma unroll
-        for (int t = 0; t < RT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      int nb[RT];
+          for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int t = 0; t < RT; ++t) nb[t] = min((tile_hi(t) + col0 + tg * kCols + tile_col(t)) >> 7, Nb - 1);
-
-      for (int gi0 = 0; gi0 < G; gi0 += D) {
+            for (int t = 0; t < RT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        // the shared weight tile alternates between two buffers
+        unsigned char* wbuf = smem + par * kWBuf;
+        // granule -> LDS
 #pragma unroll
-        for (int s = 0; s < D; ++s) {
-          const int gi = gi0 + s;
-          // the shared weight tile alternates between two buffers per iteration
-          const int par = (D % 2 == 0) ? (s & 1) : odd_par;
-          if constexpr (D % 2) odd_par ^= 1;
-          unsigned char* wbuf = smem + par * kWBuf;
-          // granule -> LDS
-#pragma unroll
-          for (int i = 0; i < WL; ++i) *reinterpret_cast<u32x4*>(wlds[i] + par * kWBuf) = r[s].w[i];
+        for (int i = 0; i < WL; ++i) *reinterpret_cast<u32x4*>(wlds + par * kWBuf + i * kWldsStep) = r[s].w[i];
+        // (a wavefront without rows in this pass stages nothing: the LDS write port is the scarcest
+        // resource of the step)
+        if (wrow0 < rows_here) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int i = 0; i < NAI; ++i) *reinterpret_cast<u32x4*>(alds[mt][i]) = r[s].a[mt][i];
-          // The activation scale is taken out of the ring slot before the slot is reloaded
-          // below.  Left to the scheduler, the multiply sinks under the reload, old and new
-          // value overlap, and the loop latch gets a register copy of the NEW value, i.e. a
-          // wait for every load in flight on each turn.
-          float xs_now[MT];
+        }
+        // The activation scale is taken out of the ring slot before the slot is reloaded
+        // below.  Left to the scheduler, the multiply sinks under the reload, old and new
+        // value overlap, and the loop latch gets a register copy of the NEW value, i.e. a
+        // wait for every load in flight on each turn.
+        float xs_now[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          xs_now[mt] = A8 ? r[s].xs[mt] : 1.0f;
+          asm volatile("" : "+v"(xs_now[mt]));
+        }
+        float wsv[RT];
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+          const int row_t = tile_hi(t) + col0 + tg * kCols + tile_col(t);
+          wsv[t] = PE ? (row_t >= half ? ws_second : ws_expert)
+                      : wsc[(size_t)min(row_t >> 7, Nb - 1) * Kb + (live ? gi : 0)];
+        }
+        // prefetch D steps ahead, across the tile-group boundary
+        load_granule(r[s], ptg, pgi);
+        if (++pgi == G) { pgi = 0; ++ptg; }
+        __syncthreads();
+        if (live && wrow0 < rows_here) {             // wave-uniform: this wavefront has rows in the pass
+          // One weight tile at a time, its fragments read while the previous tile is multiplied: all
+          // eight tiles' fragments and partial sums live at once cost 90 registers, which is a
+          // workgroup per CU less and with it a third of the bytes in flight.
+          auto read_tile = [&](int t, u32x4 (&f)[2]) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+              f[i] = *reinterpret_cast<const u32x4*>(wbuf + (t * 16 + j) * kWPitch + g * 32 + i * 16);
+          };
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            xs_now[mt] = A8 ? r[s].xs[mt] : 1.0f;
-            asm volatile("" : "+v"(xs_now[mt]));
-          }
-          float wsv[RT];
+            if (MT > 1 && wrow0 + mt * 16 >= rows_here) continue;    // wave-uniform
+            const unsigned char* am = al + (mt * 16 + j) * APitch;
+            u32x4 wf[2][2];
+            read_tile(0, wf[0]);
+            if constexpr (A8) {
+              const u32x4 x0 = *reinterpret_cast<const u32x4*>(am + g * 32);
+              const u32x4 x1 = *reinterpret_cast<const u32x4*>(am + g * 32 + 16);
+              const long xa = (long)(((uint64_t)x0[1] << 32) | x0[0]);
+              const long xb = (long)(((uint64_t)x0[3] << 32) | x0[2]);
+              const long xc = (long)(((uint64_t)x1[1] << 32) | x1[0]);
+              const long xd = (long)(((uint64_t)x1[3] << 32) | x1[2]);
+              // the scaled sum of tile t - 1 follows the matrix instructions of tile t, so that only two
+              // tiles' partial sums are live
+              f32x4 tt[2];
 #pragma unroll
-          for (int t = 0; t < RT; ++t)
-            wsv[t] = PE ? (tile_hi(t) + col0 + tg * kCols + tile_col(t) >= half ? ws_second : ws_expert)
-                        : wsc[(size_t)nb[t] * Kb + gi];
-          // prefetch D granules ahead, across the tile-group boundary
-          {
-            int ngi = gi + D, ntgi = tg;
-            if (ngi >= G) { ngi -= G; ntgi += 1; }
-            load_granule(r[s], ntgi, ngi);
-          }
-          __syncthreads();
-          if (wrow0 < rows_here) {                    // wave-uniform: this wavefront has rows in the pass
-            u32x4 wf[RT][2];
-#pragma unroll
-            for (int t = 0; t < RT; ++t)
-#pragma unroll
-              for (int i = 0; i < 2; ++i)
-                wf[t][i] = *reinterpret_cast<const u32x4*>(wbuf + (t * 16 + j) * kWPitch + g * 32 + i * 16);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-              if (MT > 1 && wrow0 + mt * 16 >= rows_here) continue;    // wave-uniform
-              const unsigned char* am = al + (mt * 16 + j) * APitch;
-              if constexpr (A8) {
-                const u32x4 x0 = *reinterpret_cast<const u32x4*>(am + g * 32);
-                const u32x4 x1 = *reinterpret_cast<const u32x4*>(am + g * 32 + 16);
-                const long xa = (long)(((uint64_t)x0[1] << 32) | x0[0]);
-                const long xb = (long)(((uint64_t)x0[3] << 32) | x0[2]);
-                const long xc = (long)(((uint64_t)x1[1] << 32) | x1[0]);
-                const long xd = (long)(((uint64_t)x1[3] << 32) | x1[2]);
-#pragma unroll
-                for (int t = 0; t < RT; ++t) {
-                  const long w0 = (long)(((uint64_t)wf[t][0][1] << 32) | wf[t][0][0]);
-                  const long w1 = (long)(((uint64_t)wf[t][0][3] << 32) | wf[t][0][2]);
-                  const long w2 = (long)(((uint64_t)wf[t][1][1] << 32) | wf[t][1][0]);
-                  const long w3 = (long)(((uint64_t)wf[t][1][3] << 32) | wf[t][1][2]);
-                  f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, xa, tt, 0, 0, 0);
-                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, xb, tt, 0, 0, 0);
-                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, xc, tt, 0, 0, 0);
-                  tt = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, xd, tt, 0, 0, 0);
-                  acc[mt][t] += tt * (xs_now[mt] * wsv[t]);
-                }
-              } else {
-                V8 xf[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) xf[i] = *reinterpret_cast<const V8*>(am + g * 64 + i * 16);
-#pragma unroll
-                for (int t = 0; t < RT; ++t) {
-                  f32x4 tt = f32x4{0.f, 0.f, 0.f, 0.f};
-                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][0][0], wf[t][0][1]), xf[0], tt);
-                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][0][2], wf[t][0][3]), xf[1], tt);
-                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][1][0], wf[t][1][1]), xf[2], tt);
-                  tt = Act::mfma(fp8x8_to_act<Act>(wf[t][1][2], wf[t][1][3]), xf[3], tt);
-                  acc[mt][t] += tt * wsv[t];
-                }
+              for (int t = 0; t < RT; ++t) {
+                if (t + 1 < RT) read_tile(t + 1, wf[(t + 1) & 1]);
+                const u32x4(&f)[2] = wf[t & 1];
+                const long w0 = (long)(((uint64_t)f[0][1] << 32) | f[0][0]);
+                const long w1 = (long)(((uint64_t)f[0][3] << 32) | f[0][2]);
+                const long w2 = (long)(((uint64_t)f[1][1] << 32) | f[1][0]);
+                const long w3 = (long)(((uint64_t)f[1][3] << 32) | f[1][2]);
+                f32x4 c = f32x4{0.f, 0.f, 0.f, 0.f};
+                c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, xa, c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, xb, c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2, xc, c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w3, xd, c, 0, 0, 0);
+                tt[t & 1] = c;
+                if (t > 0) acc[mt][t - 1] += tt[(t - 1) & 1] * (xs_now[mt] * wsv[t - 1]);
+                __builtin_amdgcn_sched_barrier(0);
               }
+              acc[mt][RT - 1] += tt[(RT - 1) & 1] * (xs_now[mt] * wsv[RT - 1]);
+            } else {
+              V8 xf[4];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) xf[i] = *reinterpret_cast<const V8*>(am + g * 64 + i * 16);
+              f32x4 tt[2];
+#pragma unroll
+              for (int t = 0; t < RT; ++t) {
+                if (t + 1 < RT) read_tile(t + 1, wf[(t + 1) & 1]);
+                const u32x4(&f)[2] = wf[t & 1];
+                f32x4 c = f32x4{0.f, 0.f, 0.f, 0.f};
+                c = Act::mfma(fp8x8_to_act<Act>(f[0][0], f[0][1]), xf[0], c);
+                c = Act::mfma(fp8x8_to_act<Act>(f[0][2], f[0][3]), xf[1], c);
+                c = Act::mfma(fp8x8_to_act<Act>(f[1][0], f[1][1]), xf[2], c);
+                c = Act::mfma(fp8x8_to_act<Act>(f[1][2], f[1][3]), xf[3], c);
+                tt[t & 1] = c;
+                if (t > 0) acc[mt][t - 1] += tt[(t - 1) & 1] * wsv[t - 1];
+                __builtin_amdgcn_sched_barrier(0);
+              }
+              acc[mt][RT - 1] += tt[(RT - 1) & 1] * wsv[RT - 1];
             }
           }
         }
-      }
 
-      // ---- epilogue of this tile group: lane holds row 16 w + j, weight rows 4 g + v ----
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-      const int m = mc + wrow0 + mt * 16 + j;
-      const int dst = m < cnt ? (p.out_map ? p.out_map[r0 + m] : r0 + m) : -1;
-      if ((unsigned)dst < (unsigned)p.total_rows) {    // a mapped row outside the output is dropped
-        Elem* out = (Elem*)p.out;
-        float* out32 = (float*)p.out;
-        const size_t orow = (size_t)dst * p.n_out;
-        const float rw = p.row_weight ? Act::to_f32(((const Elem*)p.row_weight)[dst]) : 1.0f;
-        constexpr int NO = SILU ? RT / 2 : RT;
-#pragma unroll
-        for (int o = 0; o < NO; ++o) {
-          const int t = SILU ? 2 * o : o;
-          const int n = col0 + tg * kCols + tile_col(t) + g * 4;   // first of 4 output columns
-          float v4[4];
-#pragma unroll
-          for (int v = 0; v < 4; ++v) {
+        // ---- epilogue of a tile group: lane holds row 16 w + j, weight rows 4 g + v ----
+        if (live && gi == G - 1 && wrow0 < rows_here) {
+          constexpr int NO = SILU ? RT / 2 : RT;      // 16-column output tiles of the tile group
+          const int ncol0 = col0 + tg * kCols;        // first output column of the tile group
+          auto value = [&](int mt, int o, int v, float rw) -> float {
+            const int t = SILU ? 2 * o : o;
             if constexpr (SILU) {
               const float gate = acc[mt][t][v], up = acc[mt][t + 1][v];
               if (p.gelu) {
@@ -344,30 +379,112 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const MoeGemmArgs p, cons
                 float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
                 two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
                 const float ex = __expf(two_z);
-                v4[v] = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up * rw;
-              } else {
-                v4[v] = gate / (1.0f + __expf(-gate)) * up * rw;
+                return 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up * rw;
               }
+              return gate / (1.0f + __expf(-gate)) * up * rw;
             } else {
-              v4[v] = acc[mt][t][v] * rw;
+              return acc[mt][t][v] * rw;
             }
-          }
-          if (n + 3 < limit && (p.n_out & 3) == 0) {
-            if (p.out_f32) {
-              *reinterpret_cast<f32x4*>(out32 + orow + n) = f32x4{v4[0], v4[1], v4[2], v4[3]};
-            } else {
-              Elem o4[4] = {Act::from_f32(v4[0]), Act::from_f32(v4[1]), Act::from_f32(v4[2]), Act::from_f32(v4[3])};
-              *reinterpret_cast<uint64_t*>(out + orow + n) = *reinterpret_cast<const uint64_t*>(o4);
+          };
+          // Whole 128-byte lines: the cost of a store is per cache line it touches, not per byte, and in
+          // accumulator layout an instruction puts 32 or 64 bytes into each of 16 rows.  The tile goes
+          // through the wavefront's own activation tile in LDS (free until the next step stages into
+          // it; a wavefront's LDS operations complete in order, so no barrier) and leaves as 8 rows x
+          // 128 contiguous bytes per instruction.  Needs the tile group inside the matrix and rows
+          // that start on 16 bytes; anything else takes the element-wise path below.
+          const uint32_t esz = p.out_f32 ? 4u : 2u;
+          const bool lines = ncol0 + kCols <= limit && (((uint32_t)p.n_out * esz) & 15u) == 0;
+          if (lines) {
+            constexpr int kOPitch = 128 + 16;
+            static_assert(kOPitch <= APitch, "the output tile is staged in the activation tile");
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              if (MT > 1 && wrow0 + mt * 16 >= rows_here) continue;    // wave-uniform
+              unsigned char* ol = al + mt * 16 * APitch;
+              const float rw = dst_w[mt];
+              if (p.out_f32) {
+                constexpr int TPR = 2;                 // tiles per 128-byte row piece
+#pragma unroll
+                for (int rd = 0; rd < NO / TPR; ++rd) {
+#pragma unroll
+                  for (int ot = 0; ot < TPR; ++ot) {
+                    const int o = rd * TPR + ot;
+                    *reinterpret_cast<f32x4*>(ol + j * kOPitch + (ot * 16 + g * 4) * 4) =
+                        f32x4{value(mt, o, 0, rw), value(mt, o, 1, rw), value(mt, o, 2, rw), value(mt, o, 3, rw)};
+                  }
+#pragma unroll
+                  for (int h = 0; h < 2; ++h) {
+                    const u32x4 d = *reinterpret_cast<const u32x4*>(ol + ((lane >> 3) + 8 * h) * kOPitch + (lane & 7) * 16);
+                    const int dst = dst_line[mt][h];
+                    if (dst >= 0) {
+                      u32x4* q = reinterpret_cast<u32x4*>((unsigned char*)p.out + ((size_t)dst * p.n_out + ncol0 + rd * 32) * 4 +
+                                                (lane & 7) * 16);
+                      *q = d;
+                    }
+                  }
+                }
+              } else {
+                constexpr int TPR = NO < 4 ? NO : 4;
+#pragma unroll
+                for (int rd = 0; rd < NO / TPR; ++rd) {
+#pragma unroll
+                  for (int ot = 0; ot < TPR; ++ot) {
+                    const int o = rd * TPR + ot;
+                    Elem o4[4] = {Act::from_f32(value(mt, o, 0, rw)), Act::from_f32(value(mt, o, 1, rw)),
+                                  Act::from_f32(value(mt, o, 2, rw)), Act::from_f32(value(mt, o, 3, rw))};
+                    *reinterpret_cast<uint64_t*>(ol + j * kOPitch + (ot * 16 + g * 4) * 2) = *reinterpret_cast<const uint64_t*>(o4);
+                  }
+                  constexpr int kChunks = TPR * 2;     // 16-byte chunks per row piece (TPR * 16 columns * 2 bytes)
+#pragma unroll
+                  for (int h = 0; h < 2; ++h) {
+                    const u32x4 d = *reinterpret_cast<const u32x4*>(ol + ((lane >> 3) + 8 * h) * kOPitch + (lane & 7) * 16);
+                    const int dst = dst_line[mt][h];
+                    if (dst >= 0 && (lane & 7) < kChunks) {
+                      u32x4* q = reinterpret_cast<u32x4*>((unsigned char*)p.out + ((size_t)dst * p.n_out + ncol0 + rd * TPR * 16) * 2 +
+                                                (lane & 7) * 16);
+                      *q = d;
+                    }
+                  }
+                }
+              }
             }
           } else {
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-              if (n + v < limit) {
-                if (p.out_f32) out32[orow + n + v] = v4[v]; else out[orow + n + v] = Act::from_f32(v4[v]);
+          for (int mt = 0; mt < MT; ++mt) {
+            const int dst = dst_row[mt];
+            if (dst >= 0) {
+              Elem* out = (Elem*)p.out;
+              float* out32 = (float*)p.out;
+              const size_t orow = (size_t)dst * p.n_out;
+              const float rw = dst_w[mt];
+#pragma unroll
+              for (int o = 0; o < NO; ++o) {
+                const int t = SILU ? 2 * o : o;
+                const int n = ncol0 + tile_col(t) + g * 4;   // first of 4 output columns
+                float v4[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) v4[v] = value(mt, o, v, rw);
+                if (n + 3 < limit && (p.n_out & 3) == 0) {
+                  if (p.out_f32) {
+                    *reinterpret_cast<f32x4*>(out32 + orow + n) = f32x4{v4[0], v4[1], v4[2], v4[3]};
+                  } else {
+                    Elem o4[4] = {Act::from_f32(v4[0]), Act::from_f32(v4[1]), Act::from_f32(v4[2]), Act::from_f32(v4[3])};
+                    *reinterpret_cast<uint64_t*>(out + orow + n) = *reinterpret_cast<const uint64_t*>(o4);
+                  }
+                } else {
+#pragma unroll
+                  for (int v = 0; v < 4; ++v)
+                    if (n + v < limit) {
+                      if (p.out_f32) out32[orow + n + v] = v4[v]; else out[orow + n + v] = Act::from_f32(v4[v]);
+                    }
+                }
               }
+            }
+          }
           }
         }
-      }
+        par ^= 1;
+        if (++gi == G) { gi = 0; ++tg; }
       }
     }
     __syncthreads();                                  // LDS is rewritten by the next pass
@@ -417,7 +534,9 @@ static int dispatch_moe2(const MoeGemmArgs& p, hipStream_t st) {
   const int rt = wgs_with(8) >= 1024 ? 8 : (wgs_with(4) >= 1024 ? 4 : 2);
   // short K: walk two tile groups per workgroup so the prefetch pipeline stays filled
   const int tpw = (G < 16 && wgs_with(rt) >= 2048) ? 2 : 1;
-  const bool d2 = (G % 2) == 0;                       // two granules in flight need an even count
+  // two granules in flight per thread (more do not pay: the register ring then costs a resident
+  // workgroup); a single granule has nothing to prefetch
+  const bool d2 = G >= 2;
   if (rt == 8) return d2 ? launch_moe<Act, A8, SILU, 8, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 8, 1>(p, tpw, st);
   if (rt == 4) return d2 ? launch_moe<Act, A8, SILU, 4, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 4, 1>(p, tpw, st);
   return d2 ? launch_moe<Act, A8, SILU, 2, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 2, 1>(p, tpw, st);

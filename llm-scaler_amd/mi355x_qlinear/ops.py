@@ -1068,7 +1068,15 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
     dev = x.device
     top_w = torch.empty(T, k, dtype=x.dtype, device=dev)
     top_ids = torch.empty(T, k, dtype=torch.int32, device=dev)
-    esimd_moe_topk(logits, top_w, top_ids, T)
+    if act_quant:
+        # the routing and the quantisation of x do not depend on each other: one launch
+        _chk(E <= 1024 and 0 < k <= min(E, 64), f"{who}: top_k={k} of {E} experts is not supported")
+        xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
+        xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)
+        capi.call("mi_moe_topk_quant", logits, capi.ptr(logits), capi.ptr(top_w), capi.ptr(top_ids), T, E, k, 1,
+                  capi.ptr(x), capi.ptr(xq), capi.ptr(xs), H, capi.act_dtype(x))
+    else:
+        esimd_moe_topk(logits, top_w, top_ids, T)
     sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
     start = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(P, dtype=torch.int32, device=dev)
@@ -1078,15 +1086,7 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
     # tiled grouped GEMM takes over, which writes the activation type
     prefill = (not act_quant) and P >= 96 * E
     y = torch.empty(P, H, dtype=x.dtype if prefill else torch.float32, device=dev)
-    if act_quant:
-        xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
-        xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)
-        # the expert sort and the quantisation of x do not depend on each other: one launch
-        capi.call("mi_moe_sort_quant", top_ids, capi.ptr(top_ids), capi.ptr(sorted_pairs), capi.ptr(start),
-                  capi.ptr(inv), capi.ptr(sorted_token), None, T, k, E, capi.ptr(x), capi.ptr(xq), capi.ptr(xs),
-                  T, H, capi.act_dtype(x))
-    else:
-        moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
+    moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
     if act_quant:
         moe_gemm_fp8_block(xq, xs, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
         iq = torch.empty(P, I, dtype=torch.uint8, device=dev)
