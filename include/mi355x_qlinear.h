@@ -267,7 +267,8 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
  *   scattered_w[pos] = top_w[sorted_pairs[pos]]   (esimd_moe_scatter, moe_ops.h:522-569).
  * mi_moe_combine: out[t] = sum_j w * y[inv[t*topk + j]], weights indexed by sorted
  *   position (weights_by_position = 1, esimd_moe_gather, moe_ops.h:627-676) or by
- *   pair; y is in the activation dtype, or fp32 when y_f32 = 1.  w may be null: the rows are
+ *   pair; y is in the activation dtype (y_f32 = 0), fp32 (1) or fp16 beside any activation
+ *   dtype (2).  w may be null: the rows are
  *   summed unweighted (moe_accumulate, V/csrc/moe_batch/moe.sycl:1177-1230).
  *   inv may be null: y is then already in pair order (row t*topk + j), as
  *   moe_prefill_accumulate_forward_fp8 takes it
@@ -436,7 +437,8 @@ int mi_gemm_q4k_tiled_ws(const void* x, const void* ql, const void* scale, const
  * a_scale != NULL: a is e4m3 with per-row per-128 scales [a_rows, K/128]; native
  *   fp8 MFMA.  fuse_silu_mul: weight rows [0, N/2) are gate, [N/2, N) up; out is
  *   [total_rows, N/2] = silu(gate) * up.  Both have no reference counterpart.
- * out is in the activation dtype (act_dtype), or fp32 when out_f32 = 1. */
+ * out is in the activation dtype (out_f32 = 0), fp32 (1), or fp16 whatever the activation dtype (2:
+ * values beyond the fp16 range saturate at +-65504). */
 int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* row_map, const void* w,
                           const float* w_scale, const int32_t* expert_start, void* out, int a_rows,
                           int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,

@@ -2,6 +2,8 @@
 // permutation, dynamic activation quantisation, SiLU*mul, row scatter and the
 // weighted top-k combine.  All are small, HBM- or latency-bound integer / byte /
 // elementwise kernels; none of them is reshaped into a GEMM.
+#include <type_traits>
+
 #include "qlinear_common.hpp"
 #include "../../include/mi355x_qlinear.h"
 
@@ -632,7 +634,7 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const u32x4* __restri
 // row) or 8 columns of 16-bit rows.  The positions, weights and row pieces of up to 8 routes are
 // requested before any is used: walked one route at a time, every route is a dependent pair of
 // round trips (position, then row), and eight of those in sequence were the whole run time.
-template <class Act, bool Y32>
+template <class Act, int YK>                        // rows of y: 0 activation type, 1 fp32, 2 fp16
 __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ yv,
                                                       const int32_t* __restrict__ inv,
                                                       const typename Act::elem* __restrict__ w,
@@ -641,6 +643,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
                                                       const void* __restrict__ sharedv,
                                                       const float* __restrict__ gate) {
   using Elem = typename Act::elem;
+  constexpr bool Y32 = YK == 1;
+  using YAct = typename std::conditional<YK == 2, ActF16, Act>::type;   // element type of 16-bit rows
   constexpr int CW = Y32 ? 4 : 8;                     // columns per thread
   constexpr int kBatch = 8;                           // routes in flight
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -673,14 +677,14 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
           for (int e = 0; e < 4; ++e) acc[e] += wj[b] * v[b][e];
         }
     } else {
-      typename Act::v8 v[kBatch];
+      typename YAct::v8 v[kBatch];
 #pragma unroll
-      for (int b = 0; b < kBatch; ++b) v[b] = ((const typename Act::v8*)yv)[(size_t)pos[b] * HC + c];
+      for (int b = 0; b < kBatch; ++b) v[b] = ((const typename YAct::v8*)yv)[(size_t)pos[b] * HC + c];
 #pragma unroll
       for (int b = 0; b < kBatch; ++b)
         if (j0 + b < topk) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] += wj[b] * Act::to_f32(v[b][e]);
+          for (int e = 0; e < 8; ++e) acc[e] += wj[b] * YAct::to_f32(v[b][e]);
         }
     }
   }
@@ -975,15 +979,18 @@ int mi_moe_combine_shared(const void* y, const int32_t* inv, const void* w, void
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
   if (!T) return MI_OK;
   hipStream_t st = (hipStream_t)stream;
-  const int HC = y_f32 ? H / 4 : H / 8;               // column groups per row: 4 columns of fp32, 8 of 16 bit
+  if (y_f32 < 0 || y_f32 > 2) return MI_ERR_ARG;
+  const int HC = y_f32 == 1 ? H / 4 : H / 8;          // column groups per row: 4 columns of fp32, 8 of 16 bit
   const dim3 grid = grid1d((size_t)T * HC);
-#define QLIN_COMBINE(ACT, Y32, WT)                                                                         \
-  hipLaunchKernelGGL((combine_kernel<ACT, Y32>), grid, dim3(256), 0, st, y, inv, (const WT*)w, out, HC, topk, T, \
+#define QLIN_COMBINE(ACT, YK, WT)                                                                          \
+  hipLaunchKernelGGL((combine_kernel<ACT, YK>), grid, dim3(256), 0, st, y, inv, (const WT*)w, out, HC, topk, T, \
                      weights_by_position, shared, gate)
   if (act_dtype == DT_F16) {
-    if (y_f32) QLIN_COMBINE(ActF16, true, _Float16); else QLIN_COMBINE(ActF16, false, _Float16);
+    if (y_f32 == 1) QLIN_COMBINE(ActF16, 1, _Float16); else QLIN_COMBINE(ActF16, 0, _Float16);
   } else {
-    if (y_f32) QLIN_COMBINE(ActBF16, true, __bf16); else QLIN_COMBINE(ActBF16, false, __bf16);
+    if (y_f32 == 1) QLIN_COMBINE(ActBF16, 1, __bf16);
+    else if (y_f32 == 2) QLIN_COMBINE(ActBF16, 2, __bf16);
+    else QLIN_COMBINE(ActBF16, 0, __bf16);
   }
 #undef QLIN_COMBINE
   return launch_status();

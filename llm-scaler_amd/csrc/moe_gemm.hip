@@ -37,7 +37,7 @@ struct MoeGemmArgs {
   const void* w;              // [E, N, K] e4m3
   const float* w_scale;       // [E, ceil(N/128), ceil(K/128)], or [E]
   const int32_t* start;       // [E+1]
-  void* out;                  // [total_rows, N_out], activation dtype or fp32 (out_f32)
+  void* out;                  // [total_rows, N_out]: activation dtype (out_f32 = 0), fp32 (1) or fp16 (2)
   const int32_t* out_map;     // optional: sorted position -> row of `out`
   const void* row_weight;     // optional, activation dtype: factor per row of `out`
   int out_f32;
@@ -370,6 +370,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
         if (live && gi == G - 1 && wrow0 < rows_here) {
           constexpr int NO = SILU ? RT / 2 : RT;      // 16-column output tiles of the tile group
           const int ncol0 = col0 + tg * kCols;        // first output column of the tile group
+          // four results as 16-bit words: the activation type, or fp16 whatever the activation type
+          // (out_f32 = 2; held to the fp16 range, so an overflow is a large number and not an infinity)
+          auto to_f16_sat = [](float f) -> _Float16 { return (_Float16)fminf(fmaxf(f, -65504.0f), 65504.0f); };
+          auto pack4 = [&](float a0, float a1, float a2, float a3) -> uint64_t {
+            if (p.out_f32 == 2) {
+              _Float16 h4[4] = {to_f16_sat(a0), to_f16_sat(a1), to_f16_sat(a2), to_f16_sat(a3)};
+              return *reinterpret_cast<const uint64_t*>(h4);
+            }
+            Elem o4[4] = {Act::from_f32(a0), Act::from_f32(a1), Act::from_f32(a2), Act::from_f32(a3)};
+            return *reinterpret_cast<const uint64_t*>(o4);
+          };
           auto value = [&](int mt, int o, int v, float rw) -> float {
             const int t = SILU ? 2 * o : o;
             if constexpr (SILU) {
@@ -392,7 +403,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
           // it; a wavefront's LDS operations complete in order, so no barrier) and leaves as 8 rows x
           // 128 contiguous bytes per instruction.  Needs the tile group inside the matrix and rows
           // that start on 16 bytes; anything else takes the element-wise path below.
-          const uint32_t esz = p.out_f32 ? 4u : 2u;
+          const uint32_t esz = p.out_f32 == 1 ? 4u : 2u;
           const bool lines = ncol0 + kCols <= limit && (((uint32_t)p.n_out * esz) & 15u) == 0;
           if (lines) {
             constexpr int kOPitch = 128 + 16;
@@ -402,7 +413,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
               if (MT > 1 && wrow0 + mt * 16 >= rows_here) continue;    // wave-uniform
               unsigned char* ol = al + mt * 16 * APitch;
               const float rw = dst_w[mt];
-              if (p.out_f32) {
+              if (p.out_f32 == 1) {
                 constexpr int TPR = 2;                 // tiles per 128-byte row piece
 #pragma unroll
                 for (int rd = 0; rd < NO / TPR; ++rd) {
@@ -430,9 +441,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
 #pragma unroll
                   for (int ot = 0; ot < TPR; ++ot) {
                     const int o = rd * TPR + ot;
-                    Elem o4[4] = {Act::from_f32(value(mt, o, 0, rw)), Act::from_f32(value(mt, o, 1, rw)),
-                                  Act::from_f32(value(mt, o, 2, rw)), Act::from_f32(value(mt, o, 3, rw))};
-                    *reinterpret_cast<uint64_t*>(ol + j * kOPitch + (ot * 16 + g * 4) * 2) = *reinterpret_cast<const uint64_t*>(o4);
+                    *reinterpret_cast<uint64_t*>(ol + j * kOPitch + (ot * 16 + g * 4) * 2) =
+                        pack4(value(mt, o, 0, rw), value(mt, o, 1, rw), value(mt, o, 2, rw), value(mt, o, 3, rw));
                   }
                   constexpr int kChunks = TPR * 2;     // 16-byte chunks per row piece (TPR * 16 columns * 2 bytes)
 #pragma unroll
@@ -465,17 +475,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) v4[v] = value(mt, o, v, rw);
                 if (n + 3 < limit && (p.n_out & 3) == 0) {
-                  if (p.out_f32) {
+                  if (p.out_f32 == 1) {
                     *reinterpret_cast<f32x4*>(out32 + orow + n) = f32x4{v4[0], v4[1], v4[2], v4[3]};
                   } else {
-                    Elem o4[4] = {Act::from_f32(v4[0]), Act::from_f32(v4[1]), Act::from_f32(v4[2]), Act::from_f32(v4[3])};
-                    *reinterpret_cast<uint64_t*>(out + orow + n) = *reinterpret_cast<const uint64_t*>(o4);
+                    *reinterpret_cast<uint64_t*>(out + orow + n) = pack4(v4[0], v4[1], v4[2], v4[3]);
                   }
                 } else {
 #pragma unroll
                   for (int v = 0; v < 4; ++v)
                     if (n + v < limit) {
-                      if (p.out_f32) out32[orow + n + v] = v4[v]; else out[orow + n + v] = Act::from_f32(v4[v]);
+                      if (p.out_f32 == 1) out32[orow + n + v] = v4[v];
+                      else if (p.out_f32 == 2) ((_Float16*)p.out)[orow + n + v] = to_f16_sat(v4[v]);
+                      else out[orow + n + v] = Act::from_f32(v4[v]);
                     }
                 }
               }
@@ -559,7 +570,7 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
                             int N, int K, int fuse_act, int act_dtype, int out_f32, void* stream) {
   if (!a || !w || !w_scale || !expert_start || !out) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (fuse_act < 0 || fuse_act > 2) return MI_ERR_ARG;
+  if (fuse_act < 0 || fuse_act > 2 || out_f32 < 0 || out_f32 > 2) return MI_ERR_ARG;
   if (E < 0 || N <= 0 || K <= 0 || (K % 16) || a_rows < 0 || total_rows < 0) return MI_ERR_SHAPE;
   if (a_scale && (K % 128)) return MI_ERR_SHAPE;      // quantised activations carry whole 128-groups
   if (fuse_act && (N % 2)) return MI_ERR_SHAPE;
@@ -571,7 +582,7 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
     return MI_ERR_SHAPE;
   if (!E || !total_rows) return MI_OK;
   // prefill (experts averaging 96 rows or more, 16-bit activations and output): the tiled matrix-core GEMM
-  if (!a_scale && !out_f32 && (K % 128) == 0 && E <= 1024 && (long)total_rows >= 96L * E) {
+  if (!a_scale && out_f32 == 0 && (K % 128) == 0 && E <= 1024 && (long)total_rows >= 96L * E) {
     long long bytes = 0;
     // MI_ERR_SHAPE here means the re-tiled activations would pass 2 GiB: the streaming kernel below,
     // which only bounds a_rows * K, takes such a launch

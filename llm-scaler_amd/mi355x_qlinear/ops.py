@@ -944,6 +944,14 @@ def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, t
 _ACT_NONE, _ACT_SILU, _ACT_GELU_TANH = 0, 1, 2
 
 
+def _out_kind(out, adt):
+    """The library's code for the element type of expert outputs: 0 the activation type, 1 fp32,
+    2 fp16 beside bf16 activations (three more mantissa bits than bf16 at half the bytes of fp32)."""
+    if out.dtype == torch.float32:
+        return 1
+    return 2 if (out.dtype == torch.float16 and adt == capi.DT_BF16) else 0
+
+
 def _moe_tiled_workspace(w8a16, out16, total, E, K):
     """Workspace bytes of the tiled (prefill) grouped GEMM when that route takes the launch, else None:
     16-bit activations and output, whole 128-granules, at most 1024 experts averaging 96 rows or more,
@@ -989,7 +997,7 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
     a_rows = a.numel() // K
     if a_scale is None:
         adt = capi.act_dtype(a)
-        _chk(out.dtype in (a.dtype, torch.float32), f"{who}: output must be fp32 or share the activation dtype")
+        _chk(out.dtype in (a.dtype, torch.float32, torch.float16), f"{who}: output must be fp32, fp16 or share the activation dtype")
     else:
         adt = capi.act_dtype(out) if out.dtype != torch.float32 else capi.DT_BF16
     if out_map is not None:
@@ -997,7 +1005,7 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
     if row_weight is not None:
         _chk(out.dtype != torch.float32 and row_weight.dtype == out.dtype and row_weight.is_contiguous() and
              row_weight.numel() >= total, f"{who}: row weights must share the output dtype, one per output row")
-    need = _moe_tiled_workspace(a_scale is None, out.dtype != torch.float32, total, E, K)
+    need = _moe_tiled_workspace(a_scale is None, _out_kind(out, adt) == 0, total, E, K)
     if need is not None:
         # prefill: the tiled matrix-core GEMM, workspace from the caching allocator (graph-capturable)
         buf = torch.empty(need, dtype=torch.uint8, device=out.device)
@@ -1007,7 +1015,7 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
         return out
     capi.call("mi_moe_gemm_fp8_grouped", out, capi.ptr(a), capi.ptr(a_scale), capi.ptr(row_map), int(row_map_div),
               capi.ptr(w), capi.ptr(w_scale), per_expert, capi.ptr(expert_start), capi.ptr(out), capi.ptr(out_map),
-              capi.ptr(row_weight), a_rows, total, E, N, K, fuse, adt, 1 if out.dtype == torch.float32 else 0)
+              capi.ptr(row_weight), a_rows, total, E, N, K, fuse, adt, _out_kind(out, adt))
     return out
 
 
@@ -1179,12 +1187,13 @@ def moe_combine(y, inv, top_w, output, top_k):
     who = "moe_combine"
     T, H = output.shape
     _chk(output.dtype in (torch.float16, torch.bfloat16) and output.is_contiguous(), f"{who}: output must be contiguous fp16/bf16 [T, H]")
-    _chk(y.dtype in (output.dtype, torch.float32) and y.is_contiguous() and y.shape[-1] == H, f"{who}: y must be [T*k, H] fp32 or activation dtype")
+    _chk(y.dtype in (output.dtype, torch.float32, torch.float16) and y.is_contiguous() and y.shape[-1] == H,
+         f"{who}: y must be [T*k, H] fp32, fp16 or the activation dtype")
     _chk(inv.dtype == torch.int32 and inv.numel() >= T * int(top_k), f"{who}: inv must be int32 [T*k]")
     _chk(top_w.dtype == output.dtype and top_w.is_contiguous(), f"{who}: top_w must share the output dtype")
     _chk(H % 8 == 0, f"{who}: H must be a multiple of 8")
     capi.call("mi_moe_combine", y, capi.ptr(y), capi.ptr(inv), capi.ptr(top_w), capi.ptr(output), H, int(top_k), T, 0,
-              capi.act_dtype(output), 1 if y.dtype == torch.float32 else 0)
+              capi.act_dtype(output), _out_kind(y, capi.act_dtype(output)))
     return output
 
 

@@ -475,6 +475,32 @@ def test_moe_forward_w8a16_prefill(v, dev, T, E, K, H, I, dt):
     assert bool(((o - ref).abs() <= bound).all()), ((o - ref).abs() / bound).max()
 
 
+@pytest.mark.parametrize("aq", [True, False])
+def test_expert_outputs_in_fp16_beside_bf16(v, dev, aq):
+    """The grouped GEMM can write fp16 whatever the activation type and the combine reads it: half the bytes
+    of fp32 rows at 11 significant bits.  The fused forward keeps fp32 (near-zero outputs, sums of cancelling
+    terms, are 6 x closer to the oracle with it); this covers the mode for callers that trade that for speed."""
+    T, E, K, H, I = 24, 8, 2, 256, 128
+    x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I, seed=77)
+    assert x.dtype == torch.bfloat16
+    g = _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq)
+    P = T * K
+    st = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    sp, inv, tok = (torch.empty(P, dtype=torch.int32, device=dev) for _ in range(3))
+    v.moe_sort(g["ti"], E, sp, st, inv, tok)
+    y16 = torch.empty(P, H, dtype=torch.float16, device=dev)
+    if aq:
+        v.moe_gemm_fp8_block(g["iq"], g["isc"], None, w2q.to(dev), w2s.to(dev), st, y16, H, I, E, False)
+    else:
+        v.moe_gemm_fp8_block(g["inter"], None, None, w2q.to(dev), w2s.to(dev), st, y16, H, I, E, False)
+    assert torch.equal(y16, g["y"].half())                     # the fp32 result, rounded once
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    v.moe_combine(y16, inv, g["tw"], out, K)
+    ref = (g["tw"].float().reshape(T, K, 1) * y16.float()[inv.long()].reshape(T, K, H)).sum(1)
+    assert O.max_rel_err(out.cpu(), ref.cpu()) < 4e-3          # one bf16 rounding of the fp32 sum
+    assert O.max_rel_err(out.cpu(), g["out"].float().cpu()) < TOL
+
+
 def test_cfg3_moe_forward(v, dev):
     # the stage-wise 1e-2 bars (mean floor) are inside _check_forward; it also prints the staged and the
     # free-running maxima under both denominators (free-running, this shape: 4e-2 with the mean floor)
