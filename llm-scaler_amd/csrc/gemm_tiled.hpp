@@ -208,7 +208,7 @@ struct WQ4K {
   };
   struct Stage {
     u32x4 b[B_CH];
-    uint16_t s[B_CH], m[B_CH];
+    uint32_t s[B_CH], m[B_CH];                        // fp16 bits (32-bit slots: 16-bit members end up on the stack)
   };
   struct Dq {
     uint32_t e, o, t;
@@ -240,8 +240,8 @@ struct WQ4K {
   static __device__ __forceinline__ void begin(const Res&, const Stage& st, Dq& q) {
 #pragma unroll
     for (int i = 0; i < B_CH; ++i) {
-      const _Float16 mn = __builtin_bit_cast(_Float16, st.m[i]);
-      q.sf[i] = (float)__builtin_bit_cast(_Float16, st.s[i]) * 512.0f;   // exact: a power of two
+      const _Float16 mn = __builtin_bit_cast(_Float16, (uint16_t)st.m[i]);
+      q.sf[i] = (float)__builtin_bit_cast(_Float16, (uint16_t)st.s[i]) * 512.0f;   // exact: a power of two
       q.mv[i] = f16x2{mn, mn};
     }
   }

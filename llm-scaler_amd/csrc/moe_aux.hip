@@ -441,14 +441,15 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 // plus a popcount inside the thread's own mask.  One dependent round trip to memory instead of the
 // single workgroup's clear / mark / scan / place sequence.  Ids outside [0, E) are held into the
 // range like in the other paths; every pair gets a position of its own.
-constexpr int kSortExpertThreads = 256;
-constexpr int kSortExpertMaxPairs = 32 * kSortExpertThreads;
+constexpr int kSortExpertMaxPairs = 32 * 1024;       // 32 pairs per thread, at most 1024 threads
 
-__global__ __launch_bounds__(kSortExpertThreads) void moe_sort_expert_kernel(
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void moe_sort_expert_kernel(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
     int P, int K, int E, int chunk) {
-  __shared__ int32_t wave_lt[4], wave_eq[4];
+  constexpr int NWV = THREADS / 64;
+  __shared__ int32_t wave_lt[NWV], wave_eq[NWV];
   const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int q0 = tid * chunk;
   uint32_t mask = 0;
@@ -472,14 +473,16 @@ __global__ __launch_bounds__(kSortExpertThreads) void moe_sort_expert_kernel(
   }
   if (lane == 63) { wave_eq[wave] = incl; wave_lt[wave] = lsum; }
   __syncthreads();
-  int start = 0, before = incl - eq;                  // pairs of this expert in earlier threads
-  for (int w = 0; w < 4; ++w) {
+  int start = 0, before = incl - eq, count = 0;       // `before`: pairs of this expert in earlier threads
+#pragma unroll
+  for (int w = 0; w < NWV; ++w) {
     start += wave_lt[w];
+    count += wave_eq[w];
     if (w < wave) before += wave_eq[w];
   }
   if (tid == 0) {
     expert_start[e] = start;
-    if (e == E - 1) expert_start[E] = start + wave_eq[0] + wave_eq[1] + wave_eq[2] + wave_eq[3];
+    if (e == E - 1) expert_start[E] = start + count;
   }
   int pos = start + before;
   while (mask) {
@@ -878,9 +881,16 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
   const long P = (long)T * K;
   if (!max_count && P > 0 && P <= kSortExpertMaxPairs && (long)P * E <= (4l << 20)) {
     // one workgroup per expert; each reads all ids (at most 16 MiB from L2 over the whole launch)
-    const int chunk = (int)((P + kSortExpertThreads - 1) / kSortExpertThreads);
-    hipLaunchKernelGGL(moe_sort_expert_kernel, dim3((unsigned)E), dim3(kSortExpertThreads), 0, (hipStream_t)stream,
-                       top_ids, sorted_pairs, expert_start, inv, sorted_token, (int)P, K, E, chunk);
+    hipStream_t st = (hipStream_t)stream;
+    if (P <= 32 * 256) {
+      const int chunk = (int)((P + 255) / 256);
+      hipLaunchKernelGGL(moe_sort_expert_kernel<256>, dim3((unsigned)E), dim3(256), 0, st, top_ids, sorted_pairs,
+                         expert_start, inv, sorted_token, (int)P, K, E, chunk);
+    } else {
+      const int chunk = (int)((P + 1023) / 1024);
+      hipLaunchKernelGGL(moe_sort_expert_kernel<1024>, dim3((unsigned)E), dim3(1024), 0, st, top_ids, sorted_pairs,
+                         expert_start, inv, sorted_token, (int)P, K, E, chunk);
+    }
     return launch_status();
   }
   const int S = sort_wide_span(T, E);
