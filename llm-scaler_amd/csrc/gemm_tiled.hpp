@@ -104,8 +104,7 @@ struct WInt4 {
   };
   struct Stage {
     u32x4 b[B_CH];
-    uint16_t s[B_CH];
-    uint8_t z[B_CH];
+    uint32_t s[B_CH], z[B_CH];                        // fp16 scale bits, zero-point: 32-bit slots, one register each
   };
   struct Dq {
     uint32_t e, o;
@@ -142,7 +141,7 @@ struct WInt4 {
   static __device__ __forceinline__ void begin(const Res& r, const Stage& st, Dq& q) {
 #pragma unroll
     for (int i = 0; i < B_CH; ++i) {
-      const _Float16 sc = __builtin_bit_cast(_Float16, st.s[i]);
+      const _Float16 sc = __builtin_bit_cast(_Float16, (uint16_t)st.s[i]);
       const float z = r.has_zp ? (float)st.z[i] : 8.0f;
       q.sf[i] = (float)sc * 512.0f;
       q.nzs[i] = -z * (float)sc;
