@@ -394,7 +394,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 15, g = lane >> 4;
-  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+  const int wn0 = (wave & 1) * WN;
 
   // Tile order.  The 8 XCDs take workgroups round-robin and each has its own L2, so the tile of a
   // workgroup is derived from (XCD = id % 8, slot on that XCD = id / 8):

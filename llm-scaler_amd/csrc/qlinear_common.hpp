@@ -16,6 +16,7 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) int32_t i32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 enum : int { DT_F16 = 0, DT_BF16 = 1 };
