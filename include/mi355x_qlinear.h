@@ -443,6 +443,20 @@ int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* ro
                           const float* w_scale, const int32_t* expert_start, void* out, int a_rows,
                           int total_rows, int E, int N, int K, int fuse_silu_mul, int act_dtype,
                           int out_f32, void* stream);
+/* mi_moe_sort and the gate_up mi_moe_gemm_fp8_block (quantised activations, fused silu(gate) * up) in
+ * one launch, for up to 8192 (token, route) pairs: every workgroup of an expert finds the expert's
+ * pairs in top_ids [T, topk] itself (the same stable counting sort: lower experts' pairs first, pair
+ * order inside an expert; ids outside [0, E) are held into the range) and gathers its rows of
+ * a [T, K] e4m3 / a_scale [T, K/128] by token = pair / topk; out [T*topk, N/2] is in expert-sorted
+ * order, and expert_start [E+1], inv [T*topk] and (optional) sorted_pairs [T*topk] are written as
+ * mi_moe_sort writes them, for the stages that follow.  K % 128 == 0, K >= 256, (N/2) % 16 == 0;
+ * MI_ERR_SHAPE beyond 8192 pairs (sort and GEMM are then two calls).  Takes the place of the
+ * reference's scatter + grouped up GEMM sequence (V/csrc/xpu/esimd_kernels/moe_ops.h:437-569,
+ * V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:123-334). */
+int mi_moe_gate_up_fp8_routed(const void* a, const float* a_scale, const int32_t* top_ids, int T, int topk,
+                              const void* w, const float* w_scale, int32_t* expert_start, int32_t* inv,
+                              int32_t* sorted_pairs, void* out, int E, int N, int K, int act_dtype,
+                              void* stream);
 
 /* The same GEMM with the per-expert-scalar scale of the reference's per-tensor MoE
  * kernels and their epilogues:

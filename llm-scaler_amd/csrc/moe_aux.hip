@@ -5,6 +5,7 @@
 #include <type_traits>
 
 #include "qlinear_common.hpp"
+#include "moe_sort_expert.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -443,72 +444,19 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 // range like in the other paths; every pair gets a position of its own.
 constexpr int kSortExpertMaxPairs = 32 * 1024;       // 32 pairs per thread, at most 1024 threads
 
-template <int THREADS, bool VEC>
+template <int THREADS>
 __global__ __launch_bounds__(THREADS) void moe_sort_expert_kernel(
     const int32_t* __restrict__ top_ids, int32_t* __restrict__ sorted_pairs,
     int32_t* __restrict__ expert_start, int32_t* __restrict__ inv, int32_t* __restrict__ sorted_token,
     int P, int K, int E, int chunk) {
   constexpr int NWV = THREADS / 64;
   __shared__ int32_t wave_lt[NWV], wave_eq[NWV];
-  const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e = blockIdx.x, tid = threadIdx.x;
   const int q0 = tid * chunk;
-  uint32_t mask = 0;
-  int lt = 0;
-  if constexpr (VEC) {
-    // chunk is a multiple of 4 and top_ids is 16-byte aligned: a thread's ids are whole 16-byte words,
-    // all eight loads in flight together
-    i32x4 v[8];
-#pragma unroll
-    for (int b4 = 0; b4 < 8; ++b4) {
-      const int q = q0 + 4 * b4;
-      v[b4] = i32x4{-1, -1, -1, -1};
-      if (4 * b4 < chunk && q + 3 < P) v[b4] = *reinterpret_cast<const i32x4*>(top_ids + q);
-      else if (4 * b4 < chunk) {
-        for (int z = 0; z < 4; ++z)
-          if (q + z < P) v[b4][z] = top_ids[q + z];
-      }
-    }
-#pragma unroll
-    for (int b4 = 0; b4 < 8; ++b4) {
-#pragma unroll
-      for (int z = 0; z < 4; ++z) {
-        const int b = 4 * b4 + z;
-        if (b < chunk && q0 + b < P) {
-          const int raw = v[b4][z];
-          const int id = raw < 0 ? 0 : (raw >= E ? E - 1 : raw);
-          lt += id < e;
-          mask |= (uint32_t)(id == e) << b;
-        }
-      }
-    }
-  } else {
-    for (int b = 0; b < chunk; ++b) {
-      const int q = q0 + b;
-      if (q < P) {
-        const int id = sort_expert(top_ids, q, E);
-        lt += id < e;
-        mask |= (uint32_t)(id == e) << b;
-      }
-    }
-  }
-  const int eq = __popc(mask);
-  // wave-inclusive scan of eq, wave sum of lt
-  int incl = eq, lsum = lt;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const int o = __shfl_up(incl, off, 64);
-    if (lane >= off) incl += o;
-    lsum += __shfl_xor(lsum, off, 64);
-  }
-  if (lane == 63) { wave_eq[wave] = incl; wave_lt[wave] = lsum; }
-  __syncthreads();
-  int start = 0, before = incl - eq, count = 0;       // `before`: pairs of this expert in earlier threads
-#pragma unroll
-  for (int w = 0; w < NWV; ++w) {
-    start += wave_lt[w];
-    count += wave_eq[w];
-    if (w < wave) before += wave_eq[w];
-  }
+  uint32_t mask;
+  int lt, start, count, before;                       // `before`: pairs of this expert in earlier threads
+  expert_pairs_of_thread(top_ids, P, E, e, chunk, tid, mask, lt);
+  expert_scan<NWV>(mask, lt, tid, wave_lt, wave_eq, start, count, before);
   if (tid == 0) {
     expert_start[e] = start;
     if (e == E - 1) expert_start[E] = start + count;
@@ -911,16 +859,14 @@ int mi_moe_sort(const int32_t* top_ids, int32_t* sorted_pairs, int32_t* expert_s
   if (!max_count && P > 0 && P <= kSortExpertMaxPairs && (long)P * E <= (4l << 20)) {
     // one workgroup per expert; each reads all ids (at most 16 MiB from L2 over the whole launch)
     hipStream_t st = (hipStream_t)stream;
-    const bool vec = ((uintptr_t)top_ids & 15) == 0;
     const int threads = P <= 32 * 256 ? 256 : 1024;
-    int chunk = (int)((P + threads - 1) / threads);
-    if (vec) chunk = (chunk + 3) & ~3;
-#define QLIN_SORTE(TH, V)                                                                                          \
-  hipLaunchKernelGGL((moe_sort_expert_kernel<TH, V>), dim3((unsigned)E), dim3(TH), 0, st, top_ids, sorted_pairs, \
-                     expert_start, inv, sorted_token, (int)P, K, E, chunk)
-    if (threads == 256) { if (vec) QLIN_SORTE(256, true); else QLIN_SORTE(256, false); }
-    else { if (vec) QLIN_SORTE(1024, true); else QLIN_SORTE(1024, false); }
-#undef QLIN_SORTE
+    const int chunk = ((int)((P + threads - 1) / threads) + 3) & ~3;     // whole 16-byte words of ids per thread
+    if (threads == 256)
+      hipLaunchKernelGGL(moe_sort_expert_kernel<256>, dim3((unsigned)E), dim3(256), 0, st, top_ids, sorted_pairs,
+                         expert_start, inv, sorted_token, (int)P, K, E, chunk);
+    else
+      hipLaunchKernelGGL(moe_sort_expert_kernel<1024>, dim3((unsigned)E), dim3(1024), 0, st, top_ids, sorted_pairs,
+                         expert_start, inv, sorted_token, (int)P, K, E, chunk);
     return launch_status();
   }
   const int S = sort_wide_span(T, E);

@@ -25,6 +25,7 @@
 // and scaled by a per-destination-row weight.
 #include "qlinear_common.hpp"
 #include "scratch.hpp"
+#include "moe_sort_expert.hpp"
 #include "../../include/mi355x_qlinear.h"
 
 namespace qlin {
@@ -49,6 +50,12 @@ struct MoeGemmArgs {
   int tpw;                    // tile groups walked by one workgroup
   int a_rows;                 // rows in `a` (bounds the buffer)
   int total_rows;             // rows in `out`
+  // SORT kernels: the expert grouping is derived from the routing table inside the launch
+  const int32_t* top_ids;     // [P] expert of pair q = token * topk + route
+  int32_t* sort_start;        // out [E + 1]
+  int32_t* sort_inv;          // out [P]: pair -> expert-sorted position
+  int32_t* sort_pairs;        // out [P] or null: expert-sorted position -> pair
+  int P, topk, chunk;         // pairs, routes per token, pairs owned by one thread (a multiple of 4)
 };
 
 // LDS staging geometry.  Global loads are row-coalesced (8 or 16 consecutive lanes
@@ -59,6 +66,7 @@ struct MoeGemmArgs {
 // bytes so that the 16 lanes of an operand read (row stride 144 / 272 bytes) fall
 // into distinct banks.
 constexpr int kWPitch = 128 + 16;                    // fp8 weight / activation row of one granule
+constexpr long kRoutedMaxPairs = 32 * 256;           // pairs a routed (SORT) launch takes: 32 per thread
 constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of one granule
 
 // Workgroup = 4 wavefronts.  The workgroup owns RT 16-row weight tiles of one
@@ -78,7 +86,13 @@ constexpr int kA16Pitch = 256 + 16;                  // 16-bit activation row of
 // MT = 16-row activation tiles per wavefront and pass.  Only MT = 1 (up to 64 rows per pass) is
 // launched: with 4 the kernel is bound by its LDS traffic and gained nothing for experts with
 // hundreds of rows, which run on the tiled matrix-core GEMM instead (moe_gemm_tiled.hip).
-template <class Act, bool A8, bool SILU, int RT, int D, bool PE, int MT = 1>
+// SORT: the launch takes the routing table (expert per (token, route) pair) instead of expert-sorted
+// rows.  Every workgroup of expert e finds the expert's pairs itself -- it reads all P ids, the number
+// of pairs of lower experts is the expert's first sorted position and a pair's rank is the number of
+// earlier pairs of the same expert: the stable counting sort of mi_moe_sort, one round trip to memory,
+// overlapped with the resident workgroups that already stream -- gathers its rows by token = pair / topk,
+// and the expert's first workgroup writes expert_start / inv / sorted_pairs for the later stages.
+template <class Act, bool A8, bool SILU, int RT, int D, bool PE, int MT = 1, bool SORT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2))) void moe_gemm_kernel(const MoeGemmArgs p, const float* __restrict__ w_scale,
                                                         const int32_t* __restrict__ expert_start) {
   static_assert(RT == 2 || RT == 4 || RT == 8, "two, four or eight weight tiles");
@@ -98,13 +112,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
   const int e = (slot / p.tiles_per_expert) * 8 + xcd;
   const int wg = slot % p.tiles_per_expert;
   if (e >= p.E) return;
-  const int r0 = expert_start[e];
-  const int cnt = expert_start[e + 1] - r0;
-  if (cnt <= 0) return;
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int r0 = 0, cnt = 0;
+
   const int j = lane & 15, g = lane >> 4;
   const int K = p.K, N = p.N;
   const int G = (K + 127) >> 7, Kb = G;
@@ -158,17 +170,103 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
   };
   constexpr int kPassRows = 64 * MT;                  // rows of the expert per pass over its weights
 
+  // weight loads of granule gi of tile group tg (dead beyond the last one)
+  auto load_weights = [&](Regs& r, int tg, int gi) {
+    const uint32_t dead = tg < ntg ? 0u : 0x80000000u;
+    const uint32_t wso = (uint32_t)tg * tg_stride + (uint32_t)gi * 128u;
+    // quantised activations come in whole 128-groups: no partial granule there
+    const int kext = (!A8 && gi == G - 1) ? ktail : 128;   // uniform
+    const uint32_t wv = wvoff | dead | ((uint32_t)(wch >= kext) << 31);
+    const int wc = wcol + tg * kCols;
+#pragma unroll
+    for (int i = 0; i < WL; ++i)
+      r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wv | ((uint32_t)(wc + i * 16 * (SILU ? 1 : 2) >= limit) << 31),
+                                                     wso + (uint32_t)i * wistep, 2);
+  };
+
+  Regs r[D];
+  uint32_t smask = 0;                                  // SORT: bit b = pair tid * chunk + b belongs to expert e
+  int sbefore = 0;                                     // SORT: rank of this thread's first pair inside the expert
+  __shared__ int32_t pass_token[SORT ? 64 * MT : 1];   // SORT: token of each row of the current pass
+  // The weights do not depend on the expert's rows: when most experts are in use, the first granules
+  // are requested before the workgroup knows its rows, so that its stream already runs while it finds
+  // them.  (With few rows per launch most workgroups find none and leave; those request nothing.)
+  bool early_w;                                        // the first pass's weight prefetch is already in flight
+  u32x4 ids[SORT ? kSortExpertChunkMax / 4 : 1];
+  if constexpr (SORT) {
+    static_assert(MT == 1, "one activation tile per wavefront");
+    expert_ids_load(p.top_ids, p.P, p.chunk, tid, ids);   // ahead of the weights: the sort waits for these only
+    early_w = p.P >= 2 * p.E;
+  } else {
+    early_w = p.total_rows >= 2 * p.E;
+  }
+  if (early_w) {
+    int etg = 0, egi = 0;
+#pragma unroll
+    for (int st = 0; st < D; ++st) {
+      load_weights(r[st], etg, egi);
+      if (++egi == G) { egi = 0; ++etg; }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  if constexpr (SORT) {
+    __shared__ int32_t wave_lt[4], wave_eq[4];
+    const int E = p.E, q0 = tid * p.chunk;
+    int lt, start, count;
+    expert_ids_count(ids, p.P, E, e, p.chunk, tid, smask, lt);
+    expert_scan<4>(smask, lt, tid, wave_lt, wave_eq, start, count, sbefore);
+    r0 = start;
+    cnt = count;
+    if (wg == 0) {                                     // the expert's first workgroup publishes the grouping
+      if (tid == 0) {
+        p.sort_start[e] = start;
+        if (e == E - 1) p.sort_start[E] = start + count;
+      }
+      uint32_t m2 = smask;
+      int pos = start + sbefore;
+      while (m2) {
+        const int b = __ffs(m2) - 1;
+        m2 &= m2 - 1;
+        p.sort_inv[q0 + b] = pos;
+        if (p.sort_pairs) p.sort_pairs[pos] = q0 + b;
+        ++pos;
+      }
+    }
+  } else {
+    r0 = expert_start[e];
+    cnt = expert_start[e + 1] - r0;
+  }
+  if (cnt <= 0) return;
+
   for (int mc = 0; mc < cnt; mc += kPassRows) {
     const int rows_here = min(kPassRows, cnt - mc);
     const int wrow0 = wave * 16 * MT;                 // first row of this wavefront inside the pass
+    if constexpr (SORT) {
+      // tokens of the pass's rows, from the threads that own the pairs (the previous pass's readers
+      // have passed the barrier that ends a pass)
+      uint32_t m2 = smask;
+      int rank = sbefore - mc;
+      while (m2) {
+        const int b = __ffs(m2) - 1;
+        m2 &= m2 - 1;
+        if (rank >= 0 && rank < kPassRows) pass_token[rank] = (tid * p.chunk + b) / p.topk;
+        ++rank;
+      }
+      __syncthreads();
+    }
+    // source row (of `a` / `a_scale`) of row m of the expert, m inside this pass
+    auto src_row = [&](int m, bool ok) -> uint32_t {
+      if constexpr (SORT) return (uint32_t)pass_token[ok ? m - mc : 0];
+      const int pos = r0 + (ok ? m : 0);
+      return p.row_map ? (uint32_t)p.row_map[pos] / (uint32_t)p.row_div : (uint32_t)pos;
+    };
     // source row of this lane's activation row (MFMA layout) and staging slots
     uint32_t xsoff[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = mc + wrow0 + mt * 16 + j;
       const bool ok = m < cnt;
-      const int pos = r0 + (ok ? m : 0);
-      const uint32_t src = p.row_map ? (uint32_t)p.row_map[pos] / (uint32_t)p.row_div : (uint32_t)pos;
+      const uint32_t src = src_row(m, ok);
       xsoff[mt] = (src * (uint32_t)Kb * 4u) | ((uint32_t)(!ok) << 31);
     }
     uint32_t aoff[MT][NAI];
@@ -182,25 +280,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
         const int ch = A8 ? (lane & 7) : (lane & 15);
         const int m = mc + wrow0 + mt * 16 + row;
         const bool ok = m < cnt;
-        const int pos = r0 + (ok ? m : 0);
-        const uint32_t src = p.row_map ? (uint32_t)p.row_map[pos] / (uint32_t)p.row_div : (uint32_t)pos;
+        const uint32_t src = src_row(m, ok);
         aoff[mt][i] = (src * (uint32_t)K * a_esz + (uint32_t)ch * 16u) | ((uint32_t)(!ok) << 31);
         alds[mt][i] = al + (mt * 16 + row) * APitch + ch * 16;
         ach[i] = A8 ? ch * 16 : ch * 8;               // first k of the chunk inside the granule
       }
 
-    // issue the loads of granule gi of tile group tg (dead beyond the last one)
-    auto load_granule = [&](Regs& r, int tg, int gi) {
+    // activation loads of granule gi of tile group tg (dead beyond the last one)
+    auto load_acts = [&](Regs& r, int tg, int gi) {
       const uint32_t dead = tg < ntg ? 0u : 0x80000000u;
-      const uint32_t wso = (uint32_t)tg * tg_stride + (uint32_t)gi * 128u;
-      // quantised activations come in whole 128-groups: no partial granule there
       const int kext = (!A8 && gi == G - 1) ? ktail : 128;   // uniform
-      const uint32_t wv = wvoff | dead | ((uint32_t)(wch >= kext) << 31);
-      const int wc = wcol + tg * kCols;
-#pragma unroll
-      for (int i = 0; i < WL; ++i)
-        r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wv | ((uint32_t)(wc + i * 16 * (SILU ? 1 : 2) >= limit) << 31),
-                                                       wso + (uint32_t)i * wistep, 2);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -211,6 +300,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
           r.xs[mt] = __builtin_bit_cast(float,
                                         __builtin_amdgcn_raw_buffer_load_b32(xsr, xsoff[mt] | dead, (uint32_t)gi * 4u, 0));
       }
+    };
+    auto load_granule = [&](Regs& r, int tg, int gi) {
+      load_weights(r, tg, gi);
+      load_acts(r, tg, gi);
     };
 
     // destination row and routing weight of this lane's activation row: fetched once per pass, ahead
@@ -243,11 +336,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
     // flight in a register ring.  Steps past the end (the sequence is walked in multiples of D) load
     // nothing and compute nothing.
     const int total = ntg * G;
-    Regs r[D];
     int ptg = 0, pgi = 0;                             // position of the next step to fetch
 #pragma unroll
     for (int s = 0; s < D; ++s) {
-      load_granule(r[s], ptg, pgi);
+      if (early_w && mc == 0) load_acts(r[s], ptg, pgi);
+      else load_granule(r[s], ptg, pgi);
       if (++pgi == G) { pgi = 0; ++ptg; }
       // keep the stages' loads in issue order: the counter of outstanding loads
       // retires in order, and the loop waits for "all but the younger stages"
@@ -511,10 +604,10 @@ static void launch_moe_kernel(K kern, size_t lds, long wgs, const MoeGemmArgs& p
   hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(256), lds, st, p, p.w_scale, p.start);
 }
 
-template <class Act, bool A8, bool SILU, int RT, int D, int MT = 1>
+template <class Act, bool A8, bool SILU, int RT, int D, int MT = 1, bool SORT = false>
 static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
   // quantised activations only come with block scales (the per-expert form is the reference's w8a16 mode)
-  constexpr bool kHasPE = !A8;
+  constexpr bool kHasPE = !A8 && !SORT;
   const int cols = SILU ? p.N / 2 : p.N;
   const int cols_per_group = SILU ? (RT / 2) * 16 : RT * 16;
   const int groups = (cols + cols_per_group - 1) / cols_per_group;
@@ -531,11 +624,11 @@ static int launch_moe(MoeGemmArgs p, int tpw, hipStream_t st) {
       return launch_status();
     }
   }
-  launch_moe_kernel(moe_gemm_kernel<Act, A8, SILU, RT, D, false, MT>, lds, wgs, p, st, raised_block);
+  launch_moe_kernel(moe_gemm_kernel<Act, A8, SILU, RT, D, false, MT, SORT>, lds, wgs, p, st, raised_block);
   return launch_status();
 }
 
-template <class Act, bool A8, bool SILU>
+template <class Act, bool A8, bool SILU, bool SORT = false>
 static int dispatch_moe2(const MoeGemmArgs& p, hipStream_t st) {
   const int G = (p.K + 127) / 128;
   const int cols = SILU ? p.N / 2 : p.N;
@@ -548,9 +641,17 @@ static int dispatch_moe2(const MoeGemmArgs& p, hipStream_t st) {
   // two granules in flight per thread (more do not pay: the register ring then costs a resident
   // workgroup); a single granule has nothing to prefetch
   const bool d2 = G >= 2;
-  if (rt == 8) return d2 ? launch_moe<Act, A8, SILU, 8, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 8, 1>(p, tpw, st);
-  if (rt == 4) return d2 ? launch_moe<Act, A8, SILU, 4, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 4, 1>(p, tpw, st);
-  return d2 ? launch_moe<Act, A8, SILU, 2, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 2, 1>(p, tpw, st);
+  if constexpr (SORT) {
+    // the routed launch is instantiated for the shapes that have several granules (K >= 256)
+    if (!d2) return MI_ERR_SHAPE;
+    if (rt == 8) return launch_moe<Act, A8, SILU, 8, 2, 1, true>(p, tpw, st);
+    if (rt == 4) return launch_moe<Act, A8, SILU, 4, 2, 1, true>(p, tpw, st);
+    return launch_moe<Act, A8, SILU, 2, 2, 1, true>(p, tpw, st);
+  } else {
+    if (rt == 8) return d2 ? launch_moe<Act, A8, SILU, 8, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 8, 1>(p, tpw, st);
+    if (rt == 4) return d2 ? launch_moe<Act, A8, SILU, 4, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 4, 1>(p, tpw, st);
+    return d2 ? launch_moe<Act, A8, SILU, 2, 2>(p, tpw, st) : launch_moe<Act, A8, SILU, 2, 1>(p, tpw, st);
+  }
 }
 
 template <class Act, bool A8>
@@ -609,6 +710,27 @@ int mi_moe_gemm_fp8_grouped(const void* a, const float* a_scale, const int32_t* 
   }
   return act_dtype == DT_F16 ? dispatch_moe<ActF16, false>(p, fuse_act, st)
                              : dispatch_moe<ActBF16, false>(p, fuse_act, st);
+}
+
+int mi_moe_gate_up_fp8_routed(const void* a, const float* a_scale, const int32_t* top_ids, int T, int topk,
+                              const void* w, const float* w_scale, int32_t* expert_start, int32_t* inv,
+                              int32_t* sorted_pairs, void* out, int E, int N, int K, int act_dtype, void* stream) {
+  if (!a || !a_scale || !top_ids || !w || !w_scale || !expert_start || !inv || !out) return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (T < 0 || topk < 1 || E < 1 || E > 1024 || N <= 0 || K < 256 || (K % 128) || (N % 2) || (N / 2) % 16)
+    return MI_ERR_SHAPE;
+  const long P = (long)T * topk;
+  if (P > kRoutedMaxPairs) return MI_ERR_SHAPE;       // 32 pairs per thread of a 256-thread workgroup
+  if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || (uint64_t)T * (uint64_t)K * 2 >= (1ull << 31)) return MI_ERR_SHAPE;
+  MoeGemmArgs p{};
+  p.a = a; p.a_scale = a_scale; p.row_div = 1; p.w = w; p.w_scale = w_scale; p.out = out;
+  p.E = E; p.N = N; p.K = K; p.a_rows = T; p.total_rows = (int)P;
+  p.top_ids = top_ids; p.sort_start = expert_start; p.sort_inv = inv; p.sort_pairs = sorted_pairs;
+  p.P = (int)P; p.topk = topk;
+  p.chunk = ((int)((P + 255) / 256) + 3) & ~3;        // whole 16-byte words of ids per thread
+  hipStream_t st = (hipStream_t)stream;
+  return act_dtype == DT_F16 ? dispatch_moe2<ActF16, true, true, true>(p, st)
+                             : dispatch_moe2<ActBF16, true, true, true>(p, st);
 }
 
 int mi_moe_gemm_fp8_block(const void* a, const float* a_scale, const int32_t* row_map, const void* w,

@@ -173,6 +173,14 @@ def moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, 
                                    N, K, num_experts, fuse_silu_mul)
 
 
+def moe_gate_up_fp8_routed(xq, xs, top_ids, weight, weight_scale, expert_start, inv, sorted_pairs, output,
+                           num_experts):
+    """moe_sort and the gate_up moe_gemm_fp8_block (e4m3 activations, fused SiLU*mul) in one launch,
+    for up to 8192 (token, route) pairs; expert_start / inv / sorted_pairs are written for later stages."""
+    return _ops.moe_gate_up_fp8_routed(xq, xs, top_ids, weight, weight_scale, expert_start, inv, sorted_pairs,
+                                       output, num_experts)
+
+
 def moe_combine(y, inv, top_w, output, top_k):
     return _ops.moe_combine(y, inv, top_w, output, top_k)
 

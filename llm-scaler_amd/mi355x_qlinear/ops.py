@@ -1048,6 +1048,51 @@ def moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, 
                      K, bool(fuse_silu_mul), who)
 
 
+ROUTED_MAX_PAIRS = 8192       # (token, route) pairs one routed gate_up launch sorts by itself
+
+
+def moe_gate_up_fp8_routed(xq, xs, top_ids, weight, weight_scale, expert_start, inv, sorted_pairs, output,
+                           num_experts):
+    """Expert sort and the gate_up grouped GEMM (quantised activations, fused silu(gate) * up) in one
+    launch.  xq [T, K] e4m3 with xs [T, K/128] fp32; top_ids [T, topk] int32; weight [E, N, K] e4m3
+    with block scales; output [T*topk, N/2] fp16/bf16 in expert-sorted order.  expert_start [E+1],
+    inv [T*topk] and (optional) sorted_pairs [T*topk] are written as moe_sort writes them."""
+    who = "moe_gate_up_fp8_routed"
+    E = int(num_experts)
+    _chk(top_ids.dim() == 2 and top_ids.dtype == torch.int32 and top_ids.is_contiguous(),
+         f"{who}: top_ids must be contiguous int32 [T, topk]")
+    T, k = top_ids.shape
+    P = T * k
+    _chk(0 < P <= ROUTED_MAX_PAIRS, f"{who}: {P} pairs (1..{ROUTED_MAX_PAIRS} are sorted inside the launch)")
+    _chk(xq.dim() == 2 and xq.shape[0] == T and xq.dtype in _FP8_TYPES and xq.is_contiguous(),
+         f"{who}: quantised activations must be contiguous e4m3/uint8 [T, K]")
+    K = xq.shape[1]
+    _chk(K % 128 == 0 and K >= 256, f"{who}: K={K} must be a multiple of 128, at least 256")
+    _chk(xs.dtype == torch.float32 and xs.is_contiguous() and xs.numel() == T * (K // 128),
+         f"{who}: activation scales must be fp32 [T, K/128]")
+    _chk_fp8(weight, who)
+    _chk(weight.dim() == 3 and weight.shape[0] == E and weight.shape[2] == K and weight.is_contiguous(),
+         f"{who}: weight must be contiguous [E, N, K]")
+    N = weight.shape[1]
+    _chk(N % 2 == 0 and (N // 2) % 16 == 0, f"{who}: N/2 must be a multiple of 16")
+    _chk(weight_scale.dtype == torch.float32 and weight_scale.is_contiguous() and
+         weight_scale.numel() == E * ((N + 127) // 128) * (K // 128),
+         f"{who}: weight_scale must be contiguous fp32 [E, ceil(N/128), K/128]")
+    _chk(1 <= E <= 1024, f"{who}: num_experts must be in 1..1024")
+    for t, n, nm in ((expert_start, E + 1, "expert_start"), (inv, P, "inv")) + \
+            (((sorted_pairs, P, "sorted_pairs"),) if sorted_pairs is not None else ()):
+        _chk(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n,
+             f"{who}: {nm} must be contiguous int32 with >= {n} entries")
+    _chk(output.dtype in (torch.float16, torch.bfloat16) and output.is_contiguous() and
+         output.numel() == P * (N // 2), f"{who}: output must be contiguous fp16/bf16 [T*topk, N/2]")
+    for t in (xs, top_ids, weight, weight_scale, expert_start, inv, output):
+        _chk(t.device == xq.device, f"{who}: all tensors must be on one device")
+    capi.call("mi_moe_gate_up_fp8_routed", output, capi.ptr(xq), capi.ptr(xs), capi.ptr(top_ids), T, k,
+              capi.ptr(weight), capi.ptr(weight_scale), capi.ptr(expert_start), capi.ptr(inv),
+              capi.ptr(sorted_pairs), capi.ptr(output), E, N, K, capi.act_dtype(output))
+    return output
+
+
 def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight, down_scale, output, top_k,
                           act_quant):
     """Routed-experts MoE forward for 128x128 block-FP8 weights (no shared expert).
@@ -1085,18 +1130,23 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
                   capi.ptr(x), capi.ptr(xq), capi.ptr(xs), H, capi.act_dtype(x))
     else:
         esimd_moe_topk(logits, top_w, top_ids, T)
-    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
     start = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(P, dtype=torch.int32, device=dev)
-    sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
     inter = torch.empty(P, I, dtype=x.dtype, device=dev)
     # fp32 expert outputs (the combine adds K rounded terms otherwise); in the w8a16 prefill regime the
     # tiled grouped GEMM takes over, which writes the activation type
     prefill = (not act_quant) and P >= 96 * E
     y = torch.empty(P, H, dtype=x.dtype if prefill else torch.float32, device=dev)
-    moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
+    routed = act_quant and 0 < P <= ROUTED_MAX_PAIRS and H >= 256
+    if not routed:
+        sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+        sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
+        moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
     if act_quant:
-        moe_gemm_fp8_block(xq, xs, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
+        if routed:      # the gate_up launch sorts the pairs itself
+            moe_gate_up_fp8_routed(xq, xs, top_ids, gate_up_weight, gate_up_scale, start, inv, None, inter, E)
+        else:
+            moe_gemm_fp8_block(xq, xs, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
         iq = torch.empty(P, I, dtype=torch.uint8, device=dev)
         isc = torch.empty(P, I // 128, dtype=torch.float32, device=dev)
         act_quant_fp8(inter, iq, isc)
@@ -2192,6 +2242,9 @@ def register():
     _define(_V, "moe_gemm_fp8_block(Tensor a, Tensor? a_scale, Tensor? row_map, Tensor weight, Tensor weight_scale, "
                 "Tensor expert_start, Tensor(a!) output, int N, int K, int num_experts, bool fuse_silu_mul) -> Tensor(a!)",
             moe_gemm_fp8_block, _ret(6))
+    _define(_V, "moe_gate_up_fp8_routed(Tensor xq, Tensor xs, Tensor top_ids, Tensor weight, Tensor weight_scale, "
+                "Tensor(b!) expert_start, Tensor(c!) inv, Tensor(d!)? sorted_pairs, Tensor(a!) output, "
+                "int num_experts) -> Tensor(a!)", moe_gate_up_fp8_routed, _ret(8))
     _define(_V, "moe_combine(Tensor y, Tensor inv, Tensor top_w, Tensor(a!) output, int top_k) -> Tensor(a!)",
             moe_combine, _ret(3))
     _define(_V, "moe_forward_fp8_block(Tensor x, Tensor logits, Tensor gate_up_weight, Tensor gate_up_scale, "

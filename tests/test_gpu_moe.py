@@ -358,6 +358,79 @@ def test_moe_gemm_prefill_tiled_matches_streaming_kernel(v, dev):
 
 
 # ------------------------------------------------------------------ full forward
+@pytest.mark.parametrize("T,E,k,H,I,dt,skew,offset", [
+    (512, 128, 8, 2048, 768, torch.bfloat16, False, 0),     # cfg3's gate_up
+    (1, 8, 2, 256, 128, torch.float16, False, 0),
+    (37, 16, 4, 384, 64, torch.float16, True, 0),           # 80 rows on one expert: two passes, empty experts
+    (200, 4, 2, 256, 128, torch.bfloat16, True, 1),         # ids on a 4-byte boundary only (scalar id loads)
+    (1024, 32, 8, 256, 48, torch.float16, True, 0),         # 8192 pairs: 32 per thread
+])
+def test_routed_gate_up_equals_sort_then_gemm(v, dev, T, E, k, H, I, dt, skew, offset):
+    """The launch that sorts the pairs itself writes the same expert_start / inv / sorted_pairs as
+    moe_sort (bit for bit, against the oracle's permutation too) and the same intermediate as the
+    grouped GEMM on moe_sort's row map (same kernel arithmetic: bit-equal)."""
+    g = torch.Generator().manual_seed(T * 7 + E + k)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    if skew:
+        for t in range(T // 2):
+            if 3 % E not in ids[t].tolist():
+                ids[t, 0] = 3 % E
+        ids[::5, -1] = torch.where(ids[::5, -1] == 3 % E, ids[::5, -1], torch.full_like(ids[::5, -1], E + 7))  # out of range
+    P = T * k
+    x = (torch.randn(T, H, generator=g) * 0.5).to(dt)
+    w = O.e4m3_quantize(torch.randn(E, 2 * I, H, generator=g) * 0.05)
+    ws = torch.rand(E, (2 * I + 127) // 128, H // 128, generator=g) * 0.02 + 0.005
+    xd, wd, wsd = x.to(dev), w.to(dev), ws.to(dev)
+    xq = torch.empty(T, H, dtype=torch.uint8, device=dev)
+    xs = torch.empty(T, H // 128, dtype=torch.float32, device=dev)
+    v.act_quant_fp8(xd, xq, xs)
+    buf = torch.zeros(P + 4, dtype=torch.int32, device=dev)
+    ids_d = buf[offset:offset + P].view(T, k)
+    ids_d.copy_(ids.to(dev))
+    # separate sort + GEMM
+    sp = torch.empty(P, dtype=torch.int32, device=dev)
+    st = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(P, dtype=torch.int32, device=dev)
+    tok = torch.empty(P, dtype=torch.int32, device=dev)
+    v.moe_sort(ids_d, E, sp, st, inv, tok)
+    ref = torch.full((P, I), 7.0, dtype=dt, device=dev)
+    v.moe_gemm_fp8_block(xq, xs, tok, wd, wsd, st, ref, 2 * I, H, E, True)
+    # one launch
+    sp2 = torch.full((P,), -1, dtype=torch.int32, device=dev)
+    st2 = torch.full((E + 1,), -1, dtype=torch.int32, device=dev)
+    inv2 = torch.full((P,), -1, dtype=torch.int32, device=dev)
+    out = torch.full((P, I), 7.0, dtype=dt, device=dev)
+    v.moe_gate_up_fp8_routed(xq, xs, ids_d, wd, wsd, st2, inv2, sp2, out, E)
+    ro, rs, ri = O.moe_sort(ids.clamp(0, E - 1), E)
+    assert torch.equal(st2.cpu(), rs) and torch.equal(st2, st)
+    assert torch.equal(sp2.cpu(), ro) and torch.equal(inv2.cpu(), ri)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    # without the optional sorted_pairs
+    out3 = torch.full((P, I), 7.0, dtype=dt, device=dev)
+    v.moe_gate_up_fp8_routed(xq, xs, ids_d, wd, wsd, st2, inv2, None, out3, E)
+    assert torch.equal(out3.view(torch.int16), ref.view(torch.int16))
+
+
+def test_routed_gate_up_argument_errors(v, dev):
+    T, E, k, H, I = 4, 8, 2, 256, 64
+    xq = torch.zeros(T, H, dtype=torch.uint8, device=dev)
+    xs = torch.ones(T, H // 128, dtype=torch.float32, device=dev)
+    ids = torch.zeros(T, k, dtype=torch.int32, device=dev)
+    w = torch.zeros(E, 2 * I, H, dtype=torch.uint8, device=dev)
+    ws = torch.ones(E, 1, H // 128, dtype=torch.float32, device=dev)
+    st = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    inv = torch.empty(T * k, dtype=torch.int32, device=dev)
+    out = torch.empty(T * k, I, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError, match="pairs"):
+        big = torch.zeros(8192 // k + 1, k, dtype=torch.int32, device=dev)
+        v.moe_gate_up_fp8_routed(xq, xs, big, w, ws, st, inv, None, out, E)
+    with pytest.raises(RuntimeError, match="K="):
+        v.moe_gate_up_fp8_routed(xq[:, :128].contiguous(), xs[:, :1].contiguous(), ids, w[:, :, :128].contiguous(),
+                                 ws[:, :, :1].contiguous(), st, inv, None, out, E)
+    with pytest.raises(RuntimeError, match="inv"):
+        v.moe_gate_up_fp8_routed(xq, xs, ids, w, ws, st, inv[:3], None, out, E)
+
+
 def _staged_forward(v, dev, x, logits, w13q, w13s, w2q, w2s, E, K, aq):
     """The fused op's own pipeline, run stage by stage through the same ops, so that the
     quantised intermediate is visible."""
