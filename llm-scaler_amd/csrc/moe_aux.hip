@@ -62,20 +62,37 @@ __device__ __forceinline__ void moe_topk_body(const typename Act::elem* __restri
   // shared expert's gate of the fused decode ops); its loads are in flight while the selection runs
   float gate_acc = 0.f;
   if (gate_out) {
-    for (int c = lane; c < H8; c += 64) {
-      const typename Act::v8 a = gate_x[(size_t)t * H8 + c], b = gate_w[c];
+    // four steps' loads are requested together (indices held inside the row, the surplus is not added)
+    for (int c0 = lane; c0 < H8; c0 += 256) {
+      typename Act::v8 a[4], b[4];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) gate_acc += Act::to_f32(a[e]) * Act::to_f32(b[e]);
+      for (int u = 0; u < 4; ++u) {
+        const int c = min(c0 + 64 * u, H8 - 1);
+        a[u] = gate_x[(size_t)t * H8 + c];
+        b[u] = gate_w[c];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (c0 + 64 * u < H8) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) gate_acc += Act::to_f32(a[u][e]) * Act::to_f32(b[u][e]);
+        }
+      }
     }
   }
   const typename Act::elem* row = logits + (size_t)t * E;
   float v[SLOTS];
   uint32_t key[SLOTS];                               // selection keys; 0 = taken or past E
   float mx = -INFINITY;
+  // unconditional loads (index held inside the row): with a branch per slot every load waits for the
+  // one before
+  typename Act::elem raws[SLOTS];
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) raws[s] = row[min(s * 64 + lane, E - 1)];
 #pragma unroll
   for (int s = 0; s < SLOTS; ++s) {
     const int e = s * 64 + lane;
-    const typename Act::elem raw = e < E ? row[e] : Act::from_f32(0.f);
+    const typename Act::elem raw = raws[s];
     v[s] = e < E ? Act::to_f32(raw) : -INFINITY;
     key[s] = e < E ? (f16_order((uint32_t)__builtin_bit_cast(uint16_t, raw)) << 16) | (0xFFFFu - (uint32_t)e) : 0u;
     mx = fmaxf(mx, v[s]);
@@ -636,20 +653,36 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
   for (int j0 = 0; j0 < topk; j0 += kBatch) {
     int pos[kBatch];
     float wj[kBatch];
+    // The weights are fetched as raw bits in ONE uniform branch and converted after the rows have
+    // been requested: a branch and a conversion per weight make every load wait for the one before
+    // (eight dependent round trips).
+    uint32_t wraw[kBatch];
+    const uint16_t* w16 = reinterpret_cast<const uint16_t*>(w);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) wraw[b] = 0;
+    if (w && !by_pos) {                                 // indexed by pair: independent of the positions
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) wraw[b] = w16[(size_t)t * topk + (j0 + b < topk ? j0 + b : topk - 1)];
+    }
 #pragma unroll
     for (int b = 0; b < kBatch; ++b) {
       const int j = j0 + b < topk ? j0 + b : topk - 1;
       pos[b] = inv ? inv[(size_t)t * topk + j] : t * topk + j;       // no map: y is in pair order
     }
+    if (w && by_pos) {
 #pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      const int j = j0 + b < topk ? j0 + b : topk - 1;
-      wj[b] = w ? Act::to_f32(w[by_pos ? pos[b] : t * topk + j]) : 1.0f;   // no weights: plain sum
+      for (int b = 0; b < kBatch; ++b) wraw[b] = w16[pos[b]];
     }
+    auto weights = [&]() {
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)   // no weights: plain sum
+        wj[b] = w ? Act::to_f32(__builtin_bit_cast(Elem, (uint16_t)wraw[b])) : 1.0f;
+    };
     if constexpr (Y32) {
       f32x4 v[kBatch];
 #pragma unroll
       for (int b = 0; b < kBatch; ++b) v[b] = ((const f32x4*)yv)[(size_t)pos[b] * HC + c];
+      weights();
 #pragma unroll
       for (int b = 0; b < kBatch; ++b)
         if (j0 + b < topk) {
@@ -660,6 +693,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const void* __restrict__ y
       typename YAct::v8 v[kBatch];
 #pragma unroll
       for (int b = 0; b < kBatch; ++b) v[b] = ((const typename YAct::v8*)yv)[(size_t)pos[b] * HC + c];
+      weights();
 #pragma unroll
       for (int b = 0; b < kBatch; ++b)
         if (j0 + b < topk) {

@@ -84,17 +84,26 @@ __global__ __launch_bounds__(256) void pack_x_grouped_kernel(const uint16_t* __r
   const int l = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q0 = (blockIdx.x - b * nq) * kPackQ;
   const int live = blk[2 * b + 1], first = blk[2 * b];
+  // Unconditional loads with indices held in range, the surplus zeroed afterwards: a branch around
+  // each (map entry, row piece) pair would make the four pairs eight dependent round trips.
   u32x4 v[4];
+  unsigned row[4];
+  const int k = q0 * 32 + l * 8;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = wave * 4 + i;
-    const int k = q0 * 32 + l * 8;
-    v[i] = u32x4{0u, 0u, 0u, 0u};
-    if (r < live && k < K) {
-      const int pos = first + r;
-      const unsigned row = row_map ? (unsigned)row_map[pos] / (unsigned)row_div : (unsigned)pos;
-      if (row < (unsigned)a_rows) v[i] = *reinterpret_cast<const u32x4*>(x + (size_t)row * K + k);
-    }
+    const int pos = first + (r < live ? r : 0);
+    row[i] = row_map ? (unsigned)row_map[pos] : (unsigned)pos;
+  }
+  if (row_map && row_div != 1) {                      // after all four entries have been requested
+#pragma unroll
+    for (int i = 0; i < 4; ++i) row[i] /= (unsigned)row_div;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const bool ok = wave * 4 + i < live && k < K && row[i] < (unsigned)a_rows;
+    v[i] = *reinterpret_cast<const u32x4*>(x + (ok ? (size_t)row[i] * K + k : (size_t)0));
+    if (!ok) v[i] = u32x4{0u, 0u, 0u, 0u};
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(tile + (wave * 4 + i) * kPackPitch + l * 16) = v[i];
