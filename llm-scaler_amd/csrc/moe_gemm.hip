@@ -200,8 +200,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
   } else {
     early_w = p.total_rows >= 2 * p.E;
   }
-  if (early_w) {
-    int etg = 0, egi = 0;
+  {
+    // issued without a branch (a launch that does not prefetch marks the loads dead, and dead loads
+    // touch no memory): behind a branch the compiler cannot count the loads in flight and makes the
+    // first use of anything loaded earlier wait for all of them
+    int etg = early_w ? 0 : ntg, egi = 0;
 #pragma unroll
     for (int st = 0; st < D; ++st) {
       load_weights(r[st], etg, egi);
@@ -591,6 +594,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(A8 ? 3 : 2)
         if (++gi == G) { gi = 0; ++tg; }
       }
     }
+    // Nothing is in flight past this point (the last steps' loads are dead ones).  Said explicitly:
+    // otherwise the top of the pass loop has to assume the loop's loads pending and waits for the
+    // first pass's early weight request before it touches any register they might target.
+    __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0)
     __syncthreads();                                  // LDS is rewritten by the next pass
   }
 }
