@@ -119,6 +119,25 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   // one that reads 1 KiB in a row (measured: 256 workgroups x 32 rows x 4096, 6.5 against 1.6 us).
   // A 16-row tile of the slice is two LDS tiles wide (16-bit elements), so it is staged in two
   // halves; slot [mt][hx NQ/2 + i / 2][i % 2] holds load i of half hx until the transposition.
+  // The output scales of the columns this wavefront finishes (see the end), requested first of all and
+  // kept as raw bits: fetched where they are used they are one more round trip at the very end of
+  // the launch, with nothing left to hide it.
+  constexpr int kOutIters = (kMaxTiles * MT + NW - 1) / NW;
+  uint32_t os_raw[kOutIters];
+#pragma unroll
+  for (int it = 0; it < kOutIters; ++it) os_raw[it] = 0;
+  float os_pert = 1.0f;
+  if constexpr (FMT == 0 && !BLOCK) {
+    if (scale_mode == SC_PERT) os_pert = ((const float*)a.s[mat])[0];
+    if (scale_mode != SC_PERT) {
+#pragma unroll
+      for (int it = 0; it < kOutIters; ++it) {
+        const int o = wave + it * NW;
+        const int n = min(n0 + (o / MT) * 16 + j, N - 1);
+        os_raw[it] = a.scale_f16 ? (uint32_t)((const uint16_t*)a.s[mat])[n] : ((const uint32_t*)a.s[mat])[n];
+      }
+    }
+  }
   u32x4 xq[MT][NQ][2];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -323,7 +342,10 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
 
   // ---- the 8 slices meet: wavefront w finishes output tile (t, mt) = w ----
   __syncthreads();
-  for (int o = wave; o < ntiles * MT; o += NW) {
+#pragma unroll
+  for (int it = 0; it < kOutIters; ++it) {
+    const int o = wave + it * NW;
+    if (o >= ntiles * MT) break;
     const int t = o / MT, mt = o - t * MT;
     f32x4 sum = red[0][t][mt][lane];
 #pragma unroll
@@ -333,8 +355,8 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
     if (n < nend) {
       float os = 1.0f;
       if constexpr (FMT == 0 && !BLOCK) {
-        if (scale_mode == SC_PERT) os = s32[0];
-        else os = a.scale_f16 ? (float)((const _Float16*)a.s[mat])[n] : s32[n];
+        if (scale_mode == SC_PERT) os = os_pert;
+        else os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)os_raw[it]) : __builtin_bit_cast(float, os_raw[it]);
       }
       Elem* out = (Elem*)a.out[mat];
 #pragma unroll

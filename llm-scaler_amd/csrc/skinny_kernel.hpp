@@ -133,6 +133,23 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // FP8 per-channel / per-tensor: the output scales of the columns this wavefront finishes (see the
+  // end), requested first of all and kept as raw bits; fetched where they are used they are one more
+  // round trip at the very end of the launch.
+  constexpr int kOutIters = (RT * MT + NW - 1) / NW;
+  uint32_t os_raw[kOutIters];
+#pragma unroll
+  for (int it = 0; it < kOutIters; ++it) os_raw[it] = 0;
+  float os_pert = 1.0f;
+  if constexpr (kIsFp8 && SC == SC_PERT) os_pert = s32[0];
+  if constexpr (kIsFp8 && SC == SC_PERN) {
+#pragma unroll
+    for (int it = 0; it < kOutIters; ++it) {
+      const int n = min(n0 + ((wave + it * NW) / MT) * 16 + j, N - 1);
+      os_raw[it] = a.scale_f16 ? (uint32_t)reinterpret_cast<const uint16_t*>(s16)[n] : reinterpret_cast<const uint32_t*>(s32)[n];
+    }
+  }
+
   // Out-of-range granules / lanes / rows load zeros for both operands, so the
   // loop body needs no branches: a zero weight times a zero activation adds 0.
   //
@@ -445,7 +462,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   __syncthreads();
   // D layout: lane holds output column n0 + 16 t + j, rows mt*16 + 4 g + v.
   Elem* out = (Elem*)a.out[mat] + (size_t)m0 * N;
-  for (int o = wave; o < RT * MT; o += NW) {
+#pragma unroll
+  for (int it = 0; it < kOutIters; ++it) {
+    const int o = wave + it * NW;
+    if (o >= RT * MT) break;
     const int t = o / MT, mt = o - t * MT;
     const int n = n0 + t * 16 + j;
     f32x4 sum = red[0][t][mt][lane];
@@ -453,8 +473,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     for (int w = 1; w < NW; ++w) sum += red[w][t][mt][lane];
     if (n < nend) {
       float os = 1.0f;
-      if constexpr (kIsFp8 && SC == SC_PERN) os = a.scale_f16 ? (float)s16[n] : s32[n];
-      if constexpr (kIsFp8 && SC == SC_PERT) os = s32[0];
+      if constexpr (kIsFp8 && SC == SC_PERN)
+        os = a.scale_f16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)os_raw[it]) : __builtin_bit_cast(float, os_raw[it]);
+      if constexpr (kIsFp8 && SC == SC_PERT) os = os_pert;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int m = mt * 16 + g * 4 + v;
