@@ -119,25 +119,6 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   // one that reads 1 KiB in a row (measured: 256 workgroups x 32 rows x 4096, 6.5 against 1.6 us).
   // A 16-row tile of the slice is two LDS tiles wide (16-bit elements), so it is staged in two
   // halves; slot [mt][hx NQ/2 + i / 2][i % 2] holds load i of half hx until the transposition.
-  // The output scales of the columns this wavefront finishes (see the end), requested first of all and
-  // kept as raw bits: fetched where they are used they are one more round trip at the very end of
-  // the launch, with nothing left to hide it.
-  constexpr int kOutIters = (kMaxTiles * MT + NW - 1) / NW;
-  uint32_t os_raw[kOutIters];
-#pragma unroll
-  for (int it = 0; it < kOutIters; ++it) os_raw[it] = 0;
-  float os_pert = 1.0f;
-  if constexpr (FMT == 0 && !BLOCK) {
-    if (scale_mode == SC_PERT) os_pert = ((const float*)a.s[mat])[0];
-    if (scale_mode != SC_PERT) {
-#pragma unroll
-      for (int it = 0; it < kOutIters; ++it) {
-        const int o = wave + it * NW;
-        const int n = min(n0 + (o / MT) * 16 + j, N - 1);
-        os_raw[it] = a.scale_f16 ? (uint32_t)((const uint16_t*)a.s[mat])[n] : ((const uint32_t*)a.s[mat])[n];
-      }
-    }
-  }
   u32x4 xq[MT][NQ][2];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -324,6 +305,28 @@ __global__ __launch_bounds__(kKsliceWaves * 64) void kslice_kernel(const SkinnyA
   Tile w0, w1;
   load_tile(w0, 0);
   load_tile(w1, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  // The output scales of the columns this wavefront finishes (see the end), requested behind the
+  // first weight tiles and kept as raw bits: fetched where they are used they are one more round
+  // trip at the very end of the launch, with nothing left to hide it.  (Not ahead of the weight
+  // loads: the compiler may pick the pending scale register as the don't-care half of a 64-bit
+  // address multiply-add, and the first weight load then waits for the scale.)
+  constexpr int kOutIters = (kMaxTiles * MT + NW - 1) / NW;
+  uint32_t os_raw[kOutIters];
+#pragma unroll
+  for (int it = 0; it < kOutIters; ++it) os_raw[it] = 0;
+  float os_pert = 1.0f;
+  if constexpr (FMT == 0 && !BLOCK) {
+    if (scale_mode == SC_PERT) os_pert = ((const float*)a.s[mat])[0];
+    if (scale_mode != SC_PERT) {
+#pragma unroll
+      for (int it = 0; it < kOutIters; ++it) {
+        const int o = wave + it * NW;
+        const int n = min(n0 + (o / MT) * 16 + j, N - 1);
+        os_raw[it] = a.scale_f16 ? (uint32_t)((const uint16_t*)a.s[mat])[n] : ((const uint32_t*)a.s[mat])[n];
+      }
+    }
+  }
   __builtin_amdgcn_sched_barrier(0);
   transpose_x();
   // Tiles 0 .. 3 with static register slots.  Every load is issued unconditionally (a tile past
