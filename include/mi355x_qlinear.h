@@ -458,6 +458,19 @@ int mi_moe_gate_up_fp8_routed(const void* a, const float* a_scale, const int32_t
                               int32_t* sorted_pairs, void* out, int E, int N, int K, int act_dtype,
                               void* stream);
 
+/* Decode form of the same product for a handful of (token, expert) routes: one GEMV per route,
+ * out[r, :] = (x[r / x_div, :] @ dequant(w[e_r])^T) * route_weight[r], e_r = route_expert[r] (held into
+ * [0, num_experts)); all routes in ONE launch of the row GEMV (a wavefront per weight row, routes as
+ * the grid's second dimension), so each expert's weights stream at the full rate instead of through
+ * the few workgroups a grouped launch has work for.  x [tokens, K] and out [routes, out_stride] in
+ * the activation type, w [E, N, K] e4m3 with 128 x 128 block scales w_scale [E, ceil(N/128), K/128],
+ * route_weight (optional) in the activation type.  K % 128 == 0; at most 65535 routes.  The
+ * small-batch form of moe_forward_full_fp8_block's expert loop
+ * (V/csrc/moe_batch/moe.sycl:1509-1663: one work-item row per (token, route)). */
+int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, const void* w, const float* w_scale, void* out,
+                                 long long out_stride, const int32_t* route_expert, const void* route_weight,
+                                 int routes, int num_experts, int N, int K, int act_dtype, void* stream);
+
 /* The same GEMM with the per-expert-scalar scale of the reference's per-tensor MoE
  * kernels and their epilogues:
  *   scale_per_expert = 1: w_scale is [E] fp32 (one factor per expert); K may then be

@@ -889,15 +889,15 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st, int routes = 1) {
 
 // Routed launch (one activation row per route, expert-indexed matrices): one row per batch,
 // activations staged through LDS; the routes are the grid's second dimension.
-template <class Act, int FMT>
+template <class Act, int FMT, int SC = 0>
 static void launch_rows_routed(RowsArgs a, int routes, hipStream_t st) {
   constexpr bool kByte = rows_byte_fmt(FMT);
   constexpr int ppl = kByte ? 2 : 4;
   constexpr int span_k = 64 * ppl * 8;
   constexpr int SPU = kByte ? 4 : 2;
   a.nspan = (a.K + span_k - 1) / span_k;
-  if (a.nspan == 1) return launch_rows_rw<Act, FMT, 0, 1, 1, 1, false, false, true>(a, st, routes);
-  launch_rows_rw<Act, FMT, 0, 1, 1, SPU, false, false, true>(a, st, routes);
+  if (a.nspan == 1) return launch_rows_rw<Act, FMT, SC, 1, 1, 1, false, false, true>(a, st, routes);
+  launch_rows_rw<Act, FMT, SC, 1, 1, SPU, false, false, true>(a, st, routes);
 }
 
 // Batch shape by row length.  Rows of up to one batch (fp8: 4 spans = 4096 k,

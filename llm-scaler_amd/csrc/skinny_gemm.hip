@@ -57,6 +57,29 @@ int mi_gemm_fp8_blockscale_multi(const void* x, int nmat, const void* const* w,
   return run<0, SC_BLOCK>(a, act_dtype, (hipStream_t)stream);
 }
 
+int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, const void* w, const float* w_scale, void* out,
+                                 long long out_stride, const int32_t* route_expert, const void* route_weight,
+                                 int routes, int num_experts, int N, int K, int act_dtype, void* stream) {
+  if (!x || !w || !w_scale || !out || !route_expert) return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (x_div < 1 || num_experts < 1) return MI_ERR_ARG;
+  if (routes < 0 || N < 0 || K <= 0 || (K % 128) || out_stride < N) return MI_ERR_SHAPE;
+  if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || routes > 65535) return MI_ERR_SHAPE;
+  if (rows_lds_bytes(RF_FP8, 1, K) > 64 * 1024) return MI_ERR_SHAPE;
+  if (!routes || !N) return MI_OK;
+  RowsArgs r{};
+  r.x = x; r.nmat = 1; r.M = 1; r.K = K;
+  r.r_expert = route_expert; r.r_out_mul = route_weight; r.r_num_experts = num_experts; r.r_x_div = x_div;
+  r.r_out_stride = out_stride;
+  r.w[0] = w; r.s[0] = w_scale; r.out[0] = out; r.N[0] = N;
+  r.r_w_stride[0] = (long long)N * K;
+  r.r_s_stride[0] = (long long)((N + 127) / 128) * (K / 128) * 4;
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == DT_F16) launch_rows_routed<ActF16, RF_FP8, RS_BLOCK>(r, routes, st);
+  else launch_rows_routed<ActBF16, RF_FP8, RS_BLOCK>(r, routes, st);
+  return launch_status();
+}
+
 int mi_gemm_fp8_blockscale(const void* x, const void* w, const float* scale, void* out, int M, int N,
                            int K, int act_dtype, void* stream) {
   return mi_gemm_fp8_blockscale_multi(x, 1, &w, &scale, &out, &N, M, K, act_dtype, stream);

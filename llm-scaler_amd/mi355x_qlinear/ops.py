@@ -1049,6 +1049,7 @@ def moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, 
 
 
 ROUTED_MAX_PAIRS = 8192       # (token, route) pairs one routed gate_up launch sorts by itself
+ROUTED_GEMV_MAX_PAIRS = 64    # (token, route) pairs up to which the fused decode op runs one GEMV per route
 
 
 def moe_gate_up_fp8_routed(xq, xs, top_ids, weight, weight_scale, expert_start, inv, sorted_pairs, output,
@@ -1211,6 +1212,27 @@ def moe_forward_full_fp8_block(x, logits, output, gate_up_weight, gate_up_scale,
     gate = torch.empty(T, dtype=torch.float32, device=dev)
     # routing and the shared expert's gate sigmoid(x . w) in one launch
     esimd_moe_topk(logits, top_w, top_ids, T, gate=(x, shared_expert_gate_weight, gate))
+    if P <= ROUTED_GEMV_MAX_PAIRS:
+        # Decode: one GEMV per (token, route), all routes in one launch per projection (no sort, no
+        # grouping: with a handful of rows a grouped launch has work for a few workgroups only and
+        # streams each expert's weights at a fraction of the device's rate).  The shared expert's rows
+        # follow the routed ones in the same buffers, so one SiLU * up launch serves both.
+        adt = capi.act_dtype(x)
+        gu = torch.empty(P + T, 2 * I, dtype=x.dtype, device=dev)
+        capi.call("mi_moe_gemv_fp8_block_routed", x, capi.ptr(x), k, capi.ptr(gate_up_weight), capi.ptr(gate_up_scale),
+                  capi.ptr(gu), 2 * I, capi.ptr(top_ids), None, P, E, 2 * I, H, adt)
+        esimd_gemm_fp8_blockscale(x, shared_gate_up_weight, shared_gate_up_scale, gu[P:], 128, 128)
+        act = torch.empty(P + T, I, dtype=x.dtype, device=dev)
+        esimd_moe_silu_mul(gu, act, 2 * I, I, P + T)
+        # the routing weight multiplies each route's row before it is rounded; the sum is then plain
+        y = torch.empty(P, H, dtype=x.dtype, device=dev)
+        capi.call("mi_moe_gemv_fp8_block_routed", act, capi.ptr(act), 1, capi.ptr(down_weight), capi.ptr(down_scale),
+                  capi.ptr(y), H, capi.ptr(top_ids), capi.ptr(top_w), P, E, H, I, adt)
+        sh_out = torch.empty(T, H, dtype=x.dtype, device=dev)
+        esimd_gemm_fp8_blockscale(act[P:], shared_down_weight, shared_down_scale, sh_out, 128, 128)
+        capi.call("mi_moe_combine_shared", y, capi.ptr(y), None, None, capi.ptr(output), capi.ptr(sh_out),
+                  capi.ptr(gate), H, k, T, 0, adt, 0)
+        return output
     sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
     start = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(P, dtype=torch.int32, device=dev)

@@ -616,6 +616,36 @@ def test_moe_forward_full_fp8_block(v, dev, T, dtype):
     assert mean_rel < bar and cos > (0.9999 if dtype == torch.float16 else 0.999)
 
 
+@pytest.mark.parametrize("routes,E,N,K,dt,weighted", [(8, 16, 1536, 2048, torch.bfloat16, False),
+                                                      (12, 8, 384, 256, torch.float16, True),
+                                                      (1, 4, 128, 1152, torch.float16, True)])
+def test_routed_fp8_block_gemv(dev, routes, E, N, K, dt, weighted):
+    """One block-scaled FP8 GEMV per (token, expert) route in one launch: each route's row against
+    the oracle's dequantised expert matrix (1e-2 with the mean floor), ids outside the range held
+    into it, the optional routing weight applied before the rounding."""
+    from mi355x_qlinear import capi
+    g = torch.Generator().manual_seed(routes * 31 + N)
+    k = 2 if routes % 2 == 0 else 1
+    T = routes // k
+    x = (torch.randn(T, K, generator=g) * 0.5).to(dt)
+    w, ws = O.fp8_quantize_block(torch.randn(E, N, K, generator=g) * 0.1)
+    ids = torch.randint(0, E, (routes,), generator=g).to(torch.int32)
+    ids[0] = E + 3                                          # held into the range: expert E - 1
+    rw = (torch.rand(routes, generator=g) + 0.25).to(dt) if weighted else None
+    xd, wd, wsd, idd = x.to(dev), w.to(dev), ws.to(dev), ids.to(dev)
+    out = torch.full((routes, N + 8), 7.0, dtype=dt, device=dev)       # rows 8 elements apart from dense
+    capi.call("mi_moe_gemv_fp8_block_routed", xd, capi.ptr(xd), k, capi.ptr(wd), capi.ptr(wsd), capi.ptr(out), N + 8,
+              capi.ptr(idd), capi.ptr(rw.to(dev)) if weighted else None, routes, E, N, K, capi.act_dtype(xd))
+    dw = O.fp8_dequant_block(w, ws)
+    for r in range(routes):
+        e = min(max(int(ids[r]), 0), E - 1)
+        ref = x[r // k].float() @ dw[e].t()
+        if weighted:
+            ref = ref * rw[r].float()
+        assert O.max_rel_err(out[r, :N].cpu(), ref) < TOL, (r, e)
+    assert bool((out[:, N:] == 7.0).all())
+
+
 def test_moe_forward_full_fp8_block_errors(v, dev):
     top_k = 4
     x, logits, w13, s13, sw13, ss13, w2, s2, sw2, ss2, gate = _full_case(4, 7, torch.float16)
