@@ -459,17 +459,25 @@ int mi_moe_gate_up_fp8_routed(const void* a, const float* a_scale, const int32_t
                               void* stream);
 
 /* Decode form of the same product for a handful of (token, expert) routes: one GEMV per route,
- * out[r, :] = (x[r / x_div, :] @ dequant(w[e_r])^T) * route_weight[r], e_r = route_expert[r] (held into
- * [0, num_experts)); all routes in ONE launch of the row GEMV (a wavefront per weight row, routes as
- * the grid's second dimension), so each expert's weights stream at the full rate instead of through
- * the few workgroups a grouped launch has work for.  x [tokens, K] and out [routes, out_stride] in
- * the activation type, w [E, N, K] e4m3 with 128 x 128 block scales w_scale [E, ceil(N/128), K/128],
- * route_weight (optional) in the activation type.  K % 128 == 0; at most 65535 routes.  The
- * small-batch form of moe_forward_full_fp8_block's expert loop
- * (V/csrc/moe_batch/moe.sycl:1509-1663: one work-item row per (token, route)). */
-int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, const void* w, const float* w_scale, void* out,
-                                 long long out_stride, const int32_t* route_expert, const void* route_weight,
-                                 int routes, int num_experts, int N, int K, int act_dtype, void* stream);
+ * out[r, :] = (act(x[r / x_div, :]) @ dequant(w[e_r])^T) * route_weight[r], e_r = route_expert[r] (held
+ * into [0, num_experts)); all routes in ONE launch of the row GEMV (a wavefront per weight row, routes
+ * as the grid's second dimension), so each expert's weights stream at the full rate instead of
+ * through the few workgroups a grouped launch has work for.  x [rows, K] and out [routes +
+ * shared_rows, out_stride] in the activation type, w [E, N, K] e4m3 with 128 x 128 block scales
+ * w_scale [E, ceil(N/128), K/128], route_weight (optional) in the activation type.
+ * x_silu = 1: a row of x is 2 K wide, gate then up, and act(row) = silu(gate) * up rounded to the
+ *   activation type (mi_moe_silu_mul fused into the staging of the row); 0: act is the identity.
+ * shared_w / shared_scale (optional, one matrix [N, K] with its block scales): shared_rows further
+ *   rows r = routes + i run against it -- the layer's shared expert in the same launch -- with
+ *   activation row shared_x_first + i and no route weight.
+ * K % 128 == 0; at most 65535 rows.  The small-batch form of moe_forward_full_fp8_block's expert loop
+ * (V/csrc/moe_batch/moe.sycl:1509-1663: one work-item row per (token, route), the shared expert
+ * beside them). */
+int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, int x_silu, const void* w, const float* w_scale,
+                                 void* out, long long out_stride, const int32_t* route_expert,
+                                 const void* route_weight, int routes, int num_experts, const void* shared_w,
+                                 const float* shared_scale, int shared_rows, int shared_x_first, int N, int K,
+                                 int act_dtype, void* stream);
 
 /* The same GEMM with the per-expert-scalar scale of the reference's per-tensor MoE
  * kernels and their epilogues:

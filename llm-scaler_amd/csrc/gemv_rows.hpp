@@ -71,6 +71,13 @@ struct RowsArgs {
   // expert e start e * r_*_stride[i] bytes into w / s / z / h, the activation row is row
   // r / r_x_div of x, the output row is r (r_out_stride elements apart) and is multiplied by
   // r_out_mul[r] when that is given.
+  // r_alt_w (optional): routes r >= r_alt_from run against this one matrix (scales r_alt_s) instead
+  // of an expert's -- a layer's shared expert in the same launch; their activation row is
+  // r_alt_x_first + (r - r_alt_from) and they are not multiplied by r_out_mul.
+  // ROUTED == 2: a row of x holds 2 K elements, gate then up, and the activation is silu(gate) * up.
+  const void* r_alt_w;
+  const void* r_alt_s;
+  int r_alt_from, r_alt_x_first;
   const int32_t* r_expert;
   const void* r_out_mul;
   int r_num_experts, r_x_div;
@@ -123,7 +130,7 @@ __device__ __forceinline__ void fp8x4_to_pairs(uint32_t w, uint32_t& p0, uint32_
 // consumed (two register buffers).  Weight loads carry the non-temporal hint:
 // every byte is used exactly once.
 template <class Act, int FMT, int SC, int MR, int NWV, int RW, int SPU, int NBUF, bool MULTI, bool XREG,
-          bool NORM = false, bool ROUTED = false>
+          bool NORM = false, int ROUTED = 0>
 __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in) {
   static_assert(!NORM || (MR == 1 && !XREG), "the fused norm stages one activation row through LDS");
   static_assert(!ROUTED || (MR == 1 && !NORM), "routed launches take one activation row per route");
@@ -134,7 +141,8 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
   if constexpr (ROUTED) {
     a_route = a_in;
     const int r = blockIdx.y;
-    int e = a_in.r_expert[r];
+    const bool alt = a_in.r_alt_w != nullptr && r >= a_in.r_alt_from;   // uniform
+    int e = a_in.r_expert[alt ? 0 : r];
     e = e < 0 ? 0 : (e >= a_in.r_num_experts ? a_in.r_num_experts - 1 : e);
 #pragma unroll
     for (int i = 0; i < kRowsMaxMat; ++i) {
@@ -144,8 +152,10 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
       a_route.h[i] = a_in.h[i] ? (const char*)a_in.h[i] + (long long)e * a_in.r_h_stride[i] : nullptr;
       a_route.out[i] = a_in.out[i] ? (char*)a_in.out[i] + (long long)r * a_in.r_out_stride * 2 : nullptr;
     }
-    a_route.x = (const char*)a_in.x + (long long)(r / a_in.r_x_div) * a_in.K * 2;
-    if (a_in.r_out_mul) route_mul = Act::to_f32(((const typename Act::elem*)a_in.r_out_mul)[r]);
+    if (alt) { a_route.w[0] = a_in.r_alt_w; a_route.s[0] = a_in.r_alt_s; }
+    const long long xrow = alt ? a_in.r_alt_x_first + (r - a_in.r_alt_from) : r / a_in.r_x_div;
+    a_route.x = (const char*)a_in.x + xrow * a_in.K * (ROUTED == 2 ? 4 : 2);
+    if (a_in.r_out_mul && !alt) route_mul = Act::to_f32(((const typename Act::elem*)a_in.r_out_mul)[r]);
   }
   const RowsArgs& a = ROUTED ? a_route : a_in;
   constexpr bool kFp8 = FMT == RF_FP8;
@@ -308,9 +318,23 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
   // issued BEFORE the weight prefetch: waiting for them then leaves the weight
   // loads in flight.  XPRE loads per thread go out up front; anything beyond
   // that (large M x K) is fetched after the prefetch and waits for it.
-  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+  constexpr bool XACT = ROUTED == 2;                  // the activation is silu(gate) * up of a 2 K wide row
+  static_assert(!XACT || !XREG, "the fused activation goes through the LDS staging");
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * (XACT ? 4u : 2u));
   const int total = MR * pieces_per_row;
   constexpr int XPRE = 4;
+  // eight gate and eight up values -> eight activations, fp32 inside, one rounding (what
+  // silu_mul_kernel computes)
+  auto act_mul = [&](u32x4 gv, u32x4 uv) -> u32x4 {
+    const typename Act::v8 g8 = as_v8<typename Act::v8>(gv), u8 = as_v8<typename Act::v8>(uv);
+    typename Act::v8 o8;
+#pragma unroll
+    for (int e2 = 0; e2 < 8; ++e2) {
+      const float gf = Act::to_f32(g8[e2]), uf = Act::to_f32(u8[e2]);
+      o8[e2] = Act::from_f32(gf / (1.0f + expf(-gf)) * uf);
+    }
+    return __builtin_bit_cast(u32x4, o8);
+  };
   auto x_offset = [&](int p) -> uint32_t {
     const int m = (p >= pieces_per_row) + (p >= 2 * pieces_per_row) + (p >= 3 * pieces_per_row);
     const int q = p - m * pieces_per_row;          // (s*PPL + i)*64 + l
@@ -387,9 +411,14 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
         }
   }
   u32x4 xpre[XPRE];
+  [[maybe_unused]] u32x4 upre[XACT ? XPRE : 1];
   if constexpr (!XREG) {
 #pragma unroll
     for (int t = 0; t < XPRE; ++t) xpre[t] = buf_load16(xr, x_offset(threadIdx.x + t * NWV * 64));
+    if constexpr (XACT) {
+#pragma unroll
+      for (int t = 0; t < XPRE; ++t) upre[t] = buf_load16(xr, x_offset(threadIdx.x + t * NWV * 64) + (uint32_t)K * 2u);
+    }
   }
   // NORM: residual, gate and norm weight of the same pieces (a null operand reads zeros)
   u32x4 nres[NORM ? XPRE : 1], ngate[NORM ? XPRE : 1], nwgt[NORM ? XPRE : 1];
@@ -551,9 +580,12 @@ __global__ __launch_bounds__(NWV * 64) void gemv_rows_kernel(const RowsArgs a_in
     __syncthreads();
   } else {
 #pragma unroll
-    for (int t = 0; t < XPRE; ++t) x_store(threadIdx.x + t * NWV * 64, xpre[t]);
-    for (int p = threadIdx.x + XPRE * NWV * 64; p < total; p += NWV * 64)
-      x_store(p, buf_load16(xr, x_offset(p)));
+    for (int t = 0; t < XPRE; ++t) x_store(threadIdx.x + t * NWV * 64, XACT ? act_mul(xpre[t], upre[t]) : xpre[t]);
+    for (int p = threadIdx.x + XPRE * NWV * 64; p < total; p += NWV * 64) {
+      const u32x4 xv = buf_load16(xr, x_offset(p));
+      if constexpr (XACT) x_store(p, act_mul(xv, buf_load16(xr, x_offset(p) + (uint32_t)K * 2u)));
+      else x_store(p, xv);
+    }
     if constexpr (kSums) {
       // per 32-k chunk sums, from the staged image
       __syncthreads();
@@ -849,7 +881,7 @@ static inline int device_cu_count() {
   return cus;
 }
 
-template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG, bool NORM = false, bool ROUTED = false>
+template <class Act, int FMT, int SC, int MR, int RW, int SPU, bool XREG, bool NORM = false, int ROUTED = 0>
 static void launch_rows_rw(RowsArgs a, hipStream_t st, int routes = 1) {
   constexpr int NWV = 8;
   constexpr int NBUF = 2;
@@ -889,15 +921,15 @@ static void launch_rows_rw(RowsArgs a, hipStream_t st, int routes = 1) {
 
 // Routed launch (one activation row per route, expert-indexed matrices): one row per batch,
 // activations staged through LDS; the routes are the grid's second dimension.
-template <class Act, int FMT, int SC = 0>
+template <class Act, int FMT, int SC = 0, int ROUTED = 1>
 static void launch_rows_routed(RowsArgs a, int routes, hipStream_t st) {
   constexpr bool kByte = rows_byte_fmt(FMT);
   constexpr int ppl = kByte ? 2 : 4;
   constexpr int span_k = 64 * ppl * 8;
   constexpr int SPU = kByte ? 4 : 2;
   a.nspan = (a.K + span_k - 1) / span_k;
-  if (a.nspan == 1) return launch_rows_rw<Act, FMT, SC, 1, 1, 1, false, false, true>(a, st, routes);
-  launch_rows_rw<Act, FMT, SC, 1, 1, SPU, false, false, true>(a, st, routes);
+  if (a.nspan == 1) return launch_rows_rw<Act, FMT, SC, 1, 1, 1, false, false, ROUTED>(a, st, routes);
+  launch_rows_rw<Act, FMT, SC, 1, 1, SPU, false, false, ROUTED>(a, st, routes);
 }
 
 // Batch shape by row length.  Rows of up to one batch (fp8: 4 spans = 4096 k,

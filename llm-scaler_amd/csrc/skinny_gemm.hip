@@ -57,16 +57,20 @@ int mi_gemm_fp8_blockscale_multi(const void* x, int nmat, const void* const* w,
   return run<0, SC_BLOCK>(a, act_dtype, (hipStream_t)stream);
 }
 
-int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, const void* w, const float* w_scale, void* out,
-                                 long long out_stride, const int32_t* route_expert, const void* route_weight,
-                                 int routes, int num_experts, int N, int K, int act_dtype, void* stream) {
+int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, int x_silu, const void* w, const float* w_scale,
+                                 void* out, long long out_stride, const int32_t* route_expert,
+                                 const void* route_weight, int routes, int num_experts, const void* shared_w,
+                                 const float* shared_scale, int shared_rows, int shared_x_first, int N, int K,
+                                 int act_dtype, void* stream) {
   if (!x || !w || !w_scale || !out || !route_expert) return MI_ERR_ARG;
   if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
-  if (x_div < 1 || num_experts < 1) return MI_ERR_ARG;
+  if (x_div < 1 || num_experts < 1 || x_silu < 0 || x_silu > 1) return MI_ERR_ARG;
+  if ((shared_w != nullptr) != (shared_scale != nullptr) || shared_rows < 0 || shared_x_first < 0) return MI_ERR_ARG;
+  if (!shared_w) shared_rows = 0;
   if (routes < 0 || N < 0 || K <= 0 || (K % 128) || out_stride < N) return MI_ERR_SHAPE;
-  if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || routes > 65535) return MI_ERR_SHAPE;
+  if ((uint64_t)N * (uint64_t)K >= (1ull << 31) || (long)routes + shared_rows > 65535) return MI_ERR_SHAPE;
   if (rows_lds_bytes(RF_FP8, 1, K) > 64 * 1024) return MI_ERR_SHAPE;
-  if (!routes || !N) return MI_OK;
+  if (!(routes + shared_rows) || !N) return MI_OK;
   RowsArgs r{};
   r.x = x; r.nmat = 1; r.M = 1; r.K = K;
   r.r_expert = route_expert; r.r_out_mul = route_weight; r.r_num_experts = num_experts; r.r_x_div = x_div;
@@ -74,9 +78,16 @@ int mi_moe_gemv_fp8_block_routed(const void* x, int x_div, const void* w, const 
   r.w[0] = w; r.s[0] = w_scale; r.out[0] = out; r.N[0] = N;
   r.r_w_stride[0] = (long long)N * K;
   r.r_s_stride[0] = (long long)((N + 127) / 128) * (K / 128) * 4;
+  if (shared_rows) { r.r_alt_w = shared_w; r.r_alt_s = shared_scale; r.r_alt_from = routes; r.r_alt_x_first = shared_x_first; }
+  const int total = routes + shared_rows;
   hipStream_t st = (hipStream_t)stream;
-  if (act_dtype == DT_F16) launch_rows_routed<ActF16, RF_FP8, RS_BLOCK>(r, routes, st);
-  else launch_rows_routed<ActBF16, RF_FP8, RS_BLOCK>(r, routes, st);
+  if (act_dtype == DT_F16) {
+    if (x_silu) launch_rows_routed<ActF16, RF_FP8, RS_BLOCK, 2>(r, total, st);
+    else launch_rows_routed<ActF16, RF_FP8, RS_BLOCK, 1>(r, total, st);
+  } else {
+    if (x_silu) launch_rows_routed<ActBF16, RF_FP8, RS_BLOCK, 2>(r, total, st);
+    else launch_rows_routed<ActBF16, RF_FP8, RS_BLOCK, 1>(r, total, st);
+  }
   return launch_status();
 }
 

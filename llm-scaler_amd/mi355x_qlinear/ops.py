@@ -1216,21 +1216,19 @@ def moe_forward_full_fp8_block(x, logits, output, gate_up_weight, gate_up_scale,
         # Decode: one GEMV per (token, route), all routes in one launch per projection (no sort, no
         # grouping: with a handful of rows a grouped launch has work for a few workgroups only and
         # streams each expert's weights at a fraction of the device's rate).  The shared expert's rows
-        # follow the routed ones in the same buffers, so one SiLU * up launch serves both.
+        # follow the routed ones in the same launches and buffers: four launches in all.
         adt = capi.act_dtype(x)
         gu = torch.empty(P + T, 2 * I, dtype=x.dtype, device=dev)
-        capi.call("mi_moe_gemv_fp8_block_routed", x, capi.ptr(x), k, capi.ptr(gate_up_weight), capi.ptr(gate_up_scale),
-                  capi.ptr(gu), 2 * I, capi.ptr(top_ids), None, P, E, 2 * I, H, adt)
-        esimd_gemm_fp8_blockscale(x, shared_gate_up_weight, shared_gate_up_scale, gu[P:], 128, 128)
-        act = torch.empty(P + T, I, dtype=x.dtype, device=dev)
-        esimd_moe_silu_mul(gu, act, 2 * I, I, P + T)
-        # the routing weight multiplies each route's row before it is rounded; the sum is then plain
-        y = torch.empty(P, H, dtype=x.dtype, device=dev)
-        capi.call("mi_moe_gemv_fp8_block_routed", act, capi.ptr(act), 1, capi.ptr(down_weight), capi.ptr(down_scale),
-                  capi.ptr(y), H, capi.ptr(top_ids), capi.ptr(top_w), P, E, H, I, adt)
-        sh_out = torch.empty(T, H, dtype=x.dtype, device=dev)
-        esimd_gemm_fp8_blockscale(act[P:], shared_down_weight, shared_down_scale, sh_out, 128, 128)
-        capi.call("mi_moe_combine_shared", y, capi.ptr(y), None, None, capi.ptr(output), capi.ptr(sh_out),
+        capi.call("mi_moe_gemv_fp8_block_routed", x, capi.ptr(x), k, 0, capi.ptr(gate_up_weight), capi.ptr(gate_up_scale),
+                  capi.ptr(gu), 2 * I, capi.ptr(top_ids), None, P, E, capi.ptr(shared_gate_up_weight),
+                  capi.ptr(shared_gate_up_scale), T, 0, 2 * I, H, adt)
+        # down projections: SiLU(gate) * up is applied while a row is staged; the routing weight
+        # multiplies each route's row before it is rounded, so the sum over routes is plain
+        y = torch.empty(P + T, H, dtype=x.dtype, device=dev)
+        capi.call("mi_moe_gemv_fp8_block_routed", gu, capi.ptr(gu), 1, 1, capi.ptr(down_weight), capi.ptr(down_scale),
+                  capi.ptr(y), H, capi.ptr(top_ids), capi.ptr(top_w), P, E, capi.ptr(shared_down_weight),
+                  capi.ptr(shared_down_scale), T, P, H, I, adt)
+        capi.call("mi_moe_combine_shared", y, capi.ptr(y), None, None, capi.ptr(output), capi.ptr(y[P:]),
                   capi.ptr(gate), H, k, T, 0, adt, 0)
         return output
     sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)

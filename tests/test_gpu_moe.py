@@ -633,9 +633,10 @@ def test_routed_fp8_block_gemv(dev, routes, E, N, K, dt, weighted):
     ids[0] = E + 3                                          # held into the range: expert E - 1
     rw = (torch.rand(routes, generator=g) + 0.25).to(dt) if weighted else None
     xd, wd, wsd, idd = x.to(dev), w.to(dev), ws.to(dev), ids.to(dev)
+    rwd = rw.to(dev) if weighted else None
     out = torch.full((routes, N + 8), 7.0, dtype=dt, device=dev)       # rows 8 elements apart from dense
-    capi.call("mi_moe_gemv_fp8_block_routed", xd, capi.ptr(xd), k, capi.ptr(wd), capi.ptr(wsd), capi.ptr(out), N + 8,
-              capi.ptr(idd), capi.ptr(rw.to(dev)) if weighted else None, routes, E, N, K, capi.act_dtype(xd))
+    capi.call("mi_moe_gemv_fp8_block_routed", xd, capi.ptr(xd), k, 0, capi.ptr(wd), capi.ptr(wsd), capi.ptr(out), N + 8,
+              capi.ptr(idd), capi.ptr(rwd), routes, E, None, None, 0, 0, N, K, capi.act_dtype(xd))
     dw = O.fp8_dequant_block(w, ws)
     for r in range(routes):
         e = min(max(int(ids[r]), 0), E - 1)
@@ -644,6 +645,24 @@ def test_routed_fp8_block_gemv(dev, routes, E, N, K, dt, weighted):
             ref = ref * rw[r].float()
         assert O.max_rel_err(out[r, :N].cpu(), ref) < TOL, (r, e)
     assert bool((out[:, N:] == 7.0).all())
+    # rows of a shared matrix in the same launch, and SiLU(gate) * up fused into the staging of x:
+    # x2 rows are [gate | up], 2 K wide; shared row i reads x2 row 1 + i
+    sw, sws = O.fp8_quantize_block(torch.randn(N, K, generator=g) * 0.1)
+    x2 = (torch.randn(routes + 3, 2 * K, generator=g) * 0.7).to(dt)
+    act = O.silu_mul(x2).to(dt)
+    x2d, swd, swsd = x2.to(dev), sw.to(dev), sws.to(dev)
+    out2 = torch.full((routes + 2, N), 7.0, dtype=dt, device=dev)
+    capi.call("mi_moe_gemv_fp8_block_routed", x2d, capi.ptr(x2d), 1, 1, capi.ptr(wd), capi.ptr(wsd), capi.ptr(out2), N,
+              capi.ptr(idd), capi.ptr(rwd), routes, E, capi.ptr(swd), capi.ptr(swsd), 2, 1, N, K, capi.act_dtype(xd))
+    dsw = O.fp8_dequant_block(sw, sws)
+    for r in range(routes):
+        e = min(max(int(ids[r]), 0), E - 1)
+        ref = act[r].float() @ dw[e].t()
+        if weighted:
+            ref = ref * rw[r].float()
+        assert O.max_rel_err(out2[r].cpu(), ref) < TOL, (r, e)
+    for i in range(2):
+        assert O.max_rel_err(out2[routes + i].cpu(), act[1 + i].float() @ dsw.t()) < TOL, i
 
 
 def test_moe_forward_full_fp8_block_errors(v, dev):
