@@ -929,6 +929,12 @@ static void launch_rows_routed(RowsArgs a, int routes, hipStream_t st) {
   constexpr int SPU = kByte ? 4 : 2;
   a.nspan = (a.K + span_k - 1) / span_k;
   if (a.nspan == 1) return launch_rows_rw<Act, FMT, SC, 1, 1, 1, false, false, ROUTED>(a, st, routes);
+  if constexpr (kByte) {
+    // a batch of exactly the row's spans: an empty span slot would still cost a dead load and a pass
+    // of arithmetic on zeros
+    if (a.nspan == 2) return launch_rows_rw<Act, FMT, SC, 1, 1, 2, false, false, ROUTED>(a, st, routes);
+    if (a.nspan == 3) return launch_rows_rw<Act, FMT, SC, 1, 1, 3, false, false, ROUTED>(a, st, routes);
+  }
   launch_rows_rw<Act, FMT, SC, 1, 1, SPU, false, false, ROUTED>(a, st, routes);
 }
 
