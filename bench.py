@@ -487,6 +487,52 @@ def wl_moe_forward_full(dev):
                 kernel="km_up_kernel", cpu=cpu)
 
 
+def wl_moe_fp8_block_decode(dev, T=1):
+    """The reference's fused small-batch MoE op for 128x128 block-FP8 weights (moe_forward_full_fp8_block,
+    vllm/custom-esimd-kernels-vllm/csrc/moe_batch/moe.sycl:1707-1853; called per layer by the patched
+    Qwen3-Next MoE block, vllm/patches/vllm_for_multi_arc.patch:9972-9989) at cfg3's layer shape: T tokens,
+    128 experts, top 8, one shared expert.  Each launch prefers eight other experts and runs on another
+    copy of the shared expert, so nothing is served from the Infinity Cache."""
+    import custom_esimd_kernels_vllm  # noqa: F401
+    from oracle import qlinear_oracle as O
+    E, K, H, I = 128, 8, 2048, 768
+    g = torch.Generator(device=dev).manual_seed(97)
+    f8 = lambda *shape: ((torch.randn(*shape, generator=g, device=dev)).clamp(-3, 3) * 60).to(torch.float8_e4m3fn)
+    x = (torch.randn(T, H, generator=g, device=dev) * 0.3).to(torch.bfloat16)
+    w13, w2 = f8(E, 2 * I, H), f8(E, H, I)
+    s13 = torch.rand(E, 2 * I // 128, H // 128, generator=g, device=dev) * 2e-4 + 1e-4
+    s2 = torch.rand(E, H // 128, I // 128, generator=g, device=dev) * 2e-4 + 1e-4
+    R = 64
+    sw13 = [f8(2 * I, H) for _ in range(R)]
+    sw2 = [f8(H, I) for _ in range(R)]
+    ss13 = torch.full((2 * I // 128, H // 128), 2e-4, device=dev)
+    ss2 = torch.full((H // 128, I // 128), 2e-4, device=dev)
+    gate = (torch.randn(1, H, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    sets = E // K
+    logits = []
+    for i in range(sets):                            # launch i prefers experts [i*K, (i+1)*K)
+        l = torch.randn(T, E, generator=g, device=dev) * 0.1
+        l[:, i * K:(i + 1) * K] += 8.0
+        logits.append(l.to(torch.bfloat16))
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+
+    def launch(i):
+        torch.ops.moe_ops.moe_forward_full_fp8_block(x, logits[i % sets], out, w13, s13, sw13[i % R], ss13, w2, s2,
+                                                     sw2[i % R], ss2, gate, K, 1, E)
+
+    def cpu():
+        u8 = lambda t: t.view(torch.uint8).cpu()
+        return O.moe_forward_full(x.cpu(), logits[0].cpu(), u8(w13), s13.cpu(), u8(sw13[0]), ss13.cpu(), u8(w2),
+                                  s2.cpu(), u8(sw2[0]), ss2.cpu(), gate.cpu(), K)
+
+    alg_bytes = (K + 1) * 3 * H * I + 2 * T * E + 4 * T * H      # T = 1: every route is its own expert
+    flops = 2 * T * (K + 1) * 3 * H * I
+    return dict(launch=launch, R=sets, bytes=alg_bytes, flops=flops, bound="hbm", dtype="bf16",
+                name=f"next: fused block-FP8 MoE decode op (topk + routed up/SiLU/down + shared expert + sum) "
+                     f"T={T} E={E} top{K} H={H} I={I} bf16 (w8a16)",
+                kernel="gemv_rows_kernel (routed)", cpu=cpu)
+
+
 def wl_gemv_fp16(dev):
     """16-bit weight GEMV at the reference test's largest router shape (tests/test_gemv_fp16.py:62-71)."""
     import custom_esimd_kernels_vllm as v
@@ -608,6 +654,7 @@ WORKLOADS = {
     "next_resadd_norm_gemv": wl_resadd_norm_gemv,
     "next_moe_gelu_grouped": wl_moe_gelu,
     "next_moe_forward_full_t1": wl_moe_forward_full,
+    "next_moe_fp8_block_decode_t1": wl_moe_fp8_block_decode,
     "next_gemv_fp16_router": wl_gemv_fp16,
     "next_moe_gguf_t1": wl_moe_gguf,
 }
