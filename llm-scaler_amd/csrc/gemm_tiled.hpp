@@ -629,46 +629,102 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) os_all[ao][v] = Fmt::out_scale(res, p, col_of(ao) + v < N ? col_of(ao) + v : N - 1);
   }
-  // Row tile outermost: the stores that follow each other fill one output row's columns from left to
-  // right (32 bytes each), so a row's 128-byte lines are completed by consecutive instructions and can be
-  // merged on their way to memory.
+  const bool two_scales = p.scale_mode == 3;
+  // the lane's 4 results of (row tile b, column tile ao), before the rounding
+  auto result4 = [&](auto gelu_c, int b, int ao, float (&r)[4]) __attribute__((always_inline)) {
+    const int a = FUSE ? 2 * ao : ao;
 #pragma unroll
-  for (int b = 0; b < TM; ++b) {
-    if (orow[b] < 0) continue;
-#pragma unroll
-    for (int ao = 0; ao < TNO; ++ao) {
-      const int a = FUSE ? 2 * ao : ao;
-      const int n = col_of(ao);
-      Elem v4[4];
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        float r;
-        if constexpr (FUSE) {
-          // one factor per tensor / expert, or one for the gate rows and one for the up rows
-          const float osv = Fmt::kOutScale ? os_all[Fmt::kOutScale ? ao : 0][v] : 1.0f;
-          const float gate = acc[a][b][v] * osv, up = acc[a + 1][b][v] * (p.scale_mode == 3 ? os_up : osv);
-          if (p.gelu) {
-            float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
-            two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
-            const float ex = __expf(two_z);
-            r = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up;
-          } else {
-            r = gate / (1.0f + __expf(-gate)) * up;
-          }
+    for (int v = 0; v < 4; ++v) {
+      const float osv = Fmt::kOutScale ? os_all[Fmt::kOutScale ? ao : 0][v] : 1.0f;
+      if constexpr (FUSE) {
+        // one factor per tensor / expert, or one for the gate rows and one for the up rows
+        const float gate = acc[a][b][v] * osv, up = acc[a + 1][b][v] * (two_scales ? os_up : osv);
+        if constexpr (decltype(gelu_c)::value) {
+          float two_z = 2.0f * (0.7978845608f * (gate + 0.044715f * (gate * gate * gate)));
+          two_z = fminf(fmaxf(two_z, -30.0f), 30.0f);
+          const float ex = __expf(two_z);
+          r[v] = 0.5f * gate * (1.0f + (ex - 1.0f) / (ex + 1.0f)) * up;
         } else {
-          r = Fmt::kOutScale ? acc[a][b][v] * os_all[Fmt::kOutScale ? ao : 0][v] : acc[a][b][v];
+          r[v] = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;   // reciprocal to 1 ulp, before a 16-bit rounding
         }
-        v4[v] = Act::from_f32(GROUPED ? r * rw[b] : r);
-      }
-      Elem* dst = out + (size_t)orow[b] * n_out + n;
-      if (n + 3 < n_out && (n_out & 3) == 0) {
-        *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(v4);
       } else {
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (n + v < n_out) dst[v] = v4[v];
+        r[v] = Fmt::kOutScale ? acc[a][b][v] * osv : acc[a][b][v];
       }
+      if constexpr (GROUPED) r[v] *= rw[b];
     }
+  };
+  const size_t out_bytes = (size_t)(GROUPED ? p.out_rows : p.M) * (size_t)n_out * 2u;
+  constexpr int WNO = FUSE ? WN / 2 : WN;             // output columns of this wavefront
+  constexpr int LPR = WNO / 8;                        // lanes, 16 bytes each, per output row of the wave tile
+  constexpr int RPP = 64 / LPR;                       // rows per store instruction
+  constexpr int PASSES = (16 + RPP - 1) / RPP;
+  constexpr int OPITCH = WNO * 2 + 16;                // a row of the wave tile + a slot for the row's offset
+  static_assert(WNO % 8 == 0 && 4 * 16 * OPITCH <= 2 * BNP * kPitch * 2, "output staging tile");
+  if ((n_out & 7) == 0 && out_bytes < (1ull << 31) && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0) {
+    // Each 16-row tile of results is rounded, turned through a tile in LDS that belongs to this
+    // wavefront alone (the weight tiles are free after the K loop's last barrier; the LDS queue of a
+    // wavefront runs in order, so no barrier) and leaves as 16 bytes per lane, a row's columns in
+    // adjacent lanes: a store instruction writes RPP rows of WNO * 2 contiguous bytes instead of 32
+    // bytes in each of 16 rows — the workgroup's path to L2 takes a request per row piece, whatever
+    // its size.  Rows and column groups outside the output get an offset past the buffer and are dropped.
+    const __amdgpu_buffer_rsrc_t orsrc = make_rsrc(p.out, (uint32_t)out_bytes);
+    unsigned char* otile = smem + wave * (16 * OPITCH);
+    unsigned char* wr_at = otile + j * OPITCH + g * 8;
+    const int rr = lane / LPR, cc = lane - rr * LPR;
+    const int colr = (FUSE ? n0 + (wn0 >> 1) : n0 + wn0) + cc * 8;     // this lane's 8 columns when it stores
+    const bool lane_ok = rr < RPP && colr < n_out;
+    auto emit = [&](auto gelu_c) __attribute__((always_inline)) {
+#pragma unroll
+      for (int b = 0; b < TM; ++b) {
+        if (GROUPED && b >= live) break;              // uniform: the tiles past the expert's rows
+        *reinterpret_cast<uint32_t*>(otile + j * OPITCH + WNO * 2) =
+            orow[b] >= 0 ? (uint32_t)orow[b] * (uint32_t)n_out * 2u : kOOB;
+#pragma unroll
+        for (int ao = 0; ao < TNO; ++ao) {
+          float r[4];
+          result4(gelu_c, b, ao, r);
+          u32x2 d;
+          if constexpr (Act::dt == DT_F16) {
+            d[0] = __builtin_bit_cast(uint32_t, f16x2{(_Float16)r[0], (_Float16)r[1]});
+            d[1] = __builtin_bit_cast(uint32_t, f16x2{(_Float16)r[2], (_Float16)r[3]});
+          } else {
+            d[0] = __builtin_bit_cast(uint32_t, bf16x2{(__bf16)r[0], (__bf16)r[1]});
+            d[1] = __builtin_bit_cast(uint32_t, bf16x2{(__bf16)r[2], (__bf16)r[3]});
+          }
+          *reinterpret_cast<u32x2*>(wr_at + ao * 32) = d;
+        }
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+          const int row = ps * RPP + rr;
+          const unsigned char* src = otile + (row < 16 ? row : 15) * OPITCH;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(src + cc * 16);
+          const uint32_t ro = *reinterpret_cast<const uint32_t*>(src + WNO * 2);
+          const bool ok = lane_ok && row < 16;
+          __builtin_amdgcn_raw_buffer_store_b128(v, orsrc, ok ? ro + (uint32_t)colr * 2u : kOOB, 0, 0);
+        }
+      }
+    };
+    if (FUSE && p.gelu) emit(std::true_type{});
+    else emit(std::false_type{});
+  } else {
+    auto emit = [&](auto gelu_c) __attribute__((always_inline)) {
+#pragma unroll
+      for (int b = 0; b < TM; ++b) {
+        if (orow[b] < 0) continue;
+#pragma unroll
+        for (int ao = 0; ao < TNO; ++ao) {
+          const int n = col_of(ao);
+          float r[4];
+          result4(gelu_c, b, ao, r);
+          Elem* dst = out + (size_t)orow[b] * n_out + n;
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (n + v < n_out) dst[v] = Act::from_f32(r[v]);
+        }
+      }
+    };
+    if (FUSE && p.gelu) emit(std::true_type{});
+    else emit(std::false_type{});
   }
 }
 

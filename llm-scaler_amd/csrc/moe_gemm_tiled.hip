@@ -169,7 +169,6 @@ static int run_grouped(const GemmArgs& p, bool per_expert, int fuse, int max_til
 using namespace qlin;
 
 extern "C" {
-
 int mi_moe_gemm_fp8_tiled_workspace(int total_rows, int E, int K, long long* bytes) {
   if (!bytes) return MI_ERR_ARG;
   if (total_rows < 0 || E < 0 || E > kMapThreads || K <= 0) return MI_ERR_SHAPE;

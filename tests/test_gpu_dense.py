@@ -308,6 +308,25 @@ def test_fp8_prefill_tiled_gemm(ops, dev, M, K, N, dt, mode):
         assert torch.equal(out2.cpu().float(), 2 * o.float())
 
 
+@pytest.mark.parametrize("shift", [1, 4])
+def test_fp8_prefill_output_off_16_byte_alignment(ops, dev, shift):
+    # the tiled GEMM stores 16 bytes per lane when the output allows it; an output that starts 2 or 8
+    # bytes off a 16-byte boundary takes the element-wise stores and must give the same values
+    v, _ = ops
+    M, K, N = 70, 256, 64
+    x, w8, s = O.make_fp8_pern_case(M, K, N, seed=5, act_dtype=torch.bfloat16)
+    xd, wd, sd = x.to(dev), w8.to(dev), s.to(dev)
+    want = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    v.esimd_gemv_fp8_pern(xd, wd, sd, want, N, K)
+    buf = torch.full((M * N + 16,), 7.0, dtype=torch.bfloat16, device=dev)
+    out = buf[shift:shift + M * N].view(M, N)
+    assert out.data_ptr() % 16 != 0
+    v.esimd_gemv_fp8_pern(xd, wd, sd, out, N, K)
+    assert _same_bits(out, want)
+    assert bool((buf[:shift] == 7.0).all()) and bool((buf[shift + M * N:] == 7.0).all())
+    assert O.max_rel_err(want.cpu(), O.matmul_ref(x, O.fp8_dequant_per_channel(w8, s))) < TOL
+
+
 def test_fp8_prefill_c_abi_scratch_route(ops, dev):
     # the C entry point without a workspace argument takes the same route with the library's
     # per-stream scratch buffer and gives the same bits as the op
