@@ -407,6 +407,22 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_
                              const int32_t* out_map, const void* row_weight, int a_rows, int total_rows,
                              int E, int N, int K, int fuse_act, int act_dtype, void* workspace,
                              long long workspace_bytes, void* stream);
+/* The expert MLP of that regime as one call: out = (act(a W13_gate^T) * (a W13_up^T)) W2^T per expert,
+ * w13 [E, 2 I, H] and w2 [E, H, I] E4M3, block scales [E, 2I/128, H/128] / [E, H/128, I/128]
+ * (scale_per_expert 0), one fp32 per expert and matrix (1), or gate / up scalars for w13 and one
+ * for w2 (2); fuse_act 1 = SiLU, 2 = tanh-GELU.  row_map / row_map_div gather the rows of `a`;
+ * out_map / row_weight apply to `out` [rows, H] as in mi_moe_gemm_fp8_tiled_ws.  Bit-identical to
+ * two mi_moe_gemm_fp8_tiled_ws calls with a row-major intermediate between them; the tile table
+ * is built once, and the first GEMM writes the intermediate in the operand order the second
+ * reads, so it is neither stored row-major nor re-tiled.  H % 128 == 0, I % 128 == 0.  Reference:
+ * the gate_up, SiLU x up, down sequence of the fused forward (V/csrc/xpu/moe.sycl:1509-1663) on
+ * the grouped prefill GEMM (V/csrc/xpu/esimd_kernels/fp8_moe_gemm_blockscale.h:304-357). */
+int mi_moe_mlp_fp8_tiled_workspace(int total_rows, int E, int H, int I, long long* bytes);
+int mi_moe_mlp_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_div, const void* w13,
+                            const float* w13_scale, const void* w2, const float* w2_scale, int scale_per_expert,
+                            const int32_t* expert_start, void* out, const int32_t* out_map, const void* row_weight,
+                            int a_rows, int total_rows, int E, int H, int I, int fuse_act, int act_dtype,
+                            void* workspace, long long workspace_bytes, void* stream);
 
 /* ---- prefill (M > 64) on FP8 and Q4_K weights: the tiled matrix-core GEMM ---------
  * The same results as mi_gemm_fp8_pern / _pert / _blockscale and mi_gemv_q4k, computed by the

@@ -60,6 +60,8 @@ struct GemmArgs {
   int n_half;                 // FUSE: weight row n (gate) pairs with row n + n_half (up); N = 2 n_half
   int gelu;                   // FUSE: tanh-GELU instead of SiLU
   int out_rows;               // rows of out (bounds mapped rows)
+  int out_packed;             // GROUPED: out is written in the re-tiled operand order of x (16-row blocks of the
+                              // tile table, n_out / 32 steps each) for a following grouped GEMM; out_rows = 16 x blocks
 };
 
 // MFMA with the accumulator pinned to the AGPR half of the register file and updated in place.
@@ -692,6 +694,23 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const GemmArgs p) {
             d[1] = __builtin_bit_cast(uint32_t, bf16x2{(__bf16)r[2], (__bf16)r[3]});
           }
           *reinterpret_cast<u32x2*>(wr_at + ao * 32) = d;
+        }
+        if constexpr (GROUPED && WNO % 32 == 0) {
+          if (p.out_packed) {
+            // block (activation tile, 32-wide step) = 1 KiB in operand order: lane 16 g + j holds row j,
+            // columns 8 g .. 8 g + 7 of the step; rows past the expert's last are zeros here (their
+            // activations were) as the re-tiling pass would write them
+            const uint32_t tile = (uint32_t)xblk0 + (uint32_t)mtile(b);
+            const int cb = FUSE ? n0 + (wn0 >> 1) : n0 + wn0;
+#pragma unroll
+            for (int qq = 0; qq < WNO / 32; ++qq) {
+              const u32x4 v = *reinterpret_cast<const u32x4*>(otile + j * OPITCH + (qq * 32 + g * 8) * 2);
+              const uint32_t q = (uint32_t)(cb >> 5) + qq;
+              __builtin_amdgcn_raw_buffer_store_b128(
+                  v, orsrc, cb + qq * 32 < n_out ? (tile * (uint32_t)(n_out >> 5) + q) * 1024u + (uint32_t)lane * 16u : kOOB, 0, 0);
+            }
+            continue;
+          }
         }
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {

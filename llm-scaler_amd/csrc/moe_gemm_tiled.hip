@@ -10,7 +10,9 @@
 //   3. the GEMM runs one workgroup per (M-tile, N-tile); the grid is the host-side upper bound
 //      of the tile count and surplus workgroups exit at once.
 // Optional fused epilogue act(gate) * up (SiLU or tanh-GELU), output row map and per-row factor
-// as in the weight-streaming kernel.
+// as in the weight-streaming kernel.  The expert MLP as one call (gate_up, act(gate) * up, down)
+// shares steps 1 and 2 between its two GEMMs: the first writes its result straight into the
+// operand order the second reads, so the intermediate is never re-tiled (nor stored row-major).
 #include "gemm_tiled.hpp"
 #include "scratch.hpp"
 #include "../../include/mi355x_qlinear.h"
@@ -22,48 +24,73 @@ template <class Act, int BN> using WFp8BlockG = WFp8<Act, BN, true>;
 
 constexpr int kMapThreads = 1024;
 
-// exclusive scan of one value per thread over the 1024-thread workgroup
-__device__ __forceinline__ int map_scan(int v, int* tmp, int tid) {
-  tmp[tid] = v;
-  __syncthreads();
-  for (int off = 1; off < kMapThreads; off <<= 1) {
-    const int add = tid >= off ? tmp[tid - off] : 0;
-    __syncthreads();
-    tmp[tid] += add;
-    __syncthreads();
+// exclusive scans of two values per thread over the workgroup (whole wavefronts): inside a wavefront by
+// shuffles, across the wavefronts through their totals
+__device__ __forceinline__ void map_scan2(int& a, int& b, int (*wsum)[2], int tid, int& total_a, int& total_b) {
+  const int lane = tid & 63, w = tid >> 6, nw = blockDim.x >> 6;
+  int ia = a, ib = b;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int ta = __shfl_up(ia, off), tb = __shfl_up(ib, off);
+    if (lane >= off) { ia += ta; ib += tb; }
   }
-  return tmp[tid] - v;
+  if (lane == 63) { wsum[w][0] = ia; wsum[w][1] = ib; }
+  __syncthreads();
+  int ba = 0, bb = 0;
+  total_a = 0; total_b = 0;
+  for (int i = 0; i < nw; ++i) {
+    if (i < w) { ba += wsum[i][0]; bb += wsum[i][1]; }
+    total_a += wsum[i][0]; total_b += wsum[i][1];
+  }
+  a = ba + ia - a;
+  b = bb + ib - b;
 }
 
 // g_tile[4 i] = {expert, first sorted row, rows, first activation block} per M-tile of `bm` rows;
 // blk[2 b] = {first sorted row, rows} per 16-row activation block; counts[0] = M-tiles,
-// counts[1] = blocks.  E <= 1024.
+// counts[1] = blocks.  One workgroup, E <= 1024: thread e scans expert e's counts, then all threads
+// share the table entries (entry -> expert by bisection of the scanned offsets).
 __global__ __launch_bounds__(kMapThreads) void moe_tile_map_kernel(const int32_t* __restrict__ start, int E, int bm,
                                                                    int32_t* __restrict__ g_tile,
                                                                    int32_t* __restrict__ blk,
                                                                    int32_t* __restrict__ counts) {
-  __shared__ int tmp[kMapThreads];
+  __shared__ int wsum[kMapThreads / 64][2];
+  __shared__ int s_boff[kMapThreads + 1], s_toff[kMapThreads + 1], s_r0[kMapThreads], s_cnt[kMapThreads];
   const int e = threadIdx.x;
   const int r0 = e < E ? start[e] : 0;
   const int cnt = e < E ? max(start[e + 1] - r0, 0) : 0;
-  const int nb = (cnt + 15) >> 4, nt = (cnt + bm - 1) / bm;
-  const int boff = map_scan(nb, tmp, e);
+  int boff = (cnt + 15) >> 4, toff = (cnt + bm - 1) / bm, blocks, tiles;
+  map_scan2(boff, toff, wsum, e, blocks, tiles);
+  s_boff[e] = boff;
+  s_toff[e] = toff;
+  s_r0[e] = r0;
+  s_cnt[e] = cnt;
   __syncthreads();
-  const int toff = map_scan(nt, tmp, e);
-  for (int i = 0; i < nt; ++i) {
-    int32_t* t = g_tile + 4 * (toff + i);
-    t[0] = e;
-    t[1] = r0 + i * bm;
-    t[2] = min(bm, cnt - i * bm);
-    t[3] = boff + i * (bm >> 4);
+  // last expert whose first entry is at or before i (experts without rows share their successor's offset)
+  auto owner = [&](const int* off, int i) {
+    int lo = 0, hi = E - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (off[mid] <= i) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+  };
+  for (int i = e; i < tiles; i += kMapThreads) {
+    const int x = owner(s_toff, i), k = i - s_toff[x];
+    int32_t* t = g_tile + 4 * i;
+    t[0] = x;
+    t[1] = s_r0[x] + k * bm;
+    t[2] = min(bm, s_cnt[x] - k * bm);
+    t[3] = s_boff[x] + k * (bm >> 4);
   }
-  for (int b = 0; b < nb; ++b) {
-    blk[2 * (boff + b)] = r0 + 16 * b;
-    blk[2 * (boff + b) + 1] = min(16, cnt - 16 * b);
+  for (int b = e; b < blocks; b += kMapThreads) {
+    const int x = owner(s_boff, b), k = b - s_boff[x];
+    blk[2 * b] = s_r0[x] + 16 * k;
+    blk[2 * b + 1] = min(16, s_cnt[x] - 16 * k);
   }
-  if (e == kMapThreads - 1) {                          // inclusive totals sit in the last thread
-    counts[0] = toff + nt;
-    counts[1] = boff + nb;
+  if (e == 0) {
+    counts[0] = tiles;
+    counts[1] = blocks;
   }
 }
 
@@ -217,6 +244,70 @@ int mi_moe_gemm_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_
   p.out_rows = total_rows;
   return act_dtype == DT_F16 ? run_grouped<ActF16>(p, scale_per_expert != 0, fuse_act, L.max_tiles, st)
                              : run_grouped<ActBF16>(p, scale_per_expert != 0, fuse_act, L.max_tiles, st);
+}
+
+int mi_moe_mlp_fp8_tiled_workspace(int total_rows, int E, int H, int I, long long* bytes) {
+  if (!bytes) return MI_ERR_ARG;
+  if (total_rows < 0 || E < 0 || E > kMapThreads || H <= 0 || I <= 0) return MI_ERR_SHAPE;
+  const TiledMoeLayout L = tiled_moe_layout(total_rows, E, H, kMoeBM);
+  const long long inter = ((long long)L.max_blocks * 16 * I * 2 + 255) & ~255LL;
+  *bytes = L.total + inter;
+  if ((uint64_t)L.x_bytes >= (1ull << 31) || (uint64_t)inter >= (1ull << 31)) return MI_ERR_SHAPE;
+  return MI_OK;
+}
+
+int mi_moe_mlp_fp8_tiled_ws(const void* a, const int32_t* row_map, int row_map_div, const void* w13,
+                            const float* w13_scale, const void* w2, const float* w2_scale, int scale_per_expert,
+                            const int32_t* expert_start, void* out, const int32_t* out_map, const void* row_weight,
+                            int a_rows, int total_rows, int E, int H, int I, int fuse_act, int act_dtype,
+                            void* workspace, long long workspace_bytes, void* stream) {
+  if (!a || !w13 || !w13_scale || !w2 || !w2_scale || !expert_start || !out) return MI_ERR_ARG;
+  if (act_dtype != DT_F16 && act_dtype != DT_BF16) return MI_ERR_ARG;
+  if (fuse_act < 1 || fuse_act > 2 || scale_per_expert < 0 || scale_per_expert > 2 || row_map_div < 1) return MI_ERR_ARG;
+  if (E < 0 || E > kMapThreads || H <= 0 || I <= 0 || (H % 128) || (I % 128) || a_rows < 0 || total_rows < 0)
+    return MI_ERR_SHAPE;
+  if ((uint64_t)2 * I * (uint64_t)H >= (1ull << 31)) return MI_ERR_SHAPE;
+  if (!E || !total_rows) return MI_OK;
+  long long need = 0;
+  const int rc = mi_moe_mlp_fp8_tiled_workspace(total_rows, E, H, I, &need);
+  if (rc != MI_OK) return rc;
+  if (!workspace || workspace_bytes < need) return MI_ERR_ARG;
+  const int bm = kMoeBM;
+  const TiledMoeLayout L = tiled_moe_layout(total_rows, E, H, bm);
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  int32_t* g_tile = (int32_t*)(ws + L.tile_off);
+  int32_t* blk = (int32_t*)(ws + L.blk_off);
+  int32_t* counts = (int32_t*)(ws + L.cnt_off);
+  char* inter = ws + L.total;                          // [blocks][I / 32][1 KiB], operand order
+  hipLaunchKernelGGL(moe_tile_map_kernel, dim3(1), dim3(kMapThreads), 0, st, expert_start, E, bm, g_tile, blk, counts);
+  const int Q = H / 32;
+  hipLaunchKernelGGL(pack_x_grouped_kernel, dim3((unsigned)(((Q + kPackQ - 1) / kPackQ) * L.max_blocks)), dim3(256), 0, st,
+                     (const uint16_t*)a, row_map, blk, counts, (u32x4*)ws, a_rows, H, Q, row_map_div);
+  GemmArgs p{};
+  p.x = ws; p.w = w13; p.scale = w13_scale; p.out = inter; p.M = total_rows; p.N = 2 * I; p.K = H;
+  p.scale_mode = scale_per_expert == 2 ? 3 : (scale_per_expert ? 1 : 2);
+  p.g_tile = g_tile; p.g_count = counts;
+  p.g_w_stride = (long long)2 * I * H;
+  p.g_s_stride = scale_per_expert ? 4 * scale_per_expert : (long long)((2 * I + 127) / 128) * (H / 128) * 4;
+  p.x_blocks = L.max_blocks;
+  p.n_half = I; p.gelu = fuse_act == 2;
+  p.out_rows = L.max_blocks * 16; p.out_packed = 1;
+  int r = act_dtype == DT_F16 ? run_grouped<ActF16>(p, scale_per_expert != 0, fuse_act, L.max_tiles, st)
+                              : run_grouped<ActBF16>(p, scale_per_expert != 0, fuse_act, L.max_tiles, st);
+  if (r != MI_OK) return r;
+  GemmArgs d{};
+  d.x = inter; d.w = w2; d.scale = w2_scale; d.out = out; d.M = total_rows; d.N = H; d.K = I;
+  d.scale_mode = scale_per_expert ? 1 : 2;
+  d.g_tile = g_tile; d.g_count = counts;
+  d.g_w_stride = (long long)H * I;
+  d.g_s_stride = scale_per_expert ? 4 : (long long)((H + 127) / 128) * (I / 128) * 4;
+  d.out_map = out_map; d.row_weight = row_weight;
+  d.x_blocks = L.max_blocks;
+  d.n_half = H / 2;
+  d.out_rows = total_rows;
+  return act_dtype == DT_F16 ? run_grouped<ActF16>(d, scale_per_expert != 0, 0, L.max_tiles, st)
+                             : run_grouped<ActBF16>(d, scale_per_expert != 0, 0, L.max_tiles, st);
 }
 
 }  // extern "C"

@@ -1019,6 +1019,25 @@ def _moe_gemm(a, a_scale, row_map, w, w_scale, expert_start, out, E, N, K, fuse,
     return out
 
 
+def _moe_mlp_tiled(x, row_map, w13, s13, w2, s2, expert_start, y, total, E, H, I):
+    """gate_up, SiLU * up and down of the w8a16 prefill regime as one library call (block scales);
+    False when the tiled route does not take the shape (the caller then runs the two GEMMs)."""
+    for w, s, n, kk in ((w13, s13, 2 * I, H), (w2, s2, H, I)):
+        _chk_fp8(w, "moe_forward_fp8_block")
+        _chk(s.dtype == torch.float32 and s.is_contiguous() and s.numel() == E * ((n + 127) // 128) * (kk // 128),
+             "moe_forward_fp8_block: weight scales must be contiguous fp32 [E, ceil(N/128), K/128]")
+    if not (H % 128 == 0 and I % 128 == 0 and E <= 1024 and y.dtype == x.dtype):
+        return False
+    need = ctypes.c_longlong(0)
+    if capi.lib().mi_moe_mlp_fp8_tiled_workspace(int(total), int(E), int(H), int(I), ctypes.byref(need)) != 0:
+        return False
+    buf = torch.empty(need.value, dtype=torch.uint8, device=y.device)
+    capi.call("mi_moe_mlp_fp8_tiled_ws", y, capi.ptr(x), capi.ptr(row_map), 1, capi.ptr(w13), capi.ptr(s13),
+              capi.ptr(w2), capi.ptr(s2), 0, capi.ptr(expert_start), capi.ptr(y), None, None, x.shape[0], int(total),
+              int(E), int(H), int(I), 1, capi.act_dtype(x), capi.ptr(buf), need.value)
+    return True
+
+
 def esimd_moe_gemm_fp8_blockscale(input, weight, weight_scale, output, expert_idx, N, K, num_experts,
                                   block_n, block_k):
     who = "esimd_moe_gemm_fp8_blockscale"
@@ -1133,7 +1152,6 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
         esimd_moe_topk(logits, top_w, top_ids, T)
     start = torch.empty(E + 1, dtype=torch.int32, device=dev)
     inv = torch.empty(P, dtype=torch.int32, device=dev)
-    inter = torch.empty(P, I, dtype=x.dtype, device=dev)
     # fp32 expert outputs (the combine adds K rounded terms otherwise); in the w8a16 prefill regime the
     # tiled grouped GEMM takes over, which writes the activation type
     prefill = (not act_quant) and P >= 96 * E
@@ -1144,6 +1162,7 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
         sorted_token = torch.empty(P, dtype=torch.int32, device=dev)
         moe_sort(top_ids, E, sorted_pairs, start, inv, sorted_token, None)
     if act_quant:
+        inter = torch.empty(P, I, dtype=x.dtype, device=dev)
         if routed:      # the gate_up launch sorts the pairs itself
             moe_gate_up_fp8_routed(xq, xs, top_ids, gate_up_weight, gate_up_scale, start, inv, None, inter, E)
         else:
@@ -1152,7 +1171,11 @@ def moe_forward_fp8_block(x, logits, gate_up_weight, gate_up_scale, down_weight,
         isc = torch.empty(P, I // 128, dtype=torch.float32, device=dev)
         act_quant_fp8(inter, iq, isc)
         moe_gemm_fp8_block(iq, isc, None, down_weight, down_scale, start, y, H, I, E, False)
+    elif prefill and _moe_mlp_tiled(x, sorted_token, gate_up_weight, gate_up_scale, down_weight, down_scale, start, y,
+                                    P, E, H, I):
+        pass            # both GEMMs in one call: the intermediate stays in the second GEMM's operand order
     else:
+        inter = torch.empty(P, I, dtype=x.dtype, device=dev)
         moe_gemm_fp8_block(x, None, sorted_token, gate_up_weight, gate_up_scale, start, inter, 2 * I, H, E, True)
         moe_gemm_fp8_block(inter, None, None, down_weight, down_scale, start, y, H, I, E, False)
     moe_combine(y, inv, top_w, output, k)

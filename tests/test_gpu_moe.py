@@ -548,6 +548,80 @@ def test_moe_forward_w8a16_prefill(v, dev, T, E, K, H, I, dt):
     assert bool(((o - ref).abs() <= bound).all()), ((o - ref).abs() / bound).max()
 
 
+@pytest.mark.parametrize("counts,H,I,dt,per_expert,act", [
+    ([300, 0, 17, 256, 0, 0, 513, 1], 256, 128, torch.bfloat16, 0, 1),       # empty experts, one row, tile edges
+    ([120, 200, 90, 310], 384, 256, torch.float16, 0, 2),                      # tanh-GELU
+    ([260, 250], 256, 384, torch.bfloat16, 2, 1),                              # gate / up scalars, one for down
+    ([100] * 40, 128, 128, torch.float16, 1, 1)])
+def test_moe_mlp_tiled_equals_two_grouped_gemms(v, dev, counts, H, I, dt, per_expert, act):
+    """The expert MLP as one library call (tile table built once, the intermediate written straight into the
+    second GEMM's operand order) against two calls of the tiled grouped GEMM with a row-major intermediate:
+    the same bits, with a row map on the input and a row map + row weights on the output; and the
+    two-call result against the oracle."""
+    import ctypes
+    from mi355x_qlinear import capi
+    E = len(counts)
+    total = sum(counts)
+    g = torch.Generator().manual_seed(total + H)
+    start = torch.zeros(E + 1, dtype=torch.int32)
+    start[1:] = torch.tensor(counts).cumsum(0).to(torch.int32)
+    T = total // 2 + 3
+    x = (torch.randn(T, H, generator=g) * 0.3).to(dt)
+    row_map = torch.randint(0, T, (total,), generator=g, dtype=torch.int32)
+    out_map = torch.randperm(total, generator=g).to(torch.int32)
+    row_w = (torch.rand(total, generator=g) + 0.5).to(dt)
+    if per_expert:
+        w13 = (torch.randn(E, 2 * I, H, generator=g) * 20).to(torch.float8_e4m3fn)
+        w2 = (torch.randn(E, H, I, generator=g) * 20).to(torch.float8_e4m3fn)
+        s13 = torch.rand(E, per_expert, generator=g) * 0.004 + 0.002
+        s2 = torch.rand(E, generator=g) * 0.004 + 0.002
+        w13b, w2b = w13.view(torch.uint8), w2.view(torch.uint8)
+    else:
+        w13b, s13 = O.fp8_quantize_block(torch.randn(E, 2 * I, H, generator=g) * 0.15)
+        w2b, s2 = O.fp8_quantize_block(torch.randn(E, H, I, generator=g) * 0.15)
+    xd, rmd, omd, rwd, std = x.to(dev), row_map.to(dev), out_map.to(dev), row_w.to(dev), start.to(dev)
+    w13d, s13d, w2d, s2d = w13b.to(dev), s13.to(dev), w2b.to(dev), s2.to(dev)
+    adt = capi.act_dtype(xd)
+
+    def ws_of(fn, *dims):
+        need = ctypes.c_longlong(0)
+        assert getattr(capi.lib(), fn)(*dims, ctypes.byref(need)) == 0
+        return torch.empty(need.value, dtype=torch.uint8, device=dev), need.value
+
+    inter = torch.empty(total, I, dtype=dt, device=dev)
+    two = torch.full((total, H), 3.0, dtype=dt, device=dev)
+    b1, n1 = ws_of("mi_moe_gemm_fp8_tiled_workspace", total, E, H)
+    capi.call("mi_moe_gemm_fp8_tiled_ws", xd, capi.ptr(xd), capi.ptr(rmd), 1, capi.ptr(w13d), capi.ptr(s13d), per_expert,
+              capi.ptr(std), capi.ptr(inter), None, None, T, total, E, 2 * I, H, act, adt, capi.ptr(b1), n1)
+    b2, n2 = ws_of("mi_moe_gemm_fp8_tiled_workspace", total, E, I)
+    capi.call("mi_moe_gemm_fp8_tiled_ws", xd, capi.ptr(inter), None, 1, capi.ptr(w2d), capi.ptr(s2d), min(per_expert, 1),
+              capi.ptr(std), capi.ptr(two), capi.ptr(omd), capi.ptr(rwd), total, total, E, H, I, 0, adt, capi.ptr(b2), n2)
+    one = torch.full((total, H), 5.0, dtype=dt, device=dev)
+    b3, n3 = ws_of("mi_moe_mlp_fp8_tiled_workspace", total, E, H, I)
+    capi.call("mi_moe_mlp_fp8_tiled_ws", xd, capi.ptr(xd), capi.ptr(rmd), 1, capi.ptr(w13d), capi.ptr(s13d), capi.ptr(w2d),
+              capi.ptr(s2d), per_expert, capi.ptr(std), capi.ptr(one), capi.ptr(omd), capi.ptr(rwd), T, total, E, H, I, act,
+              adt, capi.ptr(b3), n3)
+    assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+    # the two-call result against the oracle: per expert, weights with their scales folded in and rounded to
+    # the activation type where the scales are blocks (as the tiled kernel feeds the matrix core)
+    want = torch.zeros(total, H)
+    for e in range(E):
+        lo, hi = int(start[e]), int(start[e + 1])
+        if hi == lo:
+            continue
+        if per_expert:
+            d13 = w13[e].float()
+            d13 = torch.cat([d13[:I] * s13[e, 0], d13[I:] * s13[e, per_expert - 1]])
+            d2 = w2[e].float() * s2[e]
+        else:
+            d13 = O.fp8_dequant_block(w13b[e], s13[e], out_dtype=dt).float()
+            d2 = O.fp8_dequant_block(w2b[e], s2[e], out_dtype=dt).float()
+        gu = x[row_map[lo:hi].long()].float() @ d13.t()
+        h = (O.gelu_tanh_mul(gu) if act == 2 else O.silu_mul(gu)).to(dt).float()
+        want[out_map[lo:hi].long()] = ((h @ d2.t()) * row_w[out_map[lo:hi].long()].float()[:, None])
+    assert O.max_rel_err(two.cpu(), want) < TOL
+
+
 @pytest.mark.parametrize("aq", [True, False])
 def test_expert_outputs_in_fp16_beside_bf16(v, dev, aq):
     """The grouped GEMM can write fp16 whatever the activation type and the combine reads it: half the bytes
