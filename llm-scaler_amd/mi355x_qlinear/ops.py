@@ -1068,7 +1068,7 @@ def moe_gemm_fp8_block(a, a_scale, row_map, weight, weight_scale, expert_start, 
 
 
 ROUTED_MAX_PAIRS = 8192       # (token, route) pairs one routed gate_up launch sorts by itself
-ROUTED_GEMV_MAX_PAIRS = 64    # (token, route) pairs up to which the fused decode op runs one GEMV per route
+ROUTED_GEMV_MAX_PAIRS = 96    # (token, route) pairs up to which the fused decode op runs one GEMV per route (12 tokens x top 8)
 
 
 def moe_gate_up_fp8_routed(xq, xs, top_ids, weight, weight_scale, expert_start, inv, sorted_pairs, output,
