@@ -548,6 +548,69 @@ def test_moe_forward_w8a16_prefill(v, dev, T, E, K, H, I, dt):
     assert bool(((o - ref).abs() <= bound).all()), ((o - ref).abs() / bound).max()
 
 
+def test_moe_prefill_full_size_properties(v, dev):
+    """The w8a16 forward at the prefill benchmark's size (4096 tokens, 128 experts, top 8, H = 2048, I = 768,
+    bf16: 256 +- 16 rows per expert, so full tiles and a few-row tail tile per expert), checked through what
+    does not depend on the size: (1) a permutation of the tokens permutes the output rows bit for bit (a row's
+    arithmetic does not depend on which tile, wavefront or lane it lands in); (2) sampled tokens against the
+    oracle's per-token forward with the weights of their experts."""
+    T, E, K, H, I = 4096, 128, 8, 2048, 768
+    dt = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(77)
+    # finite E4M3 codes drawn directly (a CPU quantisation of 600 M weights takes minutes): |code| <= 0x6F
+    codes = lambda *s: (torch.randint(0, 0x70, s, generator=g, device=dev, dtype=torch.uint8) |
+                        (torch.randint(0, 2, s, generator=g, device=dev, dtype=torch.uint8) << 7))
+    w13, w2 = codes(E, 2 * I, H), codes(E, H, I)
+    s13 = torch.rand(E, 2 * I // 128, H // 128, generator=g, device=dev) * 2e-3 + 5e-4
+    s2 = torch.rand(E, H // 128, I // 128, generator=g, device=dev) * 2e-3 + 5e-4
+    x = (torch.randn(T, H, generator=g, device=dev) * 0.5).to(dt)
+    logits = torch.randn(T, E, generator=g, device=dev).to(dt)
+    f8 = lambda t: t.view(torch.float8_e4m3fn)
+    out = torch.empty(T, H, dtype=dt, device=dev)
+    v.moe_forward_fp8_block(x, logits, f8(w13), s13, f8(w2), s2, out, K, False)
+    assert torch.isfinite(out.float()).all()
+    perm = torch.randperm(T, generator=g, device=dev)
+    out_p = torch.empty_like(out)
+    v.moe_forward_fp8_block(x[perm].contiguous(), logits[perm].contiguous(), f8(w13), s13, f8(w2), s2, out_p, K, False)
+    assert torch.equal(out_p.view(torch.int16), out[perm].view(torch.int16))
+    # sampled tokens: block scales folded into weights of the activation type (the tiled kernel's arithmetic),
+    # the intermediate and every expert output rounded to it, fp32 sum of the routes
+    xc, lc = x.cpu(), logits.cpu()
+    rtw, rti = O.moe_topk(lc, K)
+    for t in (0, 1733, T - 1):
+        want = torch.zeros(H)
+        mag = torch.zeros(H)
+        for jr in range(K):
+            e = int(rti[t, jr])
+            d13 = O.fp8_dequant_block(w13[e].cpu(), s13[e].cpu(), out_dtype=dt)
+            d2 = O.fp8_dequant_block(w2[e].cpu(), s2[e].cpu(), out_dtype=dt)
+            h = O.silu_mul((xc[t].float() @ d13.t())[None, :]).to(dt).float()
+            y = (h @ d2.t())[0].to(dt).float()
+            want += rtw[t, jr].float() * y
+            mag += rtw[t, jr].float() * y.abs()
+        got = out[t].cpu().float()
+        bound = TOL * want.abs().clamp(min=want.abs().mean()) + 2.0 ** -8 * mag
+        assert bool(((got - want).abs() <= bound).all()), (t, ((got - want).abs() / bound).max())
+
+
+@pytest.mark.parametrize("T", [512, 37])
+def test_cfg3_forward_token_permutation(v, dev, T):
+    """cfg3's forward (fp8 activations; the gate_up launch sorts the pairs itself): permuting the tokens
+    permutes the output rows bit for bit, at the benchmark's size and at a ragged one."""
+    E, K, H, I = 128, 8, 2048, 768
+    x, logits, w13q, w13s, w2q, w2s = O.make_moe_case(T, E, K, H, I, seed=4242)
+    f8 = lambda t: t.view(torch.float8_e4m3fn).to(dev)
+    args = (f8(w13q), w13s.to(dev), f8(w2q), w2s.to(dev))
+    xd, ld = x.to(dev), logits.to(dev)
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    v.moe_forward_fp8_block(xd, ld, *args, out, K, True)
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(T)).to(dev)
+    out_p = torch.empty_like(out)
+    v.moe_forward_fp8_block(xd[perm].contiguous(), ld[perm].contiguous(), *args, out_p, K, True)
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out_p.view(torch.int16), out[perm].view(torch.int16))
+
+
 @pytest.mark.parametrize("counts,H,I,dt,per_expert,act", [
     ([300, 0, 17, 256, 0, 0, 513, 1], 256, 128, torch.bfloat16, 0, 1),       # empty experts, one row, tile edges
     ([120, 200, 90, 310], 384, 256, torch.float16, 0, 2),                      # tanh-GELU
