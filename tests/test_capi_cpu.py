@@ -23,6 +23,35 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, name).argtypes == types
 
 
+def test_moe_tiled_workspace_sizes_and_argument_errors():
+    """Host-side answers of the grouped tiled GEMM entry points (no launch): the workspace of the expert MLP
+    holds the single GEMM's (re-tiled x + tables) plus the re-tiled intermediate; limits and bad arguments
+    come back as error codes before anything is enqueued."""
+    lib = capi.lib()
+    one, mlp = ctypes.c_longlong(0), ctypes.c_longlong(0)
+    total, E, H, I = 32768, 128, 2048, 768
+    assert lib.mi_moe_gemm_fp8_tiled_workspace(total, E, H, ctypes.byref(one)) == 0
+    assert lib.mi_moe_mlp_fp8_tiled_workspace(total, E, H, I, ctypes.byref(mlp)) == 0
+    blocks = total // 16 + E
+    assert one.value >= blocks * 16 * H * 2 and one.value % 256 == 0
+    assert mlp.value == one.value + (blocks * 16 * I * 2 + 255) // 256 * 256
+    # re-tiled activations of 2 GiB or more: the tiled route does not apply (the size is still reported)
+    assert lib.mi_moe_mlp_fp8_tiled_workspace(1 << 19, E, 4096, I, ctypes.byref(mlp)) == -2 and mlp.value > (1 << 31)
+    assert lib.mi_moe_mlp_fp8_tiled_workspace(total, 1025, H, I, ctypes.byref(mlp)) == -2      # more than 1024 experts
+    assert lib.mi_moe_mlp_fp8_tiled_workspace(total, E, H, I, None) == -1
+    # the call itself: null pointers, unknown activation, sizes off the 128 grid, short workspace
+    ok = ctypes.c_void_p(256)                      # never dereferenced: every case below returns before a launch
+    args = lambda **kw: [kw.get("a", ok), None, kw.get("div", 1), ok, ok, ok, ok, kw.get("spe", 0), ok, ok, None, None, 64,
+                         4096, 8, kw.get("H", 256), kw.get("I", 128), kw.get("act", 1), kw.get("dt", 1), kw.get("ws", ok),
+                         ctypes.c_longlong(kw.get("wsb", 1 << 40)), None]
+    f = lib.mi_moe_mlp_fp8_tiled_ws
+    assert f(*args(a=None)) == -1
+    assert f(*args(act=0)) == -1 and f(*args(act=3)) == -1 and f(*args(dt=2)) == -1 and f(*args(spe=3)) == -1
+    assert f(*args(div=0)) == -1
+    assert f(*args(H=200)) == -2 and f(*args(I=100)) == -2
+    assert f(*args(ws=None)) == -1 and f(*args(wsb=1024)) == -1
+
+
 def test_header_pointer_and_scalar_mapping():
     p = capi.parse_header()
     assert p["mi_gemm_fp8_pern"] == [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_void_p]
