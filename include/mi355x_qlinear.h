@@ -202,6 +202,22 @@ int mi_moe_gguf_gemv(int fmt, const void* x, int x_div, int nmat, const void* co
                      const void* const* scale, const void* const* qmin, void* const* out, long long out_stride,
                      const int32_t* route_expert, const void* route_weight, int routes, int num_experts, int N,
                      int K, void* stream);
+/* Grouped form over chunks of expert-sorted rows (MoE prefill and multi-token verify):
+ * chunks [num_chunks, 3] int32 = {expert, first row t0, rows nt}; for every chunk and matrix i
+ *   out[t0 + m, i N + n] = sum_k x[row(t0 + m), k] W_i[expert][n, k],   m < min(nt, 64)   (16 when rows16)
+ * with row(p) = tok_ids[p] when tok_ids is given (the expert-sort permutation, out_rows entries; the
+ * gather of x happens inside the load) and p otherwise.  x [x_rows, K] fp16, out [out_rows, out_stride]
+ * fp16 with out_stride >= nmat N; stacks as for mi_moe_gguf_gemv ([E, N, K/2] nibbles, [E, N, K/32] fp16
+ * scales and mins).  Chunks with nt <= 0, an expert outside [0, E) or rows outside the output are
+ * skipped; rows of a chunk past the 64 (16) are not computed, as in the reference kernel; token ids
+ * outside [0, x_rows) read as zero rows.  Weights are dequantized as fp16(fp16(nibble * scale) - min)
+ * and accumulated in fp32.  fmt = 2 (Q4_K), nmat <= 2, K % 32 == 0; one kernel launch.
+ * Replaces moe_up_q4k_ggemv / moe_up_q4k_ggemv_smallm (S/csrc/moe_grouped/moe_q4k_ggemv.h:47-201, 311-321;
+ * ATen entry S/csrc/moe_grouped/moe_grouped_entry.sycl:24-60; caller sglang_for_multi_arc.patch:2899-2901). */
+int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_ids, int nmat, const void* const* ql,
+                        const void* const* qh, const void* const* scale, const void* const* qmin, void* out,
+                        long long out_stride, int out_rows, const int32_t* chunks, int num_chunks, int num_experts,
+                        int N, int K, int rows16, void* stream);
 int mi_q4_0_repack(const void* raw, void* packed, void* scale, int N, int K, void* stream);
 int mi_q8_0_repack(const void* raw, void* qs, void* scale, int N, int K, void* stream);
 int mi_q5k_repack(const void* raw, void* ql, void* qh, void* scale, void* qmin, int N, int K,

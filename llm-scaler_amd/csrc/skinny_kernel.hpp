@@ -30,6 +30,7 @@ namespace qlin {
 
 constexpr int kMaxMat = 3;
 constexpr int kSkinnyXLdsFrom = 2;                  // 16-row activation tiles from which x is staged through LDS
+constexpr bool kXLdsOf(int mt) { return mt >= kSkinnyXLdsFrom; }
 
 struct SkinnyArgs {
   const void* x;
@@ -47,6 +48,13 @@ struct SkinnyArgs {
   // msplit > 1: the rows of x are split over msplit workgroups per weight row block (16 MT rows
   // each); tiles_total = row blocks of all matrices.
   int msplit, tiles_total;
+  // Grouped launches (GRP instantiations): one (expert, first row, rows) triple per chunk; the
+  // chunk's rows of x are rows t0 .. t0 + nt - 1, or tok_ids[t0 ..] when given; output row t0 + m,
+  // out_stride elements apart; the expert's tables sit *_stride bytes after the previous expert's.
+  const int32_t* chunks;
+  const int32_t* tok_ids;
+  int num_chunks, num_experts, x_rows, out_rows;
+  long long out_stride, w_stride, s_stride, z_stride, h_stride;
 };
 
 enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
@@ -60,7 +68,8 @@ enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
 // of being fetched per tile and granule with scattered 16-bit loads: per-32 tables for Q4_K,
 // Q5_K, Q4_0, Q8_0 (needs K % 256 == 0), per-128 tables for INT4; chosen when the tables fit
 // beside the staging tiles.
-template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false>
+// GRP: the grid is (row blocks x chunks), see SkinnyArgs; all workgroups of a chunk run on one XCD.
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false, bool GRP = false>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   using V8 = typename Act::v8;
   using Elem = typename Act::elem;
@@ -91,7 +100,21 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 
   int tile = blockIdx.x;
   int m0 = 0;                                         // first row of x of this workgroup
-  if (a.msplit > 1) {
+  int eid = 0, t0 = 0, mrows = 0;
+  if constexpr (GRP) {
+    // workgroups are dealt to the 8 XCDs in turn: chunk c runs on XCD c % 8, so its rows of x enter one L2
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int rnd = slot / a.tiles_total;
+    const int cid = rnd * 8 + xcd;
+    tile = slot - rnd * a.tiles_total;
+    if (cid >= a.num_chunks) return;
+    eid = a.chunks[3 * cid];
+    t0 = a.chunks[3 * cid + 1];
+    const int nt = a.chunks[3 * cid + 2];
+    if (nt <= 0 || eid < 0 || eid >= a.num_experts || t0 < 0 || t0 >= a.out_rows) return;
+    mrows = min(min(nt, MT * 16), a.out_rows - t0);   // rows past 16 MT are not computed
+  }
+  if (!GRP && a.msplit > 1) {
     // The workgroups of a row block sit 8 apart: workgroups are dealt to the 8 XCDs in turn, so
     // the block's weights come from HBM once and from that XCD's L2 afterwards.
     const int grp = blockIdx.x / (8 * a.msplit), rem = blockIdx.x - grp * 8 * a.msplit;
@@ -105,7 +128,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     if (mat == i && i + 1 < a.nmat && tile >= a.tiles[i]) { tile -= a.tiles[i]; mat = i + 1; }
   }
   const int N = a.N[mat];
-  const int K = a.K, M = min(a.M - m0, MT * 16);
+  const int K = a.K, M = GRP ? mrows : min(a.M - m0, MT * 16);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = lane & 15, g = lane >> 4;
@@ -115,14 +138,40 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 
   const uint32_t wrow = kByteW ? (uint32_t)K : ((uint32_t)K >> 1);
   const uint32_t hrow = kIsQ5K ? ((uint32_t)K >> 3) : ((uint32_t)K >> 2);   // high-bit bytes per row
-  const __amdgpu_buffer_rsrc_t hr = make_rsrc(a.h[mat], kHigh ? (uint32_t)N * hrow : 0u);
-  const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w[mat], (uint32_t)N * wrow);
-  const __amdgpu_buffer_rsrc_t xr = make_rsrc((const char*)a.x + (size_t)m0 * K * 2, (uint32_t)M * (uint32_t)K * 2u);
+  // the expert's tables (GRP); null stays null
+  const char* hbase = (const char*)a.h[mat];
+  const char* wbase = (const char*)a.w[mat];
+  const char* sbase = (const char*)a.s[mat];
+  const char* zbase = (const char*)a.z[mat];
+  if constexpr (GRP) {
+    wbase += (long long)eid * a.w_stride;
+    sbase += (long long)eid * a.s_stride;
+    if (zbase) zbase += (long long)eid * a.z_stride;
+    if (hbase) hbase += (long long)eid * a.h_stride;
+  }
+  const __amdgpu_buffer_rsrc_t hr = make_rsrc(hbase, kHigh ? (uint32_t)N * hrow : 0u);
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(wbase, (uint32_t)N * wrow);
+  const __amdgpu_buffer_rsrc_t xr = GRP ? make_rsrc(a.x, (uint32_t)a.x_rows * (uint32_t)K * 2u)
+                                        : make_rsrc((const char*)a.x + (size_t)m0 * K * 2, (uint32_t)M * (uint32_t)K * 2u);
+  // GRP: byte offset of the row of x behind each row slot this lane loads (past the end: reads zeros)
+  constexpr int kXSlots = kXLdsOf(MT) ? 4 : 1;
+  uint32_t xro[MT][kXSlots];
+  if constexpr (GRP) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < kXSlots; ++i) {
+        const int m = mt * 16 + (kXLdsOf(MT) ? (lane >> 4) + 4 * i : j);
+        const int pos = t0 + min(m, M - 1);
+        const int tok = a.tok_ids ? a.tok_ids[pos] : pos;
+        xro[mt][i] = (m < M && tok >= 0 && tok < a.x_rows) ? (uint32_t)tok * (uint32_t)K * 2u : kOOB;
+      }
+  }
 
-  const _Float16* s16 = (const _Float16*)a.s[mat];
-  const float* s32 = (const float*)a.s[mat];
-  const uint8_t* zp = (const uint8_t*)a.z[mat];
-  const _Float16* qmin = (const _Float16*)a.z[mat];
+  const _Float16* s16 = (const _Float16*)sbase;
+  const float* s32 = (const float*)sbase;
+  const uint8_t* zp = (const uint8_t*)zbase;
+  const _Float16* qmin = (const _Float16*)zbase;
   const int Kg = K >> 7;                             // int4 groups per row
   const int Kb32 = K >> 5;                           // q4k sub-blocks per row
   const int Kb = G;                                  // fp8 block columns
@@ -245,11 +294,12 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
             const int r = (lane >> 4) + 4 * i, c = lane & 15;
             const int m = mt * 16 + r;
             const bool okx = gi < G && gi * 128 + c * 8 < K && m < M;
-            st.xa[u][mt][i] = buf_load16(xr, okx ? ((uint32_t)m * (uint32_t)K + (uint32_t)(gi * 128 + c * 8)) * 2u : kOOB);
+            if constexpr (GRP) st.xa[u][mt][i] = buf_load16(xr, okx ? xro[mt][i] + (uint32_t)(gi * 128 + c * 8) * 2u : kOOB);
+            else st.xa[u][mt][i] = buf_load16(xr, okx ? ((uint32_t)m * (uint32_t)K + (uint32_t)(gi * 128 + c * 8)) * 2u : kOOB);
           }
         } else {
           // few rows: straight into operand layout (lane (j, g): row j, 32 consecutive k)
-          const uint32_t xoff = ok ? ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u : kOOB;
+          const uint32_t xoff = !ok ? kOOB : (GRP ? xro[mt][0] + (uint32_t)kl * 2u : ((uint32_t)(mt * 16 + j) * (uint32_t)K + (uint32_t)kl) * 2u);
 #pragma unroll
           for (int i = 0; i < 4; ++i) st.xa[u][mt][i] = buf_load16(xr, ok ? xoff + 16u * i : kOOB);
         }
@@ -403,8 +453,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     __syncthreads();
   } else if constexpr (SL) {
     // tables [RT * 16 rows][K / 32] of scales, then of mins; rows past the workgroup's range are zeros
-    const __amdgpu_buffer_rsrc_t sr = make_rsrc(a.s[mat], (uint32_t)N * (uint32_t)Kb32 * 2u);
-    const __amdgpu_buffer_rsrc_t mr = make_rsrc(a.z[mat], kHasMin ? (uint32_t)N * (uint32_t)Kb32 * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t sr = make_rsrc(sbase, (uint32_t)N * (uint32_t)Kb32 * 2u);
+    const __amdgpu_buffer_rsrc_t mr = make_rsrc(zbase, kHasMin ? (uint32_t)N * (uint32_t)Kb32 * 2u : 0u);
     const int cpr = Kb32 >> 3;                        // 16-byte chunks per row
     u32x4* tab = reinterpret_cast<u32x4*>(smem + kTiles);
     const int total = RT * 16 * cpr;
@@ -461,7 +511,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
     for (int mt = 0; mt < MT; ++mt) red[wave][t][mt][lane] = acc[t][mt];
   __syncthreads();
   // D layout: lane holds output column n0 + 16 t + j, rows mt*16 + 4 g + v.
-  Elem* out = (Elem*)a.out[mat] + (size_t)m0 * N;
+  const size_t opitch = GRP ? (size_t)a.out_stride : (size_t)N;
+  Elem* out = (Elem*)a.out[mat] + (GRP ? (size_t)t0 * opitch : (size_t)m0 * N);
 #pragma unroll
   for (int it = 0; it < kOutIters; ++it) {
     const int o = wave + it * NW;
@@ -479,7 +530,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int m = mt * 16 + g * 4 + v;
-        if (m < M) out[(size_t)m * N + n] = Act::from_f32(sum[v] * os);
+        if (m < M) out[(size_t)m * opitch + n] = Act::from_f32(sum[v] * os);
       }
     }
   }

@@ -540,6 +540,47 @@ def esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hi
                           "esimd_moe_down_q6k")
 
 
+# grouped GGUF MoE GEMMs over chunks of expert-sorted rows (the reference's pybind module
+# moe_grouped_gguf_xpu: moe_up_q4k_ggemv, moe_down_q5k_ggemv, moe_down_q6k_ggemv)
+def _chk_chunks(chunks, who):
+    _chk(chunks.dim() == 2 and chunks.size(1) == 3, f"{who}: chunks [num_chunks,3]")
+    _chk(chunks.dtype == torch.int32 and chunks.is_contiguous(), f"{who}: chunks must be contiguous int32")
+
+
+def moe_up_q4k_ggemv(expert_states, gate_ql, gate_sc, gate_mn, up_ql, up_sc, up_mn, gate_buf, chunks, hidden_size,
+                     intermediate_size, tok_ids=None, smallm=False):
+    """gate_buf[t0 + m, 0:I] = x_m @ Wg[e]^T and gate_buf[t0 + m, I:2I] = x_m @ Wu[e]^T for every chunk
+    {e, t0, nt} of `chunks` and m < min(nt, 64) (16 with smallm), where x_m is row tok_ids[t0 + m] of
+    `expert_states` (row t0 + m when tok_ids is empty or None).  Q4_K stacks gate_ql / up_ql [E, I, H/2] uint8,
+    scale / min [E, I, H/32] fp16; fp16 activations and output; chunks with nt <= 0 are skipped
+    (S/csrc/moe_grouped/moe_grouped_entry.sycl:24-60, moe_q4k_ggemv.h:47-201).  Returns gate_buf."""
+    who = "moe_up_q4k_ggemv"
+    H, I = int(hidden_size), int(intermediate_size)
+    _chk_chunks(chunks, who)
+    _chk(gate_ql.dim() == 3 and H % 32 == 0, f"{who}: gate_ql must be [E, I, H/2], H a multiple of 32")
+    E = gate_ql.shape[0]
+    for q, sc, mn, nm in ((gate_ql, gate_sc, gate_mn, "gate"), (up_ql, up_sc, up_mn, "up")):
+        _chk_stack(q, torch.uint8, (E, I, H // 2), nm + "_ql", who)
+        _chk_stack(sc, torch.float16, (E, I, H // 32), nm + "_sc", who)
+        _chk_stack(mn, torch.float16, (E, I, H // 32), nm + "_mn", who)
+    _chk(expert_states.dtype == torch.float16 and expert_states.is_contiguous() and expert_states.dim() == 2
+         and expert_states.shape[1] == H, f"{who}: expert_states must be contiguous fp16 [rows, hidden]")
+    _chk(gate_buf.dtype == torch.float16 and gate_buf.is_contiguous() and gate_buf.dim() == 2
+         and gate_buf.shape[1] == 2 * I, f"{who}: gate_buf must be contiguous fp16 [total, 2 * intermediate]")
+    total = gate_buf.shape[0]
+    has_ids = tok_ids is not None and tok_ids.numel() > 0
+    if has_ids:
+        _chk(tok_ids.dtype == torch.int32 and tok_ids.is_contiguous() and tok_ids.numel() >= total,
+             f"{who}: tok_ids must be contiguous int32 with one entry per row of gate_buf")
+    if chunks.size(0) == 0 or total == 0:
+        return gate_buf
+    capi.call("mi_moe_gguf_grouped", expert_states, 2, capi.ptr(expert_states), expert_states.shape[0],
+              capi.ptr(tok_ids) if has_ids else None, 2, capi.ptr_array([gate_ql, up_ql]), None,
+              capi.ptr_array([gate_sc, up_sc]), capi.ptr_array([gate_mn, up_mn]), capi.ptr(gate_buf), 2 * I, total,
+              capi.ptr(chunks), chunks.size(0), E, I, H, 1 if smallm else 0)
+    return gate_buf
+
+
 def _gemv_q6_k(input, ql, qh, weight_scale, output, who):
     _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be contiguous uint8 [N, K/2]")
     N, K = ql.shape[0], ql.shape[1] * 2

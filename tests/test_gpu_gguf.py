@@ -318,3 +318,119 @@ def test_q4_0_quantize_feeds_int4_gemv(ops, dev):
     # and the quantization itself stays inside the Q4_0 envelope: |w - deq| <= |d|
     err = (wd.float() - w.float()).abs()
     assert bool((err <= sc.cpu().float().abs().repeat_interleave(128, dim=1) + 1e-4).all())
+
+
+# ---- grouped MoE GEMMs over chunks of expert-sorted rows (the reference's moe_grouped_gguf_xpu module) ----
+def _expert_chunks(topk_ids, E, max_m, fixed):
+    """The caller's chunk list (sglang_for_multi_arc.patch:2810-2887): routes sorted by expert (stable),
+    one {expert, first sorted row, rows} triple per non-empty expert, experts with more than max_m rows split;
+    `fixed` = the [E, 3] table with empty chunks that the small-M branch builds."""
+    T, k = topk_ids.shape
+    flat = topk_ids.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    tok_sorted = (torch.arange(T).repeat_interleave(k))[order].to(torch.int32)
+    counts = torch.bincount(flat, minlength=E)
+    start = torch.cumsum(counts, 0) - counts
+    rows = []
+    for e in range(E):
+        s, n = int(start[e]), int(counts[e])
+        if fixed:
+            rows.append([e, s, n])
+            continue
+        while n > 0:
+            c = min(max_m, n)
+            rows.append([e, s, c])
+            s += c
+            n -= c
+    return torch.tensor(rows, dtype=torch.int32).reshape(-1, 3), tok_sorted, order
+
+
+def _q4k_expert_stacks(U, I, H, seeds, emap, dev):
+    """Two Q4_K stacks (gate, up) of U distinct experts spread over len(emap) experts; returns the device
+    representations and the oracle's dequantized weights [U, I, H]."""
+    stack = lambda a: _t(a).reshape(U, -1, a.shape[-1]).to(dev)[emap.to(dev)].contiguous()
+    reps, deq = [], []
+    for seed in seeds:
+        Hp = (H + 255) // 256 * 256                       # raw super-blocks hold 256 elements
+        _, raw = O.make_q4k_case(1, Hp, U * I, seed=seed + H)
+        rep = O.q4k_repack(raw)
+        if Hp != H:                                       # K % 32 == 0: cut every row to its first H elements
+            rep = tuple(np.ascontiguousarray(a[:, :H // d]) for a, d in zip(rep, (2, 32, 32)))
+        reps.append([stack(a) for a in rep])
+        deq.append(torch.from_numpy(O.q4k_dequant(*rep).astype(np.float32)).reshape(U, I, H))
+    return reps, deq
+
+
+@pytest.mark.parametrize("T,E,k,H,I,smallm,gathered", [
+    (4, 16, 4, 2048, 512, True, False),      # multi-token verify: fixed [E, 3] table with empty chunks
+    (16, 8, 2, 512, 96, True, False),        # 16 rows per chunk at most; I not a multiple of the 64-row block
+    (200, 8, 2, 2048, 512, False, False),    # prefill: experts with more than 64 rows split into sub-chunks
+    (90, 6, 3, 2080, 128, False, False),     # K not a multiple of 128 (partial last granule), no LDS tables
+    (64, 4, 2, 256, 64, False, True),        # rows gathered by the caller (no token list)
+    (300, 128, 8, 2048, 768, False, False),  # many experts, few rows each
+])
+def test_moe_grouped_q4k_up(ops, dev, T, E, k, H, I, smallm, gathered):
+    """moe_up_q4k_ggemv (S/csrc/moe_grouped/moe_grouped_entry.sycl:24-60, moe_q4k_ggemv.h:47-201): gate and up
+    projections of every chunk against the per-chunk product on the oracle's dequantized weights; rows no
+    chunk covers keep the caller's zeros."""
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    g = torch.Generator().manual_seed(T + H + I)
+    x = (torch.randn(T, H, generator=g) * 0.1).half()
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    chunks, tok_sorted, _ = _expert_chunks(ids, E, 16 if smallm else 64, fixed=smallm)
+    U = min(E, 8)
+    emap = (7 * torch.arange(E) + 3) % U if U < E else torch.arange(E)
+    reps, deq = _q4k_expert_stacks(U, I, H, (21, 22), emap, dev)
+    P = T * k
+    buf = torch.zeros(P, 2 * I, dtype=torch.float16, device=dev)
+    if gathered:
+        xin = x[tok_sorted.long()].contiguous().to(dev)
+        ret = mg.moe_up_q4k_ggemv(xin, *reps[0], *reps[1], buf, chunks.to(dev), H, I)
+    else:
+        ret = mg.moe_up_q4k_ggemv(x.to(dev), *reps[0], *reps[1], buf, chunks.to(dev), H, I, tok_sorted.to(dev),
+                                  smallm=smallm)
+    assert ret.data_ptr() == buf.data_ptr()
+    want = torch.zeros(P, 2 * I)
+    for e, t0, nt in chunks.tolist():
+        if nt <= 0:
+            continue
+        xs = x.float()[tok_sorted[t0:t0 + nt].long()]
+        u = int(emap[e])
+        want[t0:t0 + nt, :I] = xs @ deq[0][u].t()
+        want[t0:t0 + nt, I:] = xs @ deq[1][u].t()
+    assert O.max_rel_err(buf.cpu(), want) < TOL
+    assert int(chunks[:, 2].sum()) == P                   # every row belongs to a chunk in these cases
+
+
+def test_moe_grouped_q4k_up_chunk_semantics(ops, dev):
+    """Chunks as the reference kernel treats them (moe_q4k_ggemv.h:70-73, 79-92, 173-186): nt <= 0 skipped, rows
+    past the tile height (64, or 16 with smallm) not computed, rows outside every chunk untouched; here also
+    experts outside [0, E), rows outside the output and token ids outside x are skipped or read as zero rows."""
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    E, H, I, R = 4, 512, 128, 200
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(50, H, generator=g) * 0.1).half()
+    tok = torch.randint(0, 50, (R,), generator=g).to(torch.int32)
+    tok[7] = 50                                           # past the rows of x: a zero row
+    tok[8] = -3
+    reps, deq = _q4k_expert_stacks(E, I, H, (31, 32), torch.arange(E), dev)
+    chunks = torch.tensor([[1, 0, 20], [2, 20, 0], [0, 30, 80], [5, 120, 10], [-1, 130, 5], [3, 190, 30],
+                           [2, 150, -4], [1, 400, 3]], dtype=torch.int32)
+    for smallm in (False, True):
+        cap = 16 if smallm else 64
+        buf = torch.full((R, 2 * I), 7.0, dtype=torch.float16, device=dev)
+        mg.moe_up_q4k_ggemv(x.to(dev), *reps[0], *reps[1], buf, chunks.to(dev), H, I, tok.to(dev), smallm=smallm)
+        want = torch.full((R, 2 * I), 7.0)
+        for e, t0, nt in chunks.tolist():
+            if nt <= 0 or not 0 <= e < E or not 0 <= t0 < R:
+                continue
+            n = min(nt, cap, R - t0)
+            ids = tok[t0:t0 + n].long()
+            ok = (ids >= 0) & (ids < 50)
+            xs = torch.where(ok[:, None], x.float()[ids.clamp(0, 49)], torch.zeros(1))
+            want[t0:t0 + n, :I] = xs @ deq[0][e].t()
+            want[t0:t0 + n, I:] = xs @ deq[1][e].t()
+        got = buf.cpu().float()
+        untouched = want == 7.0
+        assert torch.equal(got[untouched], want[untouched])
+        assert O.max_rel_err(got, want) < TOL
