@@ -217,6 +217,62 @@ def wl_moe_gguf(dev):
                                    "(Q4_K gate, Q4_K up, SiLU*up, Q6_K down: 4 launches)", kernel="gemv_rows_kernel", cpu=lambda: None)
 
 
+def wl_moe_gguf_grouped(dev, T=2048):
+    """Prefill through the grouped GGUF MoE stages (next-row workload): routes sorted by expert, Q4_K gate / up
+    over chunks of at most 64 rows with the token gather inside the launch, SiLU * up, Q6_K down, weighted
+    gather per token; top-8 of 128 experts, H = 2048, I = 768.  Random codes and scales (timing only; parity is
+    tests/test_gpu_gguf.py)."""
+    import custom_esimd_kernels_vllm as v
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    E, k, H, I = 128, 8, 2048, 768
+    g = torch.Generator(device="cpu").manual_seed(98)
+    u8 = lambda *shape: torch.randint(0, 256, shape, dtype=torch.uint8, generator=g).to(dev)
+    f16 = lambda hi, *shape: (torch.rand(*shape, generator=g) * hi).half().to(dev)
+    gq, uq = u8(E, I, H // 2), u8(E, I, H // 2)
+    gs, gm, us, um = f16(0.01, E, I, H // 32), f16(0.005, E, I, H // 32), f16(0.01, E, I, H // 32), f16(0.005, E, I, H // 32)
+    dq, dh, ds = u8(E, H, I // 2), u8(E, H, I // 4), f16(0.002, E, H, I // 16)
+    x = (torch.randn(T, H, generator=g) * 0.1).half().to(dev)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    flat = ids.reshape(-1)
+    order = torch.sort(flat, stable=True).indices
+    tok_sorted = torch.arange(T).repeat_interleave(k)[order].to(torch.int32).to(dev)
+    counts = torch.bincount(flat, minlength=E)
+    rows, s0 = [], 0
+    smallm = T <= 16                                      # the caller's verify branch: fixed [E, 3] table, 16-row tiles
+    for e in range(E):
+        n = int(counts[e])
+        if smallm:
+            rows.append([e, s0, n])
+            s0 += n
+            continue
+        while n > 0:
+            c = min(64, n)
+            rows.append([e, s0, c])
+            s0 += c
+            n -= c
+    chunks = torch.tensor(rows, dtype=torch.int32).to(dev)
+    P = T * k
+    pos = torch.argsort(order).to(torch.int32).reshape(T, k).contiguous().to(dev)
+    w_sorted = torch.full((P,), 1.0 / k, dtype=torch.float16, device=dev)
+    gate_buf = torch.zeros(P, 2 * I, dtype=torch.float16, device=dev)
+    inter = torch.empty(P, I, dtype=torch.float16, device=dev)
+    out_route = torch.zeros(P, H, dtype=torch.float16, device=dev)
+    final = torch.empty(T, H, dtype=torch.float16, device=dev)
+
+    def launch(i):
+        mg.moe_up_q4k_ggemv(x, gq, gs, gm, uq, us, um, gate_buf, chunks, H, I, tok_sorted, smallm=smallm)
+        v.esimd_moe_silu_mul(gate_buf, inter, 2 * I, I, P)
+        mg.moe_down_q6k_ggemv(inter, dq, dh, ds, out_route, chunks, I, H, smallm=smallm)
+        v.esimd_moe_gather(out_route, pos, w_sorted, final, H, k, T)
+
+    used = int((counts > 0).sum())                        # experts with rows: their matrices are what a launch reads
+    wbytes = used * (2 * (I * H // 2 + 2 * I * (H // 32) * 2) + H * I // 2 + H * I // 4 + H * (I // 16) * 2)
+    return dict(launch=launch, R=1, bytes=wbytes + 2 * T * H * 2, flops=2 * P * 3 * I * H,
+                bound="hbm" if smallm else "mfma", dtype="f16",
+                name=f"next: grouped GGUF MoE prefill T={T} top-{k} of {E} experts H={H} I={I} ({len(rows)} chunks; "
+                     "Q4_K gate / up, SiLU*up, Q6_K down, gather: 4 launches)", kernel="skinny_kernel", cpu=lambda: None)
+
+
 def wl_q4_0_quantize(dev):
     """On-device group-128 Q4_0 quantization of a [14336, 4096] bf16 weight (next-row workload)."""
     import custom_esimd_kernels_vllm as v
@@ -657,6 +713,9 @@ WORKLOADS = {
     "next_moe_fp8_block_decode_t1": wl_moe_fp8_block_decode,
     "next_gemv_fp16_router": wl_gemv_fp16,
     "next_moe_gguf_t1": wl_moe_gguf,
+    "next_moe_gguf_grouped_t2048": wl_moe_gguf_grouped,
+    "next_moe_gguf_grouped_t512": lambda dev: wl_moe_gguf_grouped(dev, 512),
+    "next_moe_gguf_grouped_t16": lambda dev: wl_moe_gguf_grouped(dev, 16),
 }
 HEADLINE = "cfg1_m1"
 # the other benchmark configurations: reported as `cases` of the default run

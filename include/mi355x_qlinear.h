@@ -211,9 +211,13 @@ int mi_moe_gguf_gemv(int fmt, const void* x, int x_div, int nmat, const void* co
  * scales and mins).  Chunks with nt <= 0, an expert outside [0, E) or rows outside the output are
  * skipped; rows of a chunk past the 64 (16) are not computed, as in the reference kernel; token ids
  * outside [0, x_rows) read as zero rows.  Weights are dequantized as fp16(fp16(nibble * scale) - min)
- * and accumulated in fp32.  fmt = 2 (Q4_K), nmat <= 2, K % 32 == 0; one kernel launch.
- * Replaces moe_up_q4k_ggemv / moe_up_q4k_ggemv_smallm (S/csrc/moe_grouped/moe_q4k_ggemv.h:47-201, 311-321;
- * ATen entry S/csrc/moe_grouped/moe_grouped_entry.sycl:24-60; caller sglang_for_multi_arc.patch:2899-2901). */
+ * and accumulated in fp32.  fmt = 2 (Q4_K), 5 (Q5_K: fp16(fp16(v5 * scale) - min)) or 6 (Q6_K:
+ * fp16((v6 - 32) * scale), scales [E, N, K/16]); the high bits of 5 / 6 in ELEMENT order as for
+ * mi_moe_gguf_gemv.  nmat <= 2, K % 32 == 0; one kernel launch.
+ * Replaces moe_up_q4k_ggemv / moe_up_q4k_ggemv_smallm (S/csrc/moe_grouped/moe_q4k_ggemv.h:47-201, 311-321),
+ * moe_down_q5k_ggemv / _smallm (moe_q5k_down_ggemv.h:26-191) and moe_down_q6k_ggemv / _smallm
+ * (moe_q6k_down_ggemv.h) with x = the intermediate in sorted order and no token list; ATen entries
+ * S/csrc/moe_grouped/moe_grouped_entry.sycl:24-106; callers sglang_for_multi_arc.patch:2899-2924. */
 int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_ids, int nmat, const void* const* ql,
                         const void* const* qh, const void* const* scale, const void* const* qmin, void* out,
                         long long out_stride, int out_rows, const int32_t* chunks, int num_chunks, int num_experts,

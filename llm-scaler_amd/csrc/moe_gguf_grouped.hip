@@ -2,7 +2,7 @@
 // is a small-M GEMM against that expert's repacked K-quant matrix.  The weight-streaming skinny
 // kernel runs them all in one launch (grid = row blocks x chunks): a workgroup owns 64 weight rows
 // of the chunk's expert and all of K, and multiplies them with up to 64 (or 16) rows of x, which it
-// gathers itself through the token list.
+// gathers itself through the token list.  All workgroups of a chunk run on one XCD.
 #include "skinny_kernel.hpp"
 #include "../../include/mi355x_qlinear.h"
 
@@ -10,9 +10,14 @@ using namespace qlin;
 
 namespace {
 
-template <int FMT, int MT, int UN, bool SL>
-void launch_grouped_one(const SkinnyArgs& a, hipStream_t st) {
-  constexpr int RT = 4, NW = 8;
+template <int FMT, int MT, int UN, bool SL, int RT = 4, int NW = 8>
+void launch_grouped_one(SkinnyArgs a, hipStream_t st) {
+  a.rpw = RT * 16;
+  a.tiles_total = 0;
+  for (int i = 0; i < a.nmat; ++i) {
+    a.tiles[i] = (a.N[i] + a.rpw - 1) / a.rpw;
+    a.tiles_total += a.tiles[i];
+  }
   constexpr int kStage = NW * RT * 16 * (64 + 16) + (MT >= kSkinnyXLdsFrom ? NW * 16 * (256 + 16) : 0);
   constexpr int kRed = NW * RT * MT * 1024;
   static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
@@ -30,10 +35,12 @@ void launch_grouped_one(const SkinnyArgs& a, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(NW * 64), lds, st, a);
 }
 
-template <int FMT, int MT, int UN>
+template <int FMT, int MT, int UN, int RT = 4, int NW = 8>
 void launch_grouped(const SkinnyArgs& a, hipStream_t st) {
-  if (skinny_tables_fit<FMT, MT, 4, 8>(a.K)) launch_grouped_one<FMT, MT, UN, true>(a, st);
-  else launch_grouped_one<FMT, MT, UN, false>(a, st);
+  if constexpr (FMT == 2 || FMT == 7) {               // the formats with per-32 scale and min tables
+    if (skinny_tables_fit<FMT, MT, RT, NW>(a.K)) return launch_grouped_one<FMT, MT, UN, true, RT, NW>(a, st);
+  }
+  launch_grouped_one<FMT, MT, UN, false, RT, NW>(a, st);
 }
 
 }  // namespace
@@ -45,7 +52,7 @@ int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_i
                         long long out_stride, int out_rows, const int32_t* chunks, int num_chunks, int num_experts,
                         int N, int K, int rows16, void* stream) {
   if (!x || !ql || !scale || !out || !chunks) return MI_ERR_ARG;
-  if (fmt != RF_Q4K) return MI_ERR_ARG;
+  if (fmt != RF_Q4K && fmt != RF_Q5K && fmt != RF_Q6K) return MI_ERR_ARG;
   if (nmat < 1 || nmat > 2 || num_experts < 1) return MI_ERR_ARG;
   if (x_rows < 0 || out_rows < 0 || num_chunks < 0 || N < 0 || K <= 0 || (K % 32)) return MI_ERR_SHAPE;
   if (out_stride < (long long)nmat * N) return MI_ERR_SHAPE;
@@ -56,10 +63,17 @@ int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_i
   a.chunks = chunks; a.tok_ids = tok_ids; a.num_chunks = num_chunks; a.num_experts = num_experts;
   a.x_rows = x_rows; a.out_rows = out_rows; a.out_stride = out_stride;
   const long long nk = (long long)N * K;
-  a.w_stride = nk / 2; a.s_stride = nk / 32 * 2; a.z_stride = nk / 32 * 2; a.h_stride = 0;
+  a.w_stride = nk / 2;
+  a.s_stride = fmt == RF_Q6K ? nk / 16 * 2 : nk / 32 * 2;
+  a.z_stride = nk / 32 * 2;
+  a.h_stride = fmt == RF_Q5K ? nk / 8 : nk / 4;
   for (int i = 0; i < nmat; ++i) {
-    if (!ql[i] || !scale[i] || !qmin || !qmin[i]) return MI_ERR_ARG;
-    a.w[i] = ql[i]; a.s[i] = scale[i]; a.z[i] = qmin[i]; a.h[i] = qh ? qh[i] : nullptr;
+    if (!ql[i] || !scale[i]) return MI_ERR_ARG;
+    if (fmt != RF_Q6K && (!qmin || !qmin[i])) return MI_ERR_ARG;
+    if (fmt != RF_Q4K && (!qh || !qh[i])) return MI_ERR_ARG;
+    a.w[i] = ql[i]; a.s[i] = scale[i];
+    a.z[i] = fmt != RF_Q6K ? qmin[i] : nullptr;
+    a.h[i] = fmt != RF_Q4K ? qh[i] : nullptr;
     a.out[i] = (char*)out + (size_t)i * N * 2;
     a.N[i] = N;
     a.tiles[i] = (N + 63) / 64;
@@ -67,8 +81,20 @@ int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_i
   }
   if ((long long)((num_chunks + 7) / 8) * 8 * a.tiles_total >= (1ll << 31)) return MI_ERR_SHAPE;
   hipStream_t st = (hipStream_t)stream;
-  if (rows16) launch_grouped<RF_Q4K, 1, 2>(a, st);
-  else launch_grouped<RF_Q4K, 4, 1>(a, st);
+  // 7 / 8: Q5_K / Q6_K with the high bits in element order.  Small workgroups (two or four wavefronts splitting
+  // K, one granule in flight each) so that several share a CU and overlap their load -> LDS -> MFMA chains:
+  // T=2048, top 8 of 128 experts, H=2048, I=768: Q4_K up 364 -> 273 us, Q6_K down 345 -> 196 us against eight
+  // wavefronts; 16 tokens: up 61 -> 50 us, down 122 -> 46 us.
+  if (fmt == RF_Q4K) {
+    if (rows16) launch_grouped<RF_Q4K, 1, 2, 4, 4>(a, st);
+    else launch_grouped<RF_Q4K, 4, 1, 4, 2>(a, st);
+  } else if (fmt == RF_Q5K) {
+    if (rows16) launch_grouped<7, 1, 1, 4, 2>(a, st);
+    else launch_grouped<7, 4, 1, 4, 2>(a, st);
+  } else {
+    if (rows16) launch_grouped<8, 1, 1, 4, 2>(a, st);
+    else launch_grouped<8, 4, 1, 4, 2>(a, st);
+  }
   return launch_status();
 }
 

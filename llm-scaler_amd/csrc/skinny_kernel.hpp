@@ -61,7 +61,9 @@ enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
 
 // ---------------------------------------------------------------- kernel
 // FMT: 0 = fp8 (SC selects the scale mode), 1 = int4 g128, 2 = Q4_K repacked, 3 = Q4_0,
-// 4 = Q8_0, 5 = Q5_K, 6 = Q6_K (the GGUF formats in their repacked representation, fp16).
+// 4 = Q8_0, 5 = Q5_K, 6 = Q6_K (the GGUF formats in their repacked representation, fp16);
+// 7 = Q5_K, 8 = Q6_K with the high bits in element order (the MoE down stacks: Q5_K byte j bit b =
+// fifth bit of element 8j + b, Q6_K byte j field p = top two bits of element 4j + p).
 // MT = 16-row activation tiles (M <= 16 MT), RT = 16-row weight tiles per
 // workgroup, NW = wavefronts splitting K, UN = granules in flight per wave.
 // SL: the scales (and mins / zero-points) of the workgroup's rows are staged once in LDS instead
@@ -78,8 +80,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   constexpr bool kIsQ4K = (FMT == 2);
   constexpr bool kIsQ40 = (FMT == 3);
   constexpr bool kIsQ80 = (FMT == 4);
-  constexpr bool kIsQ5K = (FMT == 5);
-  constexpr bool kIsQ6K = (FMT == 6);
+  constexpr bool kIsQ5K = (FMT == 5 || FMT == 7);
+  constexpr bool kIsQ6K = (FMT == 6 || FMT == 8);
+  constexpr bool kPlainH = (FMT == 7 || FMT == 8);    // high bits in element order
   constexpr bool kByteW = kIsFp8 || kIsQ80;           // one byte per weight: 128 bytes per row and granule
   constexpr bool kHigh = kIsQ5K || kIsQ6K;            // extra high bits per weight
   constexpr bool kBlock = kIsFp8 && SC == SC_BLOCK;
@@ -210,7 +213,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   struct Stage {
     u32x4 wa[US][RT], wb[US][RT];
     u32x4 xa[US][MT][4];
-    u32x4 ha[US][RT][kHigh ? 2 : 1];                  // q5k / q6k: the lane's 32 high-bit bytes
+    u32x4 ha[US][RT][(kHigh && !kPlainH) ? 2 : 1];    // q5k / q6k: the lane's 32 high-bit bytes (element order: 4 / 8 bytes)
     uint32_t sc[US][RT];                              // raw bits: int4 / q4k scale (fp16), block scale (fp32)
     uint32_t zz[US][RT];                              // raw: int4 zero-point byte / q4k min (fp16)
   };
@@ -277,11 +280,22 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
         if constexpr (kHigh) {
           // per 512-k tile the high bits of element b*64 + t' (Q5_K) / p*128 + t' (Q6_K) sit in
           // byte t': this lane's 32 consecutive k are 32 consecutive bytes, one bit field
+          if constexpr (kPlainH) {
+            // element order: this lane's 32 consecutive k are 4 (Q5_K) or 8 (Q6_K) consecutive bytes
+            const uint32_t ho = ok && n < nend ? (uint32_t)n * hrow + (uint32_t)gic * (kIsQ5K ? 16u : 32u) + (uint32_t)g * (kIsQ5K ? 4u : 8u) : kOOB;
+            if constexpr (kIsQ5K) {
+              st.ha[u][t][0] = u32x4{__builtin_amdgcn_raw_buffer_load_b32(hr, ho, 0, 0), 0u, 0u, 0u};
+            } else {
+              const u32x2 two = __builtin_amdgcn_raw_buffer_load_b64(hr, ho, 0, 0);
+              st.ha[u][t][0] = u32x4{two[0], two[1], 0u, 0u};
+            }
+          } else {
           const uint32_t tile = (uint32_t)gic >> 2;
           const uint32_t within = kIsQ5K ? ((uint32_t)g & 1u) * 32u : (uint32_t)g * 32u;
           const uint32_t ho = ok && n < nend ? (uint32_t)n * hrow + tile * (kIsQ5K ? 64u : 128u) + within : kOOB;
           st.ha[u][t][0] = __builtin_amdgcn_raw_buffer_load_b128(hr, ho, 0, 0);
           st.ha[u][t][1] = __builtin_amdgcn_raw_buffer_load_b128(hr, ho == kOOB ? kOOB : ho + 16u, 0, 0);
+          }
         }
       }
 #pragma unroll
@@ -400,9 +414,24 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
             const _Float16 mn = __builtin_bit_cast(_Float16, (uint16_t)st.zz[u][t]);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
+              if constexpr (kPlainH && kIsQ5K) {
+                // byte i of the word: one bit per element 8 i + b; spread to one bit per byte
+                const uint32_t hb = (st.ha[u][t][0][0] >> (8 * i)) & 0xFFu;
+                const uint32_t hA = ((hb & 0xFu) * 0x00204081u) & 0x01010101u;
+                const uint32_t hB = ((hb >> 4) * 0x00204081u) & 0x01010101u;
+                b[i] = kqx8_to_f16<1>(wa[i], hA, hB, 0u, s0, mn);
+              } else if constexpr (kPlainH) {
+                // 16 bits: a 2-bit field per element 8 i + p; spread to one field per byte
+                const uint32_t hw = (st.ha[u][t][0][i >> 1] >> (16 * (i & 1))) & 0xFFFFu;
+                auto spread = [](uint32_t x) {
+                  return (((x & 0x33u) * 0x1001u) & 0x00030003u) | (((((x >> 2) & 0x33u) * 0x1001u) & 0x00030003u) << 8);
+                };
+                b[i] = kqx8_to_f16<2>(wa[i], spread(hw & 0xFFu), spread(hw >> 8), 0u, i < 2 ? s0 : s1, (_Float16)0.0f);
+              } else {
               const uint32_t hA = st.ha[u][t][i >> 1][(i & 1) * 2], hB = st.ha[u][t][i >> 1][(i & 1) * 2 + 1];
               if constexpr (kIsQ5K) b[i] = kqx8_to_f16<1>(wa[i], hA, hB, shift, s0, mn);
               else b[i] = kqx8_to_f16<2>(wa[i], hA, hB, shift, i < 2 ? s0 : s1, (_Float16)0.0f);
+              }
             }
           }
         }
@@ -540,9 +569,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 template <int FMT, int RT>
 static inline int skinny_table_bytes(int K) {
   if (FMT == 1) return (RT * 16 * (K / 128) * 3 + 15) & ~15;   // fp16 scales + zero-point bytes
-  const bool side32 = FMT == 2 || FMT == 5 || FMT == 3 || FMT == 4;
+  const bool side32 = FMT == 2 || FMT == 5 || FMT == 7 || FMT == 3 || FMT == 4;
   if (!side32) return 0;
-  return RT * 16 * (K / 32) * 2 * ((FMT == 2 || FMT == 5) ? 2 : 1);
+  return RT * 16 * (K / 32) * 2 * ((FMT == 2 || FMT == 5 || FMT == 7) ? 2 : 1);
 }
 
 template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false>
@@ -576,7 +605,7 @@ static void launch_one(SkinnyArgs a, int rpw, hipStream_t st) {
 // and the tables fit beside the staging tiles; the plain one otherwise.
 template <int FMT, int MT, int RT, int NW>
 static inline bool skinny_tables_fit(int K) {
-  if constexpr (FMT == 1 || FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5) {
+  if constexpr (FMT == 1 || FMT == 2 || FMT == 3 || FMT == 4 || FMT == 5 || FMT == 7) {
     constexpr int kStage = NW * RT * 16 * (((FMT == 0 || FMT == 4) ? 128 : 64) + 16) + (MT >= kSkinnyXLdsFrom ? NW * 16 * (256 + 16) : 0);
     return (FMT == 1 || K % 256 == 0) && kStage + skinny_table_bytes<FMT, RT>(K) <= 160 * 1024;
   }

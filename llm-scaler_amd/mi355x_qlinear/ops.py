@@ -581,6 +581,54 @@ def moe_up_q4k_ggemv(expert_states, gate_ql, gate_sc, gate_mn, up_ql, up_sc, up_
     return gate_buf
 
 
+def _moe_down_grouped(fmt, intermediate, w_ql, w_qh, w_scale, w_min, expert_output, chunks, intermediate_size,
+                      hidden_size, smallm, who):
+    I, H = int(intermediate_size), int(hidden_size)
+    _chk_chunks(chunks, who)
+    _chk(w_ql.dim() == 3 and I % 32 == 0, f"{who}: w_ql must be [E, hidden, intermediate/2], intermediate a multiple of 32")
+    E = w_ql.shape[0]
+    _chk_stack(w_ql, torch.uint8, (E, H, I // 2), "w_ql", who)
+    if fmt == 5:
+        _chk_stack(w_qh, torch.uint8, (E, H, I // 8), "w_qh", who)
+        _chk_stack(w_scale, torch.float16, (E, H, I // 32), "w_scale", who)
+        _chk_stack(w_min, torch.float16, (E, H, I // 32), "w_min", who)
+    else:
+        _chk_stack(w_qh, torch.uint8, (E, H, I // 4), "w_qh", who)
+        _chk_stack(w_scale, torch.float16, (E, H, I // 16), "w_scale", who)
+    _chk(intermediate.dtype == torch.float16 and intermediate.is_contiguous() and intermediate.dim() == 2
+         and intermediate.shape[1] == I, f"{who}: intermediate must be contiguous fp16 [total, intermediate]")
+    _chk(expert_output.dtype == torch.float16 and expert_output.is_contiguous() and expert_output.dim() == 2
+         and expert_output.shape[1] == H, f"{who}: expert_output must be contiguous fp16 [total, hidden]")
+    total = expert_output.shape[0]
+    _chk(intermediate.shape[0] >= total, f"{who}: intermediate has fewer rows than expert_output")
+    if chunks.size(0) == 0 or total == 0:
+        return expert_output
+    capi.call("mi_moe_gguf_grouped", intermediate, fmt, capi.ptr(intermediate), intermediate.shape[0], None, 1,
+              capi.ptr_array([w_ql]), capi.ptr_array([w_qh]), capi.ptr_array([w_scale]),
+              capi.ptr_array([w_min]) if fmt == 5 else None, capi.ptr(expert_output), H, total, capi.ptr(chunks),
+              chunks.size(0), E, H, I, 1 if smallm else 0)
+    return expert_output
+
+
+def moe_down_q5k_ggemv(intermediate, w_ql, w_qh, w_scale, w_min, expert_output, chunks, intermediate_size,
+                       hidden_size, smallm=False):
+    """expert_output[t0 + m] = intermediate[t0 + m] @ Wd[e]^T for every chunk {e, t0, nt}, m < min(nt, 64)
+    (16 with smallm), on the Q5_K stack w_ql [E, H, I/2], w_qh [E, H, I/8] in ELEMENT order (byte j bit b =
+    fifth bit of element 8j + b), scale / min [E, H, I/32] fp16
+    (S/csrc/moe_grouped/moe_grouped_entry.sycl:62-84, moe_q5k_down_ggemv.h:26-191).  Returns expert_output."""
+    return _moe_down_grouped(5, intermediate, w_ql, w_qh, w_scale, w_min, expert_output, chunks, intermediate_size,
+                             hidden_size, smallm, "moe_down_q5k_ggemv")
+
+
+def moe_down_q6k_ggemv(intermediate, w_ql, w_qh, w_scale, expert_output, chunks, intermediate_size, hidden_size,
+                       smallm=False):
+    """The same on the Q6_K stack w_ql [E, H, I/2], w_qh [E, H, I/4] in ELEMENT order (byte j 2-bit field p =
+    top bits of element 4j + p), scale [E, H, I/16] fp16
+    (S/csrc/moe_grouped/moe_grouped_entry.sycl:86-106, moe_q6k_down_ggemv.h)."""
+    return _moe_down_grouped(6, intermediate, w_ql, w_qh, w_scale, None, expert_output, chunks, intermediate_size,
+                             hidden_size, smallm, "moe_down_q6k_ggemv")
+
+
 def _gemv_q6_k(input, ql, qh, weight_scale, output, who):
     _chk(ql.dtype == torch.uint8 and ql.dim() == 2 and ql.is_contiguous(), f"{who}: ql must be contiguous uint8 [N, K/2]")
     N, K = ql.shape[0], ql.shape[1] * 2

@@ -52,6 +52,54 @@ def test_moe_tiled_workspace_sizes_and_argument_errors():
     assert f(*args(ws=None)) == -1 and f(*args(wsb=1024)) == -1
 
 
+def test_moe_gguf_grouped_argument_errors():
+    """mi_moe_gguf_grouped answers bad arguments and sizes beyond its 32-bit addressing with error codes, and
+    empty inputs with success, before anything is enqueued."""
+    lib = capi.lib()
+    ok = ctypes.c_void_p(256)                      # never dereferenced: every case below returns before a launch
+    arr = (ctypes.c_void_p * 2)(256, 256)
+    none2 = (ctypes.c_void_p * 2)(None, None)
+
+    def f(**kw):
+        return lib.mi_moe_gguf_grouped(kw.get("fmt", 2), kw.get("x", ok), kw.get("x_rows", 64), None, kw.get("nmat", 2),
+                                       kw.get("ql", arr), kw.get("qh", None), kw.get("sc", arr), kw.get("mn", arr),
+                                       kw.get("out", ok), ctypes.c_longlong(kw.get("stride", 1024)), kw.get("rows", 64),
+                                       kw.get("chunks", ok), kw.get("n", 4), 8, kw.get("N", 512), kw.get("K", 2048), 0,
+                                       None)
+    assert f(x=None) == -1 and f(out=None) == -1 and f(chunks=None) == -1 and f(ql=None) == -1 and f(sc=None) == -1
+    assert f(fmt=3) == -1 and f(fmt=7) == -1 and f(nmat=0) == -1 and f(nmat=3) == -1
+    assert f(mn=None) == -1 and f(mn=none2) == -1 and f(ql=none2) == -1          # Q4_K needs mins
+    assert f(fmt=5) == -1 and f(fmt=6) == -1                                     # Q5_K / Q6_K need the high bits
+    assert f(fmt=6, qh=none2) == -1
+    assert f(K=2040) == -2 and f(K=0) == -2 and f(stride=1023) == -2 and f(rows=-1) == -2 and f(n=-1) == -2
+    assert f(N=1 << 20, stride=1 << 22) == -2                                    # N K beyond 2^31
+    assert f(x_rows=1 << 19) == -2                                               # x beyond 2 GiB
+    assert f(n=0) == 0 and f(rows=0) == 0 and f(x_rows=0) == 0 and f(N=0, stride=0) == 0
+
+
+def test_moe_grouped_module_matches_the_reference_binding():
+    """Names, argument order and defaults of the pybind module the patched SGLang imports
+    (S/csrc/moe_grouped/moe_grouped_entry.sycl:108-127, sglang_for_multi_arc.patch:2114)."""
+    import inspect
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    want = {
+        "moe_up_q4k_ggemv": ["expert_states", "gate_ql", "gate_sc", "gate_mn", "up_ql", "up_sc", "up_mn", "gate_buf",
+                             "chunks", "hidden_size", "intermediate_size", "tok_ids", "smallm"],
+        "moe_down_q5k_ggemv": ["intermediate", "w_ql", "w_qh", "w_scale", "w_min", "expert_output", "chunks",
+                               "intermediate_size", "hidden_size", "smallm"],
+        "moe_down_q6k_ggemv": ["intermediate", "w_ql", "w_qh", "w_scale", "expert_output", "chunks",
+                               "intermediate_size", "hidden_size", "smallm"],
+    }
+    for name, params in want.items():
+        sig = inspect.signature(getattr(mg, name))
+        assert list(sig.parameters) == params, name
+        assert sig.parameters["smallm"].default is False
+    # argument checks run before the library is touched
+    z = torch.zeros(1, 4, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match=r"chunks \[num_chunks,3\]"):
+        mg.moe_up_q4k_ggemv(z, z, z, z, z, z, z, z, torch.zeros(2, 2, dtype=torch.int32), 4, 4)
+
+
 def test_header_pointer_and_scalar_mapping():
     p = capi.parse_header()
     assert p["mi_gemm_fp8_pern"] == [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_void_p]
@@ -256,7 +304,6 @@ with open(_NAMES) as _f:
 # caller falls back, which is the intended behaviour for kernels outside the quantized-linear path.
 ABSENT_BY_DESIGN = {
     "sglang_decode_attn", "eagle_page_attn_decode_temp_size", "custom_esimd_kernels_prefill_dpas",
-    "moe_grouped_gguf_xpu",
     ("custom_esimd_kernels_sglang", "esimd_gdn_conv_fused_seq"),
     ("custom_esimd_kernels_sglang", "esimd_qkv_split_norm_rope"),
 }

@@ -434,3 +434,117 @@ def test_moe_grouped_q4k_up_chunk_semantics(ops, dev):
         untouched = want == 7.0
         assert torch.equal(got[untouched], want[untouched])
         assert O.max_rel_err(got, want) < TOL
+
+
+def _down_stack(kind, U, H, I, seed, emap, dev):
+    """Q5_K / Q6_K down stack [E, H, ...] with element-order high bits and its dequantized weights [U, H, I]."""
+    Ip = (I + 255) // 256 * 256                           # raw super-blocks hold 256 elements
+    raw = _raw_case(kind, U * H, Ip, seed=seed)
+    full = G.q5k_repack_plain(raw) if kind == "q5_k" else G.q6k_repack_plain(raw)
+    if Ip != I:                                           # K % 32 == 0: cut every row to its first I elements
+        per = (2, 8, 32, 32) if kind == "q5_k" else (2, 4, 16)
+        full = tuple(np.ascontiguousarray(a[:, :I // d]) for a, d in zip(full, per))
+    deq = G.q5k_dequant_plain(*full) if kind == "q5_k" else G.q6k_dequant_plain(*full)
+    stack = lambda a: _t(a).reshape(U, -1, a.shape[-1]).to(dev)[emap.to(dev)].contiguous()
+    return [stack(a) for a in full], torch.from_numpy(deq.astype(np.float32)).reshape(U, H, I)
+
+
+@pytest.mark.parametrize("kind", ["q5_k", "q6_k"])
+@pytest.mark.parametrize("T,E,k,H,I,smallm", [
+    (4, 16, 4, 2048, 512, True),
+    (16, 8, 2, 96, 512, True),               # H not a multiple of the 64-row block
+    (200, 8, 2, 2048, 512, False),
+    (90, 6, 3, 128, 2080 // 32 * 32, False),  # K = 2080: partial last granule
+    (70, 4, 2, 256, 96, False),              # K = 96: one partial granule, rows cut inside a super-block
+    (300, 128, 8, 2048, 768, False),
+])
+def test_moe_grouped_down(ops, dev, kind, T, E, k, H, I, smallm):
+    """moe_down_q5k_ggemv / moe_down_q6k_ggemv (S/csrc/moe_grouped/moe_grouped_entry.sycl:62-106): rows of the
+    intermediate in sorted order against the chunk's expert, element-order high bits."""
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    g = torch.Generator().manual_seed(T + H + I)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    chunks, _, _ = _expert_chunks(ids, E, 16 if smallm else 64, fixed=smallm)
+    U = min(E, 8)
+    emap = (7 * torch.arange(E) + 3) % U if U < E else torch.arange(E)
+    args, wd = _down_stack(kind, U, H, I, 41 + I, emap, dev)
+    P = T * k
+    inter = (torch.randn(P, I, generator=g) * 0.1).half()
+    out = torch.zeros(P, H, dtype=torch.float16, device=dev)
+    fn = mg.moe_down_q5k_ggemv if kind == "q5_k" else mg.moe_down_q6k_ggemv
+    ret = fn(inter.to(dev), *args, out, chunks.to(dev), I, H, smallm=smallm)
+    assert ret.data_ptr() == out.data_ptr()
+    want = torch.zeros(P, H)
+    for e, t0, nt in chunks.tolist():
+        if nt > 0:
+            want[t0:t0 + nt] = inter.float()[t0:t0 + nt] @ wd[int(emap[e])].t()
+    assert O.max_rel_err(out.cpu(), want) < TOL
+
+
+@pytest.mark.parametrize("kind", ["q5_k", "q6_k"])
+def test_moe_grouped_down_every_high_bit(ops, dev, kind):
+    """Weights whose low nibbles are zero and whose high bits are set for ONE element per row at a time: the
+    output then is that element's activation times (16 or 48 - 32) * scale, so a high-bit field read for the
+    wrong element shows up as a wrong column of the intermediate."""
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    E, H, I = 1, 16, 256
+    chunks = torch.tensor([[0, 0, 3]], dtype=torch.int32, device=dev)
+    inter = (torch.arange(3 * I).reshape(3, I) % 97 + 1).half() / 64          # distinct per element within a row
+    for e0 in list(range(0, 40)) + [63, 64, 127, 128, 200, 255]:
+        v = np.zeros((H, I), dtype=np.int64)
+        v[:, e0] = 16 if kind == "q5_k" else 48
+        if kind == "q5_k":
+            sc12 = O.q4k_pack_scales(np.full((H, 1, 8), 1), np.zeros((H, 1, 8), dtype=np.int64))
+            raw = G.q5k_build_raw(v + 0, sc12, np.full((H, 1), 0.5, np.float16), np.zeros((H, 1), np.float16))
+            rep = G.q5k_repack_plain(raw)
+            wd = G.q5k_dequant_plain(*rep)
+        else:
+            raw = G.q6k_build_raw(v + 32 * (v == 0), np.full((H, 1, 16), 1, np.int8), np.full((H, 1), 0.5, np.float16))
+            rep = G.q6k_repack_plain(raw)
+            wd = G.q6k_dequant_plain(*rep)
+        wd = torch.from_numpy(wd.astype(np.float32))
+        assert int((wd != 0).sum()) == H and bool((wd[:, e0] != 0).all())
+        out = torch.zeros(3, H, dtype=torch.float16, device=dev)
+        args = [_t(a).unsqueeze(0).to(dev) for a in rep]
+        fn = mg.moe_down_q5k_ggemv if kind == "q5_k" else mg.moe_down_q6k_ggemv
+        fn(inter.to(dev), *args, out, chunks, I, H)
+        assert torch.equal(out.cpu().float(), (inter.float() @ wd.t()).half().float()), e0
+
+
+def test_moe_grouped_prefill_flow(ops, dev):
+    """The caller's whole grouped prefill (sglang_for_multi_arc.patch:2810-2950): sort routes by expert -> Q4_K up
+    over chunks with the gather folded in -> SiLU * up -> Q5_K down -> gather + weighted sum per token, against
+    the same chain on the oracle's dequantized weights."""
+    v, s = ops
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    # the caller takes a name from the sglang package, else from the vLLM package (patch :2077-2087)
+    silu_mul = getattr(s, "esimd_moe_silu_mul", None) or v.esimd_moe_silu_mul
+    gather = getattr(s, "esimd_moe_gather", None) or v.esimd_moe_gather
+    T, E, k, H, I = 150, 8, 2, 512, 256
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(T, H, generator=g) * 0.1).half()
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    tw = torch.rand(T, k, generator=g).half()
+    chunks, tok_sorted, order = _expert_chunks(ids, E, 64, fixed=False)
+    reps, deq = _q4k_expert_stacks(E, I, H, (51, 52), torch.arange(E), dev)
+    dargs, wd = _down_stack("q5_k", E, H, I, 53, torch.arange(E), dev)
+    P = T * k
+    gate_buf = torch.zeros(P, 2 * I, dtype=torch.float16, device=dev)
+    mg.moe_up_q4k_ggemv(x.to(dev), *reps[0], *reps[1], gate_buf, chunks.to(dev), H, I, tok_sorted.to(dev))
+    inter = torch.empty(P, I, dtype=torch.float16, device=dev)
+    silu_mul(gate_buf, inter, 2 * I, I, P)
+    out_route = torch.zeros(P, H, dtype=torch.float16, device=dev)
+    mg.moe_down_q5k_ggemv(inter, *dargs, out_route, chunks.to(dev), I, H)
+    inv = torch.argsort(order)
+    pos = inv.to(torch.int32).reshape(T, k).contiguous()
+    w_sorted = tw.reshape(-1)[order].contiguous()
+    final = torch.empty(T, H, dtype=torch.float16, device=dev)
+    gather(out_route, pos.to(dev), w_sorted.to(dev), final, H, k, T)
+    want = torch.zeros(T, H)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            gu = x.float()[t] @ deq[0][e].t(), x.float()[t] @ deq[1][e].t()
+            h = (torch.nn.functional.silu(gu[0].half().float()) * gu[1].half().float()).half().float()
+            want[t] += float(tw[t, j]) * (h @ wd[e].t()).half().float()
+    assert O.max_rel_err(final.cpu(), want) < 2 * TOL      # three fp16 roundings on the way
