@@ -18,12 +18,16 @@ void launch_grouped_one(SkinnyArgs a, hipStream_t st) {
     a.tiles[i] = (a.N[i] + a.rpw - 1) / a.rpw;
     a.tiles_total += a.tiles[i];
   }
-  constexpr int kStage = NW * RT * 16 * (64 + 16) + (MT >= kSkinnyXLdsFrom ? NW * 16 * (256 + 16) : 0);
-  constexpr int kRed = NW * RT * MT * 1024;
+  constexpr int MTL = MT ? MT : 4;                    // tiles of x the LDS is sized for
+  constexpr int kStage = NW * RT * 16 * (64 + 16) + (MTL >= kSkinnyXLdsFrom ? NW * 16 * (256 + 16) : 0);
+  constexpr int kRed = NW * RT * MTL * 1024;
   static_assert((kStage > kRed ? kStage : kRed) <= 160 * 1024, "staging tiles exceed the 160 KiB of LDS per workgroup");
   const int with_tables = kStage + (SL ? skinny_table_bytes<FMT, RT>(a.K) : 0);
   const int lds = with_tables > kRed ? with_tables : kRed;
-  auto kern = skinny_kernel<ActF16, FMT, 0, MT, RT, NW, UN, SL, true>;
+  // MT = 0: the workgroups choose 1..4 tiles of x themselves (LDS sized for four)
+  void (*kern)(const SkinnyArgs);
+  if constexpr (MT == 0) kern = skinny_grouped_kernel<ActF16, FMT, RT, NW, SL>;
+  else kern = skinny_kernel<ActF16, FMT, 0, MT, RT, NW, UN, SL, true>;
   if (lds > 64 * 1024) {
     static int raised = 0;                            // opt in to > 64 KiB of dynamic LDS (grows with K)
     if (raised < lds) {
@@ -38,7 +42,7 @@ void launch_grouped_one(SkinnyArgs a, hipStream_t st) {
 template <int FMT, int MT, int UN, int RT = 4, int NW = 8>
 void launch_grouped(const SkinnyArgs& a, hipStream_t st) {
   if constexpr (FMT == 2 || FMT == 7) {               // the formats with per-32 scale and min tables
-    if (skinny_tables_fit<FMT, MT, RT, NW>(a.K)) return launch_grouped_one<FMT, MT, UN, true, RT, NW>(a, st);
+    if (skinny_tables_fit<FMT, MT ? MT : 4, RT, NW>(a.K)) return launch_grouped_one<FMT, MT, UN, true, RT, NW>(a, st);
   }
   launch_grouped_one<FMT, MT, UN, false, RT, NW>(a, st);
 }
@@ -87,13 +91,13 @@ int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_i
   // wavefronts; 16 tokens: up 61 -> 50 us, down 122 -> 46 us.
   if (fmt == RF_Q4K) {
     if (rows16) launch_grouped<RF_Q4K, 1, 2, 4, 4>(a, st);
-    else launch_grouped<RF_Q4K, 4, 1, 4, 2>(a, st);
+    else launch_grouped<RF_Q4K, 0, 1, 4, 2>(a, st);
   } else if (fmt == RF_Q5K) {
     if (rows16) launch_grouped<7, 1, 1, 4, 2>(a, st);
-    else launch_grouped<7, 4, 1, 4, 2>(a, st);
+    else launch_grouped<7, 0, 1, 4, 2>(a, st);
   } else {
     if (rows16) launch_grouped<8, 1, 1, 4, 2>(a, st);
-    else launch_grouped<8, 4, 1, 4, 2>(a, st);
+    else launch_grouped<8, 0, 1, 4, 2>(a, st);
   }
   return launch_status();
 }

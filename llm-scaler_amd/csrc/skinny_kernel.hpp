@@ -71,8 +71,10 @@ enum : int { SC_PERN = 0, SC_PERT = 1, SC_BLOCK = 2 };
 // Q5_K, Q4_0, Q8_0 (needs K % 256 == 0), per-128 tables for INT4; chosen when the tables fit
 // beside the staging tiles.
 // GRP: the grid is (row blocks x chunks), see SkinnyArgs; all workgroups of a chunk run on one XCD.
-template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false, bool GRP = false>
-__global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
+// The body: `tile` = row block over all matrices, m0 = first row of x (dense), {eid, t0, mrows} = the chunk (GRP).
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL, bool GRP>
+__device__ __forceinline__ void skinny_body(const SkinnyArgs& a, int tile, const int m0, const int eid, const int t0,
+                                            const int mrows) {
   using V8 = typename Act::v8;
   using Elem = typename Act::elem;
   constexpr bool kIsFp8 = (FMT == 0);
@@ -101,30 +103,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   f32x4 (*red)[RT][MT][64] = reinterpret_cast<f32x4 (*)[RT][MT][64]>(smem);
 
-  int tile = blockIdx.x;
-  int m0 = 0;                                         // first row of x of this workgroup
-  int eid = 0, t0 = 0, mrows = 0;
-  if constexpr (GRP) {
-    // workgroups are dealt to the 8 XCDs in turn: chunk c runs on XCD c % 8, so its rows of x enter one L2
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int rnd = slot / a.tiles_total;
-    const int cid = rnd * 8 + xcd;
-    tile = slot - rnd * a.tiles_total;
-    if (cid >= a.num_chunks) return;
-    eid = a.chunks[3 * cid];
-    t0 = a.chunks[3 * cid + 1];
-    const int nt = a.chunks[3 * cid + 2];
-    if (nt <= 0 || eid < 0 || eid >= a.num_experts || t0 < 0 || t0 >= a.out_rows) return;
-    mrows = min(min(nt, MT * 16), a.out_rows - t0);   // rows past 16 MT are not computed
-  }
-  if (!GRP && a.msplit > 1) {
-    // The workgroups of a row block sit 8 apart: workgroups are dealt to the 8 XCDs in turn, so
-    // the block's weights come from HBM once and from that XCD's L2 afterwards.
-    const int grp = blockIdx.x / (8 * a.msplit), rem = blockIdx.x - grp * 8 * a.msplit;
-    m0 = (rem >> 3) * (MT * 16);
-    tile = grp * 8 + (rem & 7);
-    if (tile >= a.tiles_total || m0 >= a.M) return;
-  }
   int mat = 0;
 #pragma unroll
   for (int i = 0; i + 1 < kMaxMat; ++i) {
@@ -563,6 +541,55 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
       }
     }
   }
+}
+
+template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false, bool GRP = false>
+__global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
+  int tile = blockIdx.x;
+  int m0 = 0;                                         // first row of x of this workgroup
+  int eid = 0, t0 = 0, mrows = 0;
+  if constexpr (GRP) {
+    // workgroups are dealt to the 8 XCDs in turn: chunk c runs on XCD c % 8, so its rows of x enter one L2
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int rnd = slot / a.tiles_total;
+    const int cid = rnd * 8 + xcd;
+    tile = slot - rnd * a.tiles_total;
+    if (cid >= a.num_chunks) return;
+    eid = a.chunks[3 * cid];
+    t0 = a.chunks[3 * cid + 1];
+    const int nt = a.chunks[3 * cid + 2];
+    if (nt <= 0 || eid < 0 || eid >= a.num_experts || t0 < 0 || t0 >= a.out_rows) return;
+    mrows = min(min(nt, MT * 16), a.out_rows - t0);   // rows past 16 MT are not computed
+  }
+  if (!GRP && a.msplit > 1) {
+    // The workgroups of a row block sit 8 apart: workgroups are dealt to the 8 XCDs in turn, so
+    // the block's weights come from HBM once and from that XCD's L2 afterwards.
+    const int grp = blockIdx.x / (8 * a.msplit), rem = blockIdx.x - grp * 8 * a.msplit;
+    m0 = (rem >> 3) * (MT * 16);
+    tile = grp * 8 + (rem & 7);
+    if (tile >= a.tiles_total || m0 >= a.M) return;
+  }
+  skinny_body<Act, FMT, SC, MT, RT, NW, UN, SL, GRP>(a, tile, m0, eid, t0, mrows);
+}
+
+// Grouped launch whose workgroups pick the number of 16-row tiles of x from their chunk's rows (up to 64):
+// a chunk of 20 rows costs two tiles' loads, LDS traffic and MFMAs instead of four.  One granule in flight.
+template <class Act, int FMT, int RT, int NW, bool SL>
+__global__ __launch_bounds__(NW * 64) void skinny_grouped_kernel(const SkinnyArgs a) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int rnd = slot / a.tiles_total;
+  const int cid = rnd * 8 + xcd;
+  const int tile = slot - rnd * a.tiles_total;
+  if (cid >= a.num_chunks) return;
+  const int eid = a.chunks[3 * cid];
+  const int t0 = a.chunks[3 * cid + 1];
+  const int nt = a.chunks[3 * cid + 2];
+  if (nt <= 0 || eid < 0 || eid >= a.num_experts || t0 < 0 || t0 >= a.out_rows) return;
+  const int mrows = min(min(nt, 64), a.out_rows - t0);  // rows past 64 are not computed
+  if (mrows <= 16) skinny_body<Act, FMT, 0, 1, RT, NW, 1, SL, true>(a, tile, 0, eid, t0, mrows);
+  else if (mrows <= 32) skinny_body<Act, FMT, 0, 2, RT, NW, 1, SL, true>(a, tile, 0, eid, t0, mrows);
+  else if (mrows <= 48) skinny_body<Act, FMT, 0, 3, RT, NW, 1, SL, true>(a, tile, 0, eid, t0, mrows);
+  else skinny_body<Act, FMT, 0, 4, RT, NW, 1, SL, true>(a, tile, 0, eid, t0, mrows);
 }
 
 // Bytes of the LDS scale tables of an SL instantiation (0: the format has none).
