@@ -127,3 +127,31 @@ def test_graph_q4k_gemv(ops, dev):
     xd = x.to(dev)
     out = torch.empty(1, 640, dtype=torch.float16, device=dev)
     _check_graph(dev, lambda: s.esimd_gemv_q4_k(xd, ql, sc, mn, out), [out])
+
+
+def test_graph_grouped_gguf_moe(ops, dev):
+    # the verify-step use of the grouped module (fixed [E, 3] chunk table, 16-row tiles) is what the caller
+    # captures (sglang/patches/sglang_for_multi_arc.patch:2850-2870); the 64-row form as well
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    E, H, I, T, k = 8, 512, 128, 12, 2
+    g = torch.Generator().manual_seed(41)
+    u8 = lambda *sh: torch.randint(0, 256, sh, dtype=torch.uint8, generator=g).to(dev)
+    f16 = lambda hi, *sh: (torch.rand(*sh, generator=g) * hi).half().to(dev)
+    up = [u8(E, I, H // 2), f16(0.01, E, I, H // 32), f16(0.005, E, I, H // 32)] * 2
+    down = [u8(E, H, I // 2), u8(E, H, I // 4), f16(0.002, E, H, I // 16)]
+    x = (torch.randn(T, H, generator=g) * 0.1).half().to(dev)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    flat = ids.reshape(-1)
+    order = torch.sort(flat, stable=True).indices
+    tok = torch.arange(T).repeat_interleave(k)[order].to(torch.int32).to(dev)
+    counts = torch.bincount(flat, minlength=E)
+    chunks = torch.stack([torch.arange(E), torch.cumsum(counts, 0) - counts, counts], 1).to(torch.int32).to(dev)
+    P = T * k
+    gate_buf = torch.zeros(P, 2 * I, dtype=torch.float16, device=dev)
+    out = torch.zeros(P, H, dtype=torch.float16, device=dev)
+    inter = (torch.randn(P, I, generator=g) * 0.1).half().to(dev)
+    for smallm in (True, False):
+        def run():
+            mg.moe_up_q4k_ggemv(x, *up, gate_buf, chunks, H, I, tok, smallm=smallm)
+            mg.moe_down_q6k_ggemv(inter, *down, out, chunks, I, H, smallm=smallm)
+        _check_graph(dev, run, [gate_buf, out])
