@@ -439,6 +439,37 @@ def test_cfg4_q4k(ops, dev, M):
     assert b < (0.6 if M == 1 else 0.1)
 
 
+@pytest.mark.parametrize("M,K,N", [(64, 4096, 40), (48, 2560, 100), (16, 5120, 64), (8, 1024, 48)])
+def test_q4k_mfma_dequant_bit_exact(ops, dev, M, K, N):
+    """One-hot activation rows turn the matrix-core kernels' outputs into single dequantized weights, so the
+    in-register dequantization is compared bit for bit with the oracle's fp16(fp16(nibble * scale) - min) —
+    with scales of ordinary size and, in some rows, of 64 and more (d = 4: products beyond the usual range);
+    the positions k walk the lane slots of several 128-wide granules."""
+    _, s = ops
+    rng = np.random.default_rng(K + N)
+    nsb = K // 256
+    q = rng.integers(0, 16, size=(N, nsb, 256), dtype=np.uint8)
+    sc6 = rng.integers(0, 64, size=(N, nsb, 8), dtype=np.uint8)
+    mn6 = rng.integers(0, 64, size=(N, nsb, 8), dtype=np.uint8)
+    d = rng.uniform(0.001, 0.01, size=(N, nsb)).astype(np.float16)
+    d[::5] = np.float16(4.0)                              # scales up to 252
+    d[3::7, ::2] = np.float16(1.0)                        # 64 and more for sc6 = 63 .. some sub-blocks only
+    dmin = rng.uniform(0.0, 0.005, size=(N, nsb)).astype(np.float16)
+    raw = O.q4k_build_raw(q, sc6, mn6, d, dmin)
+    ql, sc, mn = O.q4k_repack(raw)
+    w = torch.from_numpy(O.q4k_dequant(ql, sc, mn))       # [N, K] fp16
+    assert float(torch.from_numpy(sc.astype(np.float32)).abs().max()) >= 64
+    W = [torch.from_numpy(a).to(dev) for a in (ql, sc, mn)]
+    for base in (0, 77, K - 4 * M):
+        ks = (base + 3 * torch.arange(M)) % K                   # distinct k per row
+        x = torch.zeros(M, K, dtype=torch.float16)
+        x[torch.arange(M), ks] = 1.0
+        out = torch.empty(M, N, dtype=torch.float16, device=dev)
+        s.esimd_gemv_q4_k(x.to(dev), *W, out)
+        want = w[:, ks].t().contiguous()
+        assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16)), (M, K, N, base)
+
+
 @pytest.mark.parametrize("M,K,N", [(65, 512, 130), (200, 2048, 1000), (2048, 5120, 5120), (1800, 256, 6144)])
 def test_q4k_prefill_tiled_gemm(ops, dev, M, K, N):
     # M > 64: the tiled matrix-core GEMM with the two-rounding Q4_K dequantization staged through LDS
