@@ -439,7 +439,44 @@ def test_cfg4_q4k(ops, dev, M):
     assert b < (0.6 if M == 1 else 0.1)
 
 
-@pytest.mark.parametrize("M,K,N", [(64, 4096, 40), (48, 2560, 100), (16, 5120, 64), (8, 1024, 48)])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("fmt", ["int4", "int4zp", "pern", "pert", "block"])
+@pytest.mark.parametrize("M,K", [(1, 1024), (2, 4096), (4, 1024), (8, 4096), (32, 1024), (64, 4096), (64, 1024), (200, 1024)])
+def test_one_hot_activations_return_the_dequantized_weights(ops, dev, fmt, M, K, dt):
+    """With one 1.0 per activation row every output is a single weight, so each kernel family (row GEMV, K-sliced,
+    skinny, tiled GEMM) must return exactly the oracle's dequantized weight rounded to the activation type:
+    decode, scale / zero-point arithmetic and the output rounding are compared value for value (+0 == -0)."""
+    v, _ = ops
+    N = 128 if fmt == "block" else 72                          # the block quantizer of the oracle wants whole blocks
+    ks = (5 + 37 * torch.arange(M)) % K                        # 37 is coprime to K: distinct k per row
+    x = torch.zeros(M, K, dtype=dt)
+    x[torch.arange(M), ks] = 1.0
+    out = torch.empty(M, N, dtype=dt, device=dev)
+    if fmt.startswith("int4"):
+        _, packed, scale, zp = O.make_int4_case(1, K, N, seed=K + M, asym=fmt == "int4zp")
+        w = O.int4_dequant(packed, scale, out_dtype=dt, zp=zp)
+        if zp is None:
+            v.esimd_gemm_int4_pgrp(x.to(dev), packed.to(dev), scale.to(dev), out)
+        else:
+            v.esimd_gemm_int4_pgrp_zp(x.to(dev), packed.to(dev), scale.to(dev), zp.to(dev), out)
+    elif fmt == "block":
+        _, w8, sc = O.make_fp8_block_case(1, K, N, seed=K + M)
+        w = O.fp8_dequant_block(w8, sc).to(dt)
+        v.esimd_gemm_fp8_blockscale(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev), out, 128, 128)
+    else:
+        _, w8, sc = O.make_fp8_pern_case(1, K, N, seed=K + M)
+        if fmt == "pert":
+            sc = sc[:1].clone()
+            w = O.fp8_dequant_per_tensor(w8, sc).to(dt)
+            v.esimd_gemm_fp8_pert(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev), out)
+        else:
+            w = O.fp8_dequant_per_channel(w8, sc).to(dt)
+            v.esimd_gemv_fp8_pern(x.to(dev), w8.view(torch.float8_e4m3fn).to(dev), sc.to(dev), out, N, K)
+    want = w[:, ks].t().float()
+    assert torch.equal(out.cpu().float(), want)
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 4096, 40), (48, 2560, 100), (16, 5120, 64), (8, 1024, 48), (200, 2048, 100)])
 def test_q4k_mfma_dequant_bit_exact(ops, dev, M, K, N):
     """One-hot activation rows turn the matrix-core kernels' outputs into single dequantized weights, so the
     in-register dequantization is compared bit for bit with the oracle's fp16(fp16(nibble * scale) - min) —
@@ -468,6 +505,29 @@ def test_q4k_mfma_dequant_bit_exact(ops, dev, M, K, N):
         s.esimd_gemv_q4_k(x.to(dev), *W, out)
         want = w[:, ks].t().contiguous()
         assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16)), (M, K, N, base)
+
+
+@pytest.mark.parametrize("M,K", [(1, 5120), (2, 1024), (1, 14336)])
+def test_q4k_row_gemv_one_hot(ops, dev, M, K):
+    """The decode GEMV multiplies weights that are not rounded to fp16, like the reference's decode kernel (fp32
+    `d sc q - dmin m`, S/csrc/xpu/esimd_kernels/q4_k_GEMV.h:84-88): with one-hot activations its outputs are the
+    single rounding of fp32(nibble * scale - min), value for value."""
+    _, s = ops
+    N = 72
+    _, raw = O.make_q4k_case(1, K if K % 256 == 0 else (K + 255) // 256 * 256, N, seed=K + M)
+    ql, sc, mn = O.q4k_repack(raw)
+    nib = np.empty((N, ql.shape[1] * 2), dtype=np.float32)
+    nib[:, 0::2] = ql & 0xF
+    nib[:, 1::2] = ql >> 4
+    one = nib * np.repeat(sc.astype(np.float32), 32, 1) - np.repeat(mn.astype(np.float32), 32, 1)
+    wd = torch.from_numpy(one.astype(np.float16).astype(np.float32))
+    W = [torch.from_numpy(a).to(dev) for a in (ql, sc, mn)]
+    ks = (11 + 37 * torch.arange(M)) % K
+    x = torch.zeros(M, K, dtype=torch.float16)
+    x[torch.arange(M), ks] = 1.0
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    s.esimd_gemv_q4_k(x.to(dev), *W, out)
+    assert torch.equal(out.cpu().float(), wd[:, ks].t())
 
 
 @pytest.mark.parametrize("M,K,N", [(65, 512, 130), (200, 2048, 1000), (2048, 5120, 5120), (1800, 256, 6144)])

@@ -229,6 +229,32 @@ def test_moe_gguf_routed_stages(ops, dev, T, E, k, H, I):
         assert O.max_rel_err(out.cpu(), ref) < TOL
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("M,K", [(1, 1024), (2, 4096), (4, 1024), (8, 1024), (16, 4096), (40, 2048), (64, 4096), (100, 1024)])
+def test_one_hot_activations_return_the_dequantized_weights(ops, dev, kind, M, K):
+    """With one 1.0 per activation row every output is a single weight: row GEMV, K-sliced and skinny kernels
+    must return exactly the oracle's dequantized fp16 weight (decode, high-bit planes, scale and min
+    arithmetic, output rounding), value for value.  The row GEMV (up to 4 rows for these formats) multiplies
+    weights that are not rounded to fp16, like the reference's decode kernels (fp32 `d sc q - dmin m`,
+    S/csrc/xpu/esimd_kernels/q4_k_GEMV.h:84-88): for Q5_K, the one format here with two roundings, its output
+    is the single rounding of fp32(v5 * scale - min)."""
+    _, s = ops
+    N = 72
+    raw = _raw_case(kind, N, K, seed=3 * M + K)
+    rep = _repack_oracle(kind, raw)
+    wd = torch.from_numpy(_dequant_oracle(kind, rep).astype(np.float32))
+    if kind == "q5_k" and M <= 4:
+        v5, sc, mn = G.q5k_elem(raw)
+        one = v5.astype(np.float32) * np.repeat(sc.astype(np.float32), 32, 1) - np.repeat(mn.astype(np.float32), 32, 1)
+        wd = torch.from_numpy(one.astype(np.float16).astype(np.float32))
+    ks = (9 + 37 * torch.arange(M)) % K                        # 37 is coprime to K: distinct k per row
+    x = torch.zeros(M, K, dtype=torch.float16)
+    x[torch.arange(M), ks] = 1.0
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    _gemv(s, kind, x.to(dev), [_t(a).to(dev) for a in rep], out)
+    assert torch.equal(out.cpu().float(), wd[:, ks].t())
+
+
 @pytest.mark.parametrize("name,kind", [("esimd_gemm_q4_0", "q4_0"), ("esimd_gemv_q8_0_m", "q8_0"), ("esimd_gemv_q6_k_m", "q6_k")])
 def test_small_m_variants(ops, dev, name, kind):
     _, s = ops
