@@ -574,3 +574,38 @@ def test_moe_grouped_prefill_flow(ops, dev):
             h = (torch.nn.functional.silu(gu[0].half().float()) * gu[1].half().float()).half().float()
             want[t] += float(tw[t, j]) * (h @ wd[e].t()).half().float()
     assert O.max_rel_err(final.cpu(), want) < 2 * TOL      # three fp16 roundings on the way
+
+
+@pytest.mark.parametrize("smallm", [False, True])
+def test_moe_grouped_one_hot_rows_return_the_experts_weights(ops, dev, smallm):
+    """One 1.0 per row of x: every output of the grouped launches is a single dequantized weight of the chunk's
+    expert — Q4_K gate / up, Q5_K and Q6_K down with element-order high bits — compared value for value."""
+    from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
+    E, H, I, T, k = 6, 768, 512, 40, 2
+    g = torch.Generator().manual_seed(77)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    chunks, tok_sorted, _ = _expert_chunks(ids, E, 16 if smallm else 64, fixed=False)
+    P = T * k
+    e_of = torch.empty(P, dtype=torch.long)
+    for e, t0, nt in chunks.tolist():
+        e_of[t0:t0 + nt] = e
+    # up: x [T, H] one-hot per token, gathered through the token list
+    kx = (3 + 37 * torch.arange(T)) % H
+    x = torch.zeros(T, H, dtype=torch.float16)
+    x[torch.arange(T), kx] = 1.0
+    reps, deq = _q4k_expert_stacks(E, I, H, (61, 62), torch.arange(E), dev)
+    buf = torch.zeros(P, 2 * I, dtype=torch.float16, device=dev)
+    mg.moe_up_q4k_ggemv(x.to(dev), *reps[0], *reps[1], buf, chunks.to(dev), H, I, tok_sorted.to(dev), smallm=smallm)
+    kk = kx[tok_sorted.long()]
+    want = torch.cat([deq[0][e_of, :, kk], deq[1][e_of, :, kk]], 1)
+    assert torch.equal(buf.cpu().float(), want)
+    # down: the intermediate [P, I] one-hot per route
+    ki = (7 + 37 * torch.arange(P)) % I
+    inter = torch.zeros(P, I, dtype=torch.float16)
+    inter[torch.arange(P), ki] = 1.0
+    for kind in ("q5_k", "q6_k"):
+        args, wd = _down_stack(kind, E, H, I, 63, torch.arange(E), dev)
+        out = torch.zeros(P, H, dtype=torch.float16, device=dev)
+        fn = mg.moe_down_q5k_ggemv if kind == "q5_k" else mg.moe_down_q6k_ggemv
+        fn(inter.to(dev), *args, out, chunks.to(dev), I, H, smallm=smallm)
+        assert torch.equal(out.cpu().float(), wd[e_of, :, ki]), kind
