@@ -285,6 +285,28 @@ def test_moe_gemm_all_e4m3_codes_exact(v, dev, total):
         assert actual[0x80].item() == 0.0
 
 
+@pytest.mark.parametrize("counts", [[0, 5, 0, 70, 1, 16, 17, 0], [33, 40, 27, 36], [300, 0, 129, 257]])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_moe_gemm_one_hot_rows_return_the_experts_weights(v, dev, counts, dt):
+    """One 1.0 per activation row: every output of the grouped w8a16 GEMM is a single block-scaled weight of the
+    row's expert rounded to the activation type — the streaming kernel (few rows per expert) and the grouped
+    tiled GEMM (96 and more on average), value for value."""
+    E, N, K = len(counts), 256, 512
+    total = sum(counts)
+    st = torch.zeros(E + 1, dtype=torch.int32)
+    st[1:] = torch.tensor(counts).cumsum(0)
+    g = torch.Generator().manual_seed(total)
+    w8, ws = O.fp8_quantize_block(torch.randn(E, N, K, generator=g) * 0.05)
+    dw = O.fp8_dequant_block(w8, ws).to(dt).float()           # [E, N, K]
+    ks = (5 + 37 * torch.arange(total)) % K
+    x = torch.zeros(total, K, dtype=dt)
+    x[torch.arange(total), ks] = 1.0
+    e_of = torch.repeat_interleave(torch.arange(E), torch.tensor(counts))
+    out = torch.full((total, N), float("nan"), dtype=dt, device=dev)
+    v.esimd_moe_gemm_fp8_blockscale(x.to(dev), w8.to(dev), ws.to(dev), out, st.to(dev), N, K, E)
+    assert torch.equal(out.cpu().float(), dw[e_of, :, ks])
+
+
 @pytest.mark.parametrize("counts", [[0, 5, 0, 70, 1, 16, 17, 0], [130, 0, 0, 3]])
 @pytest.mark.parametrize("a8", [False, True])
 def test_moe_gemm_skewed_experts(v, dev, counts, a8):
