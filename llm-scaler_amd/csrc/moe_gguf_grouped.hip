@@ -35,7 +35,7 @@ void launch_grouped_one(SkinnyArgs a, hipStream_t st) {
       raised = lds;
     }
   }
-  const long long wgs = (long long)((a.num_chunks + 7) / 8) * 8 * a.tiles_total;
+  const long long wgs = (long long)((a.num_chunks + 8 * a.cgroup - 1) / (8 * a.cgroup)) * 8 * a.cgroup * a.tiles_total;
   hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(NW * 64), lds, st, a);
 }
 
@@ -83,7 +83,11 @@ int mi_moe_gguf_grouped(int fmt, const void* x, int x_rows, const int32_t* tok_i
     a.tiles[i] = (N + 63) / 64;
     a.tiles_total += a.tiles[i];
   }
-  if ((long long)((num_chunks + 7) / 8) * 8 * a.tiles_total >= (1ll << 31)) return MI_ERR_SHAPE;
+  // chunks of one expert follow each other in the caller's list: with about g chunks of 64 rows per expert,
+  // groups of g consecutive chunks share an XCD, so an expert's row block is fetched into one L2 once
+  const long long per_expert = (long long)out_rows / ((long long)64 * num_experts);
+  a.cgroup = rows16 ? 1 : (int)(per_expert < 1 ? 1 : (per_expert > 8 ? 8 : per_expert));
+  if ((long long)((num_chunks + 8 * a.cgroup - 1) / (8 * a.cgroup)) * 8 * a.cgroup * a.tiles_total >= (1ll << 31)) return MI_ERR_SHAPE;
   hipStream_t st = (hipStream_t)stream;
   // 7 / 8: Q5_K / Q6_K with the high bits in element order.  Small workgroups (two or four wavefronts splitting
   // K, one granule in flight each) so that several share a CU and overlap their load -> LDS -> MFMA chains:

@@ -54,6 +54,7 @@ struct SkinnyArgs {
   const int32_t* chunks;
   const int32_t* tok_ids;
   int num_chunks, num_experts, x_rows, out_rows;
+  int cgroup;                 // consecutive chunks that share an XCD (>= 1)
   long long out_stride, w_stride, s_stride, z_stride, h_stride;
 };
 
@@ -543,17 +544,25 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, int tile, const
   }
 }
 
+// Grouped launches: which chunk and row block a workgroup takes.  Workgroups are dealt to the 8 XCDs in turn;
+// an XCD walks groups of `cgroup` consecutive chunks (the caller lists an expert's chunks one after the other)
+// row block by row block, so that a chunk's rows of x enter one L2 and the chunks of a group find their
+// expert's row block there.
+__device__ __forceinline__ int grouped_chunk_of(const SkinnyArgs& a, int& tile) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int per = a.cgroup * a.tiles_total;
+  const int unit = slot / per, r = slot - unit * per;
+  tile = r / a.cgroup;
+  return (unit * 8 + xcd) * a.cgroup + (r - tile * a.cgroup);
+}
+
 template <class Act, int FMT, int SC, int MT, int RT, int NW, int UN, bool SL = false, bool GRP = false>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
   int tile = blockIdx.x;
   int m0 = 0;                                         // first row of x of this workgroup
   int eid = 0, t0 = 0, mrows = 0;
   if constexpr (GRP) {
-    // workgroups are dealt to the 8 XCDs in turn: chunk c runs on XCD c % 8, so its rows of x enter one L2
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int rnd = slot / a.tiles_total;
-    const int cid = rnd * 8 + xcd;
-    tile = slot - rnd * a.tiles_total;
+    const int cid = grouped_chunk_of(a, tile);
     if (cid >= a.num_chunks) return;
     eid = a.chunks[3 * cid];
     t0 = a.chunks[3 * cid + 1];
@@ -576,10 +585,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(const SkinnyArgs a) {
 // a chunk of 20 rows costs two tiles' loads, LDS traffic and MFMAs instead of four.  One granule in flight.
 template <class Act, int FMT, int RT, int NW, bool SL>
 __global__ __launch_bounds__(NW * 64) void skinny_grouped_kernel(const SkinnyArgs a) {
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int rnd = slot / a.tiles_total;
-  const int cid = rnd * 8 + xcd;
-  const int tile = slot - rnd * a.tiles_total;
+  int tile;
+  const int cid = grouped_chunk_of(a, tile);
   if (cid >= a.num_chunks) return;
   const int eid = a.chunks[3 * cid];
   const int t0 = a.chunks[3 * cid + 1];
