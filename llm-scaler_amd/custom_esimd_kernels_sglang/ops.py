@@ -142,6 +142,86 @@ def esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hi
     return _ops.esimd_moe_down_q6k(inter, ql, qh, sc, sel, topk_w, out_partial, n_tokens, hidden, intermediate, top_k)
 
 
+# The names below are what the reference's SGLang package re-exports besides the GGUF ones
+# (S/python/custom_esimd_kernels_sglang/__init__.py:69-147) and this library registers under
+# torch.ops.custom_esimd_kernels_sglang: the fused FP8 GEMVs, the norm + GEMV family and the MoE helpers the
+# patched GGUF path takes through its name lookup (esimd_moe_silu_mul, esimd_moe_gather;
+# sglang/patches/sglang_for_multi_arc.patch:2134-2138).  Same argument order as the reference's wrappers
+# (S/python/custom_esimd_kernels_sglang/ops.py:26-90, 421-600, 638-735).
+def esimd_gemv_fp8_pern_fused2(input, w0, s0, o0, N0, w1, s1, o1, N1, K):
+    return _ops.esimd_gemv_fp8_pern_fused2(input, w0, s0, o0, N0, w1, s1, o1, N1, K)
+
+
+def esimd_gemv_fp8_pern_fused3(input, w0, s0, o0, N0, w1, s1, o1, N1, w2, s2, o2, N2, K):
+    return _ops.esimd_gemv_fp8_pern_fused3(input, w0, s0, o0, N0, w1, s1, o1, N1, w2, s2, o2, N2, K)
+
+
+def esimd_gemv_fp8_pert_fused2(input, w0, s0, o0, w1, s1, o1):
+    return _ops.esimd_gemv_fp8_pert_fused2(input, w0, s0, o0, w1, s1, o1)
+
+
+def esimd_gemv_fp8_pert_fused3(input, w0, s0, o0, w1, s1, o1, w2, s2, o2):
+    return _ops.esimd_gemv_fp8_pert_fused3(input, w0, s0, o0, w1, s1, o1, w2, s2, o2)
+
+
+def esimd_fused_add_rms_norm(hidden_states, residual, weight, eps):
+    """residual = hidden_states + residual (in place); hidden_states = rmsnorm(residual) * weight."""
+    return _ops.esimd_fused_add_rms_norm(hidden_states, residual, weight, eps)
+
+
+def esimd_rms_norm_gated(x, z, weight, output, eps):
+    """output = rmsnorm(x) * weight * silu(z); x, z [rows, V], weight [V]."""
+    return _ops.esimd_rms_norm_gated(x, z, weight, output, eps)
+
+
+def esimd_fused_add_rms_norm_batched(hidden_states, residual, weight, eps):
+    return _ops.esimd_fused_add_rms_norm_batched(hidden_states, residual, weight, eps)
+
+
+def esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
+                                    normed_out, eps):
+    return _ops.esimd_resadd_norm_gemv_fp8_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale,
+                                                output, normed_out, eps)
+
+
+def esimd_resadd_norm_gemv_int4_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale, output,
+                                     normed_out, eps):
+    return _ops.esimd_resadd_norm_gemv_int4_pert(hidden_states, residual, norm_weight, gemv_weight, gemv_scale,
+                                                 output, normed_out, eps)
+
+
+def esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps):
+    return _ops.esimd_resadd_norm_gemv2_fp8_pert(hidden_states, residual, norm_weight, w0, s0, o0, w1, s1, o1, eps)
+
+
+def esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    return _ops.esimd_norm_gemv_fp8_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)
+
+
+def esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps):
+    return _ops.esimd_norm_gemv_int4_pert(x, z, norm_weight, gemv_weight, gemv_scale, output, HV, V, eps)
+
+
+def esimd_moe_topk(router_logits, top_values, top_indices, T):
+    """router_logits [T, E], top_values [T, K] (output, logits dtype), top_indices [T, K] int32 (output)."""
+    return _ops.esimd_moe_topk(router_logits, top_values, top_indices, T)
+
+
+def esimd_moe_scatter_fused(hidden_states, top_values, top_indices, scattered_hidden, scattered_weights,
+                            topk_ids, expert_start, max_tokens_out, K, topk, T, num_experts):
+    return _ops.esimd_moe_scatter_fused(hidden_states, top_values, top_indices, scattered_hidden,
+                                        scattered_weights, topk_ids, expert_start, max_tokens_out,
+                                        K, topk, T, num_experts)
+
+
+def esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows):
+    return _ops.esimd_moe_silu_mul(input, output, N_gate_up, N_half, total_rows)
+
+
+def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T):
+    return _ops.esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T)
+
+
 # Imported at module level by the patched SGLang's XPU attention backend
 # (sglang/patches/sglang_for_multi_arc.patch:684); paged attention is outside the quantized-linear path:
 # the name exists so that module imports, and raises when called.

@@ -13,6 +13,13 @@ Two kinds of site are recorded, each with the patch line it stands on:
     in the patches -- "guarded" when an enclosing block is a `try:`.
 An unguarded name that the package lacks breaks the caller's import; a guarded one makes the
 caller fall back.  tests/test_capi_cpu.py holds the package to that.
+
+Also recorded, as plain name lists:
+  * "sglang_package_exports": the `_EXPORTS` list of the reference's SGLang package
+    (sglang/custom-esimd-kernels/python/custom_esimd_kernels_sglang/__init__.py), the module-level
+    names it re-exports from its ops.py when their extension is built;
+  * "imp_kernels_names": the names the patched SGLang takes through its `_imp_kernels((...))` helper
+    (sglang package first, vLLM package second, else None; sglang_for_multi_arc.patch:2077-2140).
 """
 import json
 import os
@@ -111,6 +118,19 @@ def main():
                 result["imports"].append({
                     "patch": which, "line": no, "package": m.group(1), "module": m.group(2),
                     "names": [], "guarded": in_try(lines, i)})
+    init = open(os.path.join(REF, "sglang/custom-esimd-kernels/python/custom_esimd_kernels_sglang/__init__.py")).read()
+    block = init[init.index("_EXPORTS = ["):init.index("]", init.index("_EXPORTS = ["))]
+    result["sglang_package_exports"] = re.findall(r'"([A-Za-z_]\w*)"', block)
+    imp = set()
+    for _, _, text in added_lines(os.path.join(REF, PATCHES["sglang"])):
+        if "_imp_kernels(" in text and "def _imp_kernels" not in text:
+            imp.update(re.findall(r'"([A-Za-z_]\w*)"', text))
+    # multi-line calls: the tuple continues on the next line
+    lines = [t for _, _, t in added_lines(os.path.join(REF, PATCHES["sglang"]))]
+    for i, t in enumerate(lines):
+        if t.rstrip().endswith("_imp_kernels("):
+            imp.update(re.findall(r'"([A-Za-z_]\w*)"', lines[i + 1]))
+    result["imp_kernels_names"] = sorted(imp)
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "esimd_import_names.json")
     with open(out, "w") as f:
         json.dump(result, f, indent=1, sort_keys=True)

@@ -345,6 +345,27 @@ def test_patch_import_sites_resolve():
                 assert found, s
 
 
+def test_sglang_package_exports_what_the_library_registers():
+    """The reference's SGLang package re-exports a fixed list of wrapper names
+    (S/python/custom_esimd_kernels_sglang/__init__.py:69-147); every one of them that this library registers
+    under torch.ops.custom_esimd_kernels_sglang must also be an attribute of the package — the patched GGUF path
+    looks names up on the package, not on torch.ops (`_imp_kernels`, sglang_for_multi_arc.patch:2077-2140) —
+    and every name that lookup takes must resolve there."""
+    import custom_esimd_kernels_sglang as s
+    ns = torch.ops.custom_esimd_kernels_sglang
+    exports = IMPORT_NAMES["sglang_package_exports"]
+    assert len(exports) >= 60
+    registered = [n for n in exports if hasattr(ns, n)]
+    assert len(registered) >= 30
+    guarded_elsewhere = {"esimd_qkv_split_norm_rope", "esimd_gdn_conv_fused", "esimd_gdn_conv_fused_seq"}
+    for n in registered:
+        if n in guarded_elsewhere:
+            continue                                  # raising placeholders of the vLLM namespace: must stay absent here
+        assert callable(getattr(s, n, None)), n
+    for n in IMPORT_NAMES["imp_kernels_names"]:
+        assert callable(getattr(s, n, None)), n
+
+
 def test_names_outside_the_path_raise_when_called():
     import custom_esimd_kernels_vllm as v
     import custom_esimd_kernels_sglang as s

@@ -543,9 +543,8 @@ def test_moe_grouped_prefill_flow(ops, dev):
     the same chain on the oracle's dequantized weights."""
     v, s = ops
     from custom_esimd_kernels_sglang import moe_grouped_gguf_xpu as mg
-    # the caller takes a name from the sglang package, else from the vLLM package (patch :2077-2087)
-    silu_mul = getattr(s, "esimd_moe_silu_mul", None) or v.esimd_moe_silu_mul
-    gather = getattr(s, "esimd_moe_gather", None) or v.esimd_moe_gather
+    # the caller takes these names from the sglang package first (patch :2077-2087, :2134-2138)
+    silu_mul, gather = s.esimd_moe_silu_mul, s.esimd_moe_gather
     T, E, k, H, I = 150, 8, 2, 512, 256
     g = torch.Generator().manual_seed(9)
     x = (torch.randn(T, H, generator=g) * 0.1).half()
