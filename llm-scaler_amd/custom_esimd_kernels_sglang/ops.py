@@ -222,6 +222,35 @@ def esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, t
     return _ops.esimd_moe_gather(moe_output, topk_ids, scattered_weights, final_hidden, K, topk, T)
 
 
+# MoE batch helpers of torch.ops.moe_ops that the reference package re-exports
+_moe = torch.ops.moe_ops
+def moe_router_forward(x, weight, scale):
+    """Router logits on per-tensor FP8 weights: x [n_tokens, hidden], weight [num_experts, hidden] fp8,
+    scale [num_experts] fp32 -> [n_tokens, num_experts] (S/python/custom_esimd_kernels_sglang/ops.py:926-938)."""
+    return _moe.moe_router_forward(x, weight, scale)
+
+
+def moe_batch_topk(logits, top_k, norm=True):
+    """(top_values [n_tokens, top_k], top_indices [n_tokens, top_k] int32) (S/python/custom_esimd_kernels_sglang/ops.py:941-953)."""
+    return _moe.moe_topk(logits, top_k, norm)
+
+
+def moe_accumulate(partials, top_k, num_shared_experts):
+    """Unweighted sum of each token's top_k + shared rows: partials [n_tokens * (top_k + shared), hidden]
+    -> [n_tokens, hidden] (S/python/custom_esimd_kernels_sglang/ops.py:1015-1025)."""
+    return _moe.moe_accumulate(partials, top_k, num_shared_experts)
+
+
+def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight, shared_gate_up_scale,
+                     down_weight, down_scale, shared_down_weight, shared_down_scale, shared_expert_gate_weight,
+                     top_k, num_shared_experts, n_routed_experts):
+    """The fused decode MoE forward on K-major per-tensor FP8 weights (torch.ops.moe_ops.moe_forward_full)."""
+    return _moe.moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_weight,
+                                 shared_gate_up_scale, down_weight, down_scale, shared_down_weight,
+                                 shared_down_scale, shared_expert_gate_weight, top_k, num_shared_experts,
+                                 n_routed_experts)
+
+
 # Imported at module level by the patched SGLang's XPU attention backend
 # (sglang/patches/sglang_for_multi_arc.patch:684); paged attention is outside the quantized-linear path:
 # the name exists so that module imports, and raises when called.

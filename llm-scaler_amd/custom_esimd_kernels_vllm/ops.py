@@ -246,6 +246,23 @@ def moe_forward_full(x, logits, gate_up_weight, gate_up_scale, shared_gate_up_we
                                  shared_down_scale, shared_expert_gate_weight, top_k, num_shared_experts,
                                  n_routed_experts)
 
+def moe_router_forward(x, weight, scale):
+    """Router logits on per-tensor FP8 weights: x [n_tokens, hidden], weight [num_experts, hidden] fp8,
+    scale [num_experts] fp32 -> [n_tokens, num_experts] (V/python/custom_esimd_kernels_vllm/ops.py:931-943)."""
+    return _moe.moe_router_forward(x, weight, scale)
+
+
+def moe_batch_topk(logits, top_k, norm=True):
+    """(top_values [n_tokens, top_k], top_indices [n_tokens, top_k] int32) (V/python/custom_esimd_kernels_vllm/ops.py:946-958)."""
+    return _moe.moe_topk(logits, top_k, norm)
+
+
+def moe_accumulate(partials, top_k, num_shared_experts):
+    """Unweighted sum of each token's top_k + shared rows: partials [n_tokens * (top_k + shared), hidden]
+    -> [n_tokens, hidden] (V/python/custom_esimd_kernels_vllm/ops.py:1020-1030)."""
+    return _moe.moe_accumulate(partials, top_k, num_shared_experts)
+
+
 
 def precompute_moe_route(topk_weights, topk_ids, num_experts):
     """Same contract as the reference helper: (sorted_rows, sorted_weights, rows_per_expert),

@@ -364,6 +364,12 @@ def test_sglang_package_exports_what_the_library_registers():
         assert callable(getattr(s, n, None)), n
     for n in IMPORT_NAMES["imp_kernels_names"]:
         assert callable(getattr(s, n, None)), n
+    # the MoE batch helpers of torch.ops.moe_ops that the list names and this library registers
+    import custom_esimd_kernels_vllm as v
+    for n, op in (("moe_router_forward", "moe_router_forward"), ("moe_batch_topk", "moe_topk"),
+                  ("moe_accumulate", "moe_accumulate"), ("moe_forward_full", "moe_forward_full")):
+        assert n in exports and hasattr(torch.ops.moe_ops, op)
+        assert callable(getattr(s, n, None)) and callable(getattr(v, n, None)), n
 
 
 def test_names_outside_the_path_raise_when_called():

@@ -1168,3 +1168,25 @@ def test_kmajor_out_of_range_expert_ids_contribute_zero(v, dev):
     inter = (torch.nn.functional.silu(gu[:I]) * gu[I:]).half().float()
     want = 0.5 * s2[1] * (inter @ O.e4m3_decode(w2[1].reshape(-1, H)).reshape(I, H))
     assert O.max_rel_err(out.cpu().float()[0], want) < TOL
+
+
+def test_package_level_moe_batch_helpers(v, dev):
+    """moe_router_forward / moe_batch_topk / moe_accumulate as attributes of both packages, the names the
+    reference packages re-export (V/python/custom_esimd_kernels_vllm/ops.py:931-1030): same results as the
+    torch.ops.moe_ops operators they call."""
+    import custom_esimd_kernels_sglang as s
+    T, E, H, k = 5, 64, 256, 4
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, H, generator=g).half().to(dev)
+    w8, sc = O.fp8_quantize_per_channel(torch.randn(E, H, generator=g) * 0.05)
+    sc1 = sc.mean().reshape(1).expand(E).contiguous()        # per-tensor: one value for every expert
+    for pkg in (v, s):
+        logits = pkg.moe_router_forward(x, w8.view(torch.float8_e4m3fn).to(dev), sc1.to(dev))
+        want = torch.ops.moe_ops.moe_router_forward(x, w8.view(torch.float8_e4m3fn).to(dev), sc1.to(dev))
+        assert torch.equal(logits, want) and logits.shape == (T, E)
+        tv, ti = pkg.moe_batch_topk(logits, k)
+        wv, wi = O.moe_topk(logits.cpu(), k)
+        assert torch.equal(ti.cpu(), wi.to(torch.int32)) and O.max_rel_err(tv.cpu(), wv) < TOL
+        parts = torch.randn(T * k, H, generator=g).half().to(dev)
+        acc = pkg.moe_accumulate(parts, k, 0)
+        assert O.max_rel_err(acc.cpu(), parts.cpu().float().view(T, k, H).sum(1)) < TOL
