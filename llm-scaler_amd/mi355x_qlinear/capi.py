@@ -78,15 +78,22 @@ def lib():
     return _lib
 
 
+def _device_ptr(t) -> int:
+    # a host address handed to a kernel is a GPU memory fault, not an error code: refuse it here
+    if not t.is_cuda:
+        raise RuntimeError(f"mi355x_qlinear: every tensor operand must live on a ROCm device, got one on {t.device}")
+    return t.data_ptr()
+
+
 def ptr(t):
     """Device pointer of a tensor (None -> NULL)."""
     if t is None:
         return None
-    return ctypes.c_void_p(t.data_ptr())
+    return ctypes.c_void_p(_device_ptr(t))
 
 
 def ptr_array(tensors):
-    arr = (ctypes.c_void_p * len(tensors))(*[0 if t is None else t.data_ptr() for t in tensors])
+    arr = (ctypes.c_void_p * len(tensors))(*[0 if t is None else _device_ptr(t) for t in tensors])
     return arr
 
 

@@ -279,6 +279,17 @@ def test_no_cpu_fallback():
         torch.ops.custom_esimd_kernels_vllm.esimd_gemv_int4(x, w, s, out)
 
 
+def test_host_tensors_are_refused_before_any_launch():
+    """A host address handed to a kernel would be a GPU memory fault rather than an error code: the pointer
+    helpers refuse tensors that are not on a ROCm device."""
+    t = torch.zeros(4, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="must live on a ROCm device"):
+        capi.ptr(t)
+    with pytest.raises(RuntimeError, match="must live on a ROCm device"):
+        capi.ptr_array([None, t])
+    assert capi.ptr(None) is None
+
+
 def test_meta_kernels_trace():
     x = torch.zeros(1, 128, dtype=torch.float16, device="meta")
     w = torch.zeros(16, 64, dtype=torch.uint8, device="meta")
