@@ -257,8 +257,6 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, int tile, const
           st.sc[u][t] = reinterpret_cast<const uint32_t*>(s32)[(size_t)(min(n0 + t * 16, N - 1) >> 7) * Kb + gic];
         }
         if constexpr (kHigh) {
-          // per 512-k tile the high bits of element b*64 + t' (Q5_K) / p*128 + t' (Q6_K) sit in
-          // byte t': this lane's 32 consecutive k are 32 consecutive bytes, one bit field
           if constexpr (kPlainH) {
             // element order: this lane's 32 consecutive k are 4 (Q5_K) or 8 (Q6_K) consecutive bytes
             const uint32_t ho = ok && n < nend ? (uint32_t)n * hrow + (uint32_t)gic * (kIsQ5K ? 16u : 32u) + (uint32_t)g * (kIsQ5K ? 4u : 8u) : kOOB;
@@ -269,6 +267,8 @@ __device__ __forceinline__ void skinny_body(const SkinnyArgs& a, int tile, const
               st.ha[u][t][0] = u32x4{two[0], two[1], 0u, 0u};
             }
           } else {
+          // per 512-k tile the high bits of element b*64 + t' (Q5_K) / p*128 + t' (Q6_K) sit in
+          // byte t': this lane's 32 consecutive k are 32 consecutive bytes, one bit field
           const uint32_t tile = (uint32_t)gic >> 2;
           const uint32_t within = kIsQ5K ? ((uint32_t)g & 1u) * 32u : (uint32_t)g * 32u;
           const uint32_t ho = ok && n < nend ? (uint32_t)n * hrow + tile * (kIsQ5K ? 64u : 128u) + within : kOOB;
